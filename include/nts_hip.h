@@ -1,0 +1,267 @@
+/*
+ * nts_hip.h -- C ABI of libntship.so, the gfx950 (MI355X, wave64) replacement for the
+ * single-GPU graph-operator kernels of NeutronBench.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers and sizes, receives the HIP stream
+ * explicitly, returns an int status (0 = NTS_OK) and never prints or exits.  There is no global
+ * mutable state: calls on different streams are independent and the library is re-entrant, which
+ * is what the reference's pipelined mini-batch loop needs (one Cuda_Stream per host thread,
+ * toolkits/GCN_GPU_NEIGHBOR.hpp:1350-1363).
+ *
+ * Conventions: indices are uint32 (VertexId_CUDA, cuda/cuda_type.h:21), values are fp32, labels
+ * are int64.  Dense operands are row-major and contiguous: a [n, F] tensor has row stride F.
+ * All pointers are device pointers unless a comment says "mapped host" (pinned host memory that
+ * the device reads through its device alias).
+ *
+ * Each declaration cites the reference interface it replaces (file:line relative to the
+ * NeutronBench source tree).
+ */
+#ifndef NTS_HIP_H
+#define NTS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* hipStream_t is `struct ihipStream_t *`; spelled out so that C callers need no HIP headers. */
+typedef struct ihipStream_t *nts_stream_t;
+
+enum nts_status {
+  NTS_OK = 0,
+  NTS_ERR_INVALID = 1,     /* null pointer, zero width, size overflow, inconsistent arguments */
+  NTS_ERR_HIP = 2,         /* a HIP runtime call failed; see nts_last_error() */
+  NTS_ERR_UNSUPPORTED = 3, /* argument combination the reference also rejects (tensor weights) */
+  NTS_ERR_NOMEM = 4        /* allocation failed */
+};
+
+/* Text of the last error raised on the calling thread ("" if none).  Replaces the reference's
+ * CHECK_CUDA_RESULT print-and-exit (cuda/ntsCUDAGraphOP.cu:11-20). */
+const char *nts_last_error(void);
+/* ABI version: bumped when a signature changes. */
+int nts_abi_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Memory, copies, streams
+ * ------------------------------------------------------------------------------------------- */
+
+/* cudaMallocGPU (cuda/ntsCUDAGraphOP.cu:45-55), allocate_gpu_buffer / allocate_gpu_edge /
+ * alloc_gpu_data (:603-629).  Sizes are bytes in size_t: the reference's `int size` element
+ * counts overflow above 2^31 elements. */
+int nts_malloc_device(void **ptr, size_t bytes);
+/* FreeBuffer / FreeEdge / free_gpu_data (:557-601).  NULL is accepted (the reference's ~sampCSC
+ * frees pointers it never initialised, core/coocsc.hpp:100-116). */
+int nts_free_device(void *ptr);
+/* allocate_gpu_buffer_async / allocate_gpu_edge_async (:631-651): stream-ordered allocation. */
+int nts_malloc_device_async(void **ptr, size_t bytes, nts_stream_t stream);
+/* FreeBufferAsync / FreeEdgeAsync (:566-592). */
+int nts_free_device_async(void *ptr, nts_stream_t stream);
+/* cudaMallocPinned (:34-43): page-locked host memory mapped into the device address space. */
+int nts_malloc_pinned_mapped(void **host_ptr, size_t bytes);
+/* ntsFreeHost (:548-555). */
+int nts_free_pinned(void *host_ptr);
+/* getDevicePointer (:23-32): device alias of a mapped pinned host allocation. */
+int nts_host_get_device_ptr(void **dev_ptr, void *host_ptr);
+/* move_data_in / move_edge_in / move_bytes_in (:487-522): blocking host-to-device copy; when
+ * `sync` is non-zero the whole device is synchronised afterwards as the reference does. */
+int nts_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, int sync);
+/* move_bytes_in_async (:524-531), Cuda_Stream::move_data_in / move_edge_in (:132-152). */
+int nts_memcpy_h2d_async(void *dst_dev, const void *src_host, size_t bytes, nts_stream_t stream);
+/* move_result_out (:476-485): blocking device-to-host copy. */
+int nts_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, int sync);
+/* Cuda_Stream::move_result_out (:121-130). */
+int nts_memcpy_d2h_async(void *dst_host, const void *src_dev, size_t bytes, nts_stream_t stream);
+/* zero_buffer (:594-601) / NtsScheduler::ZeroVarMem (core/NtsScheduler.hpp:321-336).  Done with a
+ * fill kernel on `stream` (safe under graph capture); does not synchronise. */
+int nts_memset_zero(void *dev_ptr, size_t bytes, nts_stream_t stream);
+/* Cuda_Stream::Cuda_Stream / ~Cuda_Stream / destory_Stream (:57-93). Default priority only. */
+int nts_stream_create(nts_stream_t *stream);
+int nts_stream_destroy(nts_stream_t stream);
+/* Cuda_Stream::CUDA_DEVICE_SYNCHRONIZE (:111-119) -- which is a *stream* synchronise. */
+int nts_stream_sync(nts_stream_t stream);
+/* cudaDeviceSynchronize as used by zero_buffer / move_* with sync=true. */
+int nts_device_sync(void);
+/* get_gpu_mem / show_gpu_mem (utils/cuda_memory.hpp:6-68): free and total device bytes. */
+int nts_mem_info(size_t *free_bytes, size_t *total_bytes);
+
+/* ---------------------------------------------------------------------------------------------
+ * Aggregation (weighted / unweighted SpMM as a row gather)
+ *
+ *   out[r, :] (+)= sum_{e in [offsets[r], offsets[r+1])} w[e] * in[indices[e] - index_base, :]
+ *
+ * Forward = CSC arrays (column_offset, row_indices, edge_weight_forward), rows = destinations.
+ * Backward = CSR arrays (row_offset, column_indices, edge_weight_backward), rows = sources: the
+ * gradient scatter is executed as the transposed gather, so no float atomics are used and the
+ * result is bit-reproducible run to run.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Cuda_Stream::Gather_By_Dst_From_Src[_Optim] and Gather_By_Src_From_Dst[_Optim]
+ * (cuda/ntsCUDA.hpp:124-143; launches cuda/ntsCUDAGraphOP.cu:186-292; kernels
+ * cuda/ntsCUDAFuseKernel.cuh:147-290, 327-487).
+ *   w           NULL = unweighted (with_weight=false)
+ *   index_base  src_start (forward) or dst_start (backward); 0 for sampled layers
+ *   accumulate  0: out = sum (out need not be initialised);  non-zero: out += sum, the
+ *               reference's semantics on a pre-zeroed output
+ * Works without any preprocessing; one wavefront (or a sub-wavefront group for narrow F) per row.
+ * Intended for sampled mini-batch layers whose degrees are bounded by the fanout. */
+int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t *offsets,
+                    const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
+                    uint32_t F, int accumulate, nts_stream_t stream);
+
+/* Degree-bucketed schedule for a fixed offsets array (full-graph chunks: CSC_segment_pinned,
+ * core/GraphSegment.h:54-133).  Rows are ordered by descending degree class; rows longer than
+ * `chunk_edges` are split into chunks whose partial sums are combined by a second kernel in a
+ * fixed order (deterministic).  chunk_edges = 0 selects the default.  The call reads `offsets`
+ * back to the host once and synchronises `stream`. */
+typedef struct nts_spmm_plan nts_spmm_plan_t;
+int nts_spmm_plan_create(nts_spmm_plan_t **plan, const uint32_t *offsets, uint32_t rows,
+                         uint32_t edges, uint32_t chunk_edges, nts_stream_t stream);
+int nts_spmm_plan_destroy(nts_spmm_plan_t *plan);
+/* Number of work items, split rows and partial-sum slots of a plan (for tests and reports). */
+int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows,
+                       uint32_t *partials);
+/* Grow the plan's partial-sum scratch so that widths up to F need no allocation later. */
+int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F);
+/* NtsScheduler::GatherByDstFromSrc / GatherBySrcFromDst on a full-graph chunk
+ * (core/NtsScheduler.hpp:146-178, 239-271; core/graph.hpp:3432-3478).  `offsets` must be the
+ * array the plan was built from.  A plan must not be used by two streams at the same time (its
+ * scratch is shared). */
+int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *w,
+                            const uint32_t *offsets, const uint32_t *indices, uint32_t index_base,
+                            uint32_t F, int accumulate, nts_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Edge <-> vertex data movement (GAT building blocks).  `co` = column_offset [Vd+1],
+ * `ri` = row_indices [E] (source row of each edge), edge tensors are [E, F] in CSC edge order.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Cuda_Stream::Scatter_Src_Mirror_to_Msg (cuda/ntsCUDA.hpp:145-147; kernel
+ * cuda/ntsCUDADistKernel.cuh:23-44): msg[e,:] = feat[mirror[ri[e]], :]; mirror NULL = identity. */
+int nts_scatter_src_to_edge(float *msg, const float *feat, const uint32_t *ri, const uint32_t *co,
+                            const uint32_t *mirror, uint32_t Vd, uint32_t F, nts_stream_t stream);
+/* Cuda_Stream::Scatter_Dst_to_Msg (cuda/ntsCUDA.hpp:153-155; kernel :65-79):
+ * msg[e,:] = feat[d,:] for e in CSC(d). */
+int nts_scatter_dst_to_edge(float *msg, const float *feat, const uint32_t *co, uint32_t Vd,
+                            uint32_t F, nts_stream_t stream);
+/* Cuda_Stream::Scatter_Grad_Back_To_Message (cuda/ntsCUDA.hpp:192-196; kernel
+ * cuda/ntsCUDAFuseKernel.cuh:492-506): msg_grad[e,:] += gout[d,:] for e in CSC(d). */
+int nts_scatter_grad_to_edge(float *msg_grad, const float *gout, const uint32_t *co, uint32_t Vd,
+                             uint32_t F, nts_stream_t stream);
+/* Cuda_Stream::Gather_Msg_to_Dst (cuda/ntsCUDA.hpp:157-159; kernel
+ * cuda/ntsCUDADistKernel.cuh:81-95): out[d,:] (+)= sum_{e in CSC(d)} msg[e,:], summed in edge
+ * order.  accumulate as in nts_spmm_gather. */
+int nts_gather_edge_to_dst(float *out, const float *msg, const uint32_t *co, uint32_t Vd,
+                           uint32_t F, int accumulate, nts_stream_t stream);
+/* Cuda_Stream::Gather_Msg_To_Src_Mirror (cuda/ntsCUDA.hpp:149-151; kernel :46-63), made
+ * deterministic: out[s,:] (+)= sum_{k in CSR(s)} msg[perm[k], :] where `ro` = row_offset [Vs+1]
+ * and perm[k] is the CSC edge id of the k-th CSR edge (see nts_csr_from_csc). */
+int nts_gather_edge_to_src(float *out, const float *msg, const uint32_t *ro, const uint32_t *perm,
+                           uint32_t Vs, uint32_t F, int accumulate, nts_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Edge softmax and fused GAT attention.  H = number of heads (columns); edge tensors [E, H].
+ * ------------------------------------------------------------------------------------------- */
+
+/* Cuda_Stream::Edge_Softmax_Forward_Block (cuda/ntsCUDA.hpp:161-163; kernel
+ * cuda/ntsCUDADistKernel.cuh:166-213) with the semantics of the CPU operator SingleEdgeSoftMax
+ * (core/ntsSingleCPUGraphOp.hpp:297-319): per destination segment and per column,
+ * y = softmax(x), computed with the segment maximum subtracted.  `y` is also the cache the
+ * backward needs.  Empty segments write nothing. */
+int nts_edge_softmax_fwd(float *y, const float *x, const uint32_t *co, uint32_t Vd, uint32_t H,
+                         nts_stream_t stream);
+/* Cuda_Stream::Edge_Softmax_Backward_Block (cuda/ntsCUDA.hpp:165-167; kernel :216-260;
+ * SingleEdgeSoftMax::backward core/ntsSingleCPUGraphOp.hpp:321-341):
+ * gx[e,h] = y[e,h] * (gy[e,h] - sum_{e' in seg} gy[e',h] * y[e',h]). */
+int nts_edge_softmax_bwd(float *gx, const float *gy, const float *y, const uint32_t *co,
+                         uint32_t Vd, uint32_t H, nts_stream_t stream);
+
+/* Fused attention forward.  Replaces the chain scatter-src / scatter-dst / sum / leaky_relu /
+ * edge-softmax of toolkits/GAT_CPU_DIST_OPTM.hpp:186-228 (algebraically equal to
+ * toolkits/GAT_CPU.hpp:178-204):
+ *   s[e,h]     = el[ri[e], h] + er[d, h]              for e in CSC(d)
+ *   alpha[e,:] = softmax over CSC(d) of leaky_relu(s[e,:], slope)
+ * el: [Vs, H] per-source scalars (a_l . h_src), er: [Vd, H] per-destination scalars. */
+int nts_gat_attention_fwd(float *alpha, const float *el, const float *er, const uint32_t *co,
+                          const uint32_t *ri, uint32_t Vd, uint32_t H, float slope,
+                          nts_stream_t stream);
+/* Fused attention backward, destination side: from galpha [E,H] and the cached alpha computes
+ *   gs[e,h]  = leaky'(s[e,h]) * alpha[e,h] * (galpha[e,h] - sum_seg galpha*alpha)   (edge tensor)
+ *   ger[d,h] = sum_{e in CSC(d)} gs[e,h]
+ * The source-side gradient gel[s,h] = sum_{e: src(e)=s} gs[e,h] is nts_gather_edge_to_src(gs). */
+int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const float *alpha,
+                          const float *el, const float *er, const uint32_t *co, const uint32_t *ri,
+                          uint32_t Vd, uint32_t H, float slope, nts_stream_t stream);
+
+/* Attention-weighted aggregation, multi-head (DistAggregateDstFuseWeight::forward,
+ * core/ntsDistCPUGraphOp.hpp:401-440; composition E_msg*alpha -> SingleCPUDstAggregateOp of
+ * toolkits/GAT_CPU.hpp:196-201):
+ *   out[r, h*Fh + f] (+)= sum_{e in [offsets[r], offsets[r+1])} alpha[eid(e), h] * in[indices[e], h*Fh + f]
+ * eid(e) = e when perm is NULL (forward over CSC) or perm[e] (backward over CSR, alpha kept in
+ * CSC edge order). */
+int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
+                          const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
+                          uint32_t H, uint32_t Fh, int accumulate, nts_stream_t stream);
+/* Gradient of the aggregation with respect to alpha (get_additional_grad of
+ * DistAggregateDstFuseWeight, core/ntsDistCPUGraphOp.hpp:442-472):
+ *   galpha[e,h] = < in[ri[e], h*Fh : (h+1)*Fh], gout[d, h*Fh : (h+1)*Fh] >   for e in CSC(d) */
+int nts_sddmm_heads(float *galpha, const float *in, const float *gout, const uint32_t *co,
+                    const uint32_t *ri, uint32_t Vd, uint32_t H, uint32_t Fh, nts_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Mini-batch assembly
+ * ------------------------------------------------------------------------------------------- */
+
+/* One kernel for the three feature-gather launches of the reference:
+ *   Cuda_Stream::zero_copy_feature_move_gpu        (cuda/ntsCUDA.hpp:168-169; kernel
+ *       cuda/ntsCUDATransferKernel.cuh:96-108)      sel = NULL, remap = NULL, table = mapped host
+ *   Cuda_Stream::zero_copy_feature_move_gpu_cache  (:170-172; kernel :153-166)   sel = local_idx
+ *   Cuda_Stream::gather_feature_from_gpu_cache     (:173-175; kernel :168-182)   sel = local_idx_cache,
+ *                                                                                  remap = cache_node_hashmap
+ * For k < n:  i = sel ? sel[k] : k;  g = row_ids[i];  if (remap) g = remap[g];
+ *             out[i, :] = table[g, :]          (bit-exact copy)
+ * `table`, `sel`, `remap` may be device memory or mapped host memory. */
+int nts_gather_rows_f32(float *out, const float *table, const uint32_t *row_ids,
+                        const uint32_t *sel, const uint32_t *remap, uint32_t n, uint32_t F,
+                        nts_stream_t stream);
+/* Device-side split-and-gather that needs no host loop: for every i < n,
+ *   slot = hashmap[row_ids[i]];  out[i,:] = (slot != 0xFFFFFFFF) ? cache[slot,:] : table[row_ids[i],:]
+ * Same result as the reference's host split (core/ntsSampler.hpp:424-469) followed by its two
+ * kernels.  hits, if not NULL, receives the number of cache hits (device uint32, zeroed by the call). */
+int nts_gather_rows_cached_f32(float *out, const float *table, const float *cache,
+                               const uint32_t *row_ids, const uint32_t *hashmap, uint32_t n,
+                               uint32_t F, uint32_t *hits, nts_stream_t stream);
+/* Cuda_Stream::global_copy_label_move_gpu (classes == 1) and global_copy_mulilabel_move_gpu
+ * (cuda/ntsCUDA.hpp:176-179; kernels cuda/ntsCUDATransferKernel.cuh:184-203):
+ * out[i, :] = table[ids[i], :] with `classes` int64 values per row. */
+int nts_gather_labels_i64(int64_t *out, const int64_t *table, const uint32_t *ids, uint32_t n,
+                          uint32_t classes, nts_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Sampled-layer index construction on the device (sampCSC, core/coocsc.hpp)
+ * ------------------------------------------------------------------------------------------- */
+
+/* sampCSC::generate_csr_from_csc (core/coocsc.hpp:243-309): stable counting sort of the CSC edges
+ * by local source.  Outputs ro [Vs+1], ci [E] (local destination of each CSR edge, ascending
+ * within a source) and, if perm is not NULL, perm [E] (CSC edge id of each CSR edge).
+ * `work` is caller-provided device scratch of nts_csr_from_csc_work_bytes(Vd, Vs, E) bytes.
+ * Bit-exact with the host algorithm. */
+size_t nts_csr_from_csc_work_bytes(uint32_t Vd, uint32_t Vs, uint32_t E);
+int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co,
+                     const uint32_t *ri, uint32_t Vd, uint32_t Vs, uint32_t E, void *work,
+                     nts_stream_t stream);
+/* sampCSC::update_degree + compute_weight_forward / compute_weight_backward
+ * (core/coocsc.hpp:136-216) with nts_norm_degree (core/ntsBaseOp.hpp:183-186) evaluated from the
+ * layer's own degrees: in_deg(d) = co[d+1]-co[d], out_deg(s) = ro[s+1]-ro[s],
+ *   ewf[e] = 1 / ((float)sqrt((double)out_deg(ri[e])) * (float)sqrt((double)in_deg(d)))  e in CSC(d)
+ *   ewb[k] = same value for the k-th CSR edge.
+ * Either output may be NULL.  Bit-exact with the host computation. */
+int nts_gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t *ri,
+                         const uint32_t *ro, const uint32_t *ci, uint32_t Vd, uint32_t Vs,
+                         nts_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NTS_HIP_H */

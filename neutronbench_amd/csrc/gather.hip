@@ -1,0 +1,166 @@
+// Mini-batch assembly kernels: feature-row gather from mapped pinned host memory and / or an HBM
+// feature cache, and label gather (replaces cuda/ntsCUDATransferKernel.cuh:96-203 and the
+// launchers cuda/ntsCUDAGraphOP.cu:379-447).  Pure copies: results are bit-exact.
+//
+// A group of G lanes (G chosen so that G*VEC*4 bytes covers a row with little idle width) moves
+// one row with 4/8/16-byte accesses; 64/G rows per wavefront.  Wide accesses matter most on the
+// zero-copy path, where every wave load becomes PCIe read requests.
+#include "common.hpp"
+
+namespace nts {
+namespace {
+
+constexpr uint32_t kMiss = 0xFFFFFFFFu;
+
+template <typename V, int G>
+__global__ __launch_bounds__(256) void gather_rows_kernel(V *__restrict__ out, const V *__restrict__ table,
+                                                          const uint32_t *__restrict__ row_ids,
+                                                          const uint32_t *__restrict__ sel,
+                                                          const uint32_t *__restrict__ remap, uint32_t n,
+                                                          uint32_t Fv) {
+  const uint32_t k = (blockIdx.x * blockDim.x + threadIdx.x) / G;
+  if (k >= n) return;
+  const uint32_t gl = threadIdx.x & (G - 1);
+  const uint32_t i = sel ? sel[k] : k;
+  uint32_t g = row_ids[i];
+  if (remap) g = remap[g];
+  const V *src = table + static_cast<size_t>(g) * Fv;
+  V *dst = out + static_cast<size_t>(i) * Fv;
+  for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
+}
+
+template <typename V, int G>
+__global__ __launch_bounds__(256) void gather_rows_cached_kernel(V *__restrict__ out, const V *__restrict__ table,
+                                                                 const V *__restrict__ cache,
+                                                                 const uint32_t *__restrict__ row_ids,
+                                                                 const uint32_t *__restrict__ hashmap, uint32_t n,
+                                                                 uint32_t Fv, uint32_t *__restrict__ hits) {
+  const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) / G;
+  if (i >= n) return;
+  const uint32_t gl = threadIdx.x & (G - 1);
+  const uint32_t g = row_ids[i];
+  const uint32_t slot = hashmap[g];
+  const bool hit = slot != kMiss;
+  const V *src = hit ? cache + static_cast<size_t>(slot) * Fv : table + static_cast<size_t>(g) * Fv;
+  V *dst = out + static_cast<size_t>(i) * Fv;
+  for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
+  if (hits && hit && gl == 0) atomicAdd(hits, 1u);  // integer count: order-independent
+}
+
+__global__ __launch_bounds__(256) void gather_labels_kernel(int64_t *__restrict__ out,
+                                                            const int64_t *__restrict__ table,
+                                                            const uint32_t *__restrict__ ids, uint32_t n,
+                                                            uint32_t classes) {
+  const size_t total = static_cast<size_t>(n) * classes;
+  for (size_t t = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
+       t += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const uint32_t i = static_cast<uint32_t>(t / classes);
+    const uint32_t c = static_cast<uint32_t>(t - static_cast<size_t>(i) * classes);
+    out[t] = table[static_cast<size_t>(ids[i]) * classes + c];
+  }
+}
+
+__global__ void zero_u32_kernel(uint32_t *p) { *p = 0u; }
+
+// Lanes per row for a row of Fv vector elements: the smallest power of two >= Fv, clamped to [4, 64].
+inline int group_for(uint32_t Fv) {
+  int g = 4;
+  while (g < 64 && static_cast<uint32_t>(g) < Fv) g <<= 1;
+  return g;
+}
+
+struct RowsArgs {
+  float *out;
+  const float *table;
+  const float *cache;  // null: plain gather
+  const uint32_t *row_ids;
+  const uint32_t *sel;
+  const uint32_t *remap;  // plain gather: optional remap; cached gather: hashmap
+  uint32_t n;
+  uint32_t F;
+  uint32_t *hits;
+  hipStream_t stream;
+};
+
+template <typename V, int G>
+void launch_rows(const RowsArgs &a, uint32_t Fv) {
+  const uint32_t per_block = 256 / G;
+  const dim3 grid(ceil_div(a.n, per_block));
+  if (a.cache)
+    hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), grid, dim3(256), 0, a.stream,
+                       reinterpret_cast<V *>(a.out), reinterpret_cast<const V *>(a.table),
+                       reinterpret_cast<const V *>(a.cache), a.row_ids, a.remap, a.n, Fv, a.hits);
+  else
+    hipLaunchKernelGGL((gather_rows_kernel<V, G>), grid, dim3(256), 0, a.stream, reinterpret_cast<V *>(a.out),
+                       reinterpret_cast<const V *>(a.table), a.row_ids, a.sel, a.remap, a.n, Fv);
+}
+
+template <typename V>
+void launch_rows_v(const RowsArgs &a, uint32_t Fv) {
+  switch (group_for(Fv)) {
+    case 4: launch_rows<V, 4>(a, Fv); break;
+    case 8: launch_rows<V, 8>(a, Fv); break;
+    case 16: launch_rows<V, 16>(a, Fv); break;
+    case 32: launch_rows<V, 32>(a, Fv); break;
+    default: launch_rows<V, 64>(a, Fv); break;
+  }
+}
+
+void launch_rows_any(const RowsArgs &a) {
+  const bool c16 = !a.cache || aligned_to(a.cache, 16);
+  const bool c8 = !a.cache || aligned_to(a.cache, 8);
+  if (a.F % 4 == 0 && aligned_to(a.out, 16) && aligned_to(a.table, 16) && c16) return launch_rows_v<float4>(a, a.F / 4);
+  if (a.F % 2 == 0 && aligned_to(a.out, 8) && aligned_to(a.table, 8) && c8) return launch_rows_v<float2>(a, a.F / 2);
+  return launch_rows_v<float>(a, a.F);
+}
+
+}  // namespace
+}  // namespace nts
+
+using namespace nts;
+
+extern "C" {
+
+int nts_gather_rows_f32(float *out, const float *table, const uint32_t *row_ids, const uint32_t *sel,
+                        const uint32_t *remap, uint32_t n, uint32_t F, nts_stream_t stream) {
+  if (F == 0) return fail(NTS_ERR_INVALID, "nts_gather_rows_f32: F is 0");
+  if (n == 0) return NTS_OK;
+  if (!out || !table || !row_ids) return fail(NTS_ERR_INVALID, "nts_gather_rows_f32: null pointer");
+  RowsArgs a{out, table, nullptr, row_ids, sel, remap, n, F, nullptr, stream};
+  launch_rows_any(a);
+  NTS_LAUNCH_CHECK("nts_gather_rows_f32");
+  return NTS_OK;
+}
+
+int nts_gather_rows_cached_f32(float *out, const float *table, const float *cache, const uint32_t *row_ids,
+                               const uint32_t *hashmap, uint32_t n, uint32_t F, uint32_t *hits,
+                               nts_stream_t stream) {
+  if (F == 0) return fail(NTS_ERR_INVALID, "nts_gather_rows_cached_f32: F is 0");
+  if (hits) {
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, stream, hits);
+    NTS_LAUNCH_CHECK("zero_u32_kernel");
+  }
+  if (n == 0) return NTS_OK;
+  if (!out || !table || !cache || !row_ids || !hashmap)
+    return fail(NTS_ERR_INVALID, "nts_gather_rows_cached_f32: null pointer");
+  RowsArgs a{out, table, cache, row_ids, nullptr, hashmap, n, F, hits, stream};
+  launch_rows_any(a);
+  NTS_LAUNCH_CHECK("nts_gather_rows_cached_f32");
+  return NTS_OK;
+}
+
+int nts_gather_labels_i64(int64_t *out, const int64_t *table, const uint32_t *ids, uint32_t n, uint32_t classes,
+                          nts_stream_t stream) {
+  if (classes == 0) return fail(NTS_ERR_INVALID, "nts_gather_labels_i64: classes is 0");
+  if (n == 0) return NTS_OK;
+  if (!out || !table || !ids) return fail(NTS_ERR_INVALID, "nts_gather_labels_i64: null pointer");
+  const size_t total = static_cast<size_t>(n) * classes;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(gather_labels_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, out, table, ids,
+                     n, classes);
+  NTS_LAUNCH_CHECK("nts_gather_labels_i64");
+  return NTS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,155 @@
+// Device-side construction of a sampled layer's transposed structure and GCN edge weights
+// (sampCSC::generate_csr_from_csc, update_degree, compute_weight_forward / backward:
+// core/coocsc.hpp:136-216, 243-309).  Integer results and weights are bit-exact with the host
+// algorithms; everything is order-independent, so the outputs are deterministic.
+#include <string.h>
+
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
+
+#include "common.hpp"
+
+namespace nts {
+namespace {
+
+// Largest r such that off[r] <= pos, searched in off[0 .. n] (off ascending, off[n] > pos).
+__device__ __forceinline__ uint32_t owner_of(const uint32_t *__restrict__ off, uint32_t n, uint32_t pos) {
+  uint32_t lo = 0, hi = n;  // answer in [lo, hi)
+  while (hi - lo > 1) {
+    const uint32_t mid = lo + (hi - lo) / 2;
+    if (off[mid] <= pos) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// ro[s] = number of sorted keys < s, for s in [0, Vs]; keys ascending, E of them.
+__global__ __launch_bounds__(256) void offsets_from_sorted_kernel(uint32_t *__restrict__ ro,
+                                                                  const uint32_t *__restrict__ keys, uint32_t Vs,
+                                                                  uint32_t E) {
+  const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s > Vs) return;
+  uint32_t lo = 0, hi = E;  // first position whose key >= s
+  while (lo < hi) {
+    const uint32_t mid = lo + (hi - lo) / 2;
+    if (keys[mid] < s) lo = mid + 1; else hi = mid;
+  }
+  ro[s] = lo;
+}
+
+// ci[k] = destination that owns CSC edge perm[k].
+__global__ __launch_bounds__(256) void dst_of_perm_kernel(uint32_t *__restrict__ ci, const uint32_t *__restrict__ perm,
+                                                          const uint32_t *__restrict__ co, uint32_t Vd, uint32_t E) {
+  const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= E) return;
+  ci[k] = owner_of(co, Vd, perm[k]);
+}
+
+// 1 / ((float)sqrt((double)out_deg) * (float)sqrt((double)in_deg)) with every step rounded to
+// nearest, as nts_norm_degree evaluates it on the host (core/ntsBaseOp.hpp:183-186).
+__device__ __forceinline__ float norm_weight(uint32_t out_deg, uint32_t in_deg) {
+  const float a = static_cast<float>(__dsqrt_rn(static_cast<double>(out_deg)));
+  const float b = static_cast<float>(__dsqrt_rn(static_cast<double>(in_deg)));
+  return __fdiv_rn(1.0f, __fmul_rn(a, b));
+}
+
+// which = 0: thread per CSC edge e, owner = destination, other end = ri[e] (a source).
+// which = 1: thread per CSR edge k, owner = source, other end = ci[k] (a destination).
+__global__ __launch_bounds__(256) void edge_weights_kernel(float *__restrict__ wout,
+                                                           const uint32_t *__restrict__ own_off, uint32_t n_own,
+                                                           const uint32_t *__restrict__ other_idx,
+                                                           const uint32_t *__restrict__ other_off, uint32_t E,
+                                                           int which) {
+  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= E) return;
+  const uint32_t o = owner_of(own_off, n_own, e);
+  const uint32_t own_deg = own_off[o + 1] - own_off[o];
+  const uint32_t t = other_idx[e];
+  const uint32_t other_deg = other_off[t + 1] - other_off[t];
+  wout[e] = which == 0 ? norm_weight(other_deg, own_deg) : norm_weight(own_deg, other_deg);
+}
+
+inline unsigned bits_for(uint32_t n) {  // bits needed to represent values in [0, n)
+  unsigned b = 1;
+  while (b < 32 && (1ull << b) < n) ++b;
+  return b;
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Scratch layout: [sorted keys: E u32][rocprim temporary storage].
+hipError_t sort_temp_bytes(uint32_t E, size_t *bytes) {
+  size_t tmp = 0;
+  uint32_t *nul = nullptr;
+  hipError_t err = rocprim::radix_sort_pairs(nullptr, tmp, nul, nul, rocprim::counting_iterator<uint32_t>(0u), nul,
+                                             E ? E : 1u, 0u, 32u, static_cast<hipStream_t>(nullptr), false);
+  *bytes = tmp;
+  return err;
+}
+
+}  // namespace
+}  // namespace nts
+
+using namespace nts;
+
+extern "C" {
+
+size_t nts_csr_from_csc_work_bytes(uint32_t Vd, uint32_t Vs, uint32_t E) {
+  (void)Vd;
+  (void)Vs;
+  size_t tmp = 0;
+  if (sort_temp_bytes(E, &tmp) != hipSuccess) return 0;
+  return align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256) + align_up(tmp, 256) + 256;
+}
+
+int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, uint32_t Vd,
+                     uint32_t Vs, uint32_t E, void *work, nts_stream_t stream) {
+  if (!ro) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: null ro");
+  if (E == 0) {
+    return nts_memset_zero(ro, (static_cast<size_t>(Vs) + 1) * sizeof(uint32_t), stream);
+  }
+  if (!ci || !co || !ri || !work) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: null pointer");
+  if (!aligned_to(work, 256)) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: work must be 256-byte aligned");
+  unsigned char *w = static_cast<unsigned char *>(work);
+  uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(w);
+  size_t keys_bytes = align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256);
+  // Without a caller buffer for perm, ci doubles as the sorted edge-id array and is rewritten in
+  // place by a second pass (each thread reads its own element before writing it).
+  uint32_t *perm_out = perm ? perm : ci;
+  size_t tmp = 0;
+  NTS_HIP_TRY(sort_temp_bytes(E, &tmp));
+  // Stable LSD radix sort of (local source, CSC edge id): edge ids stay ascending within a source,
+  // which is exactly the order the host counting sort produces.
+  NTS_HIP_TRY(rocprim::radix_sort_pairs(w + keys_bytes, tmp, ri, keys_sorted,
+                                        rocprim::counting_iterator<uint32_t>(0u), perm_out, E, 0u, bits_for(Vs),
+                                        stream, false));
+  hipLaunchKernelGGL(offsets_from_sorted_kernel, dim3(ceil_div(static_cast<uint64_t>(Vs) + 1, 256)), dim3(256), 0,
+                     stream, ro, keys_sorted, Vs, E);
+  NTS_LAUNCH_CHECK("offsets_from_sorted_kernel");
+  hipLaunchKernelGGL(dst_of_perm_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ci, perm_out, co, Vd, E);
+  NTS_LAUNCH_CHECK("dst_of_perm_kernel");
+  return NTS_OK;
+}
+
+int nts_gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t *ri, const uint32_t *ro,
+                         const uint32_t *ci, uint32_t Vd, uint32_t Vs, nts_stream_t stream) {
+  if (!co || !ro) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null offsets");
+  if (Vd == 0 || Vs == 0) return NTS_OK;
+  // The edge count lives on the device; one small read-back keeps the ABI free of redundant sizes.
+  uint32_t E = 0;
+  NTS_HIP_TRY(hipMemcpyAsync(&E, co + Vd, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+  NTS_HIP_TRY(hipStreamSynchronize(stream));
+  if (E == 0) return NTS_OK;
+  if (ewf) {
+    if (!ri) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ri");
+    hipLaunchKernelGGL(edge_weights_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ewf, co, Vd, ri, ro, E, 0);
+    NTS_LAUNCH_CHECK("edge_weights_kernel(fwd)");
+  }
+  if (ewb) {
+    if (!ci) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ci");
+    hipLaunchKernelGGL(edge_weights_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ewb, ro, Vs, ci, co, E, 1);
+    NTS_LAUNCH_CHECK("edge_weights_kernel(bwd)");
+  }
+  return NTS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,169 @@
+// Memory, copy and stream entry points of libntship (replaces the free functions and the
+// Cuda_Stream plumbing of cuda/ntsCUDAGraphOP.cu:23-119, 476-653 and utils/cuda_memory.hpp).
+#include <string.h>
+
+#include "common.hpp"
+
+namespace nts {
+
+namespace {
+thread_local char g_last_error[512] = "";
+}
+
+int fail(int code, const char *msg) {
+  snprintf(g_last_error, sizeof(g_last_error), "%s", msg);
+  return code;
+}
+
+int fail_hip(hipError_t err, const char *what) {
+  snprintf(g_last_error, sizeof(g_last_error), "%s: %s (%d)", what, hipGetErrorString(err), static_cast<int>(err));
+  return err == hipErrorOutOfMemory ? NTS_ERR_NOMEM : NTS_ERR_HIP;
+}
+
+namespace {
+
+// 16-byte stores over the aligned body, byte stores over the ragged head and tail.
+__global__ __launch_bounds__(256) void fill_zero_kernel(unsigned char *p, size_t head, size_t body16, size_t tail) {
+  const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  uint4 *body = reinterpret_cast<uint4 *>(p + head);
+  for (size_t i = tid; i < body16; i += stride) body[i] = make_uint4(0u, 0u, 0u, 0u);
+  if (tid < head) p[tid] = 0;
+  if (tid < tail) p[head + body16 * 16 + tid] = 0;
+}
+
+}  // namespace
+}  // namespace nts
+
+using nts::fail;
+
+extern "C" {
+
+const char *nts_last_error(void) { return nts::g_last_error; }
+
+int nts_abi_version(void) { return 1; }
+
+int nts_malloc_device(void **ptr, size_t bytes) {
+  if (!ptr) return fail(NTS_ERR_INVALID, "nts_malloc_device: null out-pointer");
+  *ptr = nullptr;
+  if (bytes == 0) return NTS_OK;
+  NTS_HIP_TRY(hipMalloc(ptr, bytes));
+  return NTS_OK;
+}
+
+int nts_free_device(void *ptr) {
+  if (!ptr) return NTS_OK;
+  NTS_HIP_TRY(hipFree(ptr));
+  return NTS_OK;
+}
+
+int nts_malloc_device_async(void **ptr, size_t bytes, nts_stream_t stream) {
+  if (!ptr) return fail(NTS_ERR_INVALID, "nts_malloc_device_async: null out-pointer");
+  *ptr = nullptr;
+  if (bytes == 0) return NTS_OK;
+  NTS_HIP_TRY(hipMallocAsync(ptr, bytes, stream));
+  return NTS_OK;
+}
+
+int nts_free_device_async(void *ptr, nts_stream_t stream) {
+  if (!ptr) return NTS_OK;
+  NTS_HIP_TRY(hipFreeAsync(ptr, stream));
+  return NTS_OK;
+}
+
+int nts_malloc_pinned_mapped(void **host_ptr, size_t bytes) {
+  if (!host_ptr) return fail(NTS_ERR_INVALID, "nts_malloc_pinned_mapped: null out-pointer");
+  *host_ptr = nullptr;
+  if (bytes == 0) return NTS_OK;
+  NTS_HIP_TRY(hipHostMalloc(host_ptr, bytes, hipHostMallocMapped));
+  return NTS_OK;
+}
+
+int nts_free_pinned(void *host_ptr) {
+  if (!host_ptr) return NTS_OK;
+  NTS_HIP_TRY(hipHostFree(host_ptr));
+  return NTS_OK;
+}
+
+int nts_host_get_device_ptr(void **dev_ptr, void *host_ptr) {
+  if (!dev_ptr || !host_ptr) return fail(NTS_ERR_INVALID, "nts_host_get_device_ptr: null pointer");
+  NTS_HIP_TRY(hipHostGetDevicePointer(dev_ptr, host_ptr, 0));
+  return NTS_OK;
+}
+
+int nts_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, int sync) {
+  if (bytes == 0) return NTS_OK;
+  if (!dst_dev || !src_host) return fail(NTS_ERR_INVALID, "nts_memcpy_h2d: null pointer");
+  NTS_HIP_TRY(hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+  if (sync) NTS_HIP_TRY(hipDeviceSynchronize());
+  return NTS_OK;
+}
+
+int nts_memcpy_h2d_async(void *dst_dev, const void *src_host, size_t bytes, nts_stream_t stream) {
+  if (bytes == 0) return NTS_OK;
+  if (!dst_dev || !src_host) return fail(NTS_ERR_INVALID, "nts_memcpy_h2d_async: null pointer");
+  NTS_HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, stream));
+  return NTS_OK;
+}
+
+int nts_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, int sync) {
+  if (bytes == 0) return NTS_OK;
+  if (!dst_host || !src_dev) return fail(NTS_ERR_INVALID, "nts_memcpy_d2h: null pointer");
+  NTS_HIP_TRY(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+  if (sync) NTS_HIP_TRY(hipDeviceSynchronize());
+  return NTS_OK;
+}
+
+int nts_memcpy_d2h_async(void *dst_host, const void *src_dev, size_t bytes, nts_stream_t stream) {
+  if (bytes == 0) return NTS_OK;
+  if (!dst_host || !src_dev) return fail(NTS_ERR_INVALID, "nts_memcpy_d2h_async: null pointer");
+  NTS_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, stream));
+  return NTS_OK;
+}
+
+int nts_memset_zero(void *dev_ptr, size_t bytes, nts_stream_t stream) {
+  if (bytes == 0) return NTS_OK;
+  if (!dev_ptr) return fail(NTS_ERR_INVALID, "nts_memset_zero: null pointer");
+  unsigned char *p = static_cast<unsigned char *>(dev_ptr);
+  size_t head = (16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15;
+  if (head > bytes) head = bytes;
+  const size_t body16 = (bytes - head) / 16;
+  const size_t tail = bytes - head - body16 * 16;
+  size_t blocks = (body16 + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(nts::fill_zero_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p, head,
+                     body16, tail);
+  NTS_LAUNCH_CHECK("fill_zero_kernel");
+  return NTS_OK;
+}
+
+int nts_stream_create(nts_stream_t *stream) {
+  if (!stream) return fail(NTS_ERR_INVALID, "nts_stream_create: null out-pointer");
+  NTS_HIP_TRY(hipStreamCreate(stream));
+  return NTS_OK;
+}
+
+int nts_stream_destroy(nts_stream_t stream) {
+  if (!stream) return NTS_OK;
+  NTS_HIP_TRY(hipStreamDestroy(stream));
+  return NTS_OK;
+}
+
+int nts_stream_sync(nts_stream_t stream) {
+  NTS_HIP_TRY(hipStreamSynchronize(stream));
+  return NTS_OK;
+}
+
+int nts_device_sync(void) {
+  NTS_HIP_TRY(hipDeviceSynchronize());
+  return NTS_OK;
+}
+
+int nts_mem_info(size_t *free_bytes, size_t *total_bytes) {
+  if (!free_bytes || !total_bytes) return fail(NTS_ERR_INVALID, "nts_mem_info: null pointer");
+  NTS_HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));
+  return NTS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,544 @@
+// Aggregation kernels: weighted / unweighted SpMM executed as a row gather, forward over CSC and
+// backward over CSR (replaces cuda/ntsCUDAFuseKernel.cuh:147-290, 327-487 and their launchers
+// cuda/ntsCUDAGraphOP.cu:186-292).
+//
+// Mapping.  One wavefront (64 lanes) owns one work item = one output row, or one chunk of a long
+// row.  The 64 lanes span the feature dimension: lane l holds NACC register accumulators of VEC
+// consecutive floats at columns (l + 64*k)*VEC, so every row read is a fully coalesced
+// 64*VEC*4-byte wave load and each output element is written exactly once, without atomics.
+// Neighbour (index, weight) pairs are fetched 64 at a time with one coalesced load per wave and
+// then broadcast lane by lane into scalar registers, so the source-row base address is scalar and
+// every index/weight is read from memory once per row instead of once per lane.
+// Narrow rows (F <= 32*VEC) use sub-wavefront groups of G lanes per row (spmm_group_kernel).
+//
+// Accumulation order within a row is the edge order of the offsets array, one fused multiply-add
+// per edge and element -- the order of the CPU operators (core/ntsMiniBatchGraphOp.hpp:154-240),
+// so unsplit rows reproduce an FMA-contracted CPU build bit for bit.
+#include <algorithm>
+#include <new>
+#include <vector>
+
+#include "common.hpp"
+
+namespace nts {
+namespace {
+
+template <int VEC>
+struct Vec;
+template <>
+struct Vec<1> {
+  using type = float;
+};
+template <>
+struct Vec<2> {
+  using type = float2;
+};
+template <>
+struct Vec<4> {
+  using type = float4;
+};
+
+template <int VEC>
+__device__ __forceinline__ typename Vec<VEC>::type vzero();
+template <>
+__device__ __forceinline__ float vzero<1>() {
+  return 0.f;
+}
+template <>
+__device__ __forceinline__ float2 vzero<2>() {
+  return make_float2(0.f, 0.f);
+}
+template <>
+__device__ __forceinline__ float4 vzero<4>() {
+  return make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+__device__ __forceinline__ void vfma(float &a, float x, float w) { a = fmaf(x, w, a); }
+__device__ __forceinline__ void vfma(float2 &a, float2 x, float w) {
+  a.x = fmaf(x.x, w, a.x);
+  a.y = fmaf(x.y, w, a.y);
+}
+__device__ __forceinline__ void vfma(float4 &a, float4 x, float w) {
+  a.x = fmaf(x.x, w, a.x);
+  a.y = fmaf(x.y, w, a.y);
+  a.z = fmaf(x.z, w, a.z);
+  a.w = fmaf(x.w, w, a.w);
+}
+__device__ __forceinline__ void vadd(float &a, float x) { a += x; }
+__device__ __forceinline__ void vadd(float2 &a, float2 x) {
+  a.x += x.x;
+  a.y += x.y;
+}
+__device__ __forceinline__ void vadd(float4 &a, float4 x) {
+  a.x += x.x;
+  a.y += x.y;
+  a.z += x.z;
+  a.w += x.w;
+}
+
+// Edges processed per inner step: keeps 8..16 independent row loads in flight per lane.
+__host__ __device__ constexpr int unroll_for(int nacc) { return nacc >= 8 ? 1 : nacc >= 4 ? 2 : nacc >= 2 ? 4 : 8; }
+
+// Work item of a planned launch: row, first edge, one-past-last edge, partial slot (kNoSlot = the
+// item is a whole row and writes `out` directly).
+using Item = uint4;
+
+template <int VEC, int NACC>
+__global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                        const float *__restrict__ w,
+                                                        const uint32_t *__restrict__ offsets,
+                                                        const uint32_t *__restrict__ indices, uint32_t index_base,
+                                                        uint32_t n_items, uint32_t F, uint32_t col_base,
+                                                        const Item *__restrict__ items, float *__restrict__ partial,
+                                                        int accumulate) {
+  using V = typename Vec<VEC>::type;
+  constexpr int U = unroll_for(NACC);
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t item = blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
+  if (item >= n_items) return;
+
+  uint32_t row, e0, e1, slot;
+  if (items) {
+    const Item it = items[item];
+    row = wave_first(it.x);
+    e0 = wave_first(it.y);
+    e1 = wave_first(it.z);
+    slot = wave_first(it.w);
+  } else {
+    row = item;
+    e0 = wave_first(offsets[item]);
+    e1 = wave_first(offsets[item + 1]);
+    slot = kNoSlot;
+  }
+
+  // Lanes past the end of the row (only possible in the last accumulator) read the row's last
+  // VEC columns instead, so that loads need no predication; their sums are never stored.
+  uint32_t col[NACC];
+  uint32_t lcol[NACC];
+  bool live[NACC];
+  V acc[NACC];
+#pragma unroll
+  for (int k = 0; k < NACC; ++k) {
+    col[k] = col_base + (lane + kWave * k) * VEC;
+    live[k] = col[k] < F;
+    lcol[k] = live[k] ? col[k] : F - VEC;
+    acc[k] = vzero<VEC>();
+  }
+
+  // Tile of up to 64 neighbour (index, weight) pairs held one per lane; the next tile is fetched
+  // while the current one is consumed.
+  uint32_t nxt_i = 0;
+  float nxt_w = 1.f;
+  if (e0 + lane < e1) {
+    nxt_i = indices[e0 + lane] - index_base;
+    if (w) nxt_w = w[e0 + lane];
+  }
+  for (uint32_t eb = e0; eb < e1; eb += kWave) {
+    const uint32_t n = min(static_cast<uint32_t>(kWave), e1 - eb);
+    const uint32_t my_i = nxt_i;
+    const float my_w = nxt_w;
+    const uint32_t en = eb + kWave + lane;
+    if (en < e1) {
+      nxt_i = indices[en] - index_base;
+      if (w) nxt_w = w[en];
+    }
+    uint32_t j = 0;
+    for (; j + U <= n; j += U) {
+      const float *src[U];
+      float sw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        src[u] = in + static_cast<size_t>(wave_read(my_i, j + u)) * F;
+        sw[u] = wave_read(my_w, j + u);
+      }
+      V v[U][NACC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int k = 0; k < NACC; ++k) {
+          v[u][k] = *reinterpret_cast<const V *>(src[u] + lcol[k]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int k = 0; k < NACC; ++k) {
+          vfma(acc[k], v[u][k], sw[u]);
+        }
+      }
+    }
+    for (; j < n; ++j) {
+      const float *src = in + static_cast<size_t>(wave_read(my_i, j)) * F;
+      const float sw = wave_read(my_w, j);
+#pragma unroll
+      for (int k = 0; k < NACC; ++k) {
+        vfma(acc[k], *reinterpret_cast<const V *>(src + lcol[k]), sw);
+      }
+    }
+  }
+
+  float *dst = (slot == kNoSlot) ? out + static_cast<size_t>(row) * F : partial + static_cast<size_t>(slot) * F;
+  const bool add = accumulate && slot == kNoSlot;
+#pragma unroll
+  for (int k = 0; k < NACC; ++k) {
+    if (live[k]) {
+      V *p = reinterpret_cast<V *>(dst + col[k]);
+      V r = acc[k];
+      if (add) vadd(r, *p);
+      *p = r;
+    }
+  }
+}
+
+// Sub-wavefront variant for narrow rows: G lanes per row (G = 8, 16 or 32), 64/G rows per
+// wavefront, one VEC-wide accumulator per lane (F <= G*VEC).  Neighbour pairs are fetched G at a
+// time per group and broadcast inside the group with cross-lane shuffles.
+template <int G, int VEC>
+__global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict__ in, float *__restrict__ out,
+                                                         const float *__restrict__ w,
+                                                         const uint32_t *__restrict__ offsets,
+                                                         const uint32_t *__restrict__ indices, uint32_t index_base,
+                                                         uint32_t n_items, uint32_t F, const Item *__restrict__ items,
+                                                         float *__restrict__ partial, int accumulate) {
+  using V = typename Vec<VEC>::type;
+  constexpr int U = 4;
+  const uint32_t gl = threadIdx.x & (G - 1);
+  const uint32_t item = (blockIdx.x * blockDim.x + threadIdx.x) / G;
+  if (item >= n_items) return;  // whole groups leave together; shuffles stay inside a group
+
+  uint32_t row, e0, e1, slot;
+  if (items) {
+    const Item it = items[item];
+    row = it.x;
+    e0 = it.y;
+    e1 = it.z;
+    slot = it.w;
+  } else {
+    row = item;
+    e0 = offsets[item];
+    e1 = offsets[item + 1];
+    slot = kNoSlot;
+  }
+  const uint32_t col = gl * VEC;
+  const bool live = col < F;
+  const uint32_t lcol = live ? col : F - VEC;  // idle lanes re-read the last columns, never store
+  V acc = vzero<VEC>();
+
+  for (uint32_t eb = e0; eb < e1; eb += G) {
+    const uint32_t n = min(static_cast<uint32_t>(G), e1 - eb);
+    uint32_t my_i = 0;
+    float my_w = 1.f;
+    if (gl < n) {
+      my_i = indices[eb + gl] - index_base;
+      if (w) my_w = w[eb + gl];
+    }
+    uint32_t j = 0;
+    for (; j + U <= n; j += U) {
+      uint32_t si[U];
+      float sw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        si[u] = __shfl(my_i, j + u, G);
+        sw[u] = __shfl(my_w, j + u, G);
+      }
+      V v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        v[u] = *reinterpret_cast<const V *>(in + static_cast<size_t>(si[u]) * F + lcol);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        vfma(acc, v[u], sw[u]);
+      }
+    }
+    for (; j < n; ++j) {
+      const uint32_t si = __shfl(my_i, j, G);
+      const float sw = __shfl(my_w, j, G);
+      vfma(acc, *reinterpret_cast<const V *>(in + static_cast<size_t>(si) * F + lcol), sw);
+    }
+  }
+
+  if (live) {
+    float *dst = (slot == kNoSlot) ? out + static_cast<size_t>(row) * F : partial + static_cast<size_t>(slot) * F;
+    V *p = reinterpret_cast<V *>(dst + col);
+    V r = acc;
+    if (accumulate && slot == kNoSlot) vadd(r, *p);
+    *p = r;
+  }
+}
+
+// Second stage for split rows: out[row,:] (+)= partial[first,:] + partial[first+1,:] + ... in slot
+// order.  One block per split row; `splits[i]` = (row, first slot, slot count, unused).
+__global__ __launch_bounds__(256) void spmm_reduce_partials_kernel(float *__restrict__ out,
+                                                                   const float *__restrict__ partial,
+                                                                   const uint4 *__restrict__ splits, uint32_t F,
+                                                                   int accumulate) {
+  const uint4 s = splits[blockIdx.x];
+  float *dst = out + static_cast<size_t>(s.x) * F;
+  const float *src = partial + static_cast<size_t>(s.y) * F;
+  for (uint32_t c = threadIdx.x; c < F; c += blockDim.x) {
+    float a = src[c];
+    for (uint32_t k = 1; k < s.z; ++k) a += src[static_cast<size_t>(k) * F + c];
+    if (accumulate) a += dst[c];
+    dst[c] = a;
+  }
+}
+
+struct LaunchArgs {
+  const float *in;
+  float *out;
+  const float *w;
+  const uint32_t *offsets;
+  const uint32_t *indices;
+  uint32_t index_base;
+  uint32_t n_items;
+  uint32_t F;
+  const Item *items;
+  float *partial;
+  int accumulate;
+  hipStream_t stream;
+};
+
+template <int VEC, int NACC>
+void launch_wave(const LaunchArgs &a, uint32_t col_base) {
+  constexpr int kWavesPerBlock = 4;
+  const uint32_t blocks = ceil_div(a.n_items, kWavesPerBlock);
+  hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC>), dim3(blocks), dim3(kWavesPerBlock * kWave), 0, a.stream, a.in,
+                     a.out, a.w, a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial,
+                     a.accumulate);
+}
+
+template <int G, int VEC>
+void launch_group(const LaunchArgs &a) {
+  const uint32_t per_block = 256 / G;
+  const uint32_t blocks = ceil_div(a.n_items, per_block);
+  hipLaunchKernelGGL((spmm_group_kernel<G, VEC>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w, a.offsets,
+                     a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate);
+}
+
+template <int VEC>
+void launch_wave_vec(const LaunchArgs &a) {
+  // Column panels of at most 8 accumulators per lane; wider rows are covered by several launches
+  // over disjoint column ranges (each panel re-walks the edge list; outputs are disjoint).
+  constexpr uint32_t kMaxAcc = 8;
+  const uint32_t per_acc = kWave * VEC;
+  uint32_t col_base = 0;
+  while (col_base < a.F) {
+    const uint32_t remaining = a.F - col_base;
+    uint32_t nacc = ceil_div(remaining, per_acc);
+    if (nacc > kMaxAcc) nacc = kMaxAcc;
+    switch (nacc) {
+      case 1: launch_wave<VEC, 1>(a, col_base); break;
+      case 2: launch_wave<VEC, 2>(a, col_base); break;
+      case 3: launch_wave<VEC, 3>(a, col_base); break;
+      case 4: launch_wave<VEC, 4>(a, col_base); break;
+      case 5: launch_wave<VEC, 5>(a, col_base); break;
+      case 6: launch_wave<VEC, 6>(a, col_base); break;
+      case 7: launch_wave<VEC, 7>(a, col_base); break;
+      default: launch_wave<VEC, 8>(a, col_base); break;
+    }
+    col_base += nacc * per_acc;
+  }
+}
+
+// Widest vector the operands allow: rows start at multiples of F floats from the base pointers.
+int pick_vec(const LaunchArgs &a) {
+  const bool a16 = aligned_to(a.in, 16) && aligned_to(a.out, 16) && (!a.partial || aligned_to(a.partial, 16));
+  const bool a8 = aligned_to(a.in, 8) && aligned_to(a.out, 8) && (!a.partial || aligned_to(a.partial, 8));
+  if (a.F % 4 == 0 && a16) return 4;
+  if (a.F % 2 == 0 && a8) return 2;
+  return 1;
+}
+
+void launch_spmm(const LaunchArgs &a) {
+  if (a.n_items == 0) return;
+  const int vec = pick_vec(a);
+  const uint32_t F = a.F;
+  // Narrow rows: sub-wavefront groups so that lanes are not left idle.
+  if (vec == 4 && F <= 32) return launch_group<8, 4>(a);
+  if (vec == 4 && F <= 64) return launch_group<16, 4>(a);
+  if (vec == 4 && F <= 128) return launch_group<32, 4>(a);
+  if (vec == 2 && F <= 16) return launch_group<8, 2>(a);
+  if (vec == 2 && F <= 32) return launch_group<16, 2>(a);
+  if (vec == 2 && F <= 64) return launch_group<32, 2>(a);
+  if (vec == 1 && F <= 8) return launch_group<8, 1>(a);
+  if (vec == 1 && F <= 16) return launch_group<16, 1>(a);
+  if (vec == 1 && F <= 32) return launch_group<32, 1>(a);
+  // Wave per row.  Prefer the narrowest vector that still needs few accumulators: a 16-byte
+  // vector only pays off once a row spans more than one 8-byte wave load.
+  if (vec == 4) return launch_wave_vec<4>(a);
+  if (vec == 2) return launch_wave_vec<2>(a);
+  return launch_wave_vec<1>(a);
+}
+
+int check_common(const float *in, float *out, const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
+                 uint32_t edges, uint32_t F, const char *who) {
+  if (F == 0) return fail(NTS_ERR_INVALID, "spmm: feature width F is 0");
+  if (rows == 0) return NTS_OK;
+  if (!out || !offsets) return fail(NTS_ERR_INVALID, who);
+  if (edges != 0 && (!in || !indices)) return fail(NTS_ERR_INVALID, who);
+  return NTS_OK;
+}
+
+}  // namespace
+}  // namespace nts
+
+struct nts_spmm_plan {
+  uint32_t rows = 0;
+  uint32_t edges = 0;
+  uint32_t chunk = 0;
+  uint32_t n_items = 0;
+  uint32_t n_splits = 0;
+  uint32_t n_partials = 0;
+  const uint32_t *offsets = nullptr;  // identity check only
+  uint4 *items = nullptr;             // device
+  uint4 *splits = nullptr;            // device
+  float *partial = nullptr;           // device, n_partials * partial_F floats
+  uint32_t partial_F = 0;
+};
+
+extern "C" {
+
+int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t *offsets, const uint32_t *indices,
+                    uint32_t index_base, uint32_t rows, uint32_t edges, uint32_t F, int accumulate,
+                    nts_stream_t stream) {
+  if (int rc = nts::check_common(in, out, offsets, indices, rows, edges, F, "nts_spmm_gather: null pointer")) return rc;
+  if (rows == 0) return NTS_OK;
+  nts::LaunchArgs a{in, out, w, offsets, indices, index_base, rows, F, nullptr, nullptr, accumulate, stream};
+  nts::launch_spmm(a);
+  NTS_LAUNCH_CHECK("nts_spmm_gather");
+  return NTS_OK;
+}
+
+int nts_spmm_plan_create(nts_spmm_plan_t **plan_out, const uint32_t *offsets, uint32_t rows, uint32_t edges,
+                         uint32_t chunk_edges, nts_stream_t stream) {
+  if (!plan_out) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null out-pointer");
+  *plan_out = nullptr;
+  if (rows != 0 && !offsets) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null offsets");
+  const uint32_t chunk = chunk_edges ? chunk_edges : 4096u;
+
+  std::vector<uint32_t> off(static_cast<size_t>(rows) + 1, 0u);
+  if (rows) {
+    NTS_HIP_TRY(hipMemcpyAsync(off.data(), offsets, off.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    NTS_HIP_TRY(hipStreamSynchronize(stream));
+    if (off[rows] != edges) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: offsets[rows] != edges");
+    for (uint32_t r = 0; r < rows; ++r) {
+      if (off[r + 1] < off[r]) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: offsets not ascending");
+    }
+  }
+
+  // Items: first the chunks of split rows (all near `chunk` edges, the heaviest work), then the
+  // unsplit rows by descending degree (counting sort, stable in the row id).
+  std::vector<uint4> items;
+  std::vector<uint4> splits;
+  items.reserve(static_cast<size_t>(rows) + edges / chunk + 1);
+  uint32_t n_partials = 0;
+  std::vector<uint32_t> bucket(static_cast<size_t>(chunk) + 2, 0u);
+  for (uint32_t r = 0; r < rows; ++r) {
+    const uint32_t deg = off[r + 1] - off[r];
+    if (deg > chunk) {
+      const uint32_t first = n_partials;
+      for (uint32_t e = off[r]; e < off[r + 1]; e += chunk) {
+        const uint32_t end = std::min(off[r + 1], e + chunk);
+        items.push_back(make_uint4(r, e, end, n_partials++));
+      }
+      splits.push_back(make_uint4(r, first, n_partials - first, 0u));
+    } else {
+      ++bucket[chunk - deg + 1];  // descending degree
+    }
+  }
+  for (size_t i = 1; i < bucket.size(); ++i) bucket[i] += bucket[i - 1];
+  const size_t base = items.size();
+  items.resize(base + bucket.back());
+  for (uint32_t r = 0; r < rows; ++r) {
+    const uint32_t deg = off[r + 1] - off[r];
+    if (deg <= chunk) items[base + bucket[chunk - deg]++] = make_uint4(r, off[r], off[r + 1], nts::kNoSlot);
+  }
+
+  nts_spmm_plan *p = new (std::nothrow) nts_spmm_plan();
+  if (!p) return nts::fail(NTS_ERR_NOMEM, "nts_spmm_plan_create: host allocation failed");
+  p->rows = rows;
+  p->edges = edges;
+  p->chunk = chunk;
+  p->offsets = offsets;
+  p->n_items = static_cast<uint32_t>(items.size());
+  p->n_splits = static_cast<uint32_t>(splits.size());
+  p->n_partials = n_partials;
+  hipError_t err = hipSuccess;
+  if (!items.empty()) {
+    err = hipMalloc(reinterpret_cast<void **>(&p->items), items.size() * sizeof(uint4));
+    if (err == hipSuccess)
+      err = hipMemcpy(p->items, items.data(), items.size() * sizeof(uint4), hipMemcpyHostToDevice);
+  }
+  if (err == hipSuccess && !splits.empty()) {
+    err = hipMalloc(reinterpret_cast<void **>(&p->splits), splits.size() * sizeof(uint4));
+    if (err == hipSuccess)
+      err = hipMemcpy(p->splits, splits.data(), splits.size() * sizeof(uint4), hipMemcpyHostToDevice);
+  }
+  if (err != hipSuccess) {
+    nts_spmm_plan_destroy(p);
+    return nts::fail_hip(err, "nts_spmm_plan_create: device upload");
+  }
+  *plan_out = p;
+  return NTS_OK;
+}
+
+int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {
+  if (!plan) return NTS_OK;
+  hipError_t e1 = plan->items ? hipFree(plan->items) : hipSuccess;
+  hipError_t e2 = plan->splits ? hipFree(plan->splits) : hipSuccess;
+  hipError_t e3 = plan->partial ? hipFree(plan->partial) : hipSuccess;
+  delete plan;
+  if (e1 != hipSuccess) return nts::fail_hip(e1, "nts_spmm_plan_destroy");
+  if (e2 != hipSuccess) return nts::fail_hip(e2, "nts_spmm_plan_destroy");
+  if (e3 != hipSuccess) return nts::fail_hip(e3, "nts_spmm_plan_destroy");
+  return NTS_OK;
+}
+
+int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows, uint32_t *partials) {
+  if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_info: null plan");
+  if (items) *items = plan->n_items;
+  if (split_rows) *split_rows = plan->n_splits;
+  if (partials) *partials = plan->n_partials;
+  return NTS_OK;
+}
+
+int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F) {
+  if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_reserve: null plan");
+  if (plan->n_partials == 0 || F <= plan->partial_F) return NTS_OK;
+  // The old buffer may still be read by work queued earlier: hipFree waits for the device.
+  if (plan->partial) {
+    NTS_HIP_TRY(hipFree(plan->partial));
+    plan->partial = nullptr;
+    plan->partial_F = 0;
+  }
+  NTS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&plan->partial),
+                        static_cast<size_t>(plan->n_partials) * F * sizeof(float)));
+  plan->partial_F = F;
+  return NTS_OK;
+}
+
+int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *w,
+                            const uint32_t *offsets, const uint32_t *indices, uint32_t index_base, uint32_t F,
+                            int accumulate, nts_stream_t stream) {
+  if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_planned: null plan");
+  if (offsets != plan->offsets)
+    return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_planned: offsets differ from the array the plan was built from");
+  if (int rc = nts::check_common(in, out, offsets, indices, plan->rows, plan->edges, F,
+                                 "nts_spmm_gather_planned: null pointer"))
+    return rc;
+  if (plan->rows == 0) return NTS_OK;
+  if (int rc = nts_spmm_plan_reserve(plan, F)) return rc;
+  nts::LaunchArgs a{in,  out,         w,           offsets,       indices,   index_base, plan->n_items,
+                    F,   plan->items, plan->partial, accumulate, stream};
+  nts::launch_spmm(a);
+  NTS_LAUNCH_CHECK("nts_spmm_gather_planned");
+  if (plan->n_splits) {
+    hipLaunchKernelGGL(nts::spmm_reduce_partials_kernel, dim3(plan->n_splits), dim3(256), 0, stream, out,
+                       plan->partial, plan->splits, F, accumulate);
+    NTS_LAUNCH_CHECK("spmm_reduce_partials_kernel");
+  }
+  return NTS_OK;
+}
+
+}  // extern "C"

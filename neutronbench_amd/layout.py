@@ -1,0 +1,167 @@
+"""Device-resident graph structure: the full-graph chunk (CSC_segment_pinned's device fields,
+core/GraphSegment.h:54-133) and the sampled layer (sampCSC's dev_* arrays, core/coocsc.hpp:806-813).
+
+HBM layout.  Offsets and indices are uint32, weights fp32, each array contiguous:
+  column_offset [V_d+1] | row_indices [E] | edge_weight_forward [E]      (CSC, forward)
+  row_offset    [V_s+1] | column_indices [E] | edge_weight_backward [E]  (CSR, backward)
+torch has no uint32 arithmetic, so tensors are stored as int32 with the same bit pattern; the
+kernels read them as uint32.
+"""
+import ctypes
+
+import torch
+
+from .abi import call, ptr
+
+
+def _stream(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def as_u32(t):
+    """int64 tensor of values < 2^32 -> int32 tensor with the uint32 bit pattern."""
+    return (t & 0xFFFFFFFF).to(torch.int64).add_(1 << 31).remainder_(1 << 32).sub_(1 << 31).to(torch.int32)
+
+
+def u32_to_i64(t):
+    return t.to(torch.int64) & 0xFFFFFFFF
+
+
+class SpmmPlan:
+    """Degree-bucketed schedule bound to one offsets tensor."""
+
+    def __init__(self, offsets, rows, edges, chunk_edges=0):
+        self.offsets = offsets
+        handle = ctypes.c_void_p()
+        call("nts_spmm_plan_create", ctypes.byref(handle), ptr(offsets), rows, edges, chunk_edges,
+             _stream(offsets.device))
+        self.handle = handle.value
+
+    def info(self):
+        a, b, c = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+        call("nts_spmm_plan_info", self.handle, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))
+        return dict(items=a.value, split_rows=b.value, partials=c.value)
+
+    def reserve(self, F):
+        call("nts_spmm_plan_reserve", self.handle, F)
+
+    def close(self):
+        if self.handle:
+            call("nts_spmm_plan_destroy", self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class FullGraphChunk:
+    """One partition's CSC + CSR + GCN weights in HBM, plus the aggregation schedules."""
+
+    def __init__(self, V, column_offset, row_indices, ewf, row_offset, column_indices, ewb, chunk_edges=0):
+        self.V = V
+        self.E = int(row_indices.numel())
+        self.column_offset_gpu = column_offset
+        self.row_indices_gpu = row_indices
+        self.edge_weight_forward_gpu = ewf
+        self.row_offset_gpu = row_offset
+        self.column_indices_gpu = column_indices
+        self.edge_weight_backward_gpu = ewb
+        self.src_range = (0, V)
+        self.dst_range = (0, V)
+        self.plan_forward = SpmmPlan(column_offset, V, self.E, chunk_edges)
+        self.plan_backward = SpmmPlan(row_offset, V, self.E, chunk_edges)
+
+    @classmethod
+    def from_edges(cls, src, dst, V, chunk_edges=0):
+        """Builds the chunk on the device that holds `src` / `dst` (int64 edge list).
+
+        Edge order follows PartitionToChunks (core/PartitionedGraph.hpp:281-388): the COO list is
+        ordered by source (stable in the input order); CSR rows keep that order, CSC rows are the
+        stable re-ordering by destination.  Weights are nts_norm_degree of the global degrees.
+        """
+        device = src.device
+        E = src.numel()
+        order = torch.sort(src, stable=True).indices
+        coo_src = src[order]
+        coo_dst = dst[order]
+        del order
+        ro = torch.zeros(V + 1, dtype=torch.int64, device=device)
+        ro[1:] = torch.cumsum(torch.bincount(coo_src, minlength=V), 0)
+        perm = torch.sort(coo_dst, stable=True).indices
+        ri = coo_src[perm]
+        co = torch.zeros(V + 1, dtype=torch.int64, device=device)
+        co[1:] = torch.cumsum(torch.bincount(coo_dst, minlength=V), 0)
+        del perm, coo_src
+        co32, ro32 = as_u32(co), as_u32(ro)
+        ri32, ci32 = as_u32(ri), as_u32(coo_dst)
+        del co, ro, ri, coo_dst
+        ewf = torch.empty(E, dtype=torch.float32, device=device)
+        ewb = torch.empty(E, dtype=torch.float32, device=device)
+        call("nts_gcn_edge_weights", ptr(ewf), ptr(ewb), ptr(co32), ptr(ri32), ptr(ro32), ptr(ci32), V, V,
+             _stream(device))
+        return cls(V, co32, ri32, ewf, ro32, ci32, ewb, chunk_edges)
+
+
+class SampledLayer:
+    """Device mirror of one sampCSC: destination / source (global ids), CSC, CSR, weights.
+
+    `from_host_csc` takes what the sampler's host steps produce (column_offset, local row_indices,
+    source, destination) in one packed upload and builds the CSR and both weight arrays on the
+    device (generate_csr_from_csc + update_degree + compute_weight_*), replacing the reference's
+    eight host-built arrays and eight copies per layer (core/coocsc.hpp:737-773).
+    """
+
+    def __init__(self):
+        self.v_size = self.e_size = self.src_size = 0
+        self.dev_destination = self.dev_source = None
+        self.dev_column_offset = self.dev_row_indices = None
+        self.dev_row_offset = self.dev_column_indices = None
+        self.dev_edge_weight_forward = self.dev_edge_weight_backward = None
+        self.dev_csr_to_csc = None
+
+    @classmethod
+    def from_host_csc(cls, column_offset, row_indices, source, destination, device, want_perm=True):
+        self = cls()
+        Vd, E, Vs = destination.numel(), row_indices.numel(), source.numel()
+        self.v_size, self.e_size, self.src_size = Vd, E, Vs
+        packed = torch.cat([as_u32(column_offset), as_u32(row_indices), as_u32(source), as_u32(destination)])
+        if device.type == "cuda":
+            packed = packed.pin_memory().to(device, non_blocking=True)
+        co, ri, src, dst = torch.split(packed, [Vd + 1, E, Vs, Vd])
+        self.dev_column_offset, self.dev_row_indices, self.dev_source, self.dev_destination = co, ri, src, dst
+        self.dev_row_offset = torch.empty(Vs + 1, dtype=torch.int32, device=device)
+        self.dev_column_indices = torch.empty(E, dtype=torch.int32, device=device)
+        self.dev_csr_to_csc = torch.empty(E, dtype=torch.int32, device=device) if want_perm else None
+        self.dev_edge_weight_forward = torch.empty(E, dtype=torch.float32, device=device)
+        self.dev_edge_weight_backward = torch.empty(E, dtype=torch.float32, device=device)
+        stream = _stream(device)
+        work_bytes = call("nts_csr_from_csc_work_bytes", Vd, Vs, E)
+        work = torch.empty(max(work_bytes, 256) + 256, dtype=torch.uint8, device=device)
+        base = (work.data_ptr() + 255) // 256 * 256
+        call("nts_csr_from_csc", ptr(self.dev_row_offset), ptr(self.dev_column_indices), ptr(self.dev_csr_to_csc),
+             ptr(co), ptr(ri), Vd, Vs, E, base, stream)
+        call("nts_gcn_edge_weights", ptr(self.dev_edge_weight_forward), ptr(self.dev_edge_weight_backward), ptr(co),
+             ptr(ri), ptr(self.dev_row_offset), ptr(self.dev_column_indices), Vd, Vs, stream)
+        return self
+
+    # accessor names of the reference (core/coocsc.hpp: dev_c_o() ... dev_ewb())
+    def dev_c_o(self):
+        return self.dev_column_offset
+
+    def dev_r_i(self):
+        return self.dev_row_indices
+
+    def dev_r_o(self):
+        return self.dev_row_offset
+
+    def dev_c_i(self):
+        return self.dev_column_indices
+
+    def dev_ewf(self):
+        return self.dev_edge_weight_forward
+
+    def dev_ewb(self):
+        return self.dev_edge_weight_backward

@@ -1,0 +1,173 @@
+"""GPU parity of the aggregation kernels (through the C ABI) against the CPU oracle.
+
+Tolerance: max relative error <= 1e-4 in fp32 (relative to max(|a|, |b|, 1e-3 * sum of |terms|)).
+Unsplit rows are additionally required to be bit-identical to the oracle's fused-multiply-add
+variant: the kernel adds the edges of a row in the same order with one FMA each.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from neutronbench_amd import abi
+from neutronbench_amd.abi import call, ptr
+from neutronbench_amd.layout import SpmmPlan
+from util import abs_term_scale, brute_csr, random_block, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def _dev(a, device):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if t.dtype == torch.uint32:
+        t = t.view(torch.int32)
+    return t.to(device)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _run_planless(x, w, off, idx, rows, F, device, base=0, accumulate=0, out_init=None):
+    dx, doff, didx = _dev(x, device), _dev(off, device), _dev(idx, device)
+    dw = _dev(w, device) if w is not None else None
+    out = _dev(out_init, device) if out_init is not None else torch.full((rows, F), float("nan"), device=device)
+    call("nts_spmm_gather", ptr(dx), ptr(out), ptr(dw), ptr(doff), ptr(didx), base, rows, idx.size, F, accumulate,
+         _stream())
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("F", [1, 2, 7, 16, 32, 41, 47, 64, 100, 128, 130, 256, 602, 1433, 2050])
+@pytest.mark.parametrize("weighted", [True, False])
+def test_forward_matches_oracle(device, F, weighted):
+    print(f"case F={F} weighted={weighted}", flush=True)
+    Vd, Vs = 300, 500
+    co, ri = random_block(Vd, Vs, 12, seed=F, hub=400)
+    rng = np.random.default_rng(F + 1)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    w = rng.random(ri.size).astype(np.float32) if weighted else None
+    got = _run_planless(x, w, co, ri, Vd, F, device)
+    ref = oracle.spmm(x, w, co, ri, Vd)
+    scale = abs_term_scale(x, w, co, ri, Vd)
+    assert rel_err(got, ref, scale) <= TOL
+    ref_fma = oracle.spmm(x, w, co, ri, Vd, fused=True)
+    assert np.array_equal(got.view(np.uint32), ref_fma.view(np.uint32)), "edge order / FMA chain differs"
+
+
+def test_backward_is_transposed_gather(device):
+    """gin = A^T gout computed over the CSR arrays equals the oracle's pull backward, the oracle's
+    push backward (to rounding) and satisfies <A x, y> = <x, A^T y>."""
+    Vd, Vs, F = 257, 391, 128
+    co, ri = random_block(Vd, Vs, 9, seed=5, hub=300)
+    ro, ci, perm = brute_csr(co, ri, Vs)
+    rng = np.random.default_rng(6)
+    ewf = rng.random(ri.size).astype(np.float32)
+    ewb = ewf[perm]
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    gout = rng.standard_normal((Vd, F)).astype(np.float32)
+    y = _run_planless(x, ewf, co, ri, Vd, F, device)
+    gin = _run_planless(gout, ewb, ro, ci, Vs, F, device)
+    ref = oracle.spmm(gout, ewb, ro, ci, Vs)
+    assert rel_err(gin, ref, abs_term_scale(gout, ewb, ro, ci, Vs)) <= TOL
+    push = oracle.spmm_push(gout, ewf, co, ri, Vs)
+    assert rel_err(gin, push, abs_term_scale(gout, ewb, ro, ci, Vs)) <= TOL
+    lhs = float((y.astype(np.float64) * gout).sum())
+    rhs = float((x.astype(np.float64) * gin).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), abs(rhs), 1.0)
+
+
+def test_accumulate_and_index_base(device):
+    Vd, Vs, F, base = 64, 90, 100, 1000
+    co, ri = random_block(Vd, Vs, 7, seed=11)
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    w = rng.random(ri.size).astype(np.float32)
+    init = rng.standard_normal((Vd, F)).astype(np.float32)
+    got = _run_planless(x, w, co, (ri + base).astype(np.uint32), Vd, F, device, base=base, accumulate=1, out_init=init)
+    ref = oracle.spmm(x, w, co, ri, Vd) + init
+    assert rel_err(got, ref, abs_term_scale(x, w, co, ri, Vd) + np.abs(init)) <= TOL
+    # accumulate = 0 overwrites whatever the buffer held, including rows without edges
+    got0 = _run_planless(x, w, co, (ri + base).astype(np.uint32), Vd, F, device, base=base, accumulate=0, out_init=init)
+    assert np.array_equal(got0, oracle.spmm(x, w, co, ri, Vd, fused=True))
+
+
+@pytest.mark.parametrize("F,chunk", [(128, 64), (602, 100), (41, 32), (16, 16), (100, 4096)])
+def test_planned_split_rows(device, F, chunk):
+    """Degree-bucketed schedule with hub rows split into chunks: matches the oracle, reports the
+    split, and is bit-reproducible run to run (no atomics)."""
+    print(f"case F={F} chunk={chunk}", flush=True)
+    Vd, Vs = 500, 800
+    co, ri = random_block(Vd, Vs, 20, seed=F, hub=3000, dup=True)
+    rng = np.random.default_rng(F)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    w = rng.random(ri.size).astype(np.float32)
+    dx, dw, dco, dri = _dev(x, device), _dev(w, device), _dev(co, device), _dev(ri, device)
+    plan = SpmmPlan(dco, Vd, ri.size, chunk)
+    info = plan.info()
+    deg = np.diff(co.astype(np.int64))
+    assert info["split_rows"] == int((deg > chunk).sum())
+    assert info["partials"] == int(np.ceil(deg[deg > chunk] / chunk).sum())
+    assert info["items"] == int((deg <= chunk).sum()) + info["partials"]
+    outs = []
+    for _ in range(2):
+        out = torch.full((Vd, F), float("nan"), device=device)
+        call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, F, 0, _stream())
+        torch.cuda.synchronize()
+        outs.append(out.cpu().numpy())
+    ref = oracle.spmm(x, w, co, ri, Vd)
+    assert rel_err(outs[0], ref, abs_term_scale(x, w, co, ri, Vd)) <= TOL
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    # unsplit rows keep the sequential FMA chain
+    ref_fma = oracle.spmm(x, w, co, ri, Vd, fused=True)
+    keep = deg <= chunk
+    assert np.array_equal(outs[0][keep].view(np.uint32), ref_fma[keep].view(np.uint32))
+    # accumulate adds to the existing output, split rows included
+    init = rng.standard_normal((Vd, F)).astype(np.float32)
+    out = _dev(init, device)
+    call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, F, 1, _stream())
+    torch.cuda.synchronize()
+    assert rel_err(out.cpu().numpy(), ref + init, abs_term_scale(x, w, co, ri, Vd) + np.abs(init)) <= TOL
+    plan.close()
+
+
+def test_invariants(device):
+    """All-ones input with unit weights gives the degree; GCN weights on a k-regular ring average."""
+    Vd = Vs = 128
+    F = 64
+    k = 4
+    co = (np.arange(Vd + 1) * k).astype(np.uint32)
+    ri = np.concatenate([[(d + j) % Vs for j in range(k)] for d in range(Vd)]).astype(np.uint32)
+    ones = np.ones((Vs, F), dtype=np.float32)
+    got = _run_planless(ones, None, co, ri, Vd, F, device)
+    assert np.array_equal(got, np.full((Vd, F), float(k), dtype=np.float32))
+    w = np.full(ri.size, oracle.norm_degree(k, k), dtype=np.float32)
+    x = np.random.default_rng(1).standard_normal((Vs, F)).astype(np.float32)
+    got = _run_planless(x, w, co, ri, Vd, F, device)
+    mean = np.stack([x[(np.arange(Vd) + j) % Vs] for j in range(k)]).mean(0)
+    assert rel_err(got, mean) <= TOL
+
+
+def test_empty_and_error_paths(device):
+    F = 8
+    x = torch.zeros(4, F, device=device)
+    out = torch.zeros(4, F, device=device)
+    off = torch.zeros(5, dtype=torch.int32, device=device)
+    idx = torch.zeros(1, dtype=torch.int32, device=device)
+    s = _stream()
+    # rows = 0 and E = 0 are legal no-ops / zero fills
+    assert abi.status("nts_spmm_gather", ptr(x), ptr(out), 0, ptr(off), ptr(idx), 0, 0, 0, F, 0, s) == abi.NTS_OK
+    out.fill_(5.0)
+    assert abi.status("nts_spmm_gather", ptr(x), ptr(out), 0, ptr(off), 0, 0, 4, 0, F, 0, s) == abi.NTS_OK
+    torch.cuda.synchronize()
+    assert float(out.abs().sum()) == 0.0
+    # F = 0 and null pointers are rejected with a status, not a crash
+    assert abi.status("nts_spmm_gather", ptr(x), ptr(out), 0, ptr(off), ptr(idx), 0, 4, 0, 0, 0, s) == abi.NTS_ERR_INVALID
+    assert abi.status("nts_spmm_gather", ptr(x), 0, 0, ptr(off), ptr(idx), 0, 4, 0, F, 0, s) == abi.NTS_ERR_INVALID
+    assert "null" in abi.last_error() or "F" in abi.last_error()
+    # plan creation rejects inconsistent offsets
+    handle = ctypes.c_void_p()
+    assert abi.status("nts_spmm_plan_create", ctypes.byref(handle), ptr(off), 4, 7, 0, s) == abi.NTS_ERR_INVALID
