@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the aggregation hot path on one MI355X.
+
+Workload (BASELINE.json configs[2]): Reddit-shaped full-graph 2-layer GCN aggregation,
+forward + backward, whole graph resident in HBM.  232,965 vertices, 114.8 M directed R-MAT edges,
+GCN-normalised edge weights, fp32.  One step = the four aggregations of one training iteration in
+aggregate-then-transform order: layer-0 forward (F=602), layer-1 forward (F=128), layer-1 backward
+(F=128), layer-0 backward (F=602).  Forward gathers by destination over the CSC, backward gathers
+by source over the CSR.  Inputs are resident in HBM before the timed region.
+
+Prints one JSON line: edges aggregated per second (4 * E edges per step), the roofline figure of
+the dominant kernel (the F=602 gather) from HIP events recorded around that kernel, and the CPU
+oracle timed on the host cores on a bounded sample of the same graph.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+V_REDDIT = 232_965
+E_REDDIT = 114_800_000
+F_IN, F_HID = 602, 128
+HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the F=602 gather kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE
+# (profiles/spmm_wave_f602_reddit_pmc.txt); None until measured.
+TRAFFIC_BYTES_F602 = None
+
+
+def algorithmic_bytes(E, V_out, F, weighted=True):
+    """Edge-gather model of one aggregation pass: one source row, one index and one weight per
+    edge; one output row and one offset per output row."""
+    return E * (4 * F + 4 + (4 if weighted else 0)) + V_out * 4 * F + (V_out + 1) * 4
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--vertices", type=int, default=V_REDDIT)
+    ap.add_argument("--edges", type=int, default=E_REDDIT)
+    ap.add_argument("--chunk", type=int, default=0, help="edges per chunk of a split hub row (0 = library default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the oracle sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    import torch
+
+    from neutronbench_amd import synth
+    from neutronbench_amd.abi import call, ptr
+    from neutronbench_amd.layout import FullGraphChunk
+    from neutronbench_amd.ops import ForwardSingleGPUfuseOp
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the HIP library has no CPU fallback)")
+    dev = torch.device("cuda:0")
+    V, E = args.vertices, args.edges
+
+    t0 = time.time()
+    src, dst = synth.rmat_edges(V, E, 0.57, 0.19, 0.19, seed=3, device=dev)
+    chunk = FullGraphChunk.from_edges(src, dst, V, args.chunk)
+    del src, dst
+    x0 = synth.normal_features(V, F_IN, seed=31, device=dev)
+    h1 = synth.normal_features(V, F_HID, seed=32, device=dev)
+    g1 = synth.normal_features(V, F_HID, seed=33, device=dev)
+    g0 = synth.normal_features(V, F_IN, seed=34, device=dev)
+    torch.cuda.synchronize()
+    setup_s = time.time() - t0
+    op = ForwardSingleGPUfuseOp(chunk, with_weight=True)
+    chunk.plan_forward.reserve(F_IN)
+    chunk.plan_backward.reserve(F_IN)
+
+    def step():
+        y0 = op.forward(x0)    # layer 0: aggregate the 602-wide input features
+        y1 = op.forward(h1)    # layer 1: aggregate the 128-wide hidden features
+        d1 = op.backward(g1)   # layer 1 backward: gradient gather over the CSR
+        d0 = op.backward(g0)   # layer 0 backward
+        return y0, y1, d1, d0
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # Timed region: exactly `steps` steps between two synchronisations.
+    stream = torch.cuda.current_stream().cuda_stream
+    t_start = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t_start
+    ms_per_step = elapsed * 1e3 / args.steps
+    edges_per_s = 4.0 * E / (elapsed / args.steps)
+
+    # Dominant kernel: the F=602 forward gather.  HIP events recorded by the library on the launch
+    # stream immediately before and after that kernel, one launch at a time.
+    ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
+    call("nts_event_create", ctypes.byref(ev0))
+    call("nts_event_create", ctypes.byref(ev1))
+    call("nts_spmm_plan_set_events", chunk.plan_forward.handle, ev0, ev1)
+    durs = []
+    for _ in range(max(3, min(args.steps, 10))):
+        op.forward(x0)
+        ms = ctypes.c_float()
+        call("nts_event_elapsed_ms", ctypes.byref(ms), ev0, ev1)
+        durs.append(ms.value)
+    call("nts_spmm_plan_set_events", chunk.plan_forward.handle, None, None)
+    call("nts_event_destroy", ev0)
+    call("nts_event_destroy", ev1)
+    kernel_ms = sum(durs) / len(durs)
+    algo = algorithmic_bytes(E, V, F_IN)
+    achieved = algo / (kernel_ms * 1e-3) / 1e9
+    roofline = {
+        "bound": "hbm",
+        "kernel": "spmm_wave_kernel<2,5> (F=602 forward gather)",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": TRAFFIC_BYTES_F602,
+        "algorithmic_bytes": algo,
+        "kernel_ms": round(kernel_ms, 3),
+    }
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        cpu_baseline = run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, args.cpu_seconds)
+
+    out = {
+        "metric": "edges aggregated/s (fwd+bwd)",
+        "value": round(edges_per_s, 1),
+        "unit": "edges/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "Reddit-shaped full-graph 2-layer GCN aggregation fwd+bwd (F=602,128)",
+            "vertices": V,
+            "edges": E,
+            "graph": "R-MAT a=.57 b=.19 c=.19, seed 3, ids permuted",
+            "passes_per_step": 4,
+            "plan": chunk.plan_forward.info(),
+            "setup_s": round(setup_s, 2),
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+    }
+    print(json.dumps(out))
+
+
+def run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, target_s):
+    """The CPU oracle (restatement of the reference's CPU operators, OpenMP over rows) on the first
+    R output rows of each of the four passes of the same graph, all host cores."""
+    import numpy as np
+
+    import oracle
+    from neutronbench_amd.layout import u32_to_i64
+
+    threads = oracle.max_threads()
+    co = u32_to_i64(chunk.column_offset_gpu).cpu().numpy()
+    ro = u32_to_i64(chunk.row_offset_gpu).cpu().numpy()
+    xs = [t.cpu().numpy() for t in (x0, h1, g1, g0)]
+
+    def slice_rows(offsets, indices_dev, weights_dev, rows):
+        e = int(offsets[rows])
+        idx = indices_dev[:e].cpu().numpy().view(np.uint32)
+        w = weights_dev[:e].cpu().numpy()
+        return offsets[: rows + 1].astype(np.uint32), idx, w, e
+
+    def run(rows):
+        fo, fi, fw, fe = slice_rows(co, chunk.row_indices_gpu, chunk.edge_weight_forward_gpu, rows)
+        bo, bi, bw, be = slice_rows(ro, chunk.column_indices_gpu, chunk.edge_weight_backward_gpu, rows)
+        t = time.perf_counter()
+        oracle.spmm(xs[0], fw, fo, fi, rows, threads=threads)
+        oracle.spmm(xs[1], fw, fo, fi, rows, threads=threads)
+        oracle.spmm(xs[2], bw, bo, bi, rows, threads=threads)
+        oracle.spmm(xs[3], bw, bo, bi, rows, threads=threads)
+        return time.perf_counter() - t, 2 * (fe + be)
+
+    probe_rows = min(V, 512)
+    t_probe, e_probe = run(probe_rows)
+    rate = e_probe / max(t_probe, 1e-6)
+    # rows whose four passes need about target_s at the probed rate
+    want_edges = rate * target_s
+    per_row = (co[V] + ro[V]) * 2 / V
+    rows = int(max(probe_rows, min(V, want_edges / max(per_row, 1))))
+    t_run, e_run = run(rows)
+    return {
+        "value": round(e_run / t_run, 1),
+        "unit": "edges/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"first {rows} destination rows (forward) and first {rows} source rows (backward) of the same "
+                  f"graph, F=602 and F=128, {e_run} edge visits in {t_run:.2f} s",
+    }
+
+
+if __name__ == "__main__":
+    main()

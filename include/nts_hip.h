@@ -86,6 +86,15 @@ int nts_device_sync(void);
 /* get_gpu_mem / show_gpu_mem (utils/cuda_memory.hpp:6-68): free and total device bytes. */
 int nts_mem_info(size_t *free_bytes, size_t *total_bytes);
 
+/* Device-side timers (the reference only has host wall clocks, dep/gemini/time.hpp:20-26, around
+ * synchronised calls).  An event is an opaque handle; elapsed time is in milliseconds between two
+ * recorded events and synchronises on `stop`. */
+typedef struct ihipEvent_t *nts_event_t;
+int nts_event_create(nts_event_t *event);
+int nts_event_destroy(nts_event_t event);
+int nts_event_record(nts_event_t event, nts_stream_t stream);
+int nts_event_elapsed_ms(float *ms, nts_event_t start, nts_event_t stop);
+
 /* ---------------------------------------------------------------------------------------------
  * Aggregation (weighted / unweighted SpMM as a row gather)
  *
@@ -131,6 +140,10 @@ int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F);
 int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *w,
                             const uint32_t *offsets, const uint32_t *indices, uint32_t index_base,
                             uint32_t F, int accumulate, nts_stream_t stream);
+/* Profiling hook: when both events are non-NULL, every later nts_spmm_gather_planned on this plan
+ * records `start` immediately before and `stop` immediately after its main gather kernel (the
+ * partial-sum reduction of split rows follows `stop`).  NULL, NULL switches it off. */
+int nts_spmm_plan_set_events(nts_spmm_plan_t *plan, nts_event_t start, nts_event_t stop);
 
 /* ---------------------------------------------------------------------------------------------
  * Edge <-> vertex data movement (GAT building blocks).  `co` = column_offset [Vd+1],

@@ -42,6 +42,11 @@ SIGNATURES = {
     "nts_stream_sync": [_vp],
     "nts_device_sync": [],
     "nts_mem_info": [ctypes.POINTER(_sz), ctypes.POINTER(_sz)],
+    "nts_event_create": [ctypes.POINTER(_vp)],
+    "nts_event_destroy": [_vp],
+    "nts_event_record": [_vp, _vp],
+    "nts_event_elapsed_ms": [ctypes.POINTER(_f32), _vp, _vp],
+    "nts_spmm_plan_set_events": [_vp, _vp, _vp],
     "nts_spmm_gather": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
     "nts_spmm_plan_create": [ctypes.POINTER(_vp), _vp, _u32, _u32, _u32, _vp],
     "nts_spmm_plan_destroy": [_vp],

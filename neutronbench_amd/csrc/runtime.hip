@@ -160,6 +160,31 @@ int nts_device_sync(void) {
   return NTS_OK;
 }
 
+int nts_event_create(nts_event_t *event) {
+  if (!event) return fail(NTS_ERR_INVALID, "nts_event_create: null out-pointer");
+  NTS_HIP_TRY(hipEventCreate(event));
+  return NTS_OK;
+}
+
+int nts_event_destroy(nts_event_t event) {
+  if (!event) return NTS_OK;
+  NTS_HIP_TRY(hipEventDestroy(event));
+  return NTS_OK;
+}
+
+int nts_event_record(nts_event_t event, nts_stream_t stream) {
+  if (!event) return fail(NTS_ERR_INVALID, "nts_event_record: null event");
+  NTS_HIP_TRY(hipEventRecord(event, stream));
+  return NTS_OK;
+}
+
+int nts_event_elapsed_ms(float *ms, nts_event_t start, nts_event_t stop) {
+  if (!ms || !start || !stop) return fail(NTS_ERR_INVALID, "nts_event_elapsed_ms: null argument");
+  NTS_HIP_TRY(hipEventSynchronize(stop));
+  NTS_HIP_TRY(hipEventElapsedTime(ms, start, stop));
+  return NTS_OK;
+}
+
 int nts_mem_info(size_t *free_bytes, size_t *total_bytes) {
   if (!free_bytes || !total_bytes) return fail(NTS_ERR_INVALID, "nts_mem_info: null pointer");
   NTS_HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));

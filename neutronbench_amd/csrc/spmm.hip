@@ -395,6 +395,8 @@ struct nts_spmm_plan {
   uint4 *splits = nullptr;            // device
   float *partial = nullptr;           // device, n_partials * partial_F floats
   uint32_t partial_F = 0;
+  hipEvent_t ev_start = nullptr;      // optional profiling events around the main kernel
+  hipEvent_t ev_stop = nullptr;
 };
 
 extern "C" {
@@ -518,6 +520,15 @@ int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F) {
   return NTS_OK;
 }
 
+int nts_spmm_plan_set_events(nts_spmm_plan_t *plan, nts_event_t start, nts_event_t stop) {
+  if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_set_events: null plan");
+  if ((start == nullptr) != (stop == nullptr))
+    return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_set_events: pass both events or neither");
+  plan->ev_start = start;
+  plan->ev_stop = stop;
+  return NTS_OK;
+}
+
 int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *w,
                             const uint32_t *offsets, const uint32_t *indices, uint32_t index_base, uint32_t F,
                             int accumulate, nts_stream_t stream) {
@@ -531,8 +542,10 @@ int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, 
   if (int rc = nts_spmm_plan_reserve(plan, F)) return rc;
   nts::LaunchArgs a{in,  out,         w,           offsets,       indices,   index_base, plan->n_items,
                     F,   plan->items, plan->partial, accumulate, stream};
+  if (plan->ev_start && plan->ev_stop) NTS_HIP_TRY(hipEventRecord(plan->ev_start, stream));
   nts::launch_spmm(a);
   NTS_LAUNCH_CHECK("nts_spmm_gather_planned");
+  if (plan->ev_start && plan->ev_stop) NTS_HIP_TRY(hipEventRecord(plan->ev_stop, stream));
   if (plan->n_splits) {
     hipLaunchKernelGGL(nts::spmm_reduce_partials_kernel, dim3(plan->n_splits), dim3(256), 0, stream, out,
                        plan->partial, plan->splits, F, accumulate);

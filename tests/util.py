@@ -36,10 +36,12 @@ def brute_csr(co, ri, Vs):
     return ro.astype(np.uint32), dst_of[perm].astype(np.uint32), perm.astype(np.uint32)
 
 
-def rel_err(a, b, scale=None, floor=1e-3):
+def rel_err(a, b, scale=None, floor=1e-2):
     """max |a-b| / max(|a|, |b|, floor*scale): relative error that does not blow up where a sum
-    cancels to (almost) zero; `scale` is the magnitude of the terms that were added (default: the
-    largest |value| of the row)."""
+    cancels to (almost) zero; `scale` is the sum of the magnitudes of the terms that were added
+    (default: the largest |value| of the row).  With the 1e-4 tolerance this is the bound
+    |a-b| <= 1e-4 * max(|a|, |b|) + 1e-6 * sum|terms|: two fp32 summation orders of n terms differ
+    by up to ~sqrt(n) ulp of the term scale."""
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
     if a.size == 0:
