@@ -47,6 +47,8 @@ def main():
     ap.add_argument("--edges", type=int, default=E_REDDIT)
     ap.add_argument("--chunk", type=int, default=0, help="edges per chunk of a split hub row (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one plain 1 GiB row copy (identity gather) so that HBM byte counters can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the oracle sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -84,6 +86,17 @@ def main():
         d1 = op.backward(g1)   # layer 1 backward: gradient gather over the CSR
         d0 = op.backward(g0)   # layer 0 backward
         return y0, y1, d1, d0
+
+    if args.calibrate:
+        # Plain copy of known size: 2^18 rows of 1024 floats = 1 GiB read + 1 GiB written (+ 1 MiB of ids).
+        n_cal, f_cal = 1 << 18, 1024
+        cal_src = torch.ones(n_cal, f_cal, device=dev)
+        cal_dst = torch.empty_like(cal_src)
+        cal_ids = torch.arange(n_cal, dtype=torch.int32, device=dev)
+        call("nts_gather_rows_f32", ptr(cal_dst), ptr(cal_src), ptr(cal_ids), 0, 0, n_cal, f_cal,
+             torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        del cal_src, cal_dst, cal_ids
 
     for _ in range(args.warmup):
         step()
