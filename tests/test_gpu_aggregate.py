@@ -14,7 +14,7 @@ import oracle
 from neutronbench_amd import abi
 from neutronbench_amd.abi import call, ptr
 from neutronbench_amd.layout import SpmmPlan
-from util import abs_term_scale, brute_csr, random_block, rel_err
+from util import check, abs_term_scale, brute_csr, random_block, rel_err
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -53,7 +53,7 @@ def test_forward_matches_oracle(device, F, weighted):
     got = _run_planless(x, w, co, ri, Vd, F, device)
     ref = oracle.spmm(x, w, co, ri, Vd)
     scale = abs_term_scale(x, w, co, ri, Vd)
-    assert rel_err(got, ref, scale) <= TOL
+    check(got, ref, scale)
     ref_fma = oracle.spmm(x, w, co, ri, Vd, fused=True)
     assert np.array_equal(got.view(np.uint32), ref_fma.view(np.uint32)), "edge order / FMA chain differs"
 
@@ -72,9 +72,9 @@ def test_backward_is_transposed_gather(device):
     y = _run_planless(x, ewf, co, ri, Vd, F, device)
     gin = _run_planless(gout, ewb, ro, ci, Vs, F, device)
     ref = oracle.spmm(gout, ewb, ro, ci, Vs)
-    assert rel_err(gin, ref, abs_term_scale(gout, ewb, ro, ci, Vs)) <= TOL
+    check(gin, ref, abs_term_scale(gout, ewb, ro, ci, Vs))
     push = oracle.spmm_push(gout, ewf, co, ri, Vs)
-    assert rel_err(gin, push, abs_term_scale(gout, ewb, ro, ci, Vs)) <= TOL
+    check(gin, push, abs_term_scale(gout, ewb, ro, ci, Vs))
     lhs = float((y.astype(np.float64) * gout).sum())
     rhs = float((x.astype(np.float64) * gin).sum())
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), abs(rhs), 1.0)
@@ -89,7 +89,7 @@ def test_accumulate_and_index_base(device):
     init = rng.standard_normal((Vd, F)).astype(np.float32)
     got = _run_planless(x, w, co, (ri + base).astype(np.uint32), Vd, F, device, base=base, accumulate=1, out_init=init)
     ref = oracle.spmm(x, w, co, ri, Vd) + init
-    assert rel_err(got, ref, abs_term_scale(x, w, co, ri, Vd) + np.abs(init)) <= TOL
+    check(got, ref, abs_term_scale(x, w, co, ri, Vd) + np.abs(init))
     # accumulate = 0 overwrites whatever the buffer held, including rows without edges
     got0 = _run_planless(x, w, co, (ri + base).astype(np.uint32), Vd, F, device, base=base, accumulate=0, out_init=init)
     assert np.array_equal(got0, oracle.spmm(x, w, co, ri, Vd, fused=True))
@@ -119,7 +119,7 @@ def test_planned_split_rows(device, F, chunk):
         torch.cuda.synchronize()
         outs.append(out.cpu().numpy())
     ref = oracle.spmm(x, w, co, ri, Vd)
-    assert rel_err(outs[0], ref, abs_term_scale(x, w, co, ri, Vd)) <= TOL
+    check(outs[0], ref, abs_term_scale(x, w, co, ri, Vd))
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
     # unsplit rows keep the sequential FMA chain
     ref_fma = oracle.spmm(x, w, co, ri, Vd, fused=True)
@@ -130,7 +130,7 @@ def test_planned_split_rows(device, F, chunk):
     out = _dev(init, device)
     call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, F, 1, _stream())
     torch.cuda.synchronize()
-    assert rel_err(out.cpu().numpy(), ref + init, abs_term_scale(x, w, co, ri, Vd) + np.abs(init)) <= TOL
+    check(out.cpu().numpy(), ref + init, abs_term_scale(x, w, co, ri, Vd) + np.abs(init))
     plan.close()
 
 
@@ -148,7 +148,7 @@ def test_invariants(device):
     x = np.random.default_rng(1).standard_normal((Vs, F)).astype(np.float32)
     got = _run_planless(x, w, co, ri, Vd, F, device)
     mean = np.stack([x[(np.arange(Vd) + j) % Vs] for j in range(k)]).mean(0)
-    assert rel_err(got, mean) <= TOL
+    check(got, mean)
 
 
 def test_empty_and_error_paths(device):

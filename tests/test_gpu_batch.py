@@ -1,0 +1,183 @@
+"""GPU parity of mini-batch assembly (feature / label gather, HBM feature cache, zero-copy reads of
+mapped pinned host memory) and of the device-side sampled-layer construction: bit-exact."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import dev, host_u32, stream
+from neutronbench_amd import abi
+from neutronbench_amd.abi import call, ptr
+from neutronbench_amd.batch import FeatureCache, MappedHostTable, load_feature_gpu, load_feature_gpu_cache, load_label_gpu
+from neutronbench_amd.layout import SampledLayer
+from neutronbench_amd.stream import CudaStream, get_gpu_mem
+from util import brute_csr, random_block
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("F", [1, 3, 8, 100, 128, 602, 1433])
+def test_feature_gather_device_table(device, F):
+    print(f"case F={F}", flush=True)
+    rng = np.random.default_rng(F)
+    V, n = 3000, 1111
+    feat = rng.standard_normal((V, F)).astype(np.float32)
+    ids = rng.integers(0, V, n).astype(np.uint32)
+    out = torch.full((n, F), float("nan"), device=device)
+    dfeat, dids = dev(feat, device), dev(ids, device)  # keep the device copies alive across the call
+    call("nts_gather_rows_f32", ptr(out), ptr(dfeat), ptr(dids), 0, 0, n, F, stream())
+    assert out.cpu().numpy().tobytes() == oracle.get_feature(feat, ids).tobytes()
+
+
+def test_feature_gather_zero_copy_and_cache(device):
+    """The three launches of the reference (plain zero-copy, zero-copy of the miss list, cache
+    gather of the hit list) and the single device-split kernel all reproduce get_feature."""
+    rng = np.random.default_rng(1)
+    V, F, n_cache = 5000, 100, 1000
+    feat = rng.standard_normal((V, F)).astype(np.float32)
+    out_deg = rng.integers(0, 200, V)
+    feat_t = torch.from_numpy(feat)
+    table = MappedHostTable(feat_t)
+    cache = FeatureCache(feat_t, torch.from_numpy(out_deg), n_cache, device)
+    order = cache.order.numpy().astype(np.uint32)
+    hashmap_ref = oracle.mark_cache(V, order, n_cache)
+    assert np.array_equal(cache.cache_node_hashmap.numpy().view(np.uint32), hashmap_ref)
+    assert np.array_equal(cache.dev_cache_feature.cpu().numpy(), oracle.fill_cache(feat, order, n_cache, hashmap_ref))
+
+    source = np.sort(rng.choice(V, 1800, replace=False)).astype(np.uint32)
+    layer0 = SampledLayer()
+    layer0.src_size = source.size
+    layer0.dev_source = dev(source, device)
+    cs = CudaStream()
+    want, hit, miss = oracle.load_feature_cached(feat, cache.dev_cache_feature.cpu().numpy(), source, hashmap_ref)
+    assert want.tobytes() == oracle.get_feature(feat, source).tobytes()
+
+    x0 = torch.full((source.size, F), float("nan"), device=device)
+    load_feature_gpu(cs, layer0, x0, table.dev_ptr)
+    assert x0.cpu().numpy().tobytes() == want.tobytes()
+
+    x1 = torch.full((source.size, F), float("nan"), device=device)
+    n_hit = load_feature_gpu_cache(cs, layer0, x1, table.dev_ptr, cache, torch.from_numpy(source.astype(np.int64)),
+                                   device_split=False)
+    assert n_hit == hit.size and x1.cpu().numpy().tobytes() == want.tobytes()
+
+    x2 = torch.full((source.size, F), float("nan"), device=device)
+    hits = load_feature_gpu_cache(cs, layer0, x2, table.dev_ptr, cache)
+    cs.CUDA_DEVICE_SYNCHRONIZE()
+    assert int(hits.item()) == hit.size and x2.cpu().numpy().tobytes() == want.tobytes()
+    table.close()
+
+
+def test_label_gather(device):
+    rng = np.random.default_rng(2)
+    V, n = 4000, 1024
+    ids = rng.integers(0, V, n).astype(np.uint32)
+    top = SampledLayer()
+    top.v_size = n
+    top.dev_destination = dev(ids, device)
+    cs = CudaStream()
+    lab = rng.integers(0, 47, V).astype(np.int64)
+    out = torch.full((n,), -1, dtype=torch.int64, device=device)
+    dlab = dev(lab, device)
+    load_label_gpu(cs, top, out, dlab)
+    assert np.array_equal(out.cpu().numpy(), oracle.get_label(lab, ids))
+    multi = rng.integers(0, 2, (V, 121)).astype(np.int64)
+    out2 = torch.full((n, 121), -1, dtype=torch.int64, device=device)
+    dmulti = dev(multi, device)
+    load_label_gpu(cs, top, out2, dmulti)
+    assert np.array_equal(out2.cpu().numpy(), oracle.get_label(multi, ids))
+
+
+@pytest.mark.parametrize("Vd,Vs,mean,hub,dup", [(1024, 9000, 12, 0, False), (300, 50, 20, 45, False),
+                                                (2000, 700, 6, 5000, True), (1, 1, 1, 0, False)])
+def test_device_csr_and_weights(device, Vd, Vs, mean, hub, dup):
+    """generate_csr_from_csc + update_degree + compute_weight_* on the device are bit-exact with
+    the host algorithms of the oracle."""
+    print(f"case Vd={Vd} Vs={Vs}", flush=True)
+    co, ri = random_block(Vd, Vs, mean, seed=Vd + Vs, hub=hub, dup=dup, empty_frac=0.05)
+    E = ri.size
+    rng = np.random.default_rng(3)
+    V = 20000
+    glob = rng.permutation(V)
+    source = np.sort(glob[:Vs]).astype(np.uint32)
+    destination = glob[Vs:Vs + Vd].astype(np.uint32)
+    layer = SampledLayer.from_host_csc(torch.from_numpy(co.astype(np.int64)), torch.from_numpy(ri.astype(np.int64)),
+                                       torch.from_numpy(source.astype(np.int64)),
+                                       torch.from_numpy(destination.astype(np.int64)), device)
+    torch.cuda.synchronize()
+    ro_ref, ci_ref = oracle.csr_from_csc(co, ri, Vs)
+    assert np.array_equal(host_u32(layer.dev_row_offset), ro_ref)
+    assert np.array_equal(host_u32(layer.dev_column_indices), ci_ref)
+    _, _, perm = brute_csr(co, ri, Vs)
+    assert np.array_equal(host_u32(layer.dev_csr_to_csc), perm)
+    outd = np.ones(V, np.uint32)
+    ind = np.ones(V, np.uint32)
+    ewf_ref, ewb_ref = oracle.layer_weights(co, ri, ro_ref, ci_ref, source, destination, outd, ind)
+    assert layer.dev_ewf().cpu().numpy().tobytes() == ewf_ref.tobytes()
+    assert layer.dev_ewb().cpu().numpy().tobytes() == ewb_ref.tobytes()
+    assert np.array_equal(host_u32(layer.dev_source), source) and np.array_equal(host_u32(layer.dev_destination), destination)
+
+
+def test_norm_weight_table_bit_exact(device):
+    """Every (out_degree, in_degree) pair up to 64 x 64 through the device weight kernel equals
+    nts_norm_degree bit for bit: a star per source degree."""
+    n = 64
+    # destination d (1-based degree) gets d in-edges; source s gets s out-edges: build a complete
+    # bipartite-like block where source j connects to destinations j..n-1 -> out_deg(j) = n-j,
+    # in_deg(d) = d+1
+    co = np.zeros(n + 1, dtype=np.uint32)
+    ri = []
+    for d in range(n):
+        ri += list(range(0, d + 1))
+        co[d + 1] = len(ri)
+    ri = np.array(ri, dtype=np.uint32)
+    ro, ci, perm = brute_csr(co, ri, n)
+    ewf = torch.empty(ri.size, device=device)
+    ewb = torch.empty(ri.size, device=device)
+    dco, dri, dro, dci = (dev(t, device) for t in (co, ri, ro, ci))
+    call("nts_gcn_edge_weights", ptr(ewf), ptr(ewb), ptr(dco), ptr(dri), ptr(dro), ptr(dci), n, n, stream())
+    got = ewf.cpu().numpy()
+    k = 0
+    for d in range(n):
+        for s in range(d + 1):
+            assert got[k].tobytes() == oracle.norm_degree(n - s, d + 1).tobytes(), (s, d)
+            k += 1
+    assert np.array_equal(ewb.cpu().numpy(), got[perm])
+
+
+def test_memory_and_stream_entry_points(device):
+    used, total = get_gpu_mem()
+    assert 0 <= used <= total and total > 64 * 1024  # MiB: an MI355X has far more than 64 GiB
+    p = ctypes.c_void_p()
+    call("nts_malloc_device", ctypes.byref(p), 1 << 20)
+    assert p.value
+    s = ctypes.c_void_p()
+    call("nts_stream_create", ctypes.byref(s))
+    host = np.arange(1 << 18, dtype=np.uint32)
+    back = np.zeros_like(host)
+    call("nts_memcpy_h2d_async", p, host.ctypes.data, host.nbytes, s)
+    call("nts_memcpy_d2h_async", back.ctypes.data, p, host.nbytes, s)
+    call("nts_stream_sync", s)
+    assert np.array_equal(host, back)
+    # unaligned, odd-sized zero fill touches exactly the requested bytes
+    call("nts_memcpy_h2d", p, host.ctypes.data, host.nbytes, 1)
+    call("nts_memset_zero", p.value + 3, 1001, s)
+    call("nts_memcpy_d2h_async", back.ctypes.data, p, host.nbytes, s)
+    call("nts_stream_sync", s)
+    want = host.copy().view(np.uint8)
+    want[3:1004] = 0
+    assert np.array_equal(back.view(np.uint8), want)
+    q = ctypes.c_void_p()
+    call("nts_malloc_device_async", ctypes.byref(q), 4096, s)
+    call("nts_free_device_async", q, s)
+    call("nts_stream_sync", s)
+    call("nts_stream_destroy", s)
+    call("nts_free_device", p)
+    hp, dp = ctypes.c_void_p(), ctypes.c_void_p()
+    call("nts_malloc_pinned_mapped", ctypes.byref(hp), 4096)
+    call("nts_host_get_device_ptr", ctypes.byref(dp), hp)
+    assert dp.value
+    call("nts_free_pinned", hp)
+    assert abi.status("nts_memcpy_h2d", 0, host.ctypes.data, 16, 0) == abi.NTS_ERR_INVALID

@@ -62,3 +62,9 @@ def abs_term_scale(x, w, offsets, indices, rows):
         for e in range(int(offsets[r]), int(offsets[r + 1])):
             out[r] += (abs(float(w[e])) if w is not None else 1.0) * x[int(indices[e])]
     return out
+
+
+def check(a, b, scale=None, floor=1e-2, tol=1e-4):
+    """Asserts rel_err(a, b) <= tol with a short failure message (not the arrays)."""
+    err = rel_err(a, b, scale, floor)
+    assert err <= tol, f"max relative error {err:.3e} exceeds {tol:.0e}"
