@@ -135,3 +135,33 @@ def sample_neighbors(co, ri, dst, fanout, seed):
             offs.append(offs[-1] + fanout)
     rows = torch.cat(picks) if picks else torch.zeros(0, dtype=torch.int64)
     return torch.tensor(offs, dtype=torch.int64), rows
+
+
+def build_csc(src, dst, V):
+    """Whole-graph CSC (column_offset [V+1], row_indices [E] = global source ids, both int64) with
+    the edge order of the reference's layout: sources ascending inside a destination."""
+    order = torch.sort(src, stable=True).indices
+    s2, d2 = src[order], dst[order]
+    perm = torch.sort(d2, stable=True).indices
+    co = torch.zeros(V + 1, dtype=torch.int64, device=src.device)
+    co[1:] = torch.cumsum(torch.bincount(d2, minlength=V), 0)
+    return co, s2[perm]
+
+
+def sample_hop(co, ri, dst, fanout, seed):
+    """Vectorised neighbour choice for one hop: every destination takes all its in-neighbours when
+    it has at most `fanout` of them (or fanout < 0), otherwise `fanout` distinct consecutive CSC
+    positions starting at a seeded random offset (with wrap-around).  Which neighbours are chosen is
+    an input to both the oracle and the GPU path, not a parity target.
+    Returns (column_offset [n+1], row_indices with GLOBAL source ids), int64 on co's device."""
+    deg = co[dst + 1] - co[dst]
+    take = deg if fanout < 0 else torch.clamp(deg, max=fanout)
+    off = torch.zeros(dst.numel() + 1, dtype=torch.int64, device=co.device)
+    off[1:] = torch.cumsum(take, 0)
+    E = int(off[-1])
+    owner = torch.repeat_interleave(torch.arange(dst.numel(), device=co.device), take)
+    j = torch.arange(E, device=co.device) - off[owner]
+    start = uniform24(dst, seed * 977 + 5) % torch.clamp(deg, min=1)
+    start = torch.where(deg > take, start, torch.zeros_like(start))
+    pos = (start[owner] + j) % torch.clamp(deg[owner], min=1)
+    return off, ri[co[dst][owner] + pos]
