@@ -73,6 +73,9 @@ int nts_memcpy_h2d_async(void *dst_dev, const void *src_host, size_t bytes, nts_
 int nts_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, int sync);
 /* Cuda_Stream::move_result_out (:121-130). */
 int nts_memcpy_d2h_async(void *dst_host, const void *src_dev, size_t bytes, nts_stream_t stream);
+/* Device-to-device copy on a stream (the reference has none: its edge-softmax kernel writes the
+ * output and the cached copy itself, cuda/ntsCUDADistKernel.cuh:207-209). */
+int nts_memcpy_d2d_async(void *dst_dev, const void *src_dev, size_t bytes, nts_stream_t stream);
 /* zero_buffer (:594-601) / NtsScheduler::ZeroVarMem (core/NtsScheduler.hpp:321-336).  Done with a
  * fill kernel on `stream` (safe under graph capture); does not synchronise. */
 int nts_memset_zero(void *dev_ptr, size_t bytes, nts_stream_t stream);

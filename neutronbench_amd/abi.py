@@ -36,6 +36,7 @@ SIGNATURES = {
     "nts_memcpy_h2d_async": [_vp, _vp, _sz, _vp],
     "nts_memcpy_d2h": [_vp, _vp, _sz, _int],
     "nts_memcpy_d2h_async": [_vp, _vp, _sz, _vp],
+    "nts_memcpy_d2d_async": [_vp, _vp, _sz, _vp],
     "nts_memset_zero": [_vp, _sz, _vp],
     "nts_stream_create": [ctypes.POINTER(_vp)],
     "nts_stream_destroy": [_vp],

@@ -121,6 +121,13 @@ int nts_memcpy_d2h_async(void *dst_host, const void *src_dev, size_t bytes, nts_
   return NTS_OK;
 }
 
+int nts_memcpy_d2d_async(void *dst_dev, const void *src_dev, size_t bytes, nts_stream_t stream) {
+  if (bytes == 0) return NTS_OK;
+  if (!dst_dev || !src_dev) return fail(NTS_ERR_INVALID, "nts_memcpy_d2d_async: null pointer");
+  NTS_HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, stream));
+  return NTS_OK;
+}
+
 int nts_memset_zero(void *dev_ptr, size_t bytes, nts_stream_t stream) {
   if (bytes == 0) return NTS_OK;
   if (!dev_ptr) return fail(NTS_ERR_INVALID, "nts_memset_zero: null pointer");

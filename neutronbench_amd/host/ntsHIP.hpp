@@ -1,0 +1,340 @@
+// ntsHIP.hpp -- C++ host veneer over libntship's C ABI with the names and signatures the
+// NeutronBench tree already uses (cuda/ntsCUDA.hpp:26-211): the free allocation / copy helpers,
+// deviceCSC and the Cuda_Stream class.  Including this header instead of cuda/ntsCUDA.hpp lets
+// core/ and toolkits/ compile unchanged against the HIP library; nothing here launches a kernel
+// itself.
+//
+// Error behaviour follows the reference (cuda/ntsCUDAGraphOP.cu:11-20): a failing call prints the
+// library's error text and exits with status 1.  Callers that want status codes use nts_hip.h
+// directly.
+#ifndef NTS_HIP_VENEER_HPP
+#define NTS_HIP_VENEER_HPP
+
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include "nts_hip.h"
+
+typedef uint32_t VertexId_CUDA;
+// The stream type of the reference's interfaces.  hipStream_t and this typedef are the same
+// pointer type, so streams taken from libtorch-ROCm's pool can be passed straight in.
+typedef nts_stream_t cudaStream_t;
+
+const int CUDA_NUM_THREADS = 512;  // kept for source compatibility; launch shapes are chosen by the library
+const int CUDA_NUM_BLOCKS = 128;
+const int CUDA_NUM_THREADS_SOFTMAX = 32;
+const int CUDA_NUM_BLOCKS_SOFTMAX = 512;
+
+enum graph_type { CSR, CSC, PAIR };
+enum weight_type { NULL_TYPE, SCALA_TYPE, TENSOR_TYPE };
+
+#define NTS_VENEER_CHECK(call_expr)                                                        \
+  do {                                                                                     \
+    int nts_rc__ = (call_expr);                                                            \
+    if (nts_rc__ != NTS_OK) {                                                              \
+      printf("HIP call on line %d returned error %d: %s\n", __LINE__, nts_rc__, nts_last_error()); \
+      exit(1);                                                                             \
+    }                                                                                      \
+  } while (0)
+
+// ---- allocation and copies ---------------------------------------------------------------------
+
+inline void *cudaMallocPinned(long size_of_bytes) {
+  void *p = NULL;
+  NTS_VENEER_CHECK(nts_malloc_pinned_mapped(&p, (size_t)size_of_bytes));
+  return p;
+}
+inline void *getDevicePointer(void *host_data_to_device) {
+  void *d = NULL;
+  NTS_VENEER_CHECK(nts_host_get_device_ptr(&d, host_data_to_device));
+  return d;
+}
+inline void *cudaMallocGPU(long size_of_bytes) {
+  void *p = NULL;
+  NTS_VENEER_CHECK(nts_malloc_device(&p, (size_t)size_of_bytes));
+  return p;
+}
+inline void ntsFreeHost(void *buffer) { NTS_VENEER_CHECK(nts_free_pinned(buffer)); }
+inline void FreeBuffer(float *buffer) { NTS_VENEER_CHECK(nts_free_device(buffer)); }
+inline void FreeEdge(VertexId_CUDA *buffer) { NTS_VENEER_CHECK(nts_free_device(buffer)); }
+inline void FreeBufferAsync(float *buffer, cudaStream_t cs) { NTS_VENEER_CHECK(nts_free_device_async(buffer, cs)); }
+inline void FreeEdgeAsync(VertexId_CUDA *buffer, cudaStream_t cs) { NTS_VENEER_CHECK(nts_free_device_async(buffer, cs)); }
+template <typename T>
+inline void free_gpu_data(T *data) {
+  NTS_VENEER_CHECK(nts_free_device(data));
+}
+template <typename T>
+inline void alloc_gpu_data(T **input, int size) {
+  NTS_VENEER_CHECK(nts_malloc_device((void **)input, sizeof(T) * (size_t)size));
+}
+inline void allocate_gpu_buffer(float **input, int size) {
+  NTS_VENEER_CHECK(nts_malloc_device((void **)input, sizeof(float) * (size_t)size));
+}
+inline void allocate_gpu_edge(VertexId_CUDA **input, int size) {
+  NTS_VENEER_CHECK(nts_malloc_device((void **)input, sizeof(VertexId_CUDA) * (size_t)size));
+}
+inline void allocate_gpu_buffer_async(float **input, int size, cudaStream_t cs) {
+  NTS_VENEER_CHECK(nts_malloc_device_async((void **)input, sizeof(float) * (size_t)size, cs));
+}
+inline void allocate_gpu_edge_async(VertexId_CUDA **input, int size, cudaStream_t cs) {
+  NTS_VENEER_CHECK(nts_malloc_device_async((void **)input, sizeof(VertexId_CUDA) * (size_t)size, cs));
+}
+inline void move_result_out(float *output, float *input, int src, int dst, int feature_size, bool sync = true) {
+  NTS_VENEER_CHECK(nts_memcpy_d2h(output, input, (size_t)(dst - src) * feature_size * sizeof(float), sync));
+}
+inline void move_data_in(float *d_pointer, float *h_pointer, int start, int end, int feature_size, bool sync = true) {
+  NTS_VENEER_CHECK(nts_memcpy_h2d(d_pointer, h_pointer, (size_t)(end - start) * feature_size * sizeof(float), sync));
+}
+inline void move_edge_in(VertexId_CUDA *d_pointer, VertexId_CUDA *h_pointer, VertexId_CUDA start, VertexId_CUDA end,
+                         int feature_size, bool sync = true) {
+  NTS_VENEER_CHECK(
+      nts_memcpy_h2d(d_pointer, h_pointer, (size_t)(end - start) * feature_size * sizeof(VertexId_CUDA), sync));
+}
+inline void move_bytes_in(void *d_pointer, void *h_pointer, long bytes, bool sync = true) {
+  NTS_VENEER_CHECK(nts_memcpy_h2d(d_pointer, h_pointer, (size_t)bytes, sync));
+}
+inline void move_bytes_in_async(void *d_pointer, void *h_pointer, long bytes, cudaStream_t cs) {
+  NTS_VENEER_CHECK(nts_memcpy_h2d_async(d_pointer, h_pointer, (size_t)bytes, cs));
+}
+inline void zero_buffer(float *buffer, int size) {
+  NTS_VENEER_CHECK(nts_memset_zero(buffer, sizeof(float) * (size_t)size, (cudaStream_t)0));
+  NTS_VENEER_CHECK(nts_device_sync());
+}
+inline void CUDA_DEVICE_SYNCHRONIZE() { NTS_VENEER_CHECK(nts_device_sync()); }
+// The few raw runtime names that core/ calls outside cuda/ (core/ntsMiniBatchGraphOp.hpp:283,
+// core/coocsc.hpp:673-773).
+inline int cudaFree(void *p) { return nts_free_device(p); }
+inline int cudaStreamSynchronize(cudaStream_t s) { return nts_stream_sync(s); }
+
+// utils/cuda_memory.hpp: used, total in MiB.
+inline void get_gpu_mem(double &used, double &total) {
+  size_t free_b = 0, total_b = 0;
+  NTS_VENEER_CHECK(nts_mem_info(&free_b, &total_b));
+  used = (double)(total_b - free_b) / 1024.0 / 1024.0;
+  total = (double)total_b / 1024.0 / 1024.0;
+}
+
+// ---- deviceCSC (cuda/ntsCUDA.hpp:54-97) ----------------------------------------------------------
+
+class deviceCSC {
+ public:
+  VertexId_CUDA *column_offset = NULL;
+  VertexId_CUDA *row_indices = NULL;
+  VertexId_CUDA *mirror_index = NULL;
+  VertexId_CUDA v_size = 0;
+  VertexId_CUDA e_size = 0;
+  VertexId_CUDA mirror_size = 0;
+  bool require_mirror = false;
+
+  void init(VertexId_CUDA v_size_, VertexId_CUDA e_size_, bool require_mirror_ = false,
+            VertexId_CUDA mirror_size_ = 0) {
+    v_size = v_size_;
+    e_size = e_size_;
+    column_offset = (VertexId_CUDA *)cudaMallocGPU((long)(v_size_ + 1) * sizeof(VertexId_CUDA));
+    row_indices = (VertexId_CUDA *)cudaMallocGPU((long)e_size_ * sizeof(VertexId_CUDA));
+    require_mirror = require_mirror_;
+    if (require_mirror_) {
+      mirror_size = mirror_size_;
+      mirror_index = (VertexId_CUDA *)cudaMallocGPU((long)mirror_size_ * sizeof(VertexId_CUDA));
+    }
+  }
+  void load_from_host(VertexId_CUDA *h_column_offset, VertexId_CUDA *h_row_indices, VertexId_CUDA *h_mirror_index) {
+    load_from_host(h_column_offset, h_row_indices);
+    move_bytes_in(mirror_index, h_mirror_index, (long)mirror_size * sizeof(VertexId_CUDA));
+  }
+  void load_from_host(VertexId_CUDA *h_column_offset, VertexId_CUDA *h_row_indices) {
+    move_bytes_in(column_offset, h_column_offset, (long)(v_size + 1) * sizeof(VertexId_CUDA));
+    move_bytes_in(row_indices, h_row_indices, (long)e_size * sizeof(VertexId_CUDA));
+  }
+  void release() {
+    FreeEdge(column_offset);
+    FreeEdge(row_indices);
+    if (require_mirror) FreeEdge(mirror_index);
+    column_offset = row_indices = mirror_index = NULL;
+  }
+};
+
+// ---- Cuda_Stream (cuda/ntsCUDA.hpp:99-211) -------------------------------------------------------
+
+class Cuda_Stream {
+ public:
+  cudaStream_t stream = NULL;
+  bool owns_stream = false;
+
+  Cuda_Stream() {
+    NTS_VENEER_CHECK(nts_stream_create(&stream));
+    owns_stream = true;
+  }
+  ~Cuda_Stream() { destory_Stream(); }
+  void destory_Stream() {
+    if (owns_stream && stream) NTS_VENEER_CHECK(nts_stream_destroy(stream));
+    stream = NULL;
+    owns_stream = false;
+  }
+  cudaStream_t getStream() { return stream; }
+  // Adopts a stream owned by someone else (a libtorch pool stream); the previous own stream is destroyed.
+  void setNewStream(cudaStream_t cudaStream) {
+    destory_Stream();
+    stream = cudaStream;
+  }
+  void CUDA_DEVICE_SYNCHRONIZE() { NTS_VENEER_CHECK(nts_stream_sync(stream)); }
+
+  void move_result_out(float *output, float *input, VertexId_CUDA src, VertexId_CUDA dst, int feature_size,
+                       bool sync = true) {
+    (void)sync;
+    NTS_VENEER_CHECK(nts_memcpy_d2h_async(output, input, (size_t)(dst - src) * feature_size * sizeof(float), stream));
+  }
+  void move_data_in(float *d_pointer, float *h_pointer, VertexId_CUDA start, VertexId_CUDA end, int feature_size,
+                    bool sync = true) {
+    (void)sync;
+    NTS_VENEER_CHECK(
+        nts_memcpy_h2d_async(d_pointer, h_pointer, (size_t)(end - start) * feature_size * sizeof(float), stream));
+  }
+  void move_edge_in(VertexId_CUDA *d_pointer, VertexId_CUDA *h_pointer, VertexId_CUDA start, VertexId_CUDA end,
+                    int feature_size, bool sync = true) {
+    (void)sync;
+    NTS_VENEER_CHECK(nts_memcpy_h2d_async(d_pointer, h_pointer,
+                                          (size_t)(end - start) * feature_size * sizeof(VertexId_CUDA), stream));
+  }
+
+  // Aggregation.  The *_end and dst_start / src_start arguments that the reference's kernels never
+  // read are accepted and ignored.  Semantics: output += sum (output is pre-zeroed by the caller).
+  void Gather_By_Dst_From_Src(float *input, float *output, float *weight_forward, VertexId_CUDA *row_indices,
+                              VertexId_CUDA *column_offset, VertexId_CUDA src_start, VertexId_CUDA src_end,
+                              VertexId_CUDA dst_start, VertexId_CUDA dst_end, VertexId_CUDA edges,
+                              VertexId_CUDA batch_size, VertexId_CUDA feature_size, bool with_weight = false,
+                              bool tensor_weight = false) {
+    (void)src_end; (void)dst_start; (void)dst_end;
+    reject_tensor_weight(with_weight && tensor_weight);
+    NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_forward : NULL, column_offset, row_indices,
+                                     src_start, batch_size, edges, feature_size, 1, stream));
+  }
+  void Gather_By_Dst_From_Src_Optim(float *input, float *output, float *weight_forward, VertexId_CUDA *row_indices,
+                                    VertexId_CUDA *column_offset, VertexId_CUDA src_start, VertexId_CUDA src_end,
+                                    VertexId_CUDA dst_start, VertexId_CUDA dst_end, VertexId_CUDA edges,
+                                    VertexId_CUDA batch_size, VertexId_CUDA feature_size, bool with_weight = false,
+                                    bool tensor_weight = false) {
+    Gather_By_Dst_From_Src(input, output, weight_forward, row_indices, column_offset, src_start, src_end, dst_start,
+                           dst_end, edges, batch_size, feature_size, with_weight, tensor_weight);
+  }
+  void Gather_By_Src_From_Dst(float *input, float *output, float *weight_backward, VertexId_CUDA *row_offset,
+                              VertexId_CUDA *column_indices, VertexId_CUDA src_start, VertexId_CUDA src_end,
+                              VertexId_CUDA dst_start, VertexId_CUDA dst_end, VertexId_CUDA edges,
+                              VertexId_CUDA batch_size, VertexId_CUDA feature_size, bool with_weight = false,
+                              bool tensor_weight = false) {
+    (void)src_start; (void)src_end; (void)dst_end;
+    reject_tensor_weight(with_weight && tensor_weight);
+    NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_backward : NULL, row_offset, column_indices,
+                                     dst_start, batch_size, edges, feature_size, 1, stream));
+  }
+  void Gather_By_Src_From_Dst_Optim(float *input, float *output, float *weight_backward, VertexId_CUDA *row_offset,
+                                    VertexId_CUDA *column_indices, VertexId_CUDA src_start, VertexId_CUDA src_end,
+                                    VertexId_CUDA dst_start, VertexId_CUDA dst_end, VertexId_CUDA edges,
+                                    VertexId_CUDA batch_size, VertexId_CUDA feature_size, bool with_weight = false,
+                                    bool tensor_weight = false) {
+    Gather_By_Src_From_Dst(input, output, weight_backward, row_offset, column_indices, src_start, src_end, dst_start,
+                           dst_end, edges, batch_size, feature_size, with_weight, tensor_weight);
+  }
+  void Scatter_Grad_Back_To_Message(float *input, float *message_grad, VertexId_CUDA *row_indices,
+                                    VertexId_CUDA *column_offset, VertexId_CUDA src_start, VertexId_CUDA src_end,
+                                    VertexId_CUDA dst_start, VertexId_CUDA dst_end, VertexId_CUDA edges,
+                                    VertexId_CUDA batch_size, VertexId_CUDA feature_size, bool with_weight = true) {
+    (void)row_indices; (void)src_start; (void)src_end; (void)dst_start; (void)dst_end; (void)edges;
+    if (with_weight) {
+      printf("tensor_weight Scatter_Grad_Back_To_Weight not implemented\n");
+      exit(0);
+    }
+    NTS_VENEER_CHECK(nts_scatter_grad_to_edge(message_grad, input, column_offset, batch_size, feature_size, stream));
+  }
+
+  // Edge <-> vertex.
+  void Scatter_Src_Mirror_to_Msg(float *message, float *src_mirror_feature, VertexId_CUDA *row_indices,
+                                 VertexId_CUDA *column_offset, VertexId_CUDA *mirror_index, VertexId_CUDA batch_size,
+                                 VertexId_CUDA feature_size) {
+    NTS_VENEER_CHECK(nts_scatter_src_to_edge(message, src_mirror_feature, row_indices, column_offset, mirror_index,
+                                             batch_size, feature_size, stream));
+  }
+  void Scatter_Dst_to_Msg(float *message, float *dst_feature, VertexId_CUDA *row_indices,
+                          VertexId_CUDA *column_offset, VertexId_CUDA batch_size, VertexId_CUDA feature_size) {
+    (void)row_indices;
+    NTS_VENEER_CHECK(nts_scatter_dst_to_edge(message, dst_feature, column_offset, batch_size, feature_size, stream));
+  }
+  void Gather_Msg_to_Dst(float *dst_feature, float *message, VertexId_CUDA *row_indices, VertexId_CUDA *column_offset,
+                         VertexId_CUDA batch_size, VertexId_CUDA feature_size) {
+    (void)row_indices;
+    NTS_VENEER_CHECK(nts_gather_edge_to_dst(dst_feature, message, column_offset, batch_size, feature_size, 1, stream));
+  }
+  // Deterministic replacement of Gather_Msg_To_Src_Mirror: takes the transposed structure
+  // (row_offset [src_size+1], csr_to_csc [E]) instead of (row_indices, column_offset, mirror_index).
+  void Gather_Msg_To_Src(float *src_feature, float *message, VertexId_CUDA *row_offset, VertexId_CUDA *csr_to_csc,
+                         VertexId_CUDA src_size, VertexId_CUDA feature_size) {
+    NTS_VENEER_CHECK(nts_gather_edge_to_src(src_feature, message, row_offset, csr_to_csc, src_size, feature_size, 1,
+                                            stream));
+  }
+  void Edge_Softmax_Forward_Block(float *msg_output, float *msg_input, float *msg_cached, VertexId_CUDA *row_indices,
+                                  VertexId_CUDA *column_offset, VertexId_CUDA batch_size,
+                                  VertexId_CUDA feature_size) {
+    (void)row_indices;
+    NTS_VENEER_CHECK(nts_edge_softmax_fwd(msg_output, msg_input, column_offset, batch_size, feature_size, stream));
+    if (msg_cached && msg_cached != msg_output) {
+      // The edge count is only known on the device: copy column_offset[batch_size] back once.
+      VertexId_CUDA edges = 0;
+      NTS_VENEER_CHECK(nts_memcpy_d2h_async(&edges, column_offset + batch_size, sizeof(edges), stream));
+      NTS_VENEER_CHECK(nts_stream_sync(stream));
+      NTS_VENEER_CHECK(
+          nts_memcpy_d2d_async(msg_cached, msg_output, (size_t)edges * feature_size * sizeof(float), stream));
+    }
+  }
+  void Edge_Softmax_Backward_Block(float *msg_input_grad, float *msg_output_grad, float *msg_cached,
+                                   VertexId_CUDA *row_indices, VertexId_CUDA *column_offset, VertexId_CUDA batch_size,
+                                   VertexId_CUDA feature_size) {
+    (void)row_indices;
+    NTS_VENEER_CHECK(nts_edge_softmax_bwd(msg_input_grad, msg_output_grad, msg_cached, column_offset, batch_size,
+                                          feature_size, stream));
+  }
+
+  // Mini-batch assembly; like the reference these return with the result complete.
+  void zero_copy_feature_move_gpu(float *dev_feature, float *pinned_host_feature, VertexId_CUDA *src_vertex,
+                                  VertexId_CUDA feature_size, VertexId_CUDA vertex_size) {
+    NTS_VENEER_CHECK(nts_gather_rows_f32(dev_feature, pinned_host_feature, src_vertex, NULL, NULL, vertex_size,
+                                         feature_size, stream));
+    CUDA_DEVICE_SYNCHRONIZE();
+  }
+  void zero_copy_feature_move_gpu_cache(float *dev_feature, float *host_pinned_feature, VertexId_CUDA *src_vertex,
+                                        VertexId_CUDA feature_size, VertexId_CUDA vertex_size,
+                                        VertexId_CUDA *local_idx) {
+    NTS_VENEER_CHECK(nts_gather_rows_f32(dev_feature, host_pinned_feature, src_vertex, local_idx, NULL, vertex_size,
+                                         feature_size, stream));
+    CUDA_DEVICE_SYNCHRONIZE();
+  }
+  void gather_feature_from_gpu_cache(float *dev_feature, float *dev_cache_feature, VertexId_CUDA *src_vertex,
+                                     VertexId_CUDA feature_size, VertexId_CUDA vertex_size,
+                                     VertexId_CUDA *local_idx_cache, VertexId_CUDA *cache_node_hashmap) {
+    NTS_VENEER_CHECK(nts_gather_rows_f32(dev_feature, dev_cache_feature, src_vertex, local_idx_cache,
+                                         cache_node_hashmap, vertex_size, feature_size, stream));
+    CUDA_DEVICE_SYNCHRONIZE();
+  }
+  void global_copy_label_move_gpu(long *dev_label, long *global_dev_label, VertexId_CUDA *dst_vertex,
+                                  VertexId_CUDA vertex_size) {
+    NTS_VENEER_CHECK(nts_gather_labels_i64((int64_t *)dev_label, (const int64_t *)global_dev_label, dst_vertex,
+                                           vertex_size, 1, stream));
+    CUDA_DEVICE_SYNCHRONIZE();
+  }
+  void global_copy_mulilabel_move_gpu(long *dev_label, long *global_dev_label, VertexId_CUDA *dst_vertex,
+                                      VertexId_CUDA vertex_size, VertexId_CUDA label_size) {
+    NTS_VENEER_CHECK(nts_gather_labels_i64((int64_t *)dev_label, (const int64_t *)global_dev_label, dst_vertex,
+                                           vertex_size, label_size, stream));
+    CUDA_DEVICE_SYNCHRONIZE();
+  }
+
+ private:
+  static void reject_tensor_weight(bool tensor) {
+    if (tensor) {
+      printf("tensor-weight aggregation is a legacy implementation\n");
+      exit(0);
+    }
+  }
+};
+
+#endif  // NTS_HIP_VENEER_HPP

@@ -1,0 +1,125 @@
+// Exercises the C++ veneer (neutronbench_amd/host/ntsHIP.hpp) the way the reference's operators do
+// (core/ntsMiniBatchGraphOp.hpp:288-375, core/ntsSampler.hpp:353-529): raw device pointers, a
+// Cuda_Stream, pre-zeroed outputs.  Results are compared with plain loops written here (a binding
+// test; numerical parity against the oracle lives in the Python tests).  Exit status 0 = pass.
+#include <math.h>
+#include <string.h>
+
+#include <vector>
+
+#include "ntsHIP.hpp"
+
+static int failures = 0;
+#define EXPECT(cond)                                            \
+  do {                                                          \
+    if (!(cond)) {                                              \
+      printf("FAILED line %d: %s\n", __LINE__, #cond);          \
+      ++failures;                                               \
+    }                                                           \
+  } while (0)
+
+int main() {
+  const VertexId_CUDA Vd = 300, Vs = 500, F = 100;
+  std::vector<VertexId_CUDA> co(Vd + 1, 0), ri;
+  uint64_t state = 12345;
+  auto next = [&]() {
+    state = state * 6364136223846793005ull + 1442695040888963407ull;
+    return (uint32_t)(state >> 33);
+  };
+  for (VertexId_CUDA d = 0; d < Vd; ++d) {
+    const uint32_t deg = next() % 20;
+    for (uint32_t k = 0; k < deg; ++k) ri.push_back(next() % Vs);
+    co[d + 1] = (VertexId_CUDA)ri.size();
+  }
+  const VertexId_CUDA E = (VertexId_CUDA)ri.size();
+  std::vector<float> x((size_t)Vs * F), w(E), ref((size_t)Vd * F, 0.f), got((size_t)Vd * F);
+  for (auto &v : x) v = (float)(next() % 2001) / 1000.f - 1.f;
+  for (auto &v : w) v = (float)(next() % 1000) / 1000.f;
+  for (VertexId_CUDA d = 0; d < Vd; ++d)
+    for (VertexId_CUDA e = co[d]; e < co[d + 1]; ++e)
+      for (VertexId_CUDA f = 0; f < F; ++f) ref[(size_t)d * F + f] = fmaf(x[(size_t)ri[e] * F + f], w[e], ref[(size_t)d * F + f]);
+
+  Cuda_Stream cs;
+  deviceCSC csc;
+  csc.init(Vd, E);
+  csc.load_from_host(co.data(), ri.data());
+  float *dx, *dw, *dout;
+  allocate_gpu_buffer(&dx, (int)x.size());
+  allocate_gpu_buffer(&dw, (int)E);
+  allocate_gpu_buffer(&dout, (int)got.size());
+  move_data_in(dx, x.data(), 0, Vs, F);
+  move_data_in(dw, w.data(), 0, E, 1);
+  zero_buffer(dout, (int)got.size());
+  cs.Gather_By_Dst_From_Src(dx, dout, dw, csc.row_indices, csc.column_offset, 0, 0, 0, 0, E, Vd, F, true, false);
+  cs.CUDA_DEVICE_SYNCHRONIZE();
+  move_result_out(got.data(), dout, 0, Vd, F);
+  EXPECT(memcmp(got.data(), ref.data(), got.size() * sizeof(float)) == 0);
+
+  // second call accumulates into the same buffer (the reference's += semantics)
+  cs.Gather_By_Dst_From_Src_Optim(dx, dout, dw, csc.row_indices, csc.column_offset, 0, 0, 0, 0, E, Vd, F, true, false);
+  cs.CUDA_DEVICE_SYNCHRONIZE();
+  move_result_out(got.data(), dout, 0, Vd, F);
+  bool twice = true;
+  for (size_t i = 0; i < got.size(); ++i) twice = twice && fabsf(got[i] - 2.f * ref[i]) <= 1e-5f * (1.f + fabsf(ref[i]));
+  EXPECT(twice);
+
+  // zero-copy feature gather from mapped pinned host memory + label gather
+  float *pinned = (float *)cudaMallocPinned((long)x.size() * sizeof(float));
+  memcpy(pinned, x.data(), x.size() * sizeof(float));
+  float *pinned_dev = (float *)getDevicePointer(pinned);
+  std::vector<VertexId_CUDA> ids(200);
+  for (auto &v : ids) v = next() % Vs;
+  VertexId_CUDA *dids;
+  allocate_gpu_edge(&dids, (int)ids.size());
+  move_edge_in(dids, ids.data(), 0, (VertexId_CUDA)ids.size(), 1);
+  float *dbatch;
+  allocate_gpu_buffer(&dbatch, (int)(ids.size() * F));
+  cs.zero_copy_feature_move_gpu(dbatch, pinned_dev, dids, F, (VertexId_CUDA)ids.size());
+  std::vector<float> batch(ids.size() * F);
+  move_result_out(batch.data(), dbatch, 0, (int)ids.size(), F);
+  bool rows_ok = true;
+  for (size_t i = 0; i < ids.size(); ++i)
+    rows_ok = rows_ok && memcmp(&batch[i * F], &x[(size_t)ids[i] * F], F * sizeof(float)) == 0;
+  EXPECT(rows_ok);
+  std::vector<long> labels(Vs), lab_out(ids.size());
+  for (VertexId_CUDA v = 0; v < Vs; ++v) labels[v] = (long)(v * 7 % 41);
+  long *dlab, *dlab_out;
+  alloc_gpu_data(&dlab, (int)Vs);
+  alloc_gpu_data(&dlab_out, (int)ids.size());
+  move_bytes_in(dlab, labels.data(), (long)labels.size() * sizeof(long));
+  cs.global_copy_label_move_gpu(dlab_out, dlab, dids, (VertexId_CUDA)ids.size());
+  NTS_VENEER_CHECK(nts_memcpy_d2h(lab_out.data(), dlab_out, lab_out.size() * sizeof(long), 1));
+  bool lab_ok = true;
+  for (size_t i = 0; i < ids.size(); ++i) lab_ok = lab_ok && lab_out[i] == labels[ids[i]];
+  EXPECT(lab_ok);
+
+  // edge softmax through the veneer, with a separate cache buffer
+  std::vector<float> logits(E), alpha(E), cached(E);
+  for (auto &v : logits) v = (float)(next() % 4001) / 1000.f - 2.f;
+  float *dlog, *dalpha, *dcache;
+  allocate_gpu_buffer(&dlog, (int)E);
+  allocate_gpu_buffer(&dalpha, (int)E);
+  allocate_gpu_buffer(&dcache, (int)E);
+  move_data_in(dlog, logits.data(), 0, E, 1);
+  cs.Edge_Softmax_Forward_Block(dalpha, dlog, dcache, csc.row_indices, csc.column_offset, Vd, 1);
+  cs.CUDA_DEVICE_SYNCHRONIZE();
+  move_result_out(alpha.data(), dalpha, 0, E, 1);
+  move_result_out(cached.data(), dcache, 0, E, 1);
+  bool sm_ok = memcmp(alpha.data(), cached.data(), E * sizeof(float)) == 0;
+  for (VertexId_CUDA d = 0; d < Vd; ++d) {
+    double s = 0;
+    for (VertexId_CUDA e = co[d]; e < co[d + 1]; ++e) s += alpha[e];
+    if (co[d + 1] > co[d]) sm_ok = sm_ok && fabs(s - 1.0) < 1e-5;
+  }
+  EXPECT(sm_ok);
+
+  double used = 0, total = 0;
+  get_gpu_mem(used, total);
+  EXPECT(total > 1024.0 && used >= 0.0);
+
+  csc.release();
+  FreeBuffer(dx); FreeBuffer(dw); FreeBuffer(dout); FreeBuffer(dbatch); FreeBuffer(dlog); FreeBuffer(dalpha);
+  FreeBuffer(dcache); FreeEdge(dids); free_gpu_data(dlab); free_gpu_data(dlab_out); ntsFreeHost(pinned);
+  printf(failures ? "veneer test: %d failure(s)\n" : "veneer test: ok\n", failures);
+  return failures ? 1 : 0;
+}
