@@ -45,7 +45,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--vertices", type=int, default=V_REDDIT)
     ap.add_argument("--edges", type=int, default=E_REDDIT)
-    ap.add_argument("--chunk", type=int, default=0, help="edges per chunk of a split hub row (0 = library default)")
+    ap.add_argument("--chunk", type=int, default=1024, help="largest number of edges in one piece of a split hub row")
+    ap.add_argument("--slabs", type=int, default=16,
+                    help="source ranges of the cache-aware schedule (1 = split hub rows by edge count only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB row copy (identity gather) so that HBM byte counters can be scaled")
@@ -67,8 +69,8 @@ def main():
     V, E = args.vertices, args.edges
 
     t0 = time.time()
-    src, dst = synth.rmat_edges(V, E, 0.57, 0.19, 0.19, seed=3, device=dev)
-    chunk = FullGraphChunk.from_edges(src, dst, V, args.chunk)
+    src, dst = synth.rmat_edges(V, E, 0.57, 0.19, 0.19, seed=3, device=dev, sort=True)
+    chunk = FullGraphChunk.from_edges(src, dst, V, args.chunk, args.slabs)
     del src, dst
     x0 = synth.normal_features(V, F_IN, seed=31, device=dev)
     h1 = synth.normal_features(V, F_HID, seed=32, device=dev)
@@ -102,37 +104,57 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    # Timed region: exactly `steps` steps between two synchronisations.
+    # One HIP event pair per aggregation launch of the timed region (4 per step).  The library records
+    # them on the launch stream immediately before and after its main gather kernel; nothing waits on
+    # them until the timed region is over.
     stream = torch.cuda.current_stream().cuda_stream
+    n_ev = 4 * args.steps
+    events = []
+    for _ in range(n_ev):
+        a, b = ctypes.c_void_p(), ctypes.c_void_p()
+        call("nts_event_create", ctypes.byref(a))
+        call("nts_event_create", ctypes.byref(b))
+        events.append((a, b))
+    fwd, bwd = chunk.plan_forward.handle, chunk.plan_backward.handle
+
+    def timed_step(i):
+        call("nts_spmm_plan_set_events", fwd, *events[4 * i + 0])
+        op.forward(x0)
+        call("nts_spmm_plan_set_events", fwd, *events[4 * i + 1])
+        op.forward(h1)
+        call("nts_spmm_plan_set_events", bwd, *events[4 * i + 2])
+        op.backward(g1)
+        call("nts_spmm_plan_set_events", bwd, *events[4 * i + 3])
+        op.backward(g0)
+
+    # Timed region: exactly `steps` steps between two synchronisations.
+    torch.cuda.synchronize()
     t_start = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        timed_step(i)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t_start
     ms_per_step = elapsed * 1e3 / args.steps
     edges_per_s = 4.0 * E / (elapsed / args.steps)
+    call("nts_spmm_plan_set_events", fwd, None, None)
+    call("nts_spmm_plan_set_events", bwd, None, None)
 
-    # Dominant kernel: the F=602 forward gather.  HIP events recorded by the library on the launch
-    # stream immediately before and after that kernel, one launch at a time.
-    ev0, ev1 = ctypes.c_void_p(), ctypes.c_void_p()
-    call("nts_event_create", ctypes.byref(ev0))
-    call("nts_event_create", ctypes.byref(ev1))
-    call("nts_spmm_plan_set_events", chunk.plan_forward.handle, ev0, ev1)
     durs = []
-    for _ in range(max(3, min(args.steps, 10))):
-        op.forward(x0)
+    for a, b in events:
         ms = ctypes.c_float()
-        call("nts_event_elapsed_ms", ctypes.byref(ms), ev0, ev1)
+        call("nts_event_elapsed_ms", ctypes.byref(ms), a, b)
         durs.append(ms.value)
-    call("nts_spmm_plan_set_events", chunk.plan_forward.handle, None, None)
-    call("nts_event_destroy", ev0)
-    call("nts_event_destroy", ev1)
-    kernel_ms = sum(durs) / len(durs)
+        call("nts_event_destroy", a)
+        call("nts_event_destroy", b)
+    per_pass = [sum(durs[k::4]) / args.steps for k in range(4)]  # fwd602, fwd128, bwd128, bwd602
+    # Dominant kernel: the F=602 gather (spmm_wave_kernel<2,5>), launched twice per step: forward
+    # over the CSC and backward over the CSR.  Same algorithmic bytes per launch for both.
+    kernel_ms = (per_pass[0] + per_pass[3]) / 2
     algo = algorithmic_bytes(E, V, F_IN)
     achieved = algo / (kernel_ms * 1e-3) / 1e9
     roofline = {
         "bound": "hbm",
-        "kernel": "spmm_wave_kernel<2,5> (F=602 forward gather)",
+        "kernel": "spmm_wave_kernel<2,5> (F=602 gather, forward and backward launches)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -140,6 +162,8 @@ def main():
         "traffic": TRAFFIC_BYTES_F602,
         "algorithmic_bytes": algo,
         "kernel_ms": round(kernel_ms, 3),
+        "per_pass_ms": {"fwd_F602": round(per_pass[0], 3), "fwd_F128": round(per_pass[1], 3),
+                        "bwd_F128": round(per_pass[2], 3), "bwd_F602": round(per_pass[3], 3)},
     }
 
     cpu_baseline = None
@@ -163,9 +187,9 @@ def main():
             "workload": "Reddit-shaped full-graph 2-layer GCN aggregation fwd+bwd (F=602,128)",
             "vertices": V,
             "edges": E,
-            "graph": "R-MAT a=.57 b=.19 c=.19, seed 3, ids permuted",
+            "graph": "R-MAT a=.57 b=.19 c=.19, seed 3, ids permuted, edge list in (src, dst) order, duplicates kept",
             "passes_per_step": 4,
-            "plan": chunk.plan_forward.info(),
+            "plan": dict(chunk.plan_forward.info(), chunk_edges=args.chunk, slabs=args.slabs),
             "setup_s": round(setup_s, 2),
         },
         "roofline": roofline,

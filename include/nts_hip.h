@@ -130,6 +130,16 @@ int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t 
 typedef struct nts_spmm_plan nts_spmm_plan_t;
 int nts_spmm_plan_create(nts_spmm_plan_t **plan, const uint32_t *offsets, uint32_t rows,
                          uint32_t edges, uint32_t chunk_edges, nts_stream_t stream);
+/* The same schedule, made cache-aware: `indices` (the gather index array that belongs to `offsets`)
+ * is read back once as well, and the pieces of split rows whose indices ascend are cut at the
+ * boundaries of `n_slabs` equal ranges of [index_base, index_base + n_index) and issued slab by slab,
+ * so that concurrently running wavefronts gather from the same range of source rows (each XCD's
+ * L2 then holds that range's hot rows).  n_slabs = 0 selects the default; rows whose indices do
+ * not ascend are split by edge count as above.  Results differ from nts_spmm_plan_create only in
+ * where split rows are cut. */
+int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan, const uint32_t *offsets, const uint32_t *indices,
+                               uint32_t index_base, uint32_t n_index, uint32_t rows, uint32_t edges,
+                               uint32_t chunk_edges, uint32_t n_slabs, nts_stream_t stream);
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan);
 /* Number of work items, split rows and partial-sum slots of a plan (for tests and reports). */
 int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows,

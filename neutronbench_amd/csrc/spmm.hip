@@ -412,43 +412,64 @@ int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t 
   return NTS_OK;
 }
 
-int nts_spmm_plan_create(nts_spmm_plan_t **plan_out, const uint32_t *offsets, uint32_t rows, uint32_t edges,
-                         uint32_t chunk_edges, nts_stream_t stream) {
-  if (!plan_out) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null out-pointer");
-  *plan_out = nullptr;
-  if (rows != 0 && !offsets) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null offsets");
-  const uint32_t chunk = chunk_edges ? chunk_edges : 4096u;
+namespace {
 
-  std::vector<uint32_t> off(static_cast<size_t>(rows) + 1, 0u);
-  if (rows) {
-    NTS_HIP_TRY(hipMemcpyAsync(off.data(), offsets, off.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-    NTS_HIP_TRY(hipStreamSynchronize(stream));
-    if (off[rows] != edges) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: offsets[rows] != edges");
-    for (uint32_t r = 0; r < rows; ++r) {
-      if (off[r + 1] < off[r]) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: offsets not ascending");
-    }
-  }
+struct Piece {
+  uint32_t slab, row, e0, e1, slot;
+};
 
-  // Items: first the chunks of split rows (all near `chunk` edges, the heaviest work), then the
-  // unsplit rows by descending degree (counting sort, stable in the row id).
-  std::vector<uint4> items;
+// Builds the work-item list.  Rows with more than `chunk` edges are split into pieces that write
+// partial sums (slots numbered in ascending edge order inside a row, so the second-stage sum has
+// a fixed order).  With n_slabs > 1 and a host copy of the gather indices, pieces of rows whose
+// indices ascend are additionally cut at the boundaries of n_slabs equal ranges of the gather
+// index space and the pieces are ordered slab by slab: wavefronts that run at the same time then
+// gather from the same 1/n_slabs of the source rows, which is what lets each 4 MB L2 keep that
+// range's hot rows resident.  Items: all pieces (slab-major, longest first inside a slab), then
+// the unsplit rows by descending degree.
+int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const std::vector<uint32_t> &off,
+               const uint32_t *idx, uint32_t rows, uint32_t edges, uint32_t chunk, uint32_t n_slabs,
+               uint32_t n_index) {
+  std::vector<Piece> pieces;
   std::vector<uint4> splits;
-  items.reserve(static_cast<size_t>(rows) + edges / chunk + 1);
   uint32_t n_partials = 0;
   std::vector<uint32_t> bucket(static_cast<size_t>(chunk) + 2, 0u);
+  const bool slabbed = n_slabs > 1 && idx != nullptr && n_index > 0;
+  const uint64_t slab_width = slabbed ? (static_cast<uint64_t>(n_index) + n_slabs - 1) / n_slabs : 0;
   for (uint32_t r = 0; r < rows; ++r) {
-    const uint32_t deg = off[r + 1] - off[r];
-    if (deg > chunk) {
-      const uint32_t first = n_partials;
-      for (uint32_t e = off[r]; e < off[r + 1]; e += chunk) {
-        const uint32_t end = std::min(off[r + 1], e + chunk);
-        items.push_back(make_uint4(r, e, end, n_partials++));
-      }
-      splits.push_back(make_uint4(r, first, n_partials - first, 0u));
-    } else {
+    const uint32_t b = off[r], e = off[r + 1], deg = e - b;
+    if (deg <= chunk) {
       ++bucket[chunk - deg + 1];  // descending degree
+      continue;
     }
+    const uint32_t first = n_partials;
+    bool ascending = slabbed;
+    if (slabbed)
+      for (uint32_t k = b + 1; k < e && ascending; ++k) ascending = idx[k - 1] <= idx[k];
+    if (ascending) {
+      uint32_t cut = b;
+      for (uint32_t sl = 0; sl < n_slabs && cut < e; ++sl) {
+        const uint64_t hi = (sl + 1) * slab_width;  // first index value of the next slab
+        const uint32_t stop =
+            sl + 1 == n_slabs ? e
+                              : static_cast<uint32_t>(std::lower_bound(idx + cut, idx + e, hi,
+                                                                       [](uint32_t v, uint64_t lim) { return v < lim; }) -
+                                                      idx);
+        for (uint32_t k = cut; k < stop; k += chunk)
+          pieces.push_back(Piece{sl, r, k, std::min(stop, k + chunk), n_partials++});
+        cut = stop;
+      }
+    } else {
+      for (uint32_t k = b; k < e; k += chunk) pieces.push_back(Piece{0u, r, k, std::min(e, k + chunk), n_partials++});
+    }
+    splits.push_back(make_uint4(r, first, n_partials - first, 0u));
   }
+  std::stable_sort(pieces.begin(), pieces.end(), [](const Piece &a, const Piece &b) {
+    if (a.slab != b.slab) return a.slab < b.slab;
+    return (a.e1 - a.e0) > (b.e1 - b.e0);
+  });
+  std::vector<uint4> items;
+  items.reserve(pieces.size() + rows);
+  for (const Piece &pc : pieces) items.push_back(make_uint4(pc.row, pc.e0, pc.e1, pc.slot));
   for (size_t i = 1; i < bucket.size(); ++i) bucket[i] += bucket[i - 1];
   const size_t base = items.size();
   items.resize(base + bucket.back());
@@ -462,7 +483,7 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan_out, const uint32_t *offsets, ui
   p->rows = rows;
   p->edges = edges;
   p->chunk = chunk;
-  p->offsets = offsets;
+  p->offsets = offsets_dev;
   p->n_items = static_cast<uint32_t>(items.size());
   p->n_splits = static_cast<uint32_t>(splits.size());
   p->n_partials = n_partials;
@@ -483,6 +504,50 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan_out, const uint32_t *offsets, ui
   }
   *plan_out = p;
   return NTS_OK;
+}
+
+int read_offsets(std::vector<uint32_t> &off, const uint32_t *offsets, uint32_t rows, uint32_t edges,
+                 hipStream_t stream) {
+  off.assign(static_cast<size_t>(rows) + 1, 0u);
+  if (!rows) return NTS_OK;
+  NTS_HIP_TRY(hipMemcpyAsync(off.data(), offsets, off.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+  NTS_HIP_TRY(hipStreamSynchronize(stream));
+  if (off[rows] != edges) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: offsets[rows] != edges");
+  for (uint32_t r = 0; r < rows; ++r)
+    if (off[r + 1] < off[r]) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: offsets not ascending");
+  return NTS_OK;
+}
+
+}  // namespace
+
+int nts_spmm_plan_create(nts_spmm_plan_t **plan_out, const uint32_t *offsets, uint32_t rows, uint32_t edges,
+                         uint32_t chunk_edges, nts_stream_t stream) {
+  if (!plan_out) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null out-pointer");
+  *plan_out = nullptr;
+  if (rows != 0 && !offsets) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null offsets");
+  std::vector<uint32_t> off;
+  if (int rc = read_offsets(off, offsets, rows, edges, stream)) return rc;
+  return build_plan(plan_out, offsets, off, nullptr, rows, edges, chunk_edges ? chunk_edges : 4096u, 1u, 0u);
+}
+
+int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan_out, const uint32_t *offsets, const uint32_t *indices,
+                               uint32_t index_base, uint32_t n_index, uint32_t rows, uint32_t edges,
+                               uint32_t chunk_edges, uint32_t n_slabs, nts_stream_t stream) {
+  if (!plan_out) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create_slabs: null out-pointer");
+  *plan_out = nullptr;
+  if (rows != 0 && !offsets) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create_slabs: null offsets");
+  if (edges != 0 && !indices) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create_slabs: null indices");
+  std::vector<uint32_t> off;
+  if (int rc = read_offsets(off, offsets, rows, edges, stream)) return rc;
+  std::vector<uint32_t> idx(edges);
+  if (edges) {
+    NTS_HIP_TRY(hipMemcpyAsync(idx.data(), indices, idx.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    NTS_HIP_TRY(hipStreamSynchronize(stream));
+    if (index_base)
+      for (uint32_t &v : idx) v -= index_base;
+  }
+  return build_plan(plan_out, offsets, off, idx.data(), rows, edges, chunk_edges ? chunk_edges : 4096u,
+                    n_slabs ? n_slabs : 16u, n_index);
 }
 
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {

@@ -30,11 +30,17 @@ def u32_to_i64(t):
 class SpmmPlan:
     """Degree-bucketed schedule bound to one offsets tensor."""
 
-    def __init__(self, offsets, rows, edges, chunk_edges=0):
+    def __init__(self, offsets, rows, edges, chunk_edges=0, indices=None, n_index=0, n_slabs=0):
+        """indices / n_index given: cache-aware schedule (split rows cut at source-range boundaries
+        and issued range by range); otherwise split rows are cut every chunk_edges edges."""
         self.offsets = offsets
         handle = ctypes.c_void_p()
-        call("nts_spmm_plan_create", ctypes.byref(handle), ptr(offsets), rows, edges, chunk_edges,
-             _stream(offsets.device))
+        if indices is not None:
+            call("nts_spmm_plan_create_slabs", ctypes.byref(handle), ptr(offsets), ptr(indices), 0, n_index, rows,
+                 edges, chunk_edges, n_slabs, _stream(offsets.device))
+        else:
+            call("nts_spmm_plan_create", ctypes.byref(handle), ptr(offsets), rows, edges, chunk_edges,
+                 _stream(offsets.device))
         self.handle = handle.value
 
     def info(self):
@@ -60,7 +66,7 @@ class SpmmPlan:
 class FullGraphChunk:
     """One partition's CSC + CSR + GCN weights in HBM, plus the aggregation schedules."""
 
-    def __init__(self, V, column_offset, row_indices, ewf, row_offset, column_indices, ewb, chunk_edges=0):
+    def __init__(self, V, column_offset, row_indices, ewf, row_offset, column_indices, ewb, chunk_edges=0, n_slabs=1):
         self.V = V
         self.E = int(row_indices.numel())
         self.column_offset_gpu = column_offset
@@ -71,11 +77,15 @@ class FullGraphChunk:
         self.edge_weight_backward_gpu = ewb
         self.src_range = (0, V)
         self.dst_range = (0, V)
-        self.plan_forward = SpmmPlan(column_offset, V, self.E, chunk_edges)
-        self.plan_backward = SpmmPlan(row_offset, V, self.E, chunk_edges)
+        if n_slabs == 1:
+            self.plan_forward = SpmmPlan(column_offset, V, self.E, chunk_edges)
+            self.plan_backward = SpmmPlan(row_offset, V, self.E, chunk_edges)
+        else:
+            self.plan_forward = SpmmPlan(column_offset, V, self.E, chunk_edges, row_indices, V, n_slabs)
+            self.plan_backward = SpmmPlan(row_offset, V, self.E, chunk_edges, column_indices, V, n_slabs)
 
     @classmethod
-    def from_edges(cls, src, dst, V, chunk_edges=0):
+    def from_edges(cls, src, dst, V, chunk_edges=0, n_slabs=1):
         """Builds the chunk on the device that holds `src` / `dst` (int64 edge list).
 
         Edge order follows PartitionToChunks (core/PartitionedGraph.hpp:281-388): the COO list is
@@ -102,7 +112,7 @@ class FullGraphChunk:
         ewb = torch.empty(E, dtype=torch.float32, device=device)
         call("nts_gcn_edge_weights", ptr(ewf), ptr(ewb), ptr(co32), ptr(ri32), ptr(ro32), ptr(ci32), V, V,
              _stream(device))
-        return cls(V, co32, ri32, ewf, ro32, ci32, ewb, chunk_edges)
+        return cls(V, co32, ri32, ewf, ro32, ci32, ewb, chunk_edges, n_slabs)
 
 
 class SampledLayer:

@@ -47,8 +47,10 @@ def permutation(n, seed, device="cpu"):
     return torch.argsort(keys, stable=True)
 
 
-def rmat_edges(V, E, a=0.57, b=0.19, c=0.19, seed=1, device="cpu", permute=True):
-    """R-MAT directed edge list (src, dst) as int64 tensors of length E."""
+def rmat_edges(V, E, a=0.57, b=0.19, c=0.19, seed=1, device="cpu", permute=True, sort=False):
+    """R-MAT directed edge list (src, dst) as int64 tensors of length E.  sort=True returns the list
+    in (source, destination) order, the order of an edge file exported from sorted adjacency lists;
+    duplicates are kept either way."""
     scale = max(1, math.ceil(math.log2(V)))
     ta = int(a * (1 << 24))
     tb = int((a + b) * (1 << 24))
@@ -69,6 +71,9 @@ def rmat_edges(V, E, a=0.57, b=0.19, c=0.19, seed=1, device="cpu", permute=True)
         p = permutation(V, seed, device)
         src = p[src]
         dst = p[dst]
+    if sort:
+        order = torch.sort(src * V + dst).indices
+        src, dst = src[order], dst[order]
     return src, dst
 
 

@@ -171,3 +171,40 @@ def test_empty_and_error_paths(device):
     # plan creation rejects inconsistent offsets
     handle = ctypes.c_void_p()
     assert abi.status("nts_spmm_plan_create", ctypes.byref(handle), ptr(off), 4, 7, 0, s) == abi.NTS_ERR_INVALID
+
+
+@pytest.mark.parametrize("F,chunk,slabs,sorted_rows", [(128, 64, 4, True), (602, 100, 8, True), (41, 32, 16, True),
+                                                       (100, 64, 8, False), (16, 16, 3, True)])
+def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
+    """Source-range ("slab") schedule: same results as the oracle to tolerance, bit-reproducible, and
+    rows whose indices do not ascend fall back to edge-count chunks."""
+    print(f"case F={F} chunk={chunk} slabs={slabs} sorted={sorted_rows}", flush=True)
+    Vd, Vs = 400, 900
+    co, ri = random_block(Vd, Vs, 25, seed=F + slabs, hub=2500, dup=True)
+    if sorted_rows:
+        for d in range(Vd):
+            ri[co[d]:co[d + 1]] = np.sort(ri[co[d]:co[d + 1]])
+    rng = np.random.default_rng(F)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    w = rng.random(ri.size).astype(np.float32)
+    dx, dw, dco, dri = _dev(x, device), _dev(w, device), _dev(co, device), _dev(ri, device)
+    plan = SpmmPlan(dco, Vd, ri.size, chunk, dri, Vs, slabs)
+    info = plan.info()
+    deg = np.diff(co.astype(np.int64))
+    assert info["split_rows"] == int((deg > chunk).sum())
+    plain = int(np.ceil(deg[deg > chunk] / chunk).sum())
+    if sorted_rows:
+        assert plain <= info["partials"] <= plain + info["split_rows"] * slabs
+    else:
+        assert info["partials"] == plain
+    outs = []
+    for _ in range(2):
+        out = torch.full((Vd, F), float("nan"), device=device)
+        call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, F, 0, _stream())
+        torch.cuda.synchronize()
+        outs.append(out.cpu().numpy())
+    check(outs[0], oracle.spmm(x, w, co, ri, Vd), abs_term_scale(x, w, co, ri, Vd))
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    keep = deg <= chunk
+    assert np.array_equal(outs[0][keep].view(np.uint32), oracle.spmm(x, w, co, ri, Vd, fused=True)[keep].view(np.uint32))
+    plan.close()
