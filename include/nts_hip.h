@@ -186,6 +186,14 @@ int nts_gather_edge_to_dst(float *out, const float *msg, const uint32_t *co, uin
 int nts_gather_edge_to_src(float *out, const float *msg, const uint32_t *ro, const uint32_t *perm,
                            uint32_t Vs, uint32_t F, int accumulate, nts_stream_t stream);
 
+/* The reference's own argument list of Gather_Msg_To_Src_Mirror (cuda/ntsCUDA.hpp:149-151), for
+ * callers that have no transposed structure: out[mirror ? mirror[ri[e]] : ri[e], :] += msg[e, :] for
+ * every CSC edge e.  Deterministic (edges of one target row are added in ascending edge order): the
+ * call sorts the edges by target row in stream-ordered temporary memory, so it costs a sort per
+ * call and reads co[Vd] back (synchronises `stream`).  Prefer nts_gather_edge_to_src. */
+int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t *ri, const uint32_t *co,
+                                    const uint32_t *mirror, uint32_t Vd, uint32_t F, nts_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Edge softmax and fused GAT attention.  H = number of heads (columns); edge tensors [E, H].
  * ------------------------------------------------------------------------------------------- */

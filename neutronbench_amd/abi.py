@@ -60,6 +60,7 @@ SIGNATURES = {
     "nts_scatter_grad_to_edge": [_vp, _vp, _vp, _u32, _u32, _vp],
     "nts_gather_edge_to_dst": [_vp, _vp, _vp, _u32, _u32, _int, _vp],
     "nts_gather_edge_to_src": [_vp, _vp, _vp, _vp, _u32, _u32, _int, _vp],
+    "nts_gather_edge_to_src_unsorted": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],
     "nts_edge_softmax_fwd": [_vp, _vp, _vp, _u32, _u32, _vp],
     "nts_edge_softmax_bwd": [_vp, _vp, _vp, _vp, _u32, _u32, _vp],
     "nts_gat_attention_fwd": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp],

@@ -68,6 +68,34 @@ __global__ __launch_bounds__(256) void edge_weights_kernel(float *__restrict__ w
   wout[e] = which == 0 ? norm_weight(other_deg, own_deg) : norm_weight(own_deg, other_deg);
 }
 
+// keys[e] = mirror ? mirror[ri[e]] : ri[e]
+__global__ __launch_bounds__(256) void target_keys_kernel(uint32_t *__restrict__ keys, const uint32_t *__restrict__ ri,
+                                                          const uint32_t *__restrict__ mirror, uint32_t E) {
+  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= E) return;
+  const uint32_t s = ri[e];
+  keys[e] = mirror ? mirror[s] : s;
+}
+
+// One wave per sorted position; only the first position of a run of equal keys works: it adds the
+// run's edge rows in sorted (= ascending edge id) order into out[key].
+__global__ __launch_bounds__(256) void add_runs_kernel(float *__restrict__ out, const float *__restrict__ msg,
+                                                       const uint32_t *__restrict__ keys,
+                                                       const uint32_t *__restrict__ perm, uint32_t E, uint32_t F) {
+  const uint32_t k = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (k >= E) return;
+  const uint32_t key = keys[k];
+  if (k > 0 && keys[k - 1] == key) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint32_t end = k + 1;
+  while (end < E && keys[end] == key) ++end;
+  for (uint32_t c = lane; c < F; c += kWave) {
+    float a = 0.f;
+    for (uint32_t j = k; j < end; ++j) a += msg[static_cast<size_t>(perm[j]) * F + c];
+    out[static_cast<size_t>(key) * F + c] += a;
+  }
+}
+
 inline unsigned bits_for(uint32_t n) {  // bits needed to represent values in [0, n)
   unsigned b = 1;
   while (b < 32 && (1ull << b) < n) ++b;
@@ -127,6 +155,38 @@ int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t 
   NTS_LAUNCH_CHECK("offsets_from_sorted_kernel");
   hipLaunchKernelGGL(dst_of_perm_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ci, perm_out, co, Vd, E);
   NTS_LAUNCH_CHECK("dst_of_perm_kernel");
+  return NTS_OK;
+}
+
+int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t *ri, const uint32_t *co,
+                                    const uint32_t *mirror, uint32_t Vd, uint32_t F, nts_stream_t stream) {
+  if (F == 0) return fail(NTS_ERR_INVALID, "nts_gather_edge_to_src_unsorted: F is 0");
+  if (Vd == 0) return NTS_OK;
+  if (!out || !msg || !ri || !co) return fail(NTS_ERR_INVALID, "nts_gather_edge_to_src_unsorted: null pointer");
+  uint32_t E = 0;
+  NTS_HIP_TRY(hipMemcpyAsync(&E, co + Vd, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+  NTS_HIP_TRY(hipStreamSynchronize(stream));
+  if (E == 0) return NTS_OK;
+  size_t tmp = 0;
+  NTS_HIP_TRY(sort_temp_bytes(E, &tmp));
+  const size_t arr = align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256);
+  unsigned char *work = nullptr;
+  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&work), 3 * arr + align_up(tmp, 256), stream));
+  uint32_t *keys = reinterpret_cast<uint32_t *>(work);
+  uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(work + arr);
+  uint32_t *perm = reinterpret_cast<uint32_t *>(work + 2 * arr);
+  hipLaunchKernelGGL(target_keys_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, keys, ri, mirror, E);
+  hipError_t err = hipGetLastError();
+  if (err == hipSuccess)
+    err = rocprim::radix_sort_pairs(work + 3 * arr, tmp, keys, keys_sorted, rocprim::counting_iterator<uint32_t>(0u),
+                                    perm, E, 0u, 32u, stream, false);
+  if (err == hipSuccess) {
+    hipLaunchKernelGGL(add_runs_kernel, dim3(ceil_div(E, 4)), dim3(256), 0, stream, out, msg, keys_sorted, perm, E, F);
+    err = hipGetLastError();
+  }
+  hipError_t ferr = hipFreeAsync(work, stream);
+  if (err != hipSuccess) return fail_hip(err, "nts_gather_edge_to_src_unsorted");
+  if (ferr != hipSuccess) return fail_hip(ferr, "nts_gather_edge_to_src_unsorted: hipFreeAsync");
   return NTS_OK;
 }
 

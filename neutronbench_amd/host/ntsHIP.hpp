@@ -107,12 +107,12 @@ inline void CUDA_DEVICE_SYNCHRONIZE() { NTS_VENEER_CHECK(nts_device_sync()); }
 inline int cudaFree(void *p) { return nts_free_device(p); }
 inline int cudaStreamSynchronize(cudaStream_t s) { return nts_stream_sync(s); }
 
-// utils/cuda_memory.hpp: used, total in MiB.
-inline void get_gpu_mem(double &used, double &total) {
-  size_t free_b = 0, total_b = 0;
-  NTS_VENEER_CHECK(nts_mem_info(&free_b, &total_b));
-  used = (double)(total_b - free_b) / 1024.0 / 1024.0;
-  total = (double)total_b / 1024.0 / 1024.0;
+// cudaMallocManaged as the data loader uses it (core/ntsDataloador.hpp:66-73): memory that both the
+// host and the device address.  Page-locked mapped host memory has that property; the device reads
+// it in place (zero-copy), which is how the feature table is consumed anyway.
+template <typename T>
+inline int cudaMallocManaged(T **ptr, size_t bytes) {
+  return nts_malloc_pinned_mapped((void **)ptr, bytes);
 }
 
 // ---- deviceCSC (cuda/ntsCUDA.hpp:54-97) ----------------------------------------------------------
@@ -265,7 +265,14 @@ class Cuda_Stream {
     (void)row_indices;
     NTS_VENEER_CHECK(nts_gather_edge_to_dst(dst_feature, message, column_offset, batch_size, feature_size, 1, stream));
   }
-  // Deterministic replacement of Gather_Msg_To_Src_Mirror: takes the transposed structure
+  // Reference argument list; deterministic, but sorts the edges by target row on every call.
+  void Gather_Msg_To_Src_Mirror(float *src_mirror_feature, float *message, VertexId_CUDA *row_indices,
+                                VertexId_CUDA *column_offset, VertexId_CUDA *mirror_index, VertexId_CUDA batch_size,
+                                VertexId_CUDA feature_size) {
+    NTS_VENEER_CHECK(nts_gather_edge_to_src_unsorted(src_mirror_feature, message, row_indices, column_offset,
+                                                     mirror_index, batch_size, feature_size, stream));
+  }
+  // Cheaper deterministic form of the same operation: takes the transposed structure
   // (row_offset [src_size+1], csr_to_csc [E]) instead of (row_indices, column_offset, mirror_index).
   void Gather_Msg_To_Src(float *src_feature, float *message, VertexId_CUDA *row_offset, VertexId_CUDA *csr_to_csc,
                          VertexId_CUDA src_size, VertexId_CUDA feature_size) {
@@ -292,6 +299,25 @@ class Cuda_Stream {
     (void)row_indices;
     NTS_VENEER_CHECK(nts_edge_softmax_bwd(msg_input_grad, msg_output_grad, msg_cached, column_offset, batch_size,
                                           feature_size, stream));
+  }
+
+  // Declared by the reference but never defined there (cuda/ntsCUDA.hpp:180-187); kept so that
+  // core/NtsScheduler.hpp parses.  Calling them is a link error, as it is in the reference.
+  void Gather_By_Dst_From_Message(float *input, float *output, VertexId_CUDA *src, VertexId_CUDA *dst,
+                                  VertexId_CUDA src_start, VertexId_CUDA src_end, VertexId_CUDA dst_start,
+                                  VertexId_CUDA dst_end, VertexId_CUDA edges, VertexId_CUDA batch_size,
+                                  VertexId_CUDA feature_size, bool with_weight = false, bool tensor_weight = false);
+  void zero_copy_embedding_move_gpu(float *dev_feature, float *pinned_host_feature, VertexId_CUDA feature_size,
+                                    VertexId_CUDA vertex_size);
+  // Unpacking of multi-rank MPI message buffers (cuda/ntsCUDATransferKernel.cuh:30-93): part of the
+  // distributed path, which this single-GPU library does not implement.  They fail loudly.
+  void aggregate_comm_result(float *, float *, VertexId_CUDA, int, int, bool = true) { dist_unsupported(); }
+  void aggregate_comm_result_debug(float *, float *, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA,
+                                   bool) {
+    dist_unsupported();
+  }
+  void deSerializeToGPU(float *, float *, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA, bool) {
+    dist_unsupported();
   }
 
   // Mini-batch assembly; like the reference these return with the result complete.
@@ -329,6 +355,10 @@ class Cuda_Stream {
   }
 
  private:
+  static void dist_unsupported() {
+    printf("the distributed (MPI message buffer) GPU path is not part of the single-GPU HIP library\n");
+    exit(1);
+  }
   static void reject_tensor_weight(bool tensor) {
     if (tensor) {
       printf("tensor-weight aggregation is a legacy implementation\n");

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "ntsHIP.hpp"
+#include "compat/utils/cuda_memory.hpp"
 
 static int failures = 0;
 #define EXPECT(cond)                                            \

@@ -56,6 +56,30 @@ def test_scatter_and_gather(device, F):
     assert np.array_equal(outs.cpu().numpy(), oracle.gather_to_src(em, co, ri, Vs))
 
 
+@pytest.mark.parametrize("F", [1, 4, 33, 128])
+def test_gather_to_src_with_reference_arguments(device, F):
+    """The reference's argument list (row_indices, column_offset, mirror_index; no transposed
+    structure): deterministic, accumulates into the output, equals the oracle's edge-order sum."""
+    co, ri, ro, ci, perm, Vd, Vs = _block(50 + F, hub=200, dup=True)
+    E = ri.size
+    rng = np.random.default_rng(F)
+    em = rng.standard_normal((E, F)).astype(np.float32)
+    mirror = rng.permutation(Vs).astype(np.uint32)
+    init = rng.standard_normal((Vs, F)).astype(np.float32)
+    dco, dri, dem, dmir = dev(co, device), dev(ri, device), dev(em, device), dev(mirror, device)
+    for m, dm in ((None, None), (mirror, dmir)):
+        outs = []
+        for _ in range(2):
+            out = dev(init, device)
+            call("nts_gather_edge_to_src_unsorted", ptr(out), ptr(dem), ptr(dri), ptr(dco), ptr(dm), Vd, F, stream())
+            torch.cuda.synchronize()
+            outs.append(out.cpu().numpy())
+        assert np.array_equal(outs[0], outs[1])
+        tgt = ri if m is None else m[ri]
+        want = init + oracle.gather_to_src(em, co, tgt, Vs)
+        check(outs[0], want)
+
+
 @pytest.mark.parametrize("H", [1, 2, 3, 4, 8, 64, 65])
 def test_edge_softmax(device, H):
     print(f"case H={H}", flush=True)
