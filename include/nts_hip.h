@@ -276,6 +276,15 @@ int nts_gather_labels_i64(int64_t *out, const int64_t *table, const uint32_t *id
  * Sampled-layer index construction on the device (sampCSC, core/coocsc.hpp)
  * ------------------------------------------------------------------------------------------- */
 
+/* sampCSC::postprocessing (core/coocsc.hpp:338-424): the sampled edges' GLOBAL source ids
+ * (values < V) are marked in a bitmap; `source` receives the set bits in ascending order (the
+ * distinct sampled sources), *n_source (device) their count, and local[e] the position of
+ * global_ids[e] in `source` (local may alias global_ids).  `source` needs room for min(E, V) ids;
+ * `work` is nts_relabel_sources_work_bytes(V) bytes of 256-byte-aligned device scratch.  Bit-exact
+ * with the host bitmap scan. */
+size_t nts_relabel_sources_work_bytes(uint32_t V);
+int nts_relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *local, const uint32_t *global_ids,
+                        uint32_t E, uint32_t V, void *work, nts_stream_t stream);
 /* sampCSC::generate_csr_from_csc (core/coocsc.hpp:243-309): stable counting sort of the CSC edges
  * by local source.  Outputs ro [Vs+1], ci [E] (local destination of each CSR edge, ascending
  * within a source) and, if perm is not NULL, perm [E] (CSC edge id of each CSR edge).

@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
 
 #include "common.hpp"
@@ -96,6 +97,58 @@ __global__ __launch_bounds__(256) void add_runs_kernel(float *__restrict__ out, 
   }
 }
 
+// ---- sampled-source relabelling (bitmap of sampled global ids -> sorted list + local ids) --------
+
+__global__ __launch_bounds__(256) void mark_bits_kernel(uint32_t *__restrict__ bits, const uint32_t *__restrict__ ids,
+                                                        uint32_t E) {
+  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= E) return;
+  const uint32_t g = ids[e];
+  atomicOr(&bits[g >> 5], 1u << (g & 31));  // integer OR: the result does not depend on the order
+}
+
+__global__ __launch_bounds__(256) void popcount_words_kernel(uint32_t *__restrict__ counts,
+                                                             const uint32_t *__restrict__ bits, uint32_t words) {
+  const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
+  if (w < words) counts[w] = __popc(bits[w]);
+}
+
+// source[prefix[w] + rank] = 32*w + bit for every set bit, ascending; the last word also stores the total.
+__global__ __launch_bounds__(256) void expand_bits_kernel(uint32_t *__restrict__ source,
+                                                          uint32_t *__restrict__ n_source,
+                                                          const uint32_t *__restrict__ bits,
+                                                          const uint32_t *__restrict__ prefix, uint32_t words) {
+  const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
+  if (w >= words) return;
+  uint32_t word = bits[w];
+  uint32_t pos = prefix[w];
+  if (w + 1 == words) *n_source = pos + __popc(word);
+  while (word) {
+    const uint32_t b = __ffs(word) - 1;
+    source[pos++] = (w << 5) + b;
+    word &= word - 1;
+  }
+}
+
+__global__ __launch_bounds__(256) void relabel_kernel(uint32_t *__restrict__ local, const uint32_t *__restrict__ ids,
+                                                      const uint32_t *__restrict__ bits,
+                                                      const uint32_t *__restrict__ prefix, uint32_t E) {
+  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= E) return;
+  const uint32_t g = ids[e];
+  const uint32_t w = g >> 5;
+  local[e] = prefix[w] + __popc(bits[w] & ((1u << (g & 31)) - 1u));
+}
+
+hipError_t scan_temp_bytes(uint32_t words, size_t *bytes) {
+  size_t tmp = 0;
+  uint32_t *nul = nullptr;
+  hipError_t err = rocprim::exclusive_scan(nullptr, tmp, nul, nul, 0u, words ? words : 1u, rocprim::plus<uint32_t>(),
+                                           static_cast<hipStream_t>(nullptr), false);
+  *bytes = tmp;
+  return err;
+}
+
 inline unsigned bits_for(uint32_t n) {  // bits needed to represent values in [0, n)
   unsigned b = 1;
   while (b < 32 && (1ull << b) < n) ++b;
@@ -155,6 +208,42 @@ int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t 
   NTS_LAUNCH_CHECK("offsets_from_sorted_kernel");
   hipLaunchKernelGGL(dst_of_perm_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ci, perm_out, co, Vd, E);
   NTS_LAUNCH_CHECK("dst_of_perm_kernel");
+  return NTS_OK;
+}
+
+size_t nts_relabel_sources_work_bytes(uint32_t V) {
+  const size_t words = (static_cast<size_t>(V) + 31) / 32;
+  size_t tmp = 0;
+  if (scan_temp_bytes(static_cast<uint32_t>(words), &tmp) != hipSuccess) return 0;
+  return 3 * align_up(words * sizeof(uint32_t), 256) + align_up(tmp, 256) + 256;
+}
+
+int nts_relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *local, const uint32_t *global_ids, uint32_t E,
+                        uint32_t V, void *work, nts_stream_t stream) {
+  if (!n_source) return fail(NTS_ERR_INVALID, "nts_relabel_sources: null n_source");
+  if (E == 0 || V == 0) return nts_memset_zero(n_source, sizeof(uint32_t), stream);
+  if (!source || !local || !global_ids || !work) return fail(NTS_ERR_INVALID, "nts_relabel_sources: null pointer");
+  if (!aligned_to(work, 256)) return fail(NTS_ERR_INVALID, "nts_relabel_sources: work must be 256-byte aligned");
+  const uint32_t words = (V + 31) / 32;
+  const size_t arr = align_up(static_cast<size_t>(words) * sizeof(uint32_t), 256);
+  unsigned char *w = static_cast<unsigned char *>(work);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(w);
+  uint32_t *counts = reinterpret_cast<uint32_t *>(w + arr);
+  uint32_t *prefix = reinterpret_cast<uint32_t *>(w + 2 * arr);
+  size_t tmp = 0;
+  NTS_HIP_TRY(scan_temp_bytes(words, &tmp));
+  if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
+  hipLaunchKernelGGL(mark_bits_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, bits, global_ids, E);
+  NTS_LAUNCH_CHECK("mark_bits_kernel");
+  hipLaunchKernelGGL(popcount_words_kernel, dim3(ceil_div(words, 256)), dim3(256), 0, stream, counts, bits, words);
+  NTS_LAUNCH_CHECK("popcount_words_kernel");
+  NTS_HIP_TRY(rocprim::exclusive_scan(w + 3 * arr, tmp, counts, prefix, 0u, words, rocprim::plus<uint32_t>(), stream,
+                                      false));
+  hipLaunchKernelGGL(expand_bits_kernel, dim3(ceil_div(words, 256)), dim3(256), 0, stream, source, n_source, bits,
+                     prefix, words);
+  NTS_LAUNCH_CHECK("expand_bits_kernel");
+  hipLaunchKernelGGL(relabel_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, local, global_ids, bits, prefix, E);
+  NTS_LAUNCH_CHECK("relabel_kernel");
   return NTS_OK;
 }
 

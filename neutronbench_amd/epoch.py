@@ -1,0 +1,156 @@
+"""Per-epoch time of the sampled mini-batch path with the stage breakdown of the reference's log
+line (toolkits/GCN_GPU_NEIGHBOR.hpp:1498-1506): sample / structure / gather / aggregate forward /
+aggregate backward.  Dense layers are not part of this library and are left out.
+
+    python -m neutronbench_amd.epoch --config arxiv|products|gat [--scale S]
+
+Configurations (BASELINE.json configs 2, 4, 5):
+  arxiv     169,343 nodes, 2.48M R-MAT edges, 128 features, fanout [25,10], batch 1,024, 90,941 train nodes
+  products  2,449,029 nodes, 126.2M R-MAT edges, 100 features in mapped pinned host memory, HBM cache of the
+            top 20 % out-degree nodes, fanout [15,10,5], batch 6,000, 196,615 train nodes
+  gat       same graph, fanout [10,10], batch 4,096, 4 heads x 32, fused attention + aggregation fwd+bwd
+Neighbour choice is done by the harness on the device (torch); everything after it -- relabelling,
+CSR construction, weights, gathers, aggregation -- goes through the C ABI.  Stages are separated by
+stream synchronisation, as every reference operator synchronises its stream.
+"""
+import argparse
+import json
+import time
+
+import torch
+
+from . import synth
+from .batch import FeatureCache, MappedHostTable, load_feature_gpu_cache, load_label_gpu
+from .layout import SampledLayer, as_u32
+from .ops import GATAggregateOp, GATAttentionOp, SingleGPUSampleGraphOp
+from .stream import CudaStream
+
+CONFIGS = {
+    "arxiv": dict(V=169_343, E=2_480_000, F=128, hidden=128, classes=40, fanout=[10, 25], batch=1024, train=90_941,
+                  seed=2, cache=0.0),
+    "products": dict(V=2_449_029, E=126_200_000, F=100, hidden=128, classes=47, fanout=[5, 10, 15], batch=6000,
+                     train=196_615, seed=4, cache=0.2),
+    "gat": dict(V=2_449_029, E=126_200_000, F=100, hidden=128, classes=47, fanout=[10, 10], batch=4096, train=196_615,
+                seed=4, cache=0.2, heads=4),
+}
+
+
+class Timer:
+    def __init__(self):
+        self.t = {}
+
+    def add(self, key, t0):
+        torch.cuda.synchronize()
+        self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
+
+
+def run(name, scale=1.0, max_batches=0):
+    cfg = dict(CONFIGS[name])
+    dev = torch.device("cuda:0")
+    V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
+    n_train = int(cfg["train"] * scale)
+    src, dst = synth.rmat_edges(V, E, seed=cfg["seed"], device=dev, sort=True)
+    co, ri = synth.build_csc(src, dst, V)
+    out_deg = torch.bincount(src, minlength=V)
+    del src, dst
+    feat_cpu = synth.normal_features(V, cfg["F"], seed=cfg["seed"] + 40)
+    labels = synth.uniform_labels(V, cfg["classes"], seed=cfg["seed"] + 41, device=dev)
+    table = MappedHostTable(feat_cpu)
+    cache = FeatureCache(feat_cpu, out_deg.cpu(), int(V * cfg["cache"]), dev) if cfg["cache"] > 0 else None
+    train_nodes = synth.permutation(V, cfg["seed"] + 42, dev)[:n_train]
+    cs = CudaStream()
+    tm = Timer()
+    heads = cfg.get("heads", 0)
+    n_batches = (n_train + cfg["batch"] - 1) // cfg["batch"]
+    if max_batches:
+        n_batches = min(n_batches, max_batches)
+    edges_total, hits_total, rows_total = 0, 0, 0
+    torch.cuda.synchronize()
+    t_epoch = time.perf_counter()
+    for b in range(n_batches):
+        batch = train_nodes[b * cfg["batch"]:(b + 1) * cfg["batch"]]
+        # -- sample (harness) + structure (library) -------------------------------------------
+        layers = []
+        dst_ids = batch
+        for hop, fan in enumerate(cfg["fanout"]):
+            t0 = time.perf_counter()
+            off, rows_global = synth.sample_hop(co, ri, dst_ids, fan, 1000 * b + hop)
+            tm.add("sample", t0)
+            t0 = time.perf_counter()
+            layer = SampledLayer.from_device_hop(as_u32(off), as_u32(rows_global), as_u32(dst_ids), V, want_perm=heads > 0)
+            tm.add("structure", t0)
+            layers.append(layer)
+            dst_ids = layer.dev_source.to(torch.int64)
+        layers = layers[::-1]
+        edges_total += sum(l.e_size for l in layers)
+        # -- gather --------------------------------------------------------------------------
+        t0 = time.perf_counter()
+        x = torch.empty(layers[0].src_size, cfg["F"], device=dev)
+        if cache is not None:
+            hits = load_feature_gpu_cache(cs, layers[0], x, table.dev_ptr, cache)
+        else:
+            cs.zero_copy_feature_move_gpu(x, table.dev_ptr, layers[0].dev_source, cfg["F"], layers[0].src_size)
+            hits = None
+        lab = torch.empty(layers[-1].v_size, dtype=torch.int64, device=dev)
+        load_label_gpu(cs, layers[-1], lab, labels)
+        tm.add("gather", t0)
+        rows_total += layers[0].src_size
+        if hits is not None:
+            hits_total += int(hits.item())
+        # -- aggregation forward, then backward in reverse order --------------------------------
+        ops = []
+        for l, layer in enumerate(layers):
+            width = cfg["F"] if l == 0 else cfg["hidden"]
+            if x.shape[1] != width or x.shape[0] != layer.src_size:
+                x = synth.normal_features(layer.src_size, width, seed=l, device=dev)  # stands in for the dense layer
+            t0 = time.perf_counter()
+            if heads:
+                H, Fh = heads, cfg["hidden"] // heads
+                if x.shape[1] != H * Fh:
+                    x = synth.normal_features(layer.src_size, H * Fh, seed=l, device=dev)
+                    t0 = time.perf_counter()
+                el = x.view(layer.src_size, H, Fh).sum(2).contiguous()
+                er = torch.zeros(layer.v_size, H, device=dev)
+                att, agg = GATAttentionOp(layer, 0.2), GATAggregateOp(layer, H)
+                y = agg.forward(x, att.forward(el, er))
+                ops.append((att, agg))
+            else:
+                op = SingleGPUSampleGraphOp(layers, l, cs)
+                y = op.forward(x)
+                ops.append(op)
+            tm.add("aggregate_fwd", t0)
+            x = y
+        g = torch.ones_like(x)
+        for l in reversed(range(len(layers))):
+            if g.shape[0] != layers[l].v_size or g.shape[1] != x.shape[1]:
+                g = torch.ones(layers[l].v_size, g.shape[1], device=dev)
+            t0 = time.perf_counter()
+            if heads:
+                att, agg = ops[l]
+                g = agg.backward(g)
+                att.backward(agg.get_additional_grad())
+            else:
+                g = ops[l].backward(g)
+            tm.add("aggregate_bwd", t0)
+    torch.cuda.synchronize()
+    epoch_s = time.perf_counter() - t_epoch
+    table.close()
+    out = {
+        "config": name, "scale": scale, "vertices": V, "edges": E, "batches": n_batches, "batch_size": cfg["batch"],
+        "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
+        "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
+        "library_s": round(sum(v for k, v in tm.t.items() if k != "sample"), 4),
+        "sampled_edges": edges_total, "gathered_rows": rows_total,
+        "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
+    }
+    print(json.dumps(out))
+    return out
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--config", choices=sorted(CONFIGS), required=True)
+    ap.add_argument("--scale", type=float, default=1.0)
+    ap.add_argument("--max-batches", type=int, default=0)
+    a = ap.parse_args()
+    run(a.config, a.scale, a.max_batches)

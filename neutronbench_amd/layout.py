@@ -142,6 +142,35 @@ class SampledLayer:
             packed = packed.pin_memory().to(device, non_blocking=True)
         co, ri, src, dst = torch.split(packed, [Vd + 1, E, Vs, Vd])
         self.dev_column_offset, self.dev_row_indices, self.dev_source, self.dev_destination = co, ri, src, dst
+        self._finish_on_device(want_perm)
+        return self
+
+    @classmethod
+    def from_device_hop(cls, column_offset, row_indices_global, destination, V, want_perm=True):
+        """Whole construction on the device: `column_offset` [Vd+1] and `row_indices_global` [E]
+        (global source ids of the sampled edges) and `destination` [Vd] are int32 device tensors.
+        Relabels the sources (sampCSC::postprocessing), then builds the CSR and the weights."""
+        self = cls()
+        device = column_offset.device
+        Vd, E = destination.numel(), row_indices_global.numel()
+        stream = _stream(device)
+        work_bytes = call("nts_relabel_sources_work_bytes", V)
+        work = torch.empty(work_bytes + 256, dtype=torch.uint8, device=device)
+        base = (work.data_ptr() + 255) // 256 * 256
+        source = torch.empty(max(min(E, V), 1), dtype=torch.int32, device=device)
+        n_source = torch.zeros(1, dtype=torch.int32, device=device)
+        local = torch.empty(E, dtype=torch.int32, device=device)
+        call("nts_relabel_sources", ptr(source), ptr(n_source), ptr(local), ptr(row_indices_global), E, V, base, stream)
+        Vs = int(n_source.item())  # the one read-back of the construction: sizes the CSR arrays
+        self.v_size, self.e_size, self.src_size = Vd, E, Vs
+        self.dev_column_offset, self.dev_row_indices = column_offset, local
+        self.dev_source, self.dev_destination = source[:Vs], destination
+        self._finish_on_device(want_perm)
+        return self
+
+    def _finish_on_device(self, want_perm):
+        device = self.dev_column_offset.device
+        Vd, E, Vs = self.v_size, self.e_size, self.src_size
         self.dev_row_offset = torch.empty(Vs + 1, dtype=torch.int32, device=device)
         self.dev_column_indices = torch.empty(E, dtype=torch.int32, device=device)
         self.dev_csr_to_csc = torch.empty(E, dtype=torch.int32, device=device) if want_perm else None
@@ -152,10 +181,10 @@ class SampledLayer:
         work = torch.empty(max(work_bytes, 256) + 256, dtype=torch.uint8, device=device)
         base = (work.data_ptr() + 255) // 256 * 256
         call("nts_csr_from_csc", ptr(self.dev_row_offset), ptr(self.dev_column_indices), ptr(self.dev_csr_to_csc),
-             ptr(co), ptr(ri), Vd, Vs, E, base, stream)
-        call("nts_gcn_edge_weights", ptr(self.dev_edge_weight_forward), ptr(self.dev_edge_weight_backward), ptr(co),
-             ptr(ri), ptr(self.dev_row_offset), ptr(self.dev_column_indices), Vd, Vs, stream)
-        return self
+             ptr(self.dev_column_offset), ptr(self.dev_row_indices), Vd, Vs, E, base, stream)
+        call("nts_gcn_edge_weights", ptr(self.dev_edge_weight_forward), ptr(self.dev_edge_weight_backward),
+             ptr(self.dev_column_offset), ptr(self.dev_row_indices), ptr(self.dev_row_offset),
+             ptr(self.dev_column_indices), Vd, Vs, stream)
 
     # accessor names of the reference (core/coocsc.hpp: dev_c_o() ... dev_ewb())
     def dev_c_o(self):

@@ -181,3 +181,47 @@ def test_memory_and_stream_entry_points(device):
     assert dp.value
     call("nts_free_pinned", hp)
     assert abi.status("nts_memcpy_h2d", 0, host.ctypes.data, 16, 0) == abi.NTS_ERR_INVALID
+
+
+@pytest.mark.parametrize("V,E,seed", [(5000, 3000, 1), (100, 50000, 2), (1 << 16, 200000, 3), (37, 1, 4)])
+def test_device_relabel_matches_host_bitmap_scan(device, V, E, seed):
+    """sampCSC::postprocessing on the device: sorted distinct sources and local ids, bit-exact."""
+    rng = np.random.default_rng(seed)
+    glob = rng.integers(0, V, E).astype(np.uint32)
+    glob[0] = V - 1
+    want_local, want_source, n = oracle.postprocess(glob, V)
+    dglob = dev(glob, device)
+    work = torch.empty(call("nts_relabel_sources_work_bytes", V) + 256, dtype=torch.uint8, device=device)
+    base = (work.data_ptr() + 255) // 256 * 256
+    source = torch.full((max(min(E, V), 1),), -1, dtype=torch.int32, device=device)
+    n_source = torch.zeros(1, dtype=torch.int32, device=device)
+    local = torch.empty(E, dtype=torch.int32, device=device)
+    call("nts_relabel_sources", ptr(source), ptr(n_source), ptr(local), ptr(dglob), E, V, base, stream())
+    assert int(n_source.item()) == n
+    assert np.array_equal(host_u32(source[:n]), want_source)
+    assert np.array_equal(host_u32(local), want_local)
+
+
+def test_fully_device_side_layer_construction(device):
+    """Hop sampled on the device -> relabel -> CSR -> weights, no host step: equal to the host
+    pipeline of the oracle (postprocessing, generate_csr_from_csc, update_degree + weights)."""
+    from neutronbench_amd import synth
+    from neutronbench_amd.layout import as_u32
+
+    V, E = 30000, 600000
+    src, dst = synth.rmat_edges(V, E, seed=8, device=device, sort=True)
+    co, ri = synth.build_csc(src, dst, V)
+    batch = synth.permutation(V, 9, device)[:2000]
+    off, rows_global = synth.sample_hop(co, ri, batch, 10, 3)
+    layer = SampledLayer.from_device_hop(as_u32(off), as_u32(rows_global), as_u32(batch), V)
+    torch.cuda.synchronize()
+    glob = rows_global.cpu().numpy().astype(np.uint32)
+    local, source, n = oracle.postprocess(glob, V)
+    co_h = off.cpu().numpy().astype(np.uint32)
+    assert layer.src_size == n and np.array_equal(host_u32(layer.dev_source), source)
+    assert np.array_equal(host_u32(layer.dev_row_indices), local)
+    ro_ref, ci_ref = oracle.csr_from_csc(co_h, local, n)
+    assert np.array_equal(host_u32(layer.dev_row_offset), ro_ref) and np.array_equal(host_u32(layer.dev_column_indices), ci_ref)
+    outd, ind = np.ones(V, np.uint32), np.ones(V, np.uint32)
+    ewf, ewb = oracle.layer_weights(co_h, local, ro_ref, ci_ref, source, batch.cpu().numpy().astype(np.uint32), outd, ind)
+    assert layer.dev_ewf().cpu().numpy().tobytes() == ewf.tobytes() and layer.dev_ewb().cpu().numpy().tobytes() == ewb.tobytes()
