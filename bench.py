@@ -27,9 +27,11 @@ V_REDDIT = 232_965
 E_REDDIT = 114_800_000
 F_IN, F_HID = 602, 128
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the F=602 gather kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE
-# (profiles/spmm_wave_f602_reddit_pmc.txt); None until measured.
-TRAFFIC_BYTES_F602 = None
+# Bytes per launch of the F=602 gather kernel that cross the L2 <-> fabric boundary, from rocprofv3
+# FETCH_SIZE (x1.986 calibration) + WRITE_SIZE at the default schedule
+# (profiles/spmm_wave_f602_reddit_shaped_pmc.txt).  Reported only for the configuration it was measured on.
+TRAFFIC_BYTES_F602 = 93_989_672_629
+TRAFFIC_MEASURED_AT = dict(vertices=V_REDDIT, edges=E_REDDIT, chunk=1024, slabs=16)
 
 
 def algorithmic_bytes(E, V_out, F, weighted=True):
@@ -159,7 +161,8 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": TRAFFIC_BYTES_F602,
+        "traffic": TRAFFIC_BYTES_F602 if dict(vertices=V, edges=E, chunk=args.chunk, slabs=args.slabs) ==
+        TRAFFIC_MEASURED_AT else None,
         "algorithmic_bytes": algo,
         "kernel_ms": round(kernel_ms, 3),
         "per_pass_ms": {"fwd_F602": round(per_pass[0], 3), "fwd_F128": round(per_pass[1], 3),

@@ -268,20 +268,30 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
 }
 
 // Second stage for split rows: out[row,:] (+)= partial[first,:] + partial[first+1,:] + ... in slot
-// order.  One block per split row; `splits[i]` = (row, first slot, slot count, unused).
+// order.  Block (x, y) owns 256 columns (tile y) of split row x; `splits[i]` = (row, first slot,
+// slot count, unused).  Eight slots are loaded at a time and then added one after the other, so the
+// loads overlap while the order of the additions stays fixed.
 __global__ __launch_bounds__(256) void spmm_reduce_partials_kernel(float *__restrict__ out,
                                                                    const float *__restrict__ partial,
                                                                    const uint4 *__restrict__ splits, uint32_t F,
                                                                    int accumulate) {
   const uint4 s = splits[blockIdx.x];
-  float *dst = out + static_cast<size_t>(s.x) * F;
-  const float *src = partial + static_cast<size_t>(s.y) * F;
-  for (uint32_t c = threadIdx.x; c < F; c += blockDim.x) {
-    float a = src[c];
-    for (uint32_t k = 1; k < s.z; ++k) a += src[static_cast<size_t>(k) * F + c];
-    if (accumulate) a += dst[c];
-    dst[c] = a;
+  const uint32_t c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= F) return;
+  const float *src = partial + static_cast<size_t>(s.y) * F + c;
+  float a = src[0];
+  uint32_t k = 1;
+  for (; k + 8 <= s.z; k += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[static_cast<size_t>(k + u) * F];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a += v[u];
   }
+  for (; k < s.z; ++k) a += src[static_cast<size_t>(k) * F];
+  float *dst = out + static_cast<size_t>(s.x) * F + c;
+  if (accumulate) a += *dst;
+  *dst = a;
 }
 
 struct LaunchArgs {
@@ -463,6 +473,7 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
     }
     splits.push_back(make_uint4(r, first, n_partials - first, 0u));
   }
+  std::stable_sort(splits.begin(), splits.end(), [](const uint4 &a, const uint4 &b) { return a.z > b.z; });
   std::stable_sort(pieces.begin(), pieces.end(), [](const Piece &a, const Piece &b) {
     if (a.slab != b.slab) return a.slab < b.slab;
     return (a.e1 - a.e0) > (b.e1 - b.e0);
@@ -612,8 +623,8 @@ int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, 
   NTS_LAUNCH_CHECK("nts_spmm_gather_planned");
   if (plan->ev_start && plan->ev_stop) NTS_HIP_TRY(hipEventRecord(plan->ev_stop, stream));
   if (plan->n_splits) {
-    hipLaunchKernelGGL(nts::spmm_reduce_partials_kernel, dim3(plan->n_splits), dim3(256), 0, stream, out,
-                       plan->partial, plan->splits, F, accumulate);
+    hipLaunchKernelGGL(nts::spmm_reduce_partials_kernel, dim3(plan->n_splits, nts::ceil_div(F, 256)), dim3(256), 0,
+                       stream, out, plan->partial, plan->splits, F, accumulate);
     NTS_LAUNCH_CHECK("spmm_reduce_partials_kernel");
   }
   return NTS_OK;
