@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # Bytes per launch of the F=602 gather kernel that cross the L2 <-> fabric boundary, from rocprofv3
 # FETCH_SIZE (x1.986 calibration) + WRITE_SIZE at the default schedule
 # (profiles/spmm_wave_f602_reddit_shaped_pmc.txt).  Reported only for the configuration it was measured on.
-TRAFFIC_BYTES_F602 = 93_989_672_629
+TRAFFIC_BYTES_F602 = None
 TRAFFIC_MEASURED_AT = dict(vertices=V_REDDIT, edges=E_REDDIT, chunk=1024, slabs=16)
 
 
@@ -149,14 +149,14 @@ def main():
         call("nts_event_destroy", a)
         call("nts_event_destroy", b)
     per_pass = [sum(durs[k::4]) / args.steps for k in range(4)]  # fwd602, fwd128, bwd128, bwd602
-    # Dominant kernel: the F=602 gather (spmm_wave_kernel<2,5>), launched twice per step: forward
+    # Dominant kernel: the F=602 gather (spmm_wave_kernel<1,10>), launched twice per step: forward
     # over the CSC and backward over the CSR.  Same algorithmic bytes per launch for both.
     kernel_ms = (per_pass[0] + per_pass[3]) / 2
     algo = algorithmic_bytes(E, V, F_IN)
     achieved = algo / (kernel_ms * 1e-3) / 1e9
     roofline = {
         "bound": "hbm",
-        "kernel": "spmm_wave_kernel<2,5> (F=602 gather, forward and backward launches)",
+        "kernel": "spmm_wave_kernel<1,10> (F=602 gather, forward and backward launches)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",

@@ -4,8 +4,9 @@
 //
 // Mapping.  One wavefront (64 lanes) owns one work item = one output row, or one chunk of a long
 // row.  The 64 lanes span the feature dimension: lane l holds NACC register accumulators of VEC
-// consecutive floats at columns (l + 64*k)*VEC, so every row read is a fully coalesced
-// 64*VEC*4-byte wave load and each output element is written exactly once, without atomics.
+// consecutive floats at columns (l + 64*k)*VEC (VEC = 4 when rows are 16-byte aligned, else 1), so
+// every row read is a fully coalesced 64*VEC*4-byte wave load and each output element is written
+// exactly once, without atomics.
 // Neighbour (index, weight) pairs are fetched 64 at a time with one coalesced load per wave and
 // then broadcast lane by lane into scalar registers, so the source-row base address is scalar and
 // every index/weight is read from memory once per row instead of once per lane.
@@ -77,7 +78,7 @@ __device__ __forceinline__ void vadd(float4 &a, float4 x) {
 }
 
 // Edges processed per inner step: keeps 8..16 independent row loads in flight per lane.
-__host__ __device__ constexpr int unroll_for(int nacc) { return nacc >= 8 ? 1 : nacc >= 4 ? 2 : nacc >= 2 ? 4 : 8; }
+__host__ __device__ constexpr int unroll_for(int nacc) { return nacc >= 6 ? 1 : nacc >= 4 ? 2 : nacc >= 2 ? 4 : 8; }
 
 // Work item of a planned launch: row, first edge, one-past-last edge, partial slot (kNoSlot = the
 // item is a whole row and writes `out` directly).
@@ -190,7 +191,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
   }
 }
 
-// Sub-wavefront variant for narrow rows: G lanes per row (G = 8, 16 or 32), 64/G rows per
+// Sub-wavefront variant for narrow rows: G lanes per row (G = 4, 8, 16 or 32), 64/G rows per
 // wavefront, one VEC-wide accumulator per lane (F <= G*VEC).  Neighbour pairs are fetched G at a
 // time per group and broadcast inside the group with cross-lane shuffles.
 template <int G, int VEC>
@@ -328,15 +329,18 @@ void launch_group(const LaunchArgs &a) {
 
 template <int VEC>
 void launch_wave_vec(const LaunchArgs &a) {
-  // Column panels of at most 8 accumulators per lane; wider rows are covered by several launches
-  // over disjoint column ranges (each panel re-walks the edge list; outputs are disjoint).
-  constexpr uint32_t kMaxAcc = 8;
+  // Column panels of at most 10 accumulators per lane, balanced; wider rows are covered by several
+  // launches over disjoint column ranges (each panel re-walks the edge list; outputs are disjoint).
+  constexpr uint32_t kMaxAcc = 10;
   const uint32_t per_acc = kWave * VEC;
+  const uint32_t total_acc = ceil_div(a.F, per_acc);
+  const uint32_t panels = ceil_div(total_acc, kMaxAcc);
+  const uint32_t acc_per_panel = ceil_div(total_acc, panels);
   uint32_t col_base = 0;
   while (col_base < a.F) {
     const uint32_t remaining = a.F - col_base;
     uint32_t nacc = ceil_div(remaining, per_acc);
-    if (nacc > kMaxAcc) nacc = kMaxAcc;
+    if (nacc > acc_per_panel) nacc = acc_per_panel;
     switch (nacc) {
       case 1: launch_wave<VEC, 1>(a, col_base); break;
       case 2: launch_wave<VEC, 2>(a, col_base); break;
@@ -345,18 +349,21 @@ void launch_wave_vec(const LaunchArgs &a) {
       case 5: launch_wave<VEC, 5>(a, col_base); break;
       case 6: launch_wave<VEC, 6>(a, col_base); break;
       case 7: launch_wave<VEC, 7>(a, col_base); break;
-      default: launch_wave<VEC, 8>(a, col_base); break;
+      case 8: launch_wave<VEC, 8>(a, col_base); break;
+      case 9: launch_wave<VEC, 9>(a, col_base); break;
+      default: launch_wave<VEC, 10>(a, col_base); break;
     }
     col_base += nacc * per_acc;
   }
 }
 
-// Widest vector the operands allow: rows start at multiples of F floats from the base pointers.
+// Vector width of the row loads: 16-byte lanes when every row starts 16-byte aligned (rows start
+// at multiples of F floats from the base pointers), otherwise 4-byte lanes.  8-byte lanes are not
+// used: measured on MI355X, dwordx2 gathers run ~20 % slower than either dword or dwordx4 gathers of
+// the same bytes (F=512: 15.4 ms vs 12.8 / 11.7 ms; F=602: 18.8 ms vs 15.3 ms with dword lanes).
 int pick_vec(const LaunchArgs &a) {
   const bool a16 = aligned_to(a.in, 16) && aligned_to(a.out, 16) && (!a.partial || aligned_to(a.partial, 16));
-  const bool a8 = aligned_to(a.in, 8) && aligned_to(a.out, 8) && (!a.partial || aligned_to(a.partial, 8));
   if (a.F % 4 == 0 && a16) return 4;
-  if (a.F % 2 == 0 && a8) return 2;
   return 1;
 }
 
@@ -365,19 +372,16 @@ void launch_spmm(const LaunchArgs &a) {
   const int vec = pick_vec(a);
   const uint32_t F = a.F;
   // Narrow rows: sub-wavefront groups so that lanes are not left idle.
+  if (vec == 4 && F <= 16) return launch_group<4, 4>(a);
   if (vec == 4 && F <= 32) return launch_group<8, 4>(a);
   if (vec == 4 && F <= 64) return launch_group<16, 4>(a);
   if (vec == 4 && F <= 128) return launch_group<32, 4>(a);
-  if (vec == 2 && F <= 16) return launch_group<8, 2>(a);
-  if (vec == 2 && F <= 32) return launch_group<16, 2>(a);
-  if (vec == 2 && F <= 64) return launch_group<32, 2>(a);
+  if (vec == 1 && F <= 4) return launch_group<4, 1>(a);
   if (vec == 1 && F <= 8) return launch_group<8, 1>(a);
   if (vec == 1 && F <= 16) return launch_group<16, 1>(a);
   if (vec == 1 && F <= 32) return launch_group<32, 1>(a);
-  // Wave per row.  Prefer the narrowest vector that still needs few accumulators: a 16-byte
-  // vector only pays off once a row spans more than one 8-byte wave load.
+  // Wave per row.
   if (vec == 4) return launch_wave_vec<4>(a);
-  if (vec == 2) return launch_wave_vec<2>(a);
   return launch_wave_vec<1>(a);
 }
 
