@@ -30,8 +30,8 @@ HBM_PEAK_GBS = 8000.0
 # Bytes per launch of the F=602 gather kernel that cross the L2 <-> fabric boundary, from rocprofv3
 # FETCH_SIZE (x1.986 calibration) + WRITE_SIZE at the default schedule
 # (profiles/spmm_wave_f602_reddit_shaped_pmc.txt).  Reported only for the configuration it was measured on.
-TRAFFIC_BYTES_F602 = None
-TRAFFIC_MEASURED_AT = dict(vertices=V_REDDIT, edges=E_REDDIT, chunk=1024, slabs=16)
+TRAFFIC_BYTES_F602 = 47_969_194_494
+TRAFFIC_MEASURED_AT = dict(vertices=V_REDDIT, edges=E_REDDIT, chunk=512, slabs=32)
 
 
 def algorithmic_bytes(E, V_out, F, weighted=True):
@@ -47,8 +47,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--vertices", type=int, default=V_REDDIT)
     ap.add_argument("--edges", type=int, default=E_REDDIT)
-    ap.add_argument("--chunk", type=int, default=1024, help="largest number of edges in one piece of a split hub row")
-    ap.add_argument("--slabs", type=int, default=16,
+    ap.add_argument("--chunk", type=int, default=512, help="largest number of edges in one piece of a split hub row")
+    ap.add_argument("--slabs", type=int, default=32,
                     help="source ranges of the cache-aware schedule (1 = split hub rows by edge count only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate", action="store_true",

@@ -134,7 +134,8 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan, const uint32_t *offsets, uint32
  * is read back once as well, and the pieces of split rows whose indices ascend are cut at the
  * boundaries of `n_slabs` equal ranges of [index_base, index_base + n_index) and issued slab by slab,
  * so that concurrently running wavefronts gather from the same range of source rows (each XCD's
- * L2 then holds that range's hot rows).  n_slabs = 0 selects the default; rows whose indices do
+ * L2 then holds that range's hot rows).  n_slabs = 0 and chunk_edges = 0 select the defaults (32
+ * ranges, 512 edges, tuned on a 114.8 M-edge power-law graph at F = 602); rows whose indices do
  * not ascend are split by edge count as above.  Results differ from nts_spmm_plan_create only in
  * where split rows are cut. */
 int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan, const uint32_t *offsets, const uint32_t *indices,

@@ -561,8 +561,8 @@ int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan_out, const uint32_t *offse
     if (index_base)
       for (uint32_t &v : idx) v -= index_base;
   }
-  return build_plan(plan_out, offsets, off, idx.data(), rows, edges, chunk_edges ? chunk_edges : 4096u,
-                    n_slabs ? n_slabs : 16u, n_index);
+  return build_plan(plan_out, offsets, off, idx.data(), rows, edges, chunk_edges ? chunk_edges : 512u,
+                    n_slabs ? n_slabs : 32u, n_index);
 }
 
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {
