@@ -7,14 +7,17 @@
 // consecutive floats at columns (l + 64*k)*VEC (VEC = 4 when rows are 16-byte aligned, else 1), so
 // every row read is a fully coalesced 64*VEC*4-byte wave load and each output element is written
 // exactly once, without atomics.
-// Neighbour (index, weight) pairs are fetched 64 at a time with one coalesced load per wave and
-// then broadcast lane by lane into scalar registers, so the source-row base address is scalar and
-// every index/weight is read from memory once per row instead of once per lane.
+// Neighbour (index, weight) pairs are fetched 64 at a time with one coalesced load per wave, staged
+// in a wave-private LDS tile and read back one pair at a time by all lanes at once (a broadcast
+// read), then moved to scalar registers, so the source-row base address is scalar and every
+// index/weight is read from memory once per row instead of once per lane.
 // Narrow rows (F <= 32*VEC) use sub-wavefront groups of G lanes per row (spmm_group_kernel).
 //
 // Accumulation order within a row is the edge order of the offsets array, one fused multiply-add
 // per edge and element -- the order of the CPU operators (core/ntsMiniBatchGraphOp.hpp:154-240),
 // so unsplit rows reproduce an FMA-contracted CPU build bit for bit.
+#include <stdlib.h>
+
 #include <algorithm>
 #include <new>
 #include <vector>
@@ -84,7 +87,7 @@ __host__ __device__ constexpr int unroll_for(int nacc) { return nacc >= 6 ? 1 : 
 // item is a whole row and writes `out` directly).
 using Item = uint4;
 
-template <int VEC, int NACC>
+template <int VEC, int NACC, bool LDS_TILE>
 __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                         const float *__restrict__ w,
                                                         const uint32_t *__restrict__ offsets,
@@ -126,8 +129,14 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
     acc[k] = vzero<VEC>();
   }
 
-  // Tile of up to 64 neighbour (index, weight) pairs held one per lane; the next tile is fetched
-  // while the current one is consumed.
+  // Tile of up to 64 neighbour (index, weight) pairs, fetched with one coalesced load per wave; the
+  // next tile is fetched while the current one is consumed.  The pairs are then handed to the whole
+  // wave one at a time as scalars: either straight from the registers that hold them (readlane), or
+  // (LDS_TILE) through a wave-private LDS tile that every lane reads at the same address.  The LDS
+  // region belongs to one wave and LDS operations of a wave complete in order, so no block barrier
+  // is needed -- which matters because waves of a block run different trip counts.
+  __shared__ uint2 lds_tile[LDS_TILE ? 4 : 1][LDS_TILE ? kWave : 1];
+  uint2 *tile = lds_tile[LDS_TILE ? (threadIdx.x / kWave) : 0];
   uint32_t nxt_i = 0;
   float nxt_w = 1.f;
   if (e0 + lane < e1) {
@@ -138,19 +147,37 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
     const uint32_t n = min(static_cast<uint32_t>(kWave), e1 - eb);
     const uint32_t my_i = nxt_i;
     const float my_w = nxt_w;
+    if (LDS_TILE) {
+      __builtin_amdgcn_wave_barrier();  // earlier reads of the tile are done before it is overwritten
+      tile[lane] = make_uint2(my_i, __float_as_uint(my_w));
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
     const uint32_t en = eb + kWave + lane;
     if (en < e1) {
       nxt_i = indices[en] - index_base;
       if (w) nxt_w = w[en];
     }
+    auto pair_at = [&](uint32_t j, uint32_t &idx, float &wgt) {
+      if (LDS_TILE) {
+        const uint2 p = tile[j];
+        idx = wave_first(p.x);
+        wgt = __uint_as_float(wave_first(p.y));
+      } else {
+        idx = wave_read(my_i, j);
+        wgt = wave_read(my_w, j);
+      }
+    };
     uint32_t j = 0;
     for (; j + U <= n; j += U) {
       const float *src[U];
       float sw[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        src[u] = in + static_cast<size_t>(wave_read(my_i, j + u)) * F;
-        sw[u] = wave_read(my_w, j + u);
+        uint32_t si;
+        pair_at(j + u, si, sw[u]);
+        src[u] = in + static_cast<size_t>(si) * F;
       }
       V v[U][NACC];
 #pragma unroll
@@ -169,8 +196,10 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
       }
     }
     for (; j < n; ++j) {
-      const float *src = in + static_cast<size_t>(wave_read(my_i, j)) * F;
-      const float sw = wave_read(my_w, j);
+      uint32_t si;
+      float sw;
+      pair_at(j, si, sw);
+      const float *src = in + static_cast<size_t>(si) * F;
 #pragma unroll
       for (int k = 0; k < NACC; ++k) {
         vfma(acc[k], *reinterpret_cast<const V *>(src + lcol[k]), sw);
@@ -310,13 +339,29 @@ struct LaunchArgs {
   hipStream_t stream;
 };
 
+// How the wave kernel hands neighbour pairs to its lanes: through a wave-private LDS tile (default)
+// or by register broadcast (NTS_SPMM_LDS_TILE=0).  The two measure the same on MI355X (12.44 ms vs
+// 12.40 ms for the 114.8 M-edge F=602 gather); the variable is read once per process.
+bool lds_tile_enabled() {
+  static const bool enabled = [] {
+    const char *e = getenv("NTS_SPMM_LDS_TILE");
+    return e ? e[0] != '0' : true;
+  }();
+  return enabled;
+}
+
 template <int VEC, int NACC>
 void launch_wave(const LaunchArgs &a, uint32_t col_base) {
   constexpr int kWavesPerBlock = 4;
   const uint32_t blocks = ceil_div(a.n_items, kWavesPerBlock);
-  hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC>), dim3(blocks), dim3(kWavesPerBlock * kWave), 0, a.stream, a.in,
-                     a.out, a.w, a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial,
-                     a.accumulate);
+  if (lds_tile_enabled())
+    hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, true>), dim3(blocks), dim3(kWavesPerBlock * kWave), 0, a.stream,
+                       a.in, a.out, a.w, a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items,
+                       a.partial, a.accumulate);
+  else
+    hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, false>), dim3(blocks), dim3(kWavesPerBlock * kWave), 0, a.stream,
+                       a.in, a.out, a.w, a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items,
+                       a.partial, a.accumulate);
 }
 
 template <int G, int VEC>

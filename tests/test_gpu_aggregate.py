@@ -208,3 +208,19 @@ def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
     keep = deg <= chunk
     assert np.array_equal(outs[0][keep].view(np.uint32), oracle.spmm(x, w, co, ri, Vd, fused=True)[keep].view(np.uint32))
     plan.close()
+
+
+def test_register_broadcast_variant_in_a_fresh_process(device):
+    """The library hands neighbour pairs to the lanes through an LDS tile by default and by register
+    broadcast when NTS_SPMM_LDS_TILE=0 (read once per process): the other variant passes the same
+    parity cases."""
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, NTS_SPMM_LDS_TILE="0")
+    here = os.path.dirname(os.path.abspath(__file__))
+    r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(here, "test_gpu_aggregate.py"), "-q", "-x", "-m", "gpu",
+                        "-k", "forward_matches_oracle or planned_split_rows or cache_aware", "--timeout", "120",
+                        "--timeout-method", "thread"], env=env, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-1500:]
