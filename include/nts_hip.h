@@ -277,6 +277,24 @@ int nts_gather_labels_i64(int64_t *out, const int64_t *table, const uint32_t *id
  * Sampled-layer index construction on the device (sampCSC, core/coocsc.hpp)
  * ------------------------------------------------------------------------------------------- */
 
+/* One hop of neighbour sampling over a whole-graph CSC in HBM (Sampler::sample_one's construction
+ * steps, core/ntsSampler.hpp:843-1106).  graph_co [V+1] / graph_ri [E_graph] are the whole graph's
+ * column_offset / row_indices (global source ids), dst [n] the hop's destinations (global ids).
+ *   nts_sample_hop_offsets   co[i+1]-co[i] = fanout < 0 ? deg(dst[i]) : min(deg(dst[i]), fanout), co[n] = number
+ *                            of sampled edges (init_co, core/FullyRepGraph.hpp:199-209; bit-exact).  `work` is
+ *                            nts_sample_hop_work_bytes(n) bytes of 256-byte-aligned device scratch.
+ *   nts_sample_hop_neighbors ri_global[co[i] .. co[i+1]) = all in-neighbours of dst[i] in CSC order when none is
+ *                            dropped, otherwise that many DISTINCT positions of its CSC segment chosen uniformly
+ *                            from a hash of (seed, i, dst[i]), in ascending position order.
+ * Which neighbours the reference picks depends on its RNG, thread count and container iteration
+ * order, so the pick is specified here by these properties, not by equality with the reference. */
+size_t nts_sample_hop_work_bytes(uint32_t n);
+int nts_sample_hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, uint32_t n, int32_t fanout,
+                           void *work, nts_stream_t stream);
+int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co,
+                             const uint32_t *graph_ri, const uint32_t *dst, uint32_t n, int32_t fanout,
+                             uint64_t seed, nts_stream_t stream);
+
 /* sampCSC::postprocessing (core/coocsc.hpp:338-424): the sampled edges' GLOBAL source ids
  * (values < V) are marked in a bitmap; `source` receives the set bits in ascending order (the
  * distinct sampled sources), *n_source (device) their count, and local[e] the position of

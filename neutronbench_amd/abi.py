@@ -70,6 +70,9 @@ SIGNATURES = {
     "nts_gather_rows_f32": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],
     "nts_gather_rows_cached_f32": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp],
     "nts_gather_labels_i64": [_vp, _vp, _vp, _u32, _u32, _vp],
+    "nts_sample_hop_work_bytes": [_u32],
+    "nts_sample_hop_offsets": [_vp, _vp, _vp, _u32, ctypes.c_int32, _vp, _vp],
+    "nts_sample_hop_neighbors": [_vp, _vp, _vp, _vp, _vp, _u32, ctypes.c_int32, ctypes.c_uint64, _vp],
     "nts_relabel_sources_work_bytes": [_u32],
     "nts_relabel_sources": [_vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp],
     "nts_csr_from_csc_work_bytes": [_u32, _u32, _u32],
@@ -77,9 +80,10 @@ SIGNATURES = {
     "nts_gcn_edge_weights": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],
 }
 _RESTYPES = {"nts_last_error": ctypes.c_char_p, "nts_csr_from_csc_work_bytes": _sz,
-             "nts_relabel_sources_work_bytes": _sz}
+             "nts_relabel_sources_work_bytes": _sz, "nts_sample_hop_work_bytes": _sz}
 # Entry points whose int result is a value, not a status.
-_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes"}
+_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
+              "nts_sample_hop_work_bytes"}
 
 
 class NtsError(RuntimeError):

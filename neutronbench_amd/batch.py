@@ -89,3 +89,20 @@ def load_label_gpu(cs, top_layer, local_label, global_label):
                                           classes)
     else:
         cs.global_copy_label_move_gpu(local_label, global_label, top_layer.dev_destination, top_layer.v_size)
+
+
+def sample_hop(graph_co, graph_ri, dst, fanout, seed):
+    """One hop of neighbour sampling on the device through the library: returns
+    (column_offset [n+1], row_indices with GLOBAL source ids [E]) as int32 device tensors.
+    graph_co / graph_ri / dst are int32 device tensors (uint32 bit patterns)."""
+    device = dst.device
+    n = dst.numel()
+    stream = torch.cuda.current_stream(device).cuda_stream
+    work = torch.empty(call("nts_sample_hop_work_bytes", n) + 256, dtype=torch.uint8, device=device)
+    base = (work.data_ptr() + 255) // 256 * 256
+    co = torch.empty(n + 1, dtype=torch.int32, device=device)
+    call("nts_sample_hop_offsets", ptr(co), ptr(graph_co), ptr(dst), n, fanout, base, stream)
+    E = int(co[-1].item()) & 0xFFFFFFFF  # one read-back: sizes the edge array
+    ri = torch.empty(E, dtype=torch.int32, device=device)
+    call("nts_sample_hop_neighbors", ptr(ri), ptr(co), ptr(graph_co), ptr(graph_ri), ptr(dst), n, fanout, seed, stream)
+    return co, ri

@@ -9,8 +9,8 @@ Configurations (BASELINE.json configs 2, 4, 5):
   products  2,449,029 nodes, 126.2M R-MAT edges, 100 features in mapped pinned host memory, HBM cache of the
             top 20 % out-degree nodes, fanout [15,10,5], batch 6,000, 196,615 train nodes
   gat       same graph, fanout [10,10], batch 4,096, 4 heads x 32, fused attention + aggregation fwd+bwd
-Neighbour choice is done by the harness on the device (torch); everything after it -- relabelling,
-CSR construction, weights, gathers, aggregation -- goes through the C ABI.  Stages are separated by
+Everything goes through the C ABI: neighbour sampling of each hop, relabelling, CSR construction,
+weights, gathers, aggregation (--sampler harness uses the torch sampler of the test harness instead).  Stages are separated by
 stream synchronisation, as every reference operator synchronises its stream.
 """
 import argparse
@@ -20,7 +20,7 @@ import time
 import torch
 
 from . import synth
-from .batch import FeatureCache, MappedHostTable, load_feature_gpu_cache, load_label_gpu
+from .batch import FeatureCache, MappedHostTable, load_feature_gpu_cache, load_label_gpu, sample_hop
 from .layout import SampledLayer, as_u32
 from .ops import GATAggregateOp, GATAttentionOp, SingleGPUSampleGraphOp
 from .stream import CudaStream
@@ -44,13 +44,14 @@ class Timer:
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
-def run(name, scale=1.0, max_batches=0):
+def run(name, scale=1.0, max_batches=0, sampler="library"):
     cfg = dict(CONFIGS[name])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
     n_train = int(cfg["train"] * scale)
     src, dst = synth.rmat_edges(V, E, seed=cfg["seed"], device=dev, sort=True)
     co, ri = synth.build_csc(src, dst, V)
+    gco, gri = as_u32(co), as_u32(ri)
     out_deg = torch.bincount(src, minlength=V)
     del src, dst
     feat_cpu = synth.normal_features(V, cfg["F"], seed=cfg["seed"] + 40)
@@ -74,13 +75,19 @@ def run(name, scale=1.0, max_batches=0):
         dst_ids = batch
         for hop, fan in enumerate(cfg["fanout"]):
             t0 = time.perf_counter()
-            off, rows_global = synth.sample_hop(co, ri, dst_ids, fan, 1000 * b + hop)
+            if sampler == "library":
+                dst32 = dst_ids if dst_ids.dtype == torch.int32 else as_u32(dst_ids)
+                off32, rows32 = sample_hop(gco, gri, dst32, fan, 1000 * b + hop)
+            else:
+                d64 = dst_ids.to(torch.int64) & 0xFFFFFFFF
+                off, rows_global = synth.sample_hop(co, ri, d64, fan, 1000 * b + hop)
+                off32, rows32, dst32 = as_u32(off), as_u32(rows_global), as_u32(d64)
             tm.add("sample", t0)
             t0 = time.perf_counter()
-            layer = SampledLayer.from_device_hop(as_u32(off), as_u32(rows_global), as_u32(dst_ids), V, want_perm=heads > 0)
+            layer = SampledLayer.from_device_hop(off32, rows32, dst32, V, want_perm=heads > 0)
             tm.add("structure", t0)
             layers.append(layer)
-            dst_ids = layer.dev_source.to(torch.int64)
+            dst_ids = layer.dev_source
         layers = layers[::-1]
         edges_total += sum(l.e_size for l in layers)
         # -- gather --------------------------------------------------------------------------
@@ -139,8 +146,8 @@ def run(name, scale=1.0, max_batches=0):
         "config": name, "scale": scale, "vertices": V, "edges": E, "batches": n_batches, "batch_size": cfg["batch"],
         "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
-        "library_s": round(sum(v for k, v in tm.t.items() if k != "sample"), 4),
-        "sampled_edges": edges_total, "gathered_rows": rows_total,
+        "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler == "library"), 4),
+        "sampler": sampler, "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
     }
     print(json.dumps(out))
@@ -152,5 +159,6 @@ if __name__ == "__main__":
     ap.add_argument("--config", choices=sorted(CONFIGS), required=True)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--max-batches", type=int, default=0)
+    ap.add_argument("--sampler", choices=["library", "harness"], default="library")
     a = ap.parse_args()
-    run(a.config, a.scale, a.max_batches)
+    run(a.config, a.scale, a.max_batches, a.sampler)

@@ -10,7 +10,8 @@ import oracle
 from gpu_util import dev, host_u32, stream
 from neutronbench_amd import abi
 from neutronbench_amd.abi import call, ptr
-from neutronbench_amd.batch import FeatureCache, MappedHostTable, load_feature_gpu, load_feature_gpu_cache, load_label_gpu
+from neutronbench_amd.batch import (FeatureCache, MappedHostTable, load_feature_gpu, load_feature_gpu_cache,
+                                    load_label_gpu, sample_hop)
 from neutronbench_amd.layout import SampledLayer
 from neutronbench_amd.stream import CudaStream, get_gpu_mem
 from util import brute_csr, random_block
@@ -225,3 +226,64 @@ def test_fully_device_side_layer_construction(device):
     outd, ind = np.ones(V, np.uint32), np.ones(V, np.uint32)
     ewf, ewb = oracle.layer_weights(co_h, local, ro_ref, ci_ref, source, batch.cpu().numpy().astype(np.uint32), outd, ind)
     assert layer.dev_ewf().cpu().numpy().tobytes() == ewf.tobytes() and layer.dev_ewb().cpu().numpy().tobytes() == ewb.tobytes()
+
+
+@pytest.mark.parametrize("fanout", [-1, 1, 5, 25, 64, 100])
+def test_device_sampler_properties(device, fanout):
+    """The hop sampler's contract: offsets equal init_co (bit-exact); with nothing dropped a
+    destination's neighbours come out in CSC order; otherwise `fanout` DISTINCT positions of its
+    segment, ascending; the same seed reproduces the sample and another seed changes it.  These are
+    the reference's own validity conditions (Sampler::isValidSampleGraph / sample_one asserts)."""
+    from neutronbench_amd import synth
+    from neutronbench_amd.layout import as_u32
+
+    V, E = 20000, 600000
+    src, dst = synth.rmat_edges(V, E, seed=12, device=device, sort=True)
+    co64, ri64 = synth.build_csc(src, dst, V)
+    gco, gri = as_u32(co64), as_u32(ri64)
+    batch64 = synth.permutation(V, 13, device)[:3000]
+    batch = as_u32(batch64)
+    co, ri = sample_hop(gco, gri, batch, fanout, 77)
+    torch.cuda.synchronize()
+    co_h = host_u32(co)
+    assert np.array_equal(co_h, oracle.init_co(co64.cpu().numpy().astype(np.uint32), batch64.cpu().numpy().astype(np.uint32), fanout))
+    ri_h = host_u32(ri)
+    gco_h, gri_h = co64.cpu().numpy(), ri64.cpu().numpy()
+    b = batch64.cpu().numpy()
+    partial_rows = 0
+    for i in range(b.size):
+        seg = gri_h[gco_h[b[i]]:gco_h[b[i] + 1]]
+        got = ri_h[co_h[i]:co_h[i + 1]]
+        if got.size == seg.size:
+            assert np.array_equal(got, seg)
+            continue
+        partial_rows += 1
+        assert got.size == fanout
+        # distinct positions, ascending: `got` must be a subsequence of the (sorted, duplicates kept) segment
+        pos, ok = 0, True
+        for v in got:
+            while pos < seg.size and seg[pos] != v:
+                pos += 1
+            ok = ok and pos < seg.size
+            pos += 1
+        assert ok, f"destination slot {i}: not {fanout} distinct positions of its neighbour list"
+    if 0 < fanout < 100:
+        assert partial_rows > 0
+    co2, ri2 = sample_hop(gco, gri, batch, fanout, 77)
+    assert torch.equal(ri, ri2) and torch.equal(co, co2)
+    if partial_rows:
+        _, ri3 = sample_hop(gco, gri, batch, fanout, 78)
+        assert not torch.equal(ri, ri3)
+
+
+def test_device_sampler_is_uniform(device):
+    """Every position of a long neighbour list is picked about equally often (fanout 8 of 64)."""
+    deg, n, fanout = 64, 20000, 8
+    gco = torch.tensor([0, deg], dtype=torch.int32, device=device)
+    gri = torch.arange(deg, dtype=torch.int32, device=device)
+    dst = torch.zeros(n, dtype=torch.int32, device=device)
+    co, ri = sample_hop(gco, gri, dst, fanout, 5)
+    counts = torch.bincount(ri.to(torch.int64), minlength=deg).cpu().numpy()
+    expect = n * fanout / deg
+    assert counts.sum() == n * fanout
+    assert np.all(np.abs(counts - expect) < 6 * np.sqrt(expect)), counts
