@@ -238,6 +238,11 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
 int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
                           const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
                           uint32_t H, uint32_t Fh, int accumulate, nts_stream_t stream);
+/* The same through a schedule built by nts_spmm_plan_create[_slabs] for `offsets` (full-graph GAT:
+ * hub rows are split and the sum order of split rows is the plan's). */
+int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *alpha,
+                                  const uint32_t *perm, const uint32_t *offsets, const uint32_t *indices,
+                                  uint32_t H, uint32_t Fh, int accumulate, nts_stream_t stream);
 /* Gradient of the aggregation with respect to alpha (get_additional_grad of
  * DistAggregateDstFuseWeight, core/ntsDistCPUGraphOp.hpp:442-472):
  *   galpha[e,h] = < in[ri[e], h*Fh : (h+1)*Fh], gout[d, h*Fh : (h+1)*Fh] >   for e in CSC(d) */

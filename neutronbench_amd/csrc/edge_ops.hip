@@ -277,59 +277,7 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
   }
 }
 
-// ---- attention-weighted aggregation -----------------------------------------------------------
-
-// out[r, c] (+)= sum_k alpha[eid(k), c / Fh] * in[indices[k], c];  one wave per row, lane l owns the
-// float2 / float at column l*VEC of each 64*VEC-wide column panel.  Neighbour indices are fetched
-// 64 at a time and broadcast through scalar registers as in the GCN aggregation kernel.
-template <int VEC>
-__global__ __launch_bounds__(256) void spmm_heads_kernel(const float *__restrict__ in, float *__restrict__ out,
-                                                         const float *__restrict__ alpha,
-                                                         const uint32_t *__restrict__ perm,
-                                                         const uint32_t *__restrict__ offsets,
-                                                         const uint32_t *__restrict__ indices, uint32_t rows,
-                                                         uint32_t H, uint32_t Fh, int accumulate) {
-  const uint32_t r = wave_item();
-  if (r >= rows) return;
-  const uint32_t lane = lane_id();
-  const uint32_t F = H * Fh;
-  const uint32_t e0 = wave_first(offsets[r]), e1 = wave_first(offsets[r + 1]);
-  for (uint32_t cb = 0; cb < F; cb += kWave * VEC) {
-    const uint32_t col = cb + lane * VEC;
-    const bool live = col < F;
-    const uint32_t lcol = live ? col : F - VEC;
-    const uint32_t h = lcol / Fh;
-    float a[VEC];
-#pragma unroll
-    for (int t = 0; t < VEC; ++t) a[t] = 0.f;
-    for (uint32_t eb = e0; eb < e1; eb += kWave) {
-      const uint32_t n = min(static_cast<uint32_t>(kWave), e1 - eb);
-      uint32_t my_i = 0, my_e = 0;
-      if (lane < n) {
-        my_i = indices[eb + lane];
-        my_e = perm ? perm[eb + lane] : eb + lane;
-      }
-      for (uint32_t j = 0; j < n; ++j) {
-        const uint32_t si = wave_read(my_i, j);
-        const uint32_t se = wave_read(my_e, j);
-        const float wgt = alpha[static_cast<size_t>(se) * H + h];
-        const float *src = in + static_cast<size_t>(si) * F + lcol;
-        if constexpr (VEC == 2) {
-          const float2 v = *reinterpret_cast<const float2 *>(src);
-          a[0] = fmaf(v.x, wgt, a[0]);
-          a[1] = fmaf(v.y, wgt, a[1]);
-        } else {
-          a[0] = fmaf(src[0], wgt, a[0]);
-        }
-      }
-    }
-    if (live) {
-      float *p = out + static_cast<size_t>(r) * F + col;
-#pragma unroll
-      for (int t = 0; t < VEC; ++t) p[t] = accumulate ? p[t] + a[t] : a[t];
-    }
-  }
-}
+// ---- gradient of the attention-weighted aggregation with respect to alpha ----------------------
 
 // galpha[e,h] = < in[ri[e], h-th slice], gout[d, h-th slice] > for e in CSC(d).  One wave per
 // destination; for each edge and head the lanes stride over the slice and a full-wave butterfly
@@ -549,26 +497,6 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
     hipLaunchKernelGGL((edge_softmax_bwd_kernel<true, false>), wave_grid(Vd), wave_block(), 0, stream, gs, ger, galpha,
                        alpha, el, er, co, ri, Vd, H, slope);
   NTS_LAUNCH_CHECK("nts_gat_attention_bwd");
-  return NTS_OK;
-}
-
-int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
-                          const uint32_t *offsets, const uint32_t *indices, uint32_t rows, uint32_t H, uint32_t Fh,
-                          int accumulate, nts_stream_t stream) {
-  if (H == 0 || Fh == 0) return fail(NTS_ERR_INVALID, "nts_spmm_gather_heads: H or Fh is 0");
-  if (static_cast<uint64_t>(H) * Fh > 0xFFFFFFFFull) return fail(NTS_ERR_INVALID, "nts_spmm_gather_heads: H*Fh overflows");
-  if (rows == 0) return NTS_OK;
-  if (!in || !out || !alpha || !offsets || !indices)
-    return fail(NTS_ERR_INVALID, "nts_spmm_gather_heads: null pointer");
-  // A vector must not straddle two heads: the width has to divide Fh.
-  const bool v2 = Fh % 2 == 0 && aligned_to(in, 8) && aligned_to(out, 8);
-  if (v2)
-    hipLaunchKernelGGL(spmm_heads_kernel<2>, wave_grid(rows), wave_block(), 0, stream, in, out, alpha, perm, offsets,
-                       indices, rows, H, Fh, accumulate);
-  else
-    hipLaunchKernelGGL(spmm_heads_kernel<1>, wave_grid(rows), wave_block(), 0, stream, in, out, alpha, perm, offsets,
-                       indices, rows, H, Fh, accumulate);
-  NTS_LAUNCH_CHECK("nts_spmm_gather_heads");
   return NTS_OK;
 }
 

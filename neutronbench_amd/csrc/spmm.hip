@@ -87,14 +87,22 @@ __host__ __device__ constexpr int unroll_for(int nacc) { return nacc >= 6 ? 1 : 
 // item is a whole row and writes `out` directly).
 using Item = uint4;
 
-template <int VEC, int NACC, bool LDS_TILE>
+// Per-head edge weights (attention-weighted aggregation): w is alpha [E_csc, H], a column belongs
+// to head column / Fh, and the weight of edge position e is alpha[(perm ? perm[e] : e) * H + head].
+struct HeadArgs {
+  const uint32_t *perm;
+  uint32_t H;
+  uint32_t Fh;
+};
+
+template <int VEC, int NACC, bool LDS_TILE, bool HEADS>
 __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                         const float *__restrict__ w,
                                                         const uint32_t *__restrict__ offsets,
                                                         const uint32_t *__restrict__ indices, uint32_t index_base,
                                                         uint32_t n_items, uint32_t F, uint32_t col_base,
                                                         const Item *__restrict__ items, float *__restrict__ partial,
-                                                        int accumulate) {
+                                                        int accumulate, HeadArgs heads) {
   using V = typename Vec<VEC>::type;
   constexpr int U = unroll_for(NACC);
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -119,6 +127,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
   // VEC columns instead, so that loads need no predication; their sums are never stored.
   uint32_t col[NACC];
   uint32_t lcol[NACC];
+  uint32_t head[NACC];
   bool live[NACC];
   V acc[NACC];
 #pragma unroll
@@ -126,6 +135,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
     col[k] = col_base + (lane + kWave * k) * VEC;
     live[k] = col[k] < F;
     lcol[k] = live[k] ? col[k] : F - VEC;
+    head[k] = HEADS ? lcol[k] / heads.Fh : 0u;
     acc[k] = vzero<VEC>();
   }
 
@@ -137,19 +147,25 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
   // is needed -- which matters because waves of a block run different trip counts.
   __shared__ uint2 lds_tile[LDS_TILE ? 4 : 1][LDS_TILE ? kWave : 1];
   uint2 *tile = lds_tile[LDS_TILE ? (threadIdx.x / kWave) : 0];
+  // Second component of a pair: the edge weight (as bits), or with per-head weights the id of the
+  // edge in alpha's (CSC) order.
+  auto second_of = [&](uint32_t e) -> uint32_t {
+    if (HEADS) return heads.perm ? heads.perm[e] : e;
+    return w ? __float_as_uint(w[e]) : __float_as_uint(1.f);
+  };
   uint32_t nxt_i = 0;
-  float nxt_w = 1.f;
+  uint32_t nxt_s = HEADS ? 0u : __float_as_uint(1.f);
   if (e0 + lane < e1) {
     nxt_i = indices[e0 + lane] - index_base;
-    if (w) nxt_w = w[e0 + lane];
+    nxt_s = second_of(e0 + lane);
   }
   for (uint32_t eb = e0; eb < e1; eb += kWave) {
     const uint32_t n = min(static_cast<uint32_t>(kWave), e1 - eb);
     const uint32_t my_i = nxt_i;
-    const float my_w = nxt_w;
+    const uint32_t my_s = nxt_s;
     if (LDS_TILE) {
       __builtin_amdgcn_wave_barrier();  // earlier reads of the tile are done before it is overwritten
-      tile[lane] = make_uint2(my_i, __float_as_uint(my_w));
+      tile[lane] = make_uint2(my_i, my_s);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -157,52 +173,55 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
     const uint32_t en = eb + kWave + lane;
     if (en < e1) {
       nxt_i = indices[en] - index_base;
-      if (w) nxt_w = w[en];
+      nxt_s = second_of(en);
     }
-    auto pair_at = [&](uint32_t j, uint32_t &idx, float &wgt) {
+    auto pair_at = [&](uint32_t j, uint32_t &idx, uint32_t &second) {
       if (LDS_TILE) {
         const uint2 p = tile[j];
         idx = wave_first(p.x);
-        wgt = __uint_as_float(wave_first(p.y));
+        second = wave_first(p.y);
       } else {
         idx = wave_read(my_i, j);
-        wgt = wave_read(my_w, j);
+        second = wave_read(my_s, j);
       }
     };
     uint32_t j = 0;
     for (; j + U <= n; j += U) {
       const float *src[U];
-      float sw[U];
+      uint32_t ss[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         uint32_t si;
-        pair_at(j + u, si, sw[u]);
+        pair_at(j + u, si, ss[u]);
         src[u] = in + static_cast<size_t>(si) * F;
       }
       V v[U][NACC];
+      float wv[U][HEADS ? NACC : 1];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
 #pragma unroll
         for (int k = 0; k < NACC; ++k) {
           v[u][k] = *reinterpret_cast<const V *>(src[u] + lcol[k]);
+          if (HEADS) wv[u][k] = w[static_cast<size_t>(ss[u]) * heads.H + head[k]];
         }
+        if (!HEADS) wv[u][0] = __uint_as_float(ss[u]);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
 #pragma unroll
         for (int k = 0; k < NACC; ++k) {
-          vfma(acc[k], v[u][k], sw[u]);
+          vfma(acc[k], v[u][k], wv[u][HEADS ? k : 0]);
         }
       }
     }
     for (; j < n; ++j) {
-      uint32_t si;
-      float sw;
-      pair_at(j, si, sw);
+      uint32_t si, ss;
+      pair_at(j, si, ss);
       const float *src = in + static_cast<size_t>(si) * F;
 #pragma unroll
       for (int k = 0; k < NACC; ++k) {
-        vfma(acc[k], *reinterpret_cast<const V *>(src + lcol[k]), sw);
+        const float wgt = HEADS ? w[static_cast<size_t>(ss) * heads.H + head[k]] : __uint_as_float(ss);
+        vfma(acc[k], *reinterpret_cast<const V *>(src + lcol[k]), wgt);
       }
     }
   }
@@ -223,13 +242,13 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
 // Sub-wavefront variant for narrow rows: G lanes per row (G = 4, 8, 16 or 32), 64/G rows per
 // wavefront, one VEC-wide accumulator per lane (F <= G*VEC).  Neighbour pairs are fetched G at a
 // time per group and broadcast inside the group with cross-lane shuffles.
-template <int G, int VEC>
+template <int G, int VEC, bool HEADS>
 __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                          const float *__restrict__ w,
                                                          const uint32_t *__restrict__ offsets,
                                                          const uint32_t *__restrict__ indices, uint32_t index_base,
                                                          uint32_t n_items, uint32_t F, const Item *__restrict__ items,
-                                                         float *__restrict__ partial, int accumulate) {
+                                                         float *__restrict__ partial, int accumulate, HeadArgs heads) {
   using V = typename Vec<VEC>::type;
   constexpr int U = 4;
   const uint32_t gl = threadIdx.x & (G - 1);
@@ -252,39 +271,46 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
   const uint32_t col = gl * VEC;
   const bool live = col < F;
   const uint32_t lcol = live ? col : F - VEC;  // idle lanes re-read the last columns, never store
+  const uint32_t head = HEADS ? lcol / heads.Fh : 0u;
   V acc = vzero<VEC>();
 
   for (uint32_t eb = e0; eb < e1; eb += G) {
     const uint32_t n = min(static_cast<uint32_t>(G), e1 - eb);
     uint32_t my_i = 0;
-    float my_w = 1.f;
+    uint32_t my_s = HEADS ? 0u : __float_as_uint(1.f);  // weight bits, or the edge's id in alpha's order
     if (gl < n) {
       my_i = indices[eb + gl] - index_base;
-      if (w) my_w = w[eb + gl];
+      if (HEADS)
+        my_s = heads.perm ? heads.perm[eb + gl] : eb + gl;
+      else if (w)
+        my_s = __float_as_uint(w[eb + gl]);
     }
     uint32_t j = 0;
     for (; j + U <= n; j += U) {
       uint32_t si[U];
-      float sw[U];
+      uint32_t ss[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         si[u] = __shfl(my_i, j + u, G);
-        sw[u] = __shfl(my_w, j + u, G);
+        ss[u] = __shfl(my_s, j + u, G);
       }
       V v[U];
+      float wv[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         v[u] = *reinterpret_cast<const V *>(in + static_cast<size_t>(si[u]) * F + lcol);
+        wv[u] = HEADS ? w[static_cast<size_t>(ss[u]) * heads.H + head] : __uint_as_float(ss[u]);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        vfma(acc, v[u], sw[u]);
+        vfma(acc, v[u], wv[u]);
       }
     }
     for (; j < n; ++j) {
       const uint32_t si = __shfl(my_i, j, G);
-      const float sw = __shfl(my_w, j, G);
-      vfma(acc, *reinterpret_cast<const V *>(in + static_cast<size_t>(si) * F + lcol), sw);
+      const uint32_t ss = __shfl(my_s, j, G);
+      const float wgt = HEADS ? w[static_cast<size_t>(ss) * heads.H + head] : __uint_as_float(ss);
+      vfma(acc, *reinterpret_cast<const V *>(in + static_cast<size_t>(si) * F + lcol), wgt);
     }
   }
 
@@ -337,6 +363,7 @@ struct LaunchArgs {
   float *partial;
   int accumulate;
   hipStream_t stream;
+  HeadArgs heads = HeadArgs{nullptr, 0u, 0u};  // H == 0: one weight per edge
 };
 
 // How the wave kernel hands neighbour pairs to its lanes: through a wave-private LDS tile (default)
@@ -354,22 +381,28 @@ template <int VEC, int NACC>
 void launch_wave(const LaunchArgs &a, uint32_t col_base) {
   constexpr int kWavesPerBlock = 4;
   const uint32_t blocks = ceil_div(a.n_items, kWavesPerBlock);
-  if (lds_tile_enabled())
-    hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, true>), dim3(blocks), dim3(kWavesPerBlock * kWave), 0, a.stream,
-                       a.in, a.out, a.w, a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items,
-                       a.partial, a.accumulate);
-  else
-    hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, false>), dim3(blocks), dim3(kWavesPerBlock * kWave), 0, a.stream,
-                       a.in, a.out, a.w, a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items,
-                       a.partial, a.accumulate);
+  const dim3 grid(blocks), block(kWavesPerBlock * kWave);
+#define NTS_LAUNCH_WAVE(LDS, HD)                                                                                       \
+  hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, LDS, HD>), grid, block, 0, a.stream, a.in, a.out, a.w, a.offsets,     \
+                     a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate, a.heads)
+  if (a.heads.H) {
+    if (lds_tile_enabled()) NTS_LAUNCH_WAVE(true, true); else NTS_LAUNCH_WAVE(false, true);
+  } else {
+    if (lds_tile_enabled()) NTS_LAUNCH_WAVE(true, false); else NTS_LAUNCH_WAVE(false, false);
+  }
+#undef NTS_LAUNCH_WAVE
 }
 
 template <int G, int VEC>
 void launch_group(const LaunchArgs &a) {
   const uint32_t per_block = 256 / G;
   const uint32_t blocks = ceil_div(a.n_items, per_block);
-  hipLaunchKernelGGL((spmm_group_kernel<G, VEC>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w, a.offsets,
-                     a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate);
+  if (a.heads.H)
+    hipLaunchKernelGGL((spmm_group_kernel<G, VEC, true>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
+                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads);
+  else
+    hipLaunchKernelGGL((spmm_group_kernel<G, VEC, false>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
+                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads);
 }
 
 template <int VEC>
@@ -408,7 +441,8 @@ void launch_wave_vec(const LaunchArgs &a) {
 // the same bytes (F=512: 15.4 ms vs 12.8 / 11.7 ms; F=602: 18.8 ms vs 15.3 ms with dword lanes).
 int pick_vec(const LaunchArgs &a) {
   const bool a16 = aligned_to(a.in, 16) && aligned_to(a.out, 16) && (!a.partial || aligned_to(a.partial, 16));
-  if (a.F % 4 == 0 && a16) return 4;
+  const bool heads_ok = a.heads.H == 0 || a.heads.Fh % 4 == 0;  // a 16-byte lane must stay inside one head
+  if (a.F % 4 == 0 && a16 && heads_ok) return 4;
   return 1;
 }
 
@@ -642,6 +676,55 @@ int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F) {
   NTS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&plan->partial),
                         static_cast<size_t>(plan->n_partials) * F * sizeof(float)));
   plan->partial_F = F;
+  return NTS_OK;
+}
+
+namespace {
+int check_heads(const float *alpha, uint32_t H, uint32_t Fh, const char *who) {
+  if (H == 0 || Fh == 0) return nts::fail(NTS_ERR_INVALID, who);
+  if (static_cast<uint64_t>(H) * Fh > 0xFFFFFFFFull) return nts::fail(NTS_ERR_INVALID, who);
+  if (!alpha) return nts::fail(NTS_ERR_INVALID, who);
+  return NTS_OK;
+}
+}  // namespace
+
+int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
+                          const uint32_t *offsets, const uint32_t *indices, uint32_t rows, uint32_t H, uint32_t Fh,
+                          int accumulate, nts_stream_t stream) {
+  if (int rc = check_heads(alpha, H, Fh, "nts_spmm_gather_heads: bad H / Fh / alpha")) return rc;
+  if (rows == 0) return NTS_OK;
+  if (!in || !out || !offsets || !indices) return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_heads: null pointer");
+  nts::LaunchArgs a{in, out, alpha, offsets, indices, 0u, rows, H * Fh, nullptr, nullptr, accumulate, stream};
+  a.heads = nts::HeadArgs{perm, H, Fh};
+  nts::launch_spmm(a);
+  NTS_LAUNCH_CHECK("nts_spmm_gather_heads");
+  return NTS_OK;
+}
+
+int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *alpha,
+                                  const uint32_t *perm, const uint32_t *offsets, const uint32_t *indices, uint32_t H,
+                                  uint32_t Fh, int accumulate, nts_stream_t stream) {
+  if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_heads_planned: null plan");
+  if (offsets != plan->offsets)
+    return nts::fail(NTS_ERR_INVALID,
+                     "nts_spmm_gather_heads_planned: offsets differ from the array the plan was built from");
+  if (int rc = check_heads(alpha, H, Fh, "nts_spmm_gather_heads_planned: bad H / Fh / alpha")) return rc;
+  const uint32_t F = H * Fh;
+  if (int rc = nts::check_common(in, out, offsets, indices, plan->rows, plan->edges, F,
+                                 "nts_spmm_gather_heads_planned: null pointer"))
+    return rc;
+  if (plan->rows == 0) return NTS_OK;
+  if (int rc = nts_spmm_plan_reserve(plan, F)) return rc;
+  nts::LaunchArgs a{in,  out,         alpha,         offsets,    indices, 0u, plan->n_items,
+                    F,   plan->items, plan->partial, accumulate, stream};
+  a.heads = nts::HeadArgs{perm, H, Fh};
+  nts::launch_spmm(a);
+  NTS_LAUNCH_CHECK("nts_spmm_gather_heads_planned");
+  if (plan->n_splits) {
+    hipLaunchKernelGGL(nts::spmm_reduce_partials_kernel, dim3(plan->n_splits, nts::ceil_div(F, 256)), dim3(256), 0,
+                       stream, out, plan->partial, plan->splits, F, accumulate);
+    NTS_LAUNCH_CHECK("spmm_reduce_partials_kernel");
+  }
   return NTS_OK;
 }
 
