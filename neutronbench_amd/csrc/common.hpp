@@ -45,6 +45,17 @@ __device__ __forceinline__ uint32_t wave_first(uint32_t v) {
   return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
 }
 
+// Largest r such that off[r] <= pos, searched in off[0 .. n] (off ascending, off[n] > pos): the row
+// that owns edge position `pos`.
+__device__ __forceinline__ uint32_t owner_of(const uint32_t *__restrict__ off, uint32_t n, uint32_t pos) {
+  uint32_t lo = 0, hi = n;  // answer in [lo, hi)
+  while (hi - lo > 1) {
+    const uint32_t mid = lo + (hi - lo) / 2;
+    if (off[mid] <= pos) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
 // Butterfly reductions over the `width` lanes of an aligned lane group (width = power of two <= 64).
 template <int WIDTH>
 __device__ __forceinline__ float group_max(float v) {

@@ -2,8 +2,9 @@
 // cuda/ntsCUDADistKernel.cuh:23-95, 166-260, cuda/ntsCUDAFuseKernel.cuh:492-506 and their
 // launchers cuda/ntsCUDAGraphOP.cu:294-377, 449-474).
 //
-// All kernels give one wavefront to one destination (or source) row; lanes span the feature /
-// head dimension, sums over a segment run in edge order or through fixed-shape cross-lane
+// Copies and per-edge products are edge-parallel (work per wavefront independent of any vertex's
+// degree); per-destination reductions give one wavefront to one destination (or source) row, lanes
+// spanning the feature / head dimension.  Sums run in edge order or through fixed-shape cross-lane
 // butterflies, and nothing uses float atomics, so every result is bit-reproducible.
 #include "common.hpp"
 
@@ -21,68 +22,86 @@ inline dim3 wave_grid(uint32_t items) { return dim3(ceil_div(items ? items : 1, 
 inline dim3 wave_block() { return dim3(kWavesPerBlock * kWave); }
 
 // ---- vertex -> edge copies ------------------------------------------------------------------
+//
+// Edge-parallel: the edge count is read on the device (co[Vd]); a wavefront takes 64 consecutive
+// edges per step, every lane looks up the feature row its edge copies from (the source id, or the
+// destination that owns the edge by binary search in co), and sub-wavefront groups of G lanes then
+// move 64/G rows at a time.  Work per wave does not depend on any vertex's degree.
 
-// msg[e,:] = feat[mirror ? mirror[ri[e]] : ri[e], :] for e in CSC(d); one wave per destination.
-template <typename V>
-__global__ __launch_bounds__(256) void scatter_src_to_edge_kernel(V *__restrict__ msg, const V *__restrict__ feat,
-                                                                  const uint32_t *__restrict__ ri,
-                                                                  const uint32_t *__restrict__ co,
-                                                                  const uint32_t *__restrict__ mirror, uint32_t Vd,
-                                                                  uint32_t Fv) {
-  const uint32_t d = wave_item();
-  if (d >= Vd) return;
-  const uint32_t lane = lane_id();
-  const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
-  for (uint32_t e = e0; e < e1; ++e) {
-    uint32_t s = ri[e];
-    if (mirror) s = mirror[s];
-    const V *src = feat + static_cast<size_t>(s) * Fv;
-    V *dst = msg + static_cast<size_t>(e) * Fv;
-    for (uint32_t c = lane; c < Fv; c += kWave) dst[c] = src[c];
-  }
-}
+enum CopyMode { kFromSrc = 0, kFromDst = 1, kAddFromDst = 2 };
 
-// msg[e,:] (+)= feat[d,:] for e in CSC(d); the destination row is read once per column.
-template <typename V, bool ADD>
-__global__ __launch_bounds__(256) void scatter_dst_to_edge_kernel(V *__restrict__ msg, const V *__restrict__ feat,
-                                                                  const uint32_t *__restrict__ co, uint32_t Vd,
-                                                                  uint32_t Fv) {
-  const uint32_t d = wave_item();
-  if (d >= Vd) return;
+template <typename V, int G>
+__global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, const V *__restrict__ feat,
+                                                        const uint32_t *__restrict__ ri,
+                                                        const uint32_t *__restrict__ co,
+                                                        const uint32_t *__restrict__ mirror, uint32_t Vd, uint32_t Fv,
+                                                        int mode) {
+  const uint32_t E = co[Vd];
   const uint32_t lane = lane_id();
-  const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
-  for (uint32_t c = lane; c < Fv; c += kWave) {
-    const V v = feat[static_cast<size_t>(d) * Fv + c];
-    for (uint32_t e = e0; e < e1; ++e) {
-      V *p = msg + static_cast<size_t>(e) * Fv + c;
-      if (ADD) {
-        V o = *p;
-        float *of = reinterpret_cast<float *>(&o);
-        const float *vf = reinterpret_cast<const float *>(&v);
-#pragma unroll
-        for (int t = 0; t < static_cast<int>(sizeof(V) / 4); ++t) of[t] += vf[t];
-        *p = o;
+  const uint32_t gl = lane & (G - 1), grp = lane / G;
+  constexpr uint32_t kEdgesPerStep = kWave / G;
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  for (uint64_t base = wave * kWave; base < E; base += n_waves * kWave) {
+    const uint64_t e = base + lane;
+    uint32_t row = 0;
+    if (e < E) {
+      if (mode == kFromSrc) {
+        row = ri[e];
+        if (mirror) row = mirror[row];
       } else {
-        *p = v;
+        row = owner_of(co, Vd, static_cast<uint32_t>(e));
+      }
+    }
+    for (uint32_t j = 0; j < G; ++j) {
+      const uint32_t holder = j * kEdgesPerStep + grp;  // lane that looked up this group's edge
+      const uint32_t r = __shfl(row, holder, kWave);
+      const uint64_t ee = base + holder;
+      if (ee < E) {
+        const V *src = feat + static_cast<size_t>(r) * Fv;
+        V *dst = msg + ee * Fv;
+        for (uint32_t c = gl; c < Fv; c += G) {
+          V v = src[c];
+          if (mode == kAddFromDst) {
+            const V o = dst[c];
+            float *vf = reinterpret_cast<float *>(&v);
+            const float *of = reinterpret_cast<const float *>(&o);
+#pragma unroll
+            for (int t = 0; t < static_cast<int>(sizeof(V) / 4); ++t) vf[t] = of[t] + vf[t];
+          }
+          dst[c] = v;
+        }
       }
     }
   }
 }
 
 // ---- edge -> vertex sums ----------------------------------------------------------------------
+//
+// Rows with at most `long_limit` edges: a group of G lanes per row (64/G rows per wavefront) adds
+// the row's edge rows in order.  Longer rows (power-law hubs) are left to the block kernel below,
+// which is handed the list of such rows; it spreads a row's edges over the slices of a 1024-thread
+// block and adds the slices' partial sums in a fixed order.
+
+constexpr uint32_t kNoLimit = 0xFFFFFFFFu;
+constexpr uint32_t kLongRowEdges = 1024;    // edges of a row above which the block kernel takes over
+constexpr uint32_t kLongRowValues = 4096;   // the same for softmax segments, in values (edges * heads)
+constexpr uint32_t kLongMinVertices = 16384;  // vertex count below which the extra launches are not worth it
+constexpr int kLongBlock = 1024;
 
 // out[r,:] (+)= sum_{k in [off[r], off[r+1])} msg[perm ? perm[k] : k, :], added in k order.
-template <typename V>
+template <typename V, int G>
 __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__ out, const V *__restrict__ msg,
                                                                  const uint32_t *__restrict__ off,
                                                                  const uint32_t *__restrict__ perm, uint32_t rows,
-                                                                 uint32_t Fv, int accumulate) {
-  const uint32_t r = wave_item();
+                                                                 uint32_t Fv, int accumulate, uint32_t long_limit) {
+  const uint32_t r = (blockIdx.x * blockDim.x + threadIdx.x) / G;
   if (r >= rows) return;
-  const uint32_t lane = lane_id();
-  const uint32_t e0 = wave_first(off[r]), e1 = wave_first(off[r + 1]);
+  const uint32_t gl = threadIdx.x & (G - 1);
+  const uint32_t e0 = off[r], e1 = off[r + 1];
+  if (e1 - e0 > long_limit) return;
   constexpr int NF = sizeof(V) / 4;
-  for (uint32_t c = lane; c < Fv; c += kWave) {
+  for (uint32_t c = gl; c < Fv; c += G) {
     float a[NF];
 #pragma unroll
     for (int t = 0; t < NF; ++t) a[t] = 0.f;
@@ -105,6 +124,53 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__
 #pragma unroll
     for (int t = 0; t < NF; ++t) rf[t] = a[t];
     *p = res;
+  }
+}
+
+// list[0 .. *count) = rows r with (off[r+1] - off[r]) * width > limit (any order).
+__global__ __launch_bounds__(256) void collect_long_rows_kernel(uint32_t *__restrict__ list,
+                                                                uint32_t *__restrict__ count,
+                                                                const uint32_t *__restrict__ off, uint32_t rows,
+                                                                uint32_t width, uint32_t limit) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  if (static_cast<uint64_t>(off[r + 1] - off[r]) * width > limit) list[atomicAdd(count, 1u)] = r;
+}
+
+// One 1024-thread block per listed row.  Columns are taken in tiles of `tile` (a power of two
+// <= 1024); thread t owns column t % tile of slice t / tile, a slice adds every (1024/tile)-th edge
+// of the row in ascending order, and slice 0 then adds the slices' sums in slice order.
+__global__ __launch_bounds__(kLongBlock) void gather_edge_to_row_long_kernel(
+    float *__restrict__ out, const float *__restrict__ msg, const uint32_t *__restrict__ off,
+    const uint32_t *__restrict__ perm, const uint32_t *__restrict__ list, const uint32_t *__restrict__ count,
+    uint32_t F, uint32_t tile, int accumulate) {
+  __shared__ float part[kLongBlock];
+  const uint32_t n_rows = *count;
+  const uint32_t c = threadIdx.x & (tile - 1);
+  const uint32_t slice = threadIdx.x / tile;
+  const uint32_t n_slices = kLongBlock / tile;
+  for (uint32_t i = blockIdx.x; i < n_rows; i += gridDim.x) {
+    const uint32_t r = list[i];
+    const uint32_t e0 = off[r], e1 = off[r + 1];
+    for (uint32_t cb = 0; cb < F; cb += tile) {
+      const uint32_t col = cb + c;
+      float a = 0.f;
+      if (col < F) {
+        for (uint32_t k = e0 + slice; k < e1; k += n_slices) {
+          const uint32_t e = perm ? perm[k] : k;
+          a += msg[static_cast<size_t>(e) * F + col];
+        }
+      }
+      part[threadIdx.x] = a;
+      __syncthreads();
+      if (slice == 0 && col < F) {
+        float total = part[c];
+        for (uint32_t sidx = 1; sidx < n_slices; ++sidx) total += part[sidx * tile + c];
+        float *p = out + static_cast<size_t>(r) * F + col;
+        *p = accumulate ? *p + total : total;
+      }
+      __syncthreads();
+    }
   }
 }
 
@@ -134,12 +200,13 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
                                                                const float *__restrict__ er,
                                                                const uint32_t *__restrict__ co,
                                                                const uint32_t *__restrict__ ri, uint32_t Vd,
-                                                               uint32_t H, float slope) {
+                                                               uint32_t H, float slope, uint32_t long_limit) {
   const uint32_t d = wave_item();
   if (d >= Vd) return;
   const uint32_t lane = lane_id();
   const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
   if (e0 == e1) return;
+  if (static_cast<uint64_t>(e1 - e0) * H > long_limit) return;  // left to the block kernel
   const size_t base = static_cast<size_t>(e0) * H;
   const uint32_t n = (e1 - e0) * H;
   float *ys = y + base;
@@ -215,11 +282,12 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
                                                                const float *__restrict__ er,
                                                                const uint32_t *__restrict__ co,
                                                                const uint32_t *__restrict__ ri, uint32_t Vd,
-                                                               uint32_t H, float slope) {
+                                                               uint32_t H, float slope, uint32_t long_limit) {
   const uint32_t d = wave_item();
   if (d >= Vd) return;
   const uint32_t lane = lane_id();
   const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
+  if (static_cast<uint64_t>(e1 - e0) * H > long_limit) return;  // left to the block kernel
   const size_t base = static_cast<size_t>(e0) * H;
   const uint32_t n = (e1 - e0) * H;
   const float *gys = gy + base;
@@ -277,65 +345,185 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
   }
 }
 
-// ---- gradient of the attention-weighted aggregation with respect to alpha ----------------------
+// Block kernels for long segments (power-of-two H <= 64 only; other head counts stay on the wave
+// kernels).  1024 threads walk the segment's values; thread t always meets head t mod H.  Per-head
+// maxima / sums are reduced inside each wave with the head butterfly, then across the 16 waves
+// through LDS in wave order.
+template <int MODE>  // 0 = max, 1 = sum
+__device__ __forceinline__ float block_head_reduce(float v, uint32_t H, float (*red)[kWave]) {
+  const uint32_t lane = lane_id(), wave = threadIdx.x / kWave;
+  v = head_reduce<MODE>(v, H);
+  if (lane < H) red[wave][lane] = v;
+  __syncthreads();
+  const uint32_t h = lane & (H - 1);
+  float r = red[0][h];
+  for (uint32_t wv = 1; wv < kLongBlock / kWave; ++wv) r = MODE == 0 ? fmaxf(r, red[wv][h]) : r + red[wv][h];
+  __syncthreads();
+  return r;
+}
 
-// galpha[e,h] = < in[ri[e], h-th slice], gout[d, h-th slice] > for e in CSC(d).  One wave per
-// destination; for each edge and head the lanes stride over the slice and a full-wave butterfly
-// adds the partial products.
-__global__ __launch_bounds__(256) void sddmm_heads_kernel(float *__restrict__ galpha, const float *__restrict__ in,
-                                                          const float *__restrict__ gout,
-                                                          const uint32_t *__restrict__ co,
-                                                          const uint32_t *__restrict__ ri, uint32_t Vd, uint32_t H,
-                                                          uint32_t Fh) {
-  const uint32_t d = wave_item();
-  if (d >= Vd) return;
-  const uint32_t lane = lane_id();
-  const uint32_t F = H * Fh;
-  const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
-  const float *g = gout + static_cast<size_t>(d) * F;
-  for (uint32_t e = e0; e < e1; ++e) {
-    const float *src = in + static_cast<size_t>(wave_first(ri[e])) * F;
-    for (uint32_t h = 0; h < H; ++h) {
-      float p = 0.f;
-      for (uint32_t f = lane; f < Fh; f += kWave) p = fmaf(src[h * Fh + f], g[h * Fh + f], p);
-      p = group_sum<kWave>(p);
-      if (lane == 0) galpha[static_cast<size_t>(e) * H + h] = p;
+template <bool FUSED>
+__global__ __launch_bounds__(kLongBlock) void edge_softmax_fwd_long_kernel(
+    float *__restrict__ y, const float *__restrict__ x, const float *__restrict__ el, const float *__restrict__ er,
+    const uint32_t *__restrict__ co, const uint32_t *__restrict__ ri, const uint32_t *__restrict__ list,
+    const uint32_t *__restrict__ count, uint32_t H, float slope) {
+  __shared__ float red[kLongBlock / kWave][kWave];
+  const uint32_t n_rows = *count;
+  const uint32_t h = threadIdx.x & (H - 1);
+  for (uint32_t i = blockIdx.x; i < n_rows; i += gridDim.x) {
+    const uint32_t d = list[i];
+    const uint32_t e0 = co[d], e1 = co[d + 1];
+    const size_t base = static_cast<size_t>(e0) * H;
+    const size_t n = static_cast<size_t>(e1 - e0) * H;
+    float *ys = y + base;
+    const float *xs = FUSED ? nullptr : x + base;
+    float erv = 0.f;
+    if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+    float mx = -INFINITY;
+    for (size_t j = threadIdx.x; j < n; j += kLongBlock) {
+      float sc;
+      if (FUSED) {
+        const uint32_t src = ri[e0 + j / H];
+        sc = leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
+        ys[j] = sc;
+      } else {
+        sc = xs[j];
+      }
+      mx = fmaxf(mx, sc);
+    }
+    mx = block_head_reduce<0>(mx, H, red);
+    float sum = 0.f;
+    for (size_t j = threadIdx.x; j < n; j += kLongBlock) sum += expf((FUSED ? ys[j] : xs[j]) - mx);
+    sum = block_head_reduce<1>(sum, H, red);
+    for (size_t j = threadIdx.x; j < n; j += kLongBlock) ys[j] = expf((FUSED ? ys[j] : xs[j]) - mx) / sum;
+  }
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(kLongBlock) void edge_softmax_bwd_long_kernel(
+    float *__restrict__ gx, float *__restrict__ ger, const float *__restrict__ gy, const float *__restrict__ y,
+    const float *__restrict__ el, const float *__restrict__ er, const uint32_t *__restrict__ co,
+    const uint32_t *__restrict__ ri, const uint32_t *__restrict__ list, const uint32_t *__restrict__ count, uint32_t H,
+    float slope) {
+  __shared__ float red[kLongBlock / kWave][kWave];
+  const uint32_t n_rows = *count;
+  const uint32_t h = threadIdx.x & (H - 1);
+  for (uint32_t i = blockIdx.x; i < n_rows; i += gridDim.x) {
+    const uint32_t d = list[i];
+    const uint32_t e0 = co[d], e1 = co[d + 1];
+    const size_t base = static_cast<size_t>(e0) * H;
+    const size_t n = static_cast<size_t>(e1 - e0) * H;
+    const float *gys = gy + base;
+    const float *ys = y + base;
+    float *gxs = gx + base;
+    float dot = 0.f;
+    for (size_t j = threadIdx.x; j < n; j += kLongBlock) dot += gys[j] * ys[j];
+    dot = block_head_reduce<1>(dot, H, red);
+    float erv = 0.f, gsum = 0.f;
+    if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+    for (size_t j = threadIdx.x; j < n; j += kLongBlock) {
+      float g = ys[j] * (gys[j] - dot);
+      if (FUSED) {
+        const uint32_t src = ri[e0 + j / H];
+        const float pre = el[static_cast<size_t>(src) * H + h] + erv;
+        g *= pre > 0.f ? 1.f : slope;
+        gsum += g;
+      }
+      gxs[j] = g;
+    }
+    if (FUSED) {
+      gsum = block_head_reduce<1>(gsum, H, red);
+      if (threadIdx.x < H) ger[static_cast<size_t>(d) * H + threadIdx.x] = gsum;
     }
   }
 }
 
-// Fast path of the above when every head is a power-of-two number L = Fh <= 64 of lanes wide and
-// the whole row fits one wave pass (H*Fh <= 64): lane l owns column l, the per-head sum is a
-// butterfly over L lanes.
-__global__ __launch_bounds__(256) void sddmm_heads_pow2_kernel(float *__restrict__ galpha,
-                                                               const float *__restrict__ in,
-                                                               const float *__restrict__ gout,
-                                                               const uint32_t *__restrict__ co,
-                                                               const uint32_t *__restrict__ ri, uint32_t Vd,
-                                                               uint32_t H, uint32_t Fh) {
-  const uint32_t d = wave_item();
-  if (d >= Vd) return;
-  const uint32_t lane = lane_id();
+// ---- gradient of the attention-weighted aggregation with respect to alpha ----------------------
+//
+// galpha[e,h] = < in[ri[e], h-th slice], gout[d, h-th slice] > for e in CSC(d).  Edge-parallel like
+// the copies: 64 consecutive edges per wave step, (source, owner) looked up per lane.
+
+// Fast path: G = (H*Fh)/VEC lanes cover one edge's row (G a power of two <= 64), the Fh/VEC lanes of
+// a head add their products with an xor butterfly; 64/G edges per step.
+template <int VEC>
+__global__ __launch_bounds__(256) void sddmm_edge_kernel(float *__restrict__ galpha, const float *__restrict__ in,
+                                                         const float *__restrict__ gout,
+                                                         const uint32_t *__restrict__ co,
+                                                         const uint32_t *__restrict__ ri, uint32_t Vd, uint32_t H,
+                                                         uint32_t Fh, uint32_t G, uint32_t lanes_per_head) {
+  const uint32_t E = co[Vd];
   const uint32_t F = H * Fh;
-  const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
-  const bool live = lane < F;
-  const float g = live ? gout[static_cast<size_t>(d) * F + lane] : 0.f;
-  for (uint32_t e = e0; e < e1; ++e) {
-    const float *src = in + static_cast<size_t>(wave_first(ri[e])) * F;
-    float p = live ? src[lane] * g : 0.f;
-    for (uint32_t m = Fh / 2; m >= 1; m >>= 1) p += __shfl_xor(p, m, kWave);
-    if (live && (lane & (Fh - 1)) == 0) galpha[static_cast<size_t>(e) * H + lane / Fh] = p;
+  const uint32_t lane = lane_id();
+  const uint32_t gl = lane & (G - 1), grp = lane / G;
+  const uint32_t edges_per_step = kWave / G;
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  for (uint64_t base = wave * kWave; base < E; base += n_waves * kWave) {
+    const uint64_t e = base + lane;
+    uint32_t src = 0, own = 0;
+    if (e < E) {
+      src = ri[e];
+      own = owner_of(co, Vd, static_cast<uint32_t>(e));
+    }
+    for (uint32_t j = 0; j < G; ++j) {
+      const uint32_t holder = j * edges_per_step + grp;
+      const uint32_t s = __shfl(src, holder, kWave);
+      const uint32_t d = __shfl(own, holder, kWave);
+      const uint64_t ee = base + holder;
+      const bool valid = ee < E;
+      float p = 0.f;
+      if (valid) {
+        const float *a = in + static_cast<size_t>(s) * F + gl * VEC;
+        const float *b = gout + static_cast<size_t>(d) * F + gl * VEC;
+        if (VEC == 4) {
+          const float4 x = *reinterpret_cast<const float4 *>(a);
+          const float4 y = *reinterpret_cast<const float4 *>(b);
+          p = fmaf(x.w, y.w, fmaf(x.z, y.z, fmaf(x.y, y.y, x.x * y.x)));
+        } else {
+          p = a[0] * b[0];
+        }
+      }
+      for (uint32_t m = lanes_per_head / 2; m >= 1; m >>= 1) p += __shfl_xor(p, m, kWave);
+      if (valid && (gl & (lanes_per_head - 1)) == 0) galpha[ee * H + gl / lanes_per_head] = p;
+    }
+  }
+}
+
+// General shapes: the 64 edges of a step are taken one after the other; for each edge and head the
+// lanes stride over the head's slice and a full-wave butterfly adds the partial products.
+__global__ __launch_bounds__(256) void sddmm_edge_generic_kernel(float *__restrict__ galpha,
+                                                                 const float *__restrict__ in,
+                                                                 const float *__restrict__ gout,
+                                                                 const uint32_t *__restrict__ co,
+                                                                 const uint32_t *__restrict__ ri, uint32_t Vd,
+                                                                 uint32_t H, uint32_t Fh) {
+  const uint32_t E = co[Vd];
+  const uint32_t F = H * Fh;
+  const uint32_t lane = lane_id();
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  for (uint64_t base = wave * kWave; base < E; base += n_waves * kWave) {
+    const uint64_t e = base + lane;
+    uint32_t src = 0, own = 0;
+    if (e < E) {
+      src = ri[e];
+      own = owner_of(co, Vd, static_cast<uint32_t>(e));
+    }
+    const uint32_t n = static_cast<uint32_t>(min(static_cast<uint64_t>(kWave), E - base));
+    for (uint32_t j = 0; j < n; ++j) {
+      const float *a = in + static_cast<size_t>(wave_read(src, j)) * F;
+      const float *b = gout + static_cast<size_t>(wave_read(own, j)) * F;
+      for (uint32_t h = 0; h < H; ++h) {
+        float p = 0.f;
+        for (uint32_t f = lane; f < Fh; f += kWave) p = fmaf(a[h * Fh + f], b[h * Fh + f], p);
+        p = group_sum<kWave>(p);
+        if (lane == 0) galpha[(base + j) * H + h] = p;
+      }
+    }
   }
 }
 
 inline bool is_pow2(uint32_t v) { return v && !(v & (v - 1)); }
-
-// Vector width (in floats) usable for [*, F] row-major operands at the given base pointers.
-inline int row_vec(uint32_t F, const void *a, const void *b) {
-  if (F % 4 == 0 && aligned_to(a, 16) && aligned_to(b, 16)) return 4;
-  if (F % 2 == 0 && aligned_to(a, 8) && aligned_to(b, 8)) return 2;
-  return 1;
-}
 
 }  // namespace
 }  // namespace nts
@@ -343,27 +531,99 @@ inline int row_vec(uint32_t F, const void *a, const void *b) {
 using namespace nts;
 
 namespace {
-template <bool ADD>
-int scatter_dst_impl(float *msg, const float *feat, const uint32_t *co, uint32_t Vd, uint32_t F, hipStream_t stream,
-                     const char *who) {
+// Grid for the edge-parallel kernels: the edge count lives on the device, so the grid is sized from
+// the vertex count (assuming a few dozen edges per vertex) and the kernels stride over the edges.
+inline dim3 edge_grid(uint32_t Vd) {
+  uint64_t blocks = (static_cast<uint64_t>(Vd) * 32 + 255) / 256;
+  if (blocks < 64) blocks = 64;
+  if (blocks > 8192) blocks = 8192;
+  return dim3(static_cast<unsigned>(blocks));
+}
+
+// Lanes per row for a row of Fv vector elements: the smallest power of two >= Fv, at most 64.
+inline int lanes_for(uint32_t Fv) {
+  int g = 1;
+  while (g < 64 && static_cast<uint32_t>(g) < Fv) g <<= 1;
+  return g;
+}
+
+template <typename V>
+void launch_edge_copy(V *msg, const V *feat, const uint32_t *ri, const uint32_t *co, const uint32_t *mirror,
+                      uint32_t Vd, uint32_t Fv, int mode, hipStream_t stream) {
+  const dim3 grid = edge_grid(Vd), block(256);
+#define NTS_COPY(GG)                                                                                              \
+  hipLaunchKernelGGL((edge_copy_kernel<V, GG>), grid, block, 0, stream, msg, feat, ri, co, mirror, Vd, Fv, mode)
+  switch (lanes_for(Fv)) {
+    case 1: NTS_COPY(1); break;
+    case 2: NTS_COPY(2); break;
+    case 4: NTS_COPY(4); break;
+    case 8: NTS_COPY(8); break;
+    case 16: NTS_COPY(16); break;
+    case 32: NTS_COPY(32); break;
+    default: NTS_COPY(64); break;
+  }
+#undef NTS_COPY
+}
+
+int edge_copy_impl(float *msg, const float *feat, const uint32_t *ri, const uint32_t *co, const uint32_t *mirror,
+                   uint32_t Vd, uint32_t F, int mode, hipStream_t stream, const char *who) {
   if (F == 0) return fail(NTS_ERR_INVALID, who);
   if (Vd == 0) return NTS_OK;
-  if (!msg || !feat || !co) return fail(NTS_ERR_INVALID, who);
-  switch (row_vec(F, msg, feat)) {
-    case 4:
-      hipLaunchKernelGGL((scatter_dst_to_edge_kernel<float4, ADD>), wave_grid(Vd), wave_block(), 0, stream,
-                         reinterpret_cast<float4 *>(msg), reinterpret_cast<const float4 *>(feat), co, Vd, F / 4);
-      break;
-    case 2:
-      hipLaunchKernelGGL((scatter_dst_to_edge_kernel<float2, ADD>), wave_grid(Vd), wave_block(), 0, stream,
-                         reinterpret_cast<float2 *>(msg), reinterpret_cast<const float2 *>(feat), co, Vd, F / 2);
-      break;
-    default:
-      hipLaunchKernelGGL((scatter_dst_to_edge_kernel<float, ADD>), wave_grid(Vd), wave_block(), 0, stream, msg, feat,
-                         co, Vd, F);
-  }
+  if (!msg || !feat || !co || (mode == kFromSrc && !ri)) return fail(NTS_ERR_INVALID, who);
+  if (F % 4 == 0 && aligned_to(msg, 16) && aligned_to(feat, 16))
+    launch_edge_copy(reinterpret_cast<float4 *>(msg), reinterpret_cast<const float4 *>(feat), ri, co, mirror, Vd,
+                     F / 4, mode, stream);
+  else
+    launch_edge_copy(msg, feat, ri, co, mirror, Vd, F, mode, stream);
   NTS_LAUNCH_CHECK(who);
   return NTS_OK;
+}
+
+// Scratch of the long-row path: list[rows] followed by the counter, in stream-ordered memory.
+struct LongRows {
+  uint32_t *list = nullptr;
+  uint32_t *count = nullptr;
+};
+
+// Collects the rows whose segment holds more than `limit` values (edges * width) when the vertex
+// count makes hubs likely; returns with lr.list == nullptr when the long path is not used.
+int collect_long_rows(LongRows &lr, const uint32_t *off, uint32_t rows, uint32_t width, uint32_t limit,
+                      hipStream_t stream) {
+  if (rows < kLongMinVertices) return NTS_OK;
+  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&lr.list), (static_cast<size_t>(rows) + 1) * sizeof(uint32_t),
+                             stream));
+  lr.count = lr.list + rows;
+  if (int rc = nts_memset_zero(lr.count, sizeof(uint32_t), stream)) return rc;
+  hipLaunchKernelGGL(collect_long_rows_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, stream, lr.list, lr.count, off,
+                     rows, width, limit);
+  NTS_LAUNCH_CHECK("collect_long_rows_kernel");
+  return NTS_OK;
+}
+
+int release_long_rows(LongRows &lr, hipStream_t stream) {
+  if (lr.list) NTS_HIP_TRY(hipFreeAsync(lr.list, stream));
+  lr.list = lr.count = nullptr;
+  return NTS_OK;
+}
+
+constexpr unsigned kLongGrid = 512;  // blocks of the long-row kernels; they stride over the list
+
+template <typename V>
+void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_t *perm, uint32_t rows, uint32_t Fv,
+                        int accumulate, uint32_t limit, hipStream_t stream) {
+#define NTS_GATHER(GG)                                                                                          \
+  hipLaunchKernelGGL((gather_edge_to_row_kernel<V, GG>), dim3(ceil_div(static_cast<uint64_t>(rows) * GG, 256)),  \
+                     dim3(256), 0, stream, out, msg, off, perm, rows, Fv, accumulate, limit)
+  switch (lanes_for(Fv)) {
+    case 1: NTS_GATHER(1); break;
+    case 2: NTS_GATHER(2); break;
+    case 4: NTS_GATHER(4); break;
+    case 8: NTS_GATHER(8); break;
+    case 16: NTS_GATHER(16); break;
+    case 32: NTS_GATHER(32); break;
+    default: NTS_GATHER(64); break;
+  }
+#undef NTS_GATHER
 }
 
 int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const uint32_t *perm, uint32_t rows,
@@ -371,23 +631,72 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
   if (F == 0) return fail(NTS_ERR_INVALID, who);
   if (rows == 0) return NTS_OK;
   if (!out || !msg || !off) return fail(NTS_ERR_INVALID, who);
-  switch (row_vec(F, out, msg)) {
-    case 4:
-      hipLaunchKernelGGL(gather_edge_to_row_kernel<float4>, wave_grid(rows), wave_block(), 0, stream,
-                         reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, rows,
-                         F / 4, accumulate);
-      break;
-    case 2:
-      hipLaunchKernelGGL(gather_edge_to_row_kernel<float2>, wave_grid(rows), wave_block(), 0, stream,
-                         reinterpret_cast<float2 *>(out), reinterpret_cast<const float2 *>(msg), off, perm, rows,
-                         F / 2, accumulate);
-      break;
-    default:
-      hipLaunchKernelGGL(gather_edge_to_row_kernel<float>, wave_grid(rows), wave_block(), 0, stream, out, msg, off,
-                         perm, rows, F, accumulate);
-  }
+  LongRows lr;
+  if (int rc = collect_long_rows(lr, off, rows, 1u, kLongRowEdges, stream)) return rc;
+  const uint32_t limit = lr.list ? kLongRowEdges : kNoLimit;
+  if (F % 4 == 0 && aligned_to(out, 16) && aligned_to(msg, 16))
+    launch_gather_rows(reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, rows, F / 4,
+                       accumulate, limit, stream);
+  else
+    launch_gather_rows(out, msg, off, perm, rows, F, accumulate, limit, stream);
   NTS_LAUNCH_CHECK(who);
-  return NTS_OK;
+  if (lr.list) {
+    uint32_t tile = 1;
+    while (tile < F && tile < static_cast<uint32_t>(kLongBlock)) tile <<= 1;
+    hipLaunchKernelGGL(gather_edge_to_row_long_kernel, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, msg, off,
+                       perm, lr.list, lr.count, F, tile, accumulate);
+    NTS_LAUNCH_CHECK(who);
+  }
+  return release_long_rows(lr, stream);
+}
+
+// Edge softmax / fused attention, forward (gy == nullptr) or backward; x / el / er / ri / ger are
+// null where the variant does not use them.
+int softmax_impl(bool backward, bool fused, float *out, float *ger, const float *x_or_gy, const float *y,
+                 const float *el, const float *er, const uint32_t *co, const uint32_t *ri, uint32_t Vd, uint32_t H,
+                 float slope, hipStream_t stream, const char *who) {
+  const bool pow2 = is_pow2(H) && H <= kWave;
+  LongRows lr;
+  if (pow2)
+    if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, stream)) return rc;
+  const uint32_t limit = lr.list ? kLongRowValues : kNoLimit;
+  const dim3 grid = wave_grid(Vd), block = wave_block();
+  if (!backward) {
+#define NTS_FWD(FU, P2)                                                                                          \
+  hipLaunchKernelGGL((edge_softmax_fwd_kernel<FU, P2>), grid, block, 0, stream, out, x_or_gy, el, er, co, ri, Vd, H, \
+                     slope, limit)
+    if (fused) { if (pow2) NTS_FWD(true, true); else NTS_FWD(true, false); }
+    else       { if (pow2) NTS_FWD(false, true); else NTS_FWD(false, false); }
+#undef NTS_FWD
+    NTS_LAUNCH_CHECK(who);
+    if (lr.list) {
+      if (fused)
+        hipLaunchKernelGGL(edge_softmax_fwd_long_kernel<true>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out,
+                           x_or_gy, el, er, co, ri, lr.list, lr.count, H, slope);
+      else
+        hipLaunchKernelGGL(edge_softmax_fwd_long_kernel<false>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out,
+                           x_or_gy, el, er, co, ri, lr.list, lr.count, H, slope);
+      NTS_LAUNCH_CHECK(who);
+    }
+  } else {
+#define NTS_BWD(FU, P2)                                                                                           \
+  hipLaunchKernelGGL((edge_softmax_bwd_kernel<FU, P2>), grid, block, 0, stream, out, ger, x_or_gy, y, el, er, co, ri, \
+                     Vd, H, slope, limit)
+    if (fused) { if (pow2) NTS_BWD(true, true); else NTS_BWD(true, false); }
+    else       { if (pow2) NTS_BWD(false, true); else NTS_BWD(false, false); }
+#undef NTS_BWD
+    NTS_LAUNCH_CHECK(who);
+    if (lr.list) {
+      if (fused)
+        hipLaunchKernelGGL(edge_softmax_bwd_long_kernel<true>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, ger,
+                           x_or_gy, y, el, er, co, ri, lr.list, lr.count, H, slope);
+      else
+        hipLaunchKernelGGL(edge_softmax_bwd_long_kernel<false>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, ger,
+                           x_or_gy, y, el, er, co, ri, lr.list, lr.count, H, slope);
+      NTS_LAUNCH_CHECK(who);
+    }
+  }
+  return release_long_rows(lr, stream);
 }
 }  // namespace
 
@@ -395,36 +704,19 @@ extern "C" {
 
 int nts_scatter_src_to_edge(float *msg, const float *feat, const uint32_t *ri, const uint32_t *co,
                             const uint32_t *mirror, uint32_t Vd, uint32_t F, nts_stream_t stream) {
-  if (F == 0) return fail(NTS_ERR_INVALID, "nts_scatter_src_to_edge: F is 0");
-  if (Vd == 0) return NTS_OK;
-  if (!msg || !feat || !ri || !co) return fail(NTS_ERR_INVALID, "nts_scatter_src_to_edge: null pointer");
-  switch (row_vec(F, msg, feat)) {
-    case 4:
-      hipLaunchKernelGGL(scatter_src_to_edge_kernel<float4>, wave_grid(Vd), wave_block(), 0, stream,
-                         reinterpret_cast<float4 *>(msg), reinterpret_cast<const float4 *>(feat), ri, co, mirror, Vd,
-                         F / 4);
-      break;
-    case 2:
-      hipLaunchKernelGGL(scatter_src_to_edge_kernel<float2>, wave_grid(Vd), wave_block(), 0, stream,
-                         reinterpret_cast<float2 *>(msg), reinterpret_cast<const float2 *>(feat), ri, co, mirror, Vd,
-                         F / 2);
-      break;
-    default:
-      hipLaunchKernelGGL(scatter_src_to_edge_kernel<float>, wave_grid(Vd), wave_block(), 0, stream, msg, feat, ri, co,
-                         mirror, Vd, F);
-  }
-  NTS_LAUNCH_CHECK("nts_scatter_src_to_edge");
-  return NTS_OK;
+  return edge_copy_impl(msg, feat, ri, co, mirror, Vd, F, kFromSrc, stream, "nts_scatter_src_to_edge: bad argument");
 }
 
 int nts_scatter_dst_to_edge(float *msg, const float *feat, const uint32_t *co, uint32_t Vd, uint32_t F,
                             nts_stream_t stream) {
-  return scatter_dst_impl<false>(msg, feat, co, Vd, F, stream, "nts_scatter_dst_to_edge: bad argument");
+  return edge_copy_impl(msg, feat, nullptr, co, nullptr, Vd, F, kFromDst, stream,
+                        "nts_scatter_dst_to_edge: bad argument");
 }
 
 int nts_scatter_grad_to_edge(float *msg_grad, const float *gout, const uint32_t *co, uint32_t Vd, uint32_t F,
                              nts_stream_t stream) {
-  return scatter_dst_impl<true>(msg_grad, gout, co, Vd, F, stream, "nts_scatter_grad_to_edge: bad argument");
+  return edge_copy_impl(msg_grad, gout, nullptr, co, nullptr, Vd, F, kAddFromDst, stream,
+                        "nts_scatter_grad_to_edge: bad argument");
 }
 
 int nts_gather_edge_to_dst(float *out, const float *msg, const uint32_t *co, uint32_t Vd, uint32_t F, int accumulate,
@@ -443,14 +735,8 @@ int nts_edge_softmax_fwd(float *y, const float *x, const uint32_t *co, uint32_t 
   if (H == 0) return fail(NTS_ERR_INVALID, "nts_edge_softmax_fwd: H is 0");
   if (Vd == 0) return NTS_OK;
   if (!y || !x || !co) return fail(NTS_ERR_INVALID, "nts_edge_softmax_fwd: null pointer");
-  if (is_pow2(H) && H <= kWave)
-    hipLaunchKernelGGL((edge_softmax_fwd_kernel<false, true>), wave_grid(Vd), wave_block(), 0, stream, y, x, nullptr,
-                       nullptr, co, nullptr, Vd, H, 0.f);
-  else
-    hipLaunchKernelGGL((edge_softmax_fwd_kernel<false, false>), wave_grid(Vd), wave_block(), 0, stream, y, x, nullptr,
-                       nullptr, co, nullptr, Vd, H, 0.f);
-  NTS_LAUNCH_CHECK("nts_edge_softmax_fwd");
-  return NTS_OK;
+  return softmax_impl(false, false, y, nullptr, x, nullptr, nullptr, nullptr, co, nullptr, Vd, H, 0.f, stream,
+                      "nts_edge_softmax_fwd");
 }
 
 int nts_edge_softmax_bwd(float *gx, const float *gy, const float *y, const uint32_t *co, uint32_t Vd, uint32_t H,
@@ -458,14 +744,8 @@ int nts_edge_softmax_bwd(float *gx, const float *gy, const float *y, const uint3
   if (H == 0) return fail(NTS_ERR_INVALID, "nts_edge_softmax_bwd: H is 0");
   if (Vd == 0) return NTS_OK;
   if (!gx || !gy || !y || !co) return fail(NTS_ERR_INVALID, "nts_edge_softmax_bwd: null pointer");
-  if (is_pow2(H) && H <= kWave)
-    hipLaunchKernelGGL((edge_softmax_bwd_kernel<false, true>), wave_grid(Vd), wave_block(), 0, stream, gx, nullptr, gy,
-                       y, nullptr, nullptr, co, nullptr, Vd, H, 0.f);
-  else
-    hipLaunchKernelGGL((edge_softmax_bwd_kernel<false, false>), wave_grid(Vd), wave_block(), 0, stream, gx, nullptr,
-                       gy, y, nullptr, nullptr, co, nullptr, Vd, H, 0.f);
-  NTS_LAUNCH_CHECK("nts_edge_softmax_bwd");
-  return NTS_OK;
+  return softmax_impl(true, false, gx, nullptr, gy, y, nullptr, nullptr, co, nullptr, Vd, H, 0.f, stream,
+                      "nts_edge_softmax_bwd");
 }
 
 int nts_gat_attention_fwd(float *alpha, const float *el, const float *er, const uint32_t *co, const uint32_t *ri,
@@ -473,14 +753,8 @@ int nts_gat_attention_fwd(float *alpha, const float *el, const float *er, const 
   if (H == 0) return fail(NTS_ERR_INVALID, "nts_gat_attention_fwd: H is 0");
   if (Vd == 0) return NTS_OK;
   if (!alpha || !el || !er || !co || !ri) return fail(NTS_ERR_INVALID, "nts_gat_attention_fwd: null pointer");
-  if (is_pow2(H) && H <= kWave)
-    hipLaunchKernelGGL((edge_softmax_fwd_kernel<true, true>), wave_grid(Vd), wave_block(), 0, stream, alpha, nullptr,
-                       el, er, co, ri, Vd, H, slope);
-  else
-    hipLaunchKernelGGL((edge_softmax_fwd_kernel<true, false>), wave_grid(Vd), wave_block(), 0, stream, alpha, nullptr,
-                       el, er, co, ri, Vd, H, slope);
-  NTS_LAUNCH_CHECK("nts_gat_attention_fwd");
-  return NTS_OK;
+  return softmax_impl(false, true, alpha, nullptr, nullptr, nullptr, el, er, co, ri, Vd, H, slope, stream,
+                      "nts_gat_attention_fwd");
 }
 
 int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const float *alpha, const float *el,
@@ -490,27 +764,31 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
   if (Vd == 0) return NTS_OK;
   if (!gs || !ger || !galpha || !alpha || !el || !er || !co || !ri)
     return fail(NTS_ERR_INVALID, "nts_gat_attention_bwd: null pointer");
-  if (is_pow2(H) && H <= kWave)
-    hipLaunchKernelGGL((edge_softmax_bwd_kernel<true, true>), wave_grid(Vd), wave_block(), 0, stream, gs, ger, galpha,
-                       alpha, el, er, co, ri, Vd, H, slope);
-  else
-    hipLaunchKernelGGL((edge_softmax_bwd_kernel<true, false>), wave_grid(Vd), wave_block(), 0, stream, gs, ger, galpha,
-                       alpha, el, er, co, ri, Vd, H, slope);
-  NTS_LAUNCH_CHECK("nts_gat_attention_bwd");
-  return NTS_OK;
+  return softmax_impl(true, true, gs, ger, galpha, alpha, el, er, co, ri, Vd, H, slope, stream,
+                      "nts_gat_attention_bwd");
 }
 
 int nts_sddmm_heads(float *galpha, const float *in, const float *gout, const uint32_t *co, const uint32_t *ri,
                     uint32_t Vd, uint32_t H, uint32_t Fh, nts_stream_t stream) {
   if (H == 0 || Fh == 0) return fail(NTS_ERR_INVALID, "nts_sddmm_heads: H or Fh is 0");
+  if (static_cast<uint64_t>(H) * Fh > 0xFFFFFFFFull) return fail(NTS_ERR_INVALID, "nts_sddmm_heads: H*Fh overflows");
   if (Vd == 0) return NTS_OK;
   if (!galpha || !in || !gout || !co || !ri) return fail(NTS_ERR_INVALID, "nts_sddmm_heads: null pointer");
-  if (is_pow2(Fh) && static_cast<uint64_t>(H) * Fh <= kWave)
-    hipLaunchKernelGGL(sddmm_heads_pow2_kernel, wave_grid(Vd), wave_block(), 0, stream, galpha, in, gout, co, ri, Vd,
-                       H, Fh);
-  else
-    hipLaunchKernelGGL(sddmm_heads_kernel, wave_grid(Vd), wave_block(), 0, stream, galpha, in, gout, co, ri, Vd, H,
-                       Fh);
+  const uint32_t F = H * Fh;
+  const dim3 grid = edge_grid(Vd), block(256);
+  const bool v4 = Fh % 4 == 0 && aligned_to(in, 16) && aligned_to(gout, 16);
+  const uint32_t vec = v4 ? 4 : 1;
+  const uint32_t lanes = F / vec, lanes_per_head = Fh / vec;
+  if (lanes <= kWave && is_pow2(lanes) && is_pow2(lanes_per_head)) {
+    if (v4)
+      hipLaunchKernelGGL(sddmm_edge_kernel<4>, grid, block, 0, stream, galpha, in, gout, co, ri, Vd, H, Fh, lanes,
+                         lanes_per_head);
+    else
+      hipLaunchKernelGGL(sddmm_edge_kernel<1>, grid, block, 0, stream, galpha, in, gout, co, ri, Vd, H, Fh, lanes,
+                         lanes_per_head);
+  } else {
+    hipLaunchKernelGGL(sddmm_edge_generic_kernel, grid, block, 0, stream, galpha, in, gout, co, ri, Vd, H, Fh);
+  }
   NTS_LAUNCH_CHECK("nts_sddmm_heads");
   return NTS_OK;
 }

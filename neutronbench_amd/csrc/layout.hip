@@ -13,16 +13,6 @@
 namespace nts {
 namespace {
 
-// Largest r such that off[r] <= pos, searched in off[0 .. n] (off ascending, off[n] > pos).
-__device__ __forceinline__ uint32_t owner_of(const uint32_t *__restrict__ off, uint32_t n, uint32_t pos) {
-  uint32_t lo = 0, hi = n;  // answer in [lo, hi)
-  while (hi - lo > 1) {
-    const uint32_t mid = lo + (hi - lo) / 2;
-    if (off[mid] <= pos) lo = mid; else hi = mid;
-  }
-  return lo;
-}
-
 // ro[s] = number of sorted keys < s, for s in [0, Vs]; keys ascending, E of them.
 __global__ __launch_bounds__(256) void offsets_from_sorted_kernel(uint32_t *__restrict__ ro,
                                                                   const uint32_t *__restrict__ keys, uint32_t Vs,

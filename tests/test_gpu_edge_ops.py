@@ -199,3 +199,82 @@ def test_fused_gat_layer(device, H, Fh):
     dgs_ref = dev(gs_ref, device)
     call("nts_gather_edge_to_src", ptr(gel), ptr(dgs_ref), ptr(dro), ptr(dperm), Vs, H, 0, s)
     assert np.array_equal(gel.cpu().numpy(), gel_ref)
+
+
+@pytest.mark.parametrize("H", [1, 4, 3])
+def test_long_segments_softmax_and_attention(device, H):
+    """Vertex counts at which the library hands hub segments (more than 4096 values) to its block
+    kernels: edge softmax and fused attention, forward and backward, still match the oracle."""
+    print(f"case H={H}", flush=True)
+    Vd, Vs = 17000, 2500
+    co, ri = random_block(Vd, Vs, 3, seed=300 + H, hub=7000, dup=True)
+    co, ri = co.copy(), ri.copy()
+    E = ri.size
+    rng = np.random.default_rng(H)
+    x = (rng.standard_normal((E, H)) * 3).astype(np.float32)
+    gy = rng.standard_normal((E, H)).astype(np.float32)
+    dco, dri, dx, dgy = dev(co, device), dev(ri, device), dev(x, device), dev(gy, device)
+    y = torch.full((E, H), float("nan"), device=device)
+    call("nts_edge_softmax_fwd", ptr(y), ptr(dx), ptr(dco), Vd, H, stream())
+    ref = oracle.edge_softmax(x, co)
+    got = y.cpu().numpy()
+    check(got, ref, scale=1.0, floor=1e-7)
+    gx = torch.full((E, H), float("nan"), device=device)
+    call("nts_edge_softmax_bwd", ptr(gx), ptr(dgy), ptr(y), ptr(dco), Vd, H, stream())
+    refb = oracle.edge_softmax_bwd(gy, got, co)
+    seg_abs = oracle.scatter_dst(oracle.aggregate_dst(np.abs(gy) * got, co), co, E)
+    check(gx.cpu().numpy(), refb, scale=got * (np.abs(gy) + seg_abs))
+    # fused attention
+    el = rng.standard_normal((Vs, H)).astype(np.float32)
+    er = rng.standard_normal((Vd, H)).astype(np.float32)
+    pre = (oracle.scatter_src(el, co, ri) + oracle.scatter_dst(er, co, E)).astype(np.float32)
+    m = np.where(pre > 0, pre, np.float32(0.2) * pre).astype(np.float32)
+    alpha_ref = oracle.edge_softmax(m, co)
+    del_, der = dev(el, device), dev(er, device)
+    alpha = torch.full((E, H), float("nan"), device=device)
+    call("nts_gat_attention_fwd", ptr(alpha), ptr(del_), ptr(der), ptr(dco), ptr(dri), Vd, H, 0.2, stream())
+    check(alpha.cpu().numpy(), alpha_ref, scale=1.0, floor=1e-7)
+    dalpha_ref = dev(alpha_ref, device)
+    gs = torch.full((E, H), float("nan"), device=device)
+    ger = torch.full((Vd, H), float("nan"), device=device)
+    call("nts_gat_attention_bwd", ptr(gs), ptr(ger), ptr(dgy), ptr(dalpha_ref), ptr(del_), ptr(der), ptr(dco), ptr(dri),
+         Vd, H, 0.2, stream())
+    gm = oracle.edge_softmax_bwd(gy, alpha_ref, co)
+    gs_ref = (gm * np.where(pre > 0, np.float32(1.0), np.float32(0.2))).astype(np.float32)
+    seg_abs = oracle.scatter_dst(oracle.aggregate_dst(np.abs(gy) * alpha_ref, co), co, E)
+    scale_gs = alpha_ref * (np.abs(gy) + seg_abs)
+    check(gs.cpu().numpy(), gs_ref, scale=scale_gs)
+    check(ger.cpu().numpy(), oracle.aggregate_dst(gs_ref, co), scale=oracle.aggregate_dst(scale_gs.astype(np.float32), co))
+
+
+@pytest.mark.parametrize("F", [1, 4, 33, 128, 1100])
+def test_long_rows_edge_sums(device, F):
+    """Edge -> vertex sums with hub rows beyond 1024 edges (block kernel: slices added in a fixed
+    order): within tolerance of the oracle's edge-order sum, bit-reproducible, accumulate honoured."""
+    print(f"case F={F}", flush=True)
+    Vd, Vs = 17000, 20000
+    co, ri = random_block(Vd, Vs, 2, seed=400 + F, hub=5000, dup=True)
+    ri[int(co[1]):int(co[2])] = 7  # make source 7 a hub of the transposed structure as well
+    ri[:3000] = 7
+    ro, ci, perm = brute_csr(co, ri, Vs)
+    E = ri.size
+    rng = np.random.default_rng(F)
+    em = rng.standard_normal((E, F)).astype(np.float32)
+    dco, dro, dperm, dem = dev(co, device), dev(ro, device), dev(perm, device), dev(em, device)
+    want_d = oracle.aggregate_dst(em, co)
+    want_s = oracle.gather_to_src(em, co, ri, Vs)
+    sc_d = oracle.aggregate_dst(np.abs(em), co)
+    sc_s = oracle.gather_to_src(np.abs(em), co, ri, Vs)
+    outs = []
+    for _ in range(2):
+        out = torch.full((Vd, F), float("nan"), device=device)
+        call("nts_gather_edge_to_dst", ptr(out), ptr(dem), ptr(dco), Vd, F, 0, stream())
+        outs.append(out.cpu().numpy())
+    check(outs[0], want_d, scale=sc_d)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    short = np.diff(co.astype(np.int64)) <= 1024
+    assert np.array_equal(outs[0][short], want_d[short])  # short rows keep the plain edge order
+    init = rng.standard_normal((Vs, F)).astype(np.float32)
+    outs_ = dev(init, device)
+    call("nts_gather_edge_to_src", ptr(outs_), ptr(dem), ptr(dro), ptr(dperm), Vs, F, 1, stream())
+    check(outs_.cpu().numpy(), want_s + init, scale=sc_s + np.abs(init))
