@@ -43,20 +43,22 @@ __device__ __forceinline__ float norm_weight(uint32_t out_deg, uint32_t in_deg) 
   return __fdiv_rn(1.0f, __fmul_rn(a, b));
 }
 
-// which = 0: thread per CSC edge e, owner = destination, other end = ri[e] (a source).
-// which = 1: thread per CSR edge k, owner = source, other end = ci[k] (a destination).
+// which = 0: CSC edges e, owner = destination, other end = ri[e] (a source).
+// which = 1: CSR edges k, owner = source, other end = ci[k] (a destination).
+// The edge count is read on the device (own_off[n_own]); threads stride over the edges.
 __global__ __launch_bounds__(256) void edge_weights_kernel(float *__restrict__ wout,
                                                            const uint32_t *__restrict__ own_off, uint32_t n_own,
                                                            const uint32_t *__restrict__ other_idx,
-                                                           const uint32_t *__restrict__ other_off, uint32_t E,
-                                                           int which) {
-  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= E) return;
-  const uint32_t o = owner_of(own_off, n_own, e);
-  const uint32_t own_deg = own_off[o + 1] - own_off[o];
-  const uint32_t t = other_idx[e];
-  const uint32_t other_deg = other_off[t + 1] - other_off[t];
-  wout[e] = which == 0 ? norm_weight(other_deg, own_deg) : norm_weight(own_deg, other_deg);
+                                                           const uint32_t *__restrict__ other_off, int which) {
+  const uint32_t E = own_off[n_own];
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+  for (uint64_t e = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; e < E; e += stride) {
+    const uint32_t o = owner_of(own_off, n_own, static_cast<uint32_t>(e));
+    const uint32_t own_deg = own_off[o + 1] - own_off[o];
+    const uint32_t t = other_idx[e];
+    const uint32_t other_deg = other_off[t + 1] - other_off[t];
+    wout[e] = which == 0 ? norm_weight(other_deg, own_deg) : norm_weight(own_deg, other_deg);
+  }
 }
 
 // keys[e] = mirror ? mirror[ri[e]] : ri[e]
@@ -273,19 +275,20 @@ int nts_gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint3
                          const uint32_t *ci, uint32_t Vd, uint32_t Vs, nts_stream_t stream) {
   if (!co || !ro) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null offsets");
   if (Vd == 0 || Vs == 0) return NTS_OK;
-  // The edge count lives on the device; one small read-back keeps the ABI free of redundant sizes.
-  uint32_t E = 0;
-  NTS_HIP_TRY(hipMemcpyAsync(&E, co + Vd, sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-  NTS_HIP_TRY(hipStreamSynchronize(stream));
-  if (E == 0) return NTS_OK;
+  // The edge count lives on the device: the grid is sized from the vertex counts and the kernel
+  // strides over co[Vd] edges, so the call neither needs the count nor synchronises.
+  uint64_t blocks = (static_cast<uint64_t>(Vd > Vs ? Vd : Vs) * 32 + 255) / 256;
+  if (blocks < 64) blocks = 64;
+  if (blocks > 8192) blocks = 8192;
+  const dim3 grid(static_cast<unsigned>(blocks));
   if (ewf) {
     if (!ri) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ri");
-    hipLaunchKernelGGL(edge_weights_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ewf, co, Vd, ri, ro, E, 0);
+    hipLaunchKernelGGL(edge_weights_kernel, grid, dim3(256), 0, stream, ewf, co, Vd, ri, ro, 0);
     NTS_LAUNCH_CHECK("edge_weights_kernel(fwd)");
   }
   if (ewb) {
     if (!ci) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ci");
-    hipLaunchKernelGGL(edge_weights_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ewb, ro, Vs, ci, co, E, 1);
+    hipLaunchKernelGGL(edge_weights_kernel, grid, dim3(256), 0, stream, ewb, ro, Vs, ci, co, 1);
     NTS_LAUNCH_CHECK("edge_weights_kernel(bwd)");
   }
   return NTS_OK;
