@@ -328,6 +328,65 @@ int nts_gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint3
                          const uint32_t *ro, const uint32_t *ci, uint32_t Vd, uint32_t Vs,
                          nts_stream_t stream);
 
+/* PartitionedGraph::generatePartitionedSubgraph + PartitionToChunks for one partition
+ * (core/PartitionedGraph.hpp:281-388; device arrays of CSC_segment_pinned, core/GraphSegment.h:54-133):
+ * from the edge list `pairs` (device, E records {src, dst} as the .edge file holds them, all ids < V)
+ * builds on the device
+ *   CSR  ro [V+1], ci [E]: edges ordered by source, input order kept inside a source,
+ *   CSC  co [V+1], ri [E]: that list re-ordered by destination, stably (sources ascend in a row),
+ * and, unless both are NULL, ewf [E] / ewb [E] = nts_norm_degree(out_deg(src), in_deg(dst)) in CSC /
+ * CSR order, degrees being the edge counts of the list (duplicates and self loops count).
+ * `work` is nts_chunk_from_edges_work_bytes(V, E) bytes of 256-byte-aligned device scratch.
+ * Integer outputs and weights are bit-exact with the host construction fed the same list. */
+size_t nts_chunk_from_edges_work_bytes(uint32_t V, uint32_t E);
+int nts_chunk_from_edges(uint32_t *co, uint32_t *ri, float *ewf, uint32_t *ro, uint32_t *ci, float *ewb,
+                         const uint32_t *pairs, uint32_t E, uint32_t V, void *work, nts_stream_t stream);
+
+/* ---- on-disk dataset formats (host side; all buffers are host memory) ------------------------- */
+
+/* Binary edge list: packed records {uint32 src, uint32 dst} in host byte order, no header
+ * (EdgeUnit<Empty>, dep/gemini/type.hpp:99-106; Graph::load_directed takes file bytes / 8 as the
+ * edge count, core/graph.hpp:1050-1061; written by data/generate_nts_dataset.py:340-345).
+ * nts_edge_file_read copies records [first, first+n) into pairs [2n] and, if max_id is not NULL,
+ * stores the largest vertex id among them (callers check it against their vertex count). */
+int nts_edge_file_count(const char *path, uint64_t *edges);
+int nts_edge_file_read(const char *path, uint32_t *pairs, uint64_t first, uint64_t n, uint32_t *max_id);
+
+/* GNNDatum::readFeature_Label_Mask for a partition that owns every vertex
+ * (core/ntsDataloador.hpp:264-395; readFtrFrom1, :209-262, reads the same feature and label text).
+ * All three files are white-space separated tokens.
+ *   feature file: records of 1 + F tokens "id f0 .. fF-1"; the values go to local_feature[id*F ..]
+ *     ([V, F]); a value is the nearest float of its decimal text, as `istream >> float` yields;
+ *     records whose id is >= V are skipped like vertices outside the reader's partition.
+ *   label file: records "id label" (classes <= 1, tables [V]) or "id count idx_1 .. idx_count"
+ *     (classes > 1, tables [V, classes], the named entries are set to 1).
+ *   mask file: records "id word"; train -> 0, eval / val -> 1, test -> 2, anything else -> 3.
+ * local_label / local_mask: the k-th label / mask record is stored at the vertex named by the k-th
+ * FEATURE record (the files are read in step and the id column of the label / mask file is
+ * ignored); global_label / global_mask: records are stored at their own id.  Entries the files do
+ * not name keep their value, so tables come in zeroed as the reference's constructor leaves them
+ * (:78-88).  Any of the four label / mask tables may be NULL.  Parsing runs on `threads` host
+ * threads (<= 0: all); it fails with NTS_ERR_INVALID on an unreadable file, a malformed token or an
+ * incomplete last feature record. */
+int nts_read_feature_label_mask(const char *path_f, const char *path_l, const char *path_m, uint32_t V,
+                                uint32_t F, uint32_t classes, float *local_feature, int64_t *local_label,
+                                int32_t *local_mask, int64_t *global_label, int32_t *global_mask,
+                                int threads);
+/* Comma-separated feature file of readFeature_Label_Mask_OGB (core/ntsDataloador.hpp:397-437): line k
+ * holds the F values of vertex k; each field is converted with atof and narrowed to float. */
+int nts_feature_csv_read(const char *path, float *table, uint32_t V, uint32_t F, int threads);
+/* White-space separated integers (the label column and the train / valid / test id lists of
+ * readFeature_Label_Mask_OGB, core/ntsDataloador.hpp:432, 461-469): stores the first `capacity` of them
+ * in out (may be NULL) and the number found in *count; reading ends at the first non-integer token. */
+int nts_int_list_text_read(const char *path, int64_t *out, uint64_t capacity, uint64_t *count);
+/* Binary table (no counterpart in the reference, which only reads text): a 32-byte little-endian
+ * header {"NTSTABLE", uint64 rows, uint64 cols, uint32 elem_bytes, uint32 0} followed by the
+ * row-major data.  nts_table_bin_read copies rows [row_begin, row_begin+rows) into out, e.g.
+ * straight into the pinned feature table. */
+int nts_table_bin_write(const char *path, const void *data, uint64_t rows, uint64_t cols, uint32_t elem_bytes);
+int nts_table_bin_info(const char *path, uint64_t *rows, uint64_t *cols, uint32_t *elem_bytes);
+int nts_table_bin_read(const char *path, void *out, uint64_t row_begin, uint64_t rows);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,6 +20,8 @@ _u32 = ctypes.c_uint32
 _int = ctypes.c_int
 _sz = ctypes.c_size_t
 _f32 = ctypes.c_float
+_u64 = ctypes.c_uint64
+_str = ctypes.c_char_p
 
 # name -> argument types, in the order of include/nts_hip.h.  All return int unless listed in _RESTYPES.
 SIGNATURES = {
@@ -79,12 +81,23 @@ SIGNATURES = {
     "nts_csr_from_csc_work_bytes": [_u32, _u32, _u32],
     "nts_csr_from_csc": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp, _vp],
     "nts_gcn_edge_weights": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],
+    "nts_chunk_from_edges_work_bytes": [_u32, _u32],
+    "nts_chunk_from_edges": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp],
+    "nts_edge_file_count": [_str, ctypes.POINTER(_u64)],
+    "nts_edge_file_read": [_str, _vp, _u64, _u64, ctypes.POINTER(_u32)],
+    "nts_read_feature_label_mask": [_str, _str, _str, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _int],
+    "nts_feature_csv_read": [_str, _vp, _u32, _u32, _int],
+    "nts_int_list_text_read": [_str, _vp, _u64, ctypes.POINTER(_u64)],
+    "nts_table_bin_write": [_str, _vp, _u64, _u64, _u32],
+    "nts_table_bin_info": [_str, ctypes.POINTER(_u64), ctypes.POINTER(_u64), ctypes.POINTER(_u32)],
+    "nts_table_bin_read": [_str, _vp, _u64, _u64],
 }
 _RESTYPES = {"nts_last_error": ctypes.c_char_p, "nts_csr_from_csc_work_bytes": _sz,
-             "nts_relabel_sources_work_bytes": _sz, "nts_sample_hop_work_bytes": _sz}
+             "nts_relabel_sources_work_bytes": _sz, "nts_sample_hop_work_bytes": _sz,
+             "nts_chunk_from_edges_work_bytes": _sz}
 # Entry points whose int result is a value, not a status.
 _NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
-              "nts_sample_hop_work_bytes"}
+              "nts_sample_hop_work_bytes", "nts_chunk_from_edges_work_bytes"}
 
 
 class NtsError(RuntimeError):

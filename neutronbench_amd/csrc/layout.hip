@@ -159,6 +159,25 @@ hipError_t sort_temp_bytes(uint32_t E, size_t *bytes) {
   return err;
 }
 
+// Splits the (src, dst) pairs of an edge list into two key arrays.
+__global__ __launch_bounds__(256) void split_pairs_kernel(uint32_t *__restrict__ src, uint32_t *__restrict__ dst,
+                                                          const uint2 *__restrict__ pairs, uint32_t E) {
+  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= E) return;
+  const uint2 p = pairs[e];
+  src[e] = p.x;
+  dst[e] = p.y;
+}
+
+hipError_t sort_pairs_temp_bytes(uint32_t E, size_t *bytes) {
+  size_t tmp = 0;
+  uint32_t *nul = nullptr;
+  hipError_t err = rocprim::radix_sort_pairs(nullptr, tmp, nul, nul, nul, nul, E ? E : 1u, 0u, 32u,
+                                             static_cast<hipStream_t>(nullptr), false);
+  *bytes = tmp;
+  return err;
+}
+
 }  // namespace
 }  // namespace nts
 
@@ -200,6 +219,50 @@ int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t 
   NTS_LAUNCH_CHECK("offsets_from_sorted_kernel");
   hipLaunchKernelGGL(dst_of_perm_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ci, perm_out, co, Vd, E);
   NTS_LAUNCH_CHECK("dst_of_perm_kernel");
+  return NTS_OK;
+}
+
+size_t nts_chunk_from_edges_work_bytes(uint32_t V, uint32_t E) {
+  (void)V;
+  size_t tmp = 0;
+  if (sort_pairs_temp_bytes(E, &tmp) != hipSuccess) return 0;
+  return 3 * align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256) + align_up(tmp, 256) + 256;
+}
+
+int nts_chunk_from_edges(uint32_t *co, uint32_t *ri, float *ewf, uint32_t *ro, uint32_t *ci, float *ewb,
+                         const uint32_t *pairs, uint32_t E, uint32_t V, void *work, nts_stream_t stream) {
+  if (!co || !ro) return fail(NTS_ERR_INVALID, "nts_chunk_from_edges: null offsets");
+  if (E == 0) {
+    if (int rc = nts_memset_zero(co, (static_cast<size_t>(V) + 1) * sizeof(uint32_t), stream)) return rc;
+    return nts_memset_zero(ro, (static_cast<size_t>(V) + 1) * sizeof(uint32_t), stream);
+  }
+  if (V == 0) return fail(NTS_ERR_INVALID, "nts_chunk_from_edges: edges without vertices");
+  if (!ri || !ci || !pairs || !work) return fail(NTS_ERR_INVALID, "nts_chunk_from_edges: null pointer");
+  if (!aligned_to(work, 256) || !aligned_to(pairs, 8))
+    return fail(NTS_ERR_INVALID, "nts_chunk_from_edges: work must be 256-byte and pairs 8-byte aligned");
+  const size_t arr = align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256);
+  unsigned char *w = static_cast<unsigned char *>(work);
+  uint32_t *a = reinterpret_cast<uint32_t *>(w);            // file-order sources, later destination-sorted keys
+  uint32_t *b = reinterpret_cast<uint32_t *>(w + arr);      // file-order destinations
+  uint32_t *c = reinterpret_cast<uint32_t *>(w + 2 * arr);  // sources in (source, file) order
+  void *tmp_ptr = w + 3 * arr;
+  size_t tmp = 0;
+  NTS_HIP_TRY(sort_pairs_temp_bytes(E, &tmp));
+  const unsigned bits = bits_for(V);
+  hipLaunchKernelGGL(split_pairs_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, a, b,
+                     reinterpret_cast<const uint2 *>(pairs), E);
+  NTS_LAUNCH_CHECK("split_pairs_kernel");
+  // The edge list ordered by source, file order kept inside a source (stable sort): the CSR rows.
+  NTS_HIP_TRY(rocprim::radix_sort_pairs(tmp_ptr, tmp, a, c, b, ci, E, 0u, bits, stream, false));
+  hipLaunchKernelGGL(offsets_from_sorted_kernel, dim3(ceil_div(static_cast<uint64_t>(V) + 1, 256)), dim3(256), 0,
+                     stream, ro, c, V, E);
+  NTS_LAUNCH_CHECK("offsets_from_sorted_kernel(ro)");
+  // That list re-ordered by destination, again stable: the CSC rows (sources ascending inside a row).
+  NTS_HIP_TRY(rocprim::radix_sort_pairs(tmp_ptr, tmp, ci, a, c, ri, E, 0u, bits, stream, false));
+  hipLaunchKernelGGL(offsets_from_sorted_kernel, dim3(ceil_div(static_cast<uint64_t>(V) + 1, 256)), dim3(256), 0,
+                     stream, co, a, V, E);
+  NTS_LAUNCH_CHECK("offsets_from_sorted_kernel(co)");
+  if (ewf || ewb) return nts_gcn_edge_weights(ewf, ewb, co, ri, ro, ci, V, V, stream);
   return NTS_OK;
 }
 

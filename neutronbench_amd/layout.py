@@ -92,27 +92,38 @@ class FullGraphChunk:
         ordered by source (stable in the input order); CSR rows keep that order, CSC rows are the
         stable re-ordering by destination.  Weights are nts_norm_degree of the global degrees.
         """
-        device = src.device
-        E = src.numel()
-        order = torch.sort(src, stable=True).indices
-        coo_src = src[order]
-        coo_dst = dst[order]
-        del order
-        ro = torch.zeros(V + 1, dtype=torch.int64, device=device)
-        ro[1:] = torch.cumsum(torch.bincount(coo_src, minlength=V), 0)
-        perm = torch.sort(coo_dst, stable=True).indices
-        ri = coo_src[perm]
-        co = torch.zeros(V + 1, dtype=torch.int64, device=device)
-        co[1:] = torch.cumsum(torch.bincount(coo_dst, minlength=V), 0)
-        del perm, coo_src
-        co32, ro32 = as_u32(co), as_u32(ro)
-        ri32, ci32 = as_u32(ri), as_u32(coo_dst)
-        del co, ro, ri, coo_dst
+        pairs = torch.stack([src, dst], dim=1).to(torch.int32).contiguous()
+        return cls.from_edge_pairs(pairs, V, chunk_edges, n_slabs)
+
+    @classmethod
+    def from_edge_pairs(cls, pairs, V, chunk_edges=0, n_slabs=1):
+        """`pairs`: int32 device tensor [E, 2] holding the .edge file's records (src, dst)."""
+        device = pairs.device
+        E = pairs.shape[0]
+        co32 = torch.empty(V + 1, dtype=torch.int32, device=device)
+        ro32 = torch.empty(V + 1, dtype=torch.int32, device=device)
+        ri32 = torch.empty(E, dtype=torch.int32, device=device)
+        ci32 = torch.empty(E, dtype=torch.int32, device=device)
         ewf = torch.empty(E, dtype=torch.float32, device=device)
         ewb = torch.empty(E, dtype=torch.float32, device=device)
-        call("nts_gcn_edge_weights", ptr(ewf), ptr(ewb), ptr(co32), ptr(ri32), ptr(ro32), ptr(ci32), V, V,
-             _stream(device))
+        work = torch.empty(call("nts_chunk_from_edges_work_bytes", V, E) + 256, dtype=torch.uint8, device=device)
+        wptr = (work.data_ptr() + 255) // 256 * 256
+        call("nts_chunk_from_edges", ptr(co32), ptr(ri32), ptr(ewf), ptr(ro32), ptr(ci32), ptr(ewb), ptr(pairs), E, V,
+             wptr, _stream(device))
+        torch.cuda.current_stream(device).synchronize()  # `work` and `pairs` may be released by the caller
+        del work
         return cls(V, co32, ri32, ewf, ro32, ci32, ewb, chunk_edges, n_slabs)
+
+    @classmethod
+    def from_edge_file(cls, path, V, device, chunk_edges=0, n_slabs=1):
+        """Graph::load_directed + PartitionToChunks for one partition: reads the binary edge list
+        into pinned memory, uploads it once and builds CSC, CSR and weights on the device."""
+        from .dataset import edge_file_count, read_edge_file
+
+        E = edge_file_count(path)
+        host = torch.empty((E, 2), dtype=torch.int32, pin_memory=True)
+        read_edge_file(path, vertices=V, out=host.numpy().view("uint32"))
+        return cls.from_edge_pairs(host.to(device, non_blocking=True), V, chunk_edges, n_slabs)
 
 
 class SampledLayer:

@@ -317,3 +317,43 @@ def edge_softmax_bwd(gy, y, co):
     lib().nts_oracle_edge_softmax_bwd(gx.ctypes.data_as(_f32p), pg, py, pco, ctypes.c_uint32(co.size - 1),
                                       ctypes.c_uint32(H))
     return gx
+
+
+def read_feature_label_mask(path_f, path_l, path_m, V, F, classes=1):
+    """GNNDatum::readFeature_Label_Mask for one partition owning [0, V).  Returns a dict of the five tables."""
+    width = classes if classes > 1 else 1
+    feat = np.zeros((V, F), dtype=np.float32)
+    ll = np.zeros(V * width, dtype=np.int64)
+    gl = np.zeros(V * width, dtype=np.int64)
+    lm = np.zeros(V, dtype=np.int32)
+    gm = np.zeros(V, dtype=np.int32)
+    i32p = ctypes.POINTER(ctypes.c_int32)
+    rc = lib().nts_oracle_read_feature_label_mask(
+        os.fsencode(path_f), os.fsencode(path_l), os.fsencode(path_m), ctypes.c_uint32(V), ctypes.c_uint32(F),
+        ctypes.c_uint32(classes), feat.ctypes.data_as(_f32p), ll.ctypes.data_as(_i64p), lm.ctypes.data_as(i32p),
+        gl.ctypes.data_as(_i64p), gm.ctypes.data_as(i32p))
+    if rc != 0:
+        raise IOError(f"oracle reader failed with {rc}")
+    return dict(local_feature=feat, local_label=ll, local_mask=lm, global_label=gl, global_mask=gm)
+
+
+def read_feature_label_mask_ogb(path_f, path_l, dir_m, V, F):
+    feat = np.zeros((V, F), dtype=np.float32)
+    ll = np.zeros(V, dtype=np.int64)
+    lm = np.zeros(V, dtype=np.int32)
+    rc = lib().nts_oracle_read_feature_label_mask_ogb(
+        os.fsencode(path_f), os.fsencode(path_l), os.fsencode(dir_m), ctypes.c_uint32(V), ctypes.c_uint32(F),
+        feat.ctypes.data_as(_f32p), ll.ctypes.data_as(_i64p), lm.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)))
+    if rc != 0:
+        raise IOError(f"oracle reader failed with {rc}")
+    return dict(local_feature=feat, local_label=ll, local_mask=lm)
+
+
+def read_edges(path):
+    E = os.path.getsize(path) // 8
+    src = np.empty(max(E, 1), dtype=np.uint32)
+    dst = np.empty(max(E, 1), dtype=np.uint32)
+    f = lib().nts_oracle_read_edges
+    f.restype = ctypes.c_uint64
+    n = f(os.fsencode(path), src.ctypes.data_as(_u32p), dst.ctypes.data_as(_u32p), ctypes.c_uint64(E))
+    return src[:n].copy(), dst[:n].copy()

@@ -16,7 +16,10 @@
  *   the reference holds no test vector at that boundary -> parity unpinned against the reference
  *   itself, pinned against torch.softmax / scipy as a library identity.
  */
+#define _GNU_SOURCE /* getline */
 #include <math.h>
+#include <stdio.h>
+#include <sys/types.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -391,6 +394,163 @@ NTS_EXPORT void nts_oracle_edge_softmax_bwd(float *gx, const float *gy, const fl
       }
     }
   }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * On-disk formats.  Sequential restatements of the reference's readers for one partition that
+ * owns every vertex (p_v_s = 0, p_v_e = V).  `stream >> x` is restated with fscanf, which like the
+ * stream extraction skips white space and converts with the C library's strtof / strtol.
+ * ------------------------------------------------------------------------------------------- */
+
+static int mask_word_code(const char *w) {
+  if (strcmp(w, "train") == 0) return 0;
+  if (strcmp(w, "eval") == 0 || strcmp(w, "val") == 0) return 1;
+  if (strcmp(w, "test") == 0) return 2;
+  return 3;
+}
+
+/* GNNDatum::readFeature_Label_Mask (core/ntsDataloador.hpp:264-395).  The three files are read in
+ * step: the k-th record of the label and of the mask file belongs to the vertex named by the k-th
+ * record of the feature file (local_*); afterwards label and mask files are read again on their
+ * own ids (global_*).  Tables must come in zeroed, as the constructor leaves them (:78-88). */
+NTS_EXPORT int nts_oracle_read_feature_label_mask(const char *path_f, const char *path_l, const char *path_m,
+                                                  uint32_t V, uint32_t F, uint32_t classes, float *local_feature,
+                                                  int64_t *local_label, int32_t *local_mask, int64_t *global_label,
+                                                  int32_t *global_mask) {
+  FILE *ff = fopen(path_f, "r"), *fl = fopen(path_l, "r"), *fm = fopen(path_m, "r");
+  if (!ff || !fl || !fm) {
+    if (ff) fclose(ff);
+    if (fl) fclose(fl);
+    if (fm) fclose(fm);
+    return -1;
+  }
+  char la[256], msk[256];
+  unsigned id = 0;
+  float skip;
+  while (fscanf(ff, "%u", &id) == 1) {
+    if (id < V) {
+      for (uint32_t i = 0; i < F; ++i)
+        if (fscanf(ff, "%f", &local_feature[(size_t)F * id + i]) != 1) break;
+      if (fscanf(fl, "%255s", la) != 1) la[0] = 0;
+      if (classes > 1) {
+        int sz = 0, idx = 0;
+        if (fscanf(fl, "%d", &sz) != 1) sz = 0;
+        while (sz--) {
+          if (fscanf(fl, "%d", &idx) != 1) break;
+          local_label[(size_t)id * classes + idx] = 1;
+        }
+      } else {
+        long v = 0;
+        if (fscanf(fl, "%ld", &v) == 1) local_label[id] = v;
+      }
+      if (fscanf(fm, "%255s", la) != 1) la[0] = 0;
+      if (fscanf(fm, "%255s", msk) != 1) msk[0] = 0;
+      local_mask[id] = mask_word_code(msk);
+    } else {
+      for (uint32_t i = 0; i < F; ++i)
+        if (fscanf(ff, "%f", &skip) != 1) break;
+      if (fscanf(fl, "%255s", la) != 1 || fscanf(fl, "%255s", la) != 1) la[0] = 0;
+      if (fscanf(fm, "%255s", la) != 1 || fscanf(fm, "%255s", la) != 1) la[0] = 0;
+    }
+  }
+  fclose(ff);
+  rewind(fl);
+  while (fscanf(fl, "%u", &id) == 1) {
+    if (classes > 1) {
+      int sz = 0, idx = 0;
+      if (fscanf(fl, "%d", &sz) != 1) sz = 0;
+      while (sz--) {
+        if (fscanf(fl, "%d", &idx) != 1) break;
+        if (id < V) global_label[(size_t)id * classes + idx] = 1;
+      }
+    } else {
+      long v = 0;
+      if (fscanf(fl, "%ld", &v) == 1 && id < V) global_label[id] = v;
+    }
+  }
+  rewind(fm);
+  while (fscanf(fm, "%u", &id) == 1) {
+    if (fscanf(fm, "%255s", msk) != 1) msk[0] = 0;
+    if (id < V) global_mask[id] = mask_word_code(msk);
+  }
+  fclose(fl);
+  fclose(fm);
+  return 0;
+}
+
+/* GNNDatum::readFeature_Label_Mask_OGB (core/ntsDataloador.hpp:397-471): line k of the feature file
+ * holds vertex k's values separated by commas, converted with atof; the label file holds one
+ * integer per vertex; <dir>/train.csv, valid.csv, test.csv list the vertex ids of the splits. */
+NTS_EXPORT int nts_oracle_read_feature_label_mask_ogb(const char *path_f, const char *path_l, const char *dir_m,
+                                                      uint32_t V, uint32_t F, float *local_feature,
+                                                      int64_t *local_label, int32_t *local_mask) {
+  FILE *ff = fopen(path_f, "r"), *fl = fopen(path_l, "r");
+  if (!ff || !fl) {
+    if (ff) fclose(ff);
+    if (fl) fclose(fl);
+    return -1;
+  }
+  char *line = NULL;
+  size_t cap = 0;
+  int rc = 0;
+  for (uint32_t id = 0; id < V; ++id) {
+    ssize_t len = getline(&line, &cap, ff);
+    if (len < 0) {
+      rc = -2;
+      break;
+    }
+    if (len > 0 && line[len - 1] == '\n') line[--len] = 0;
+    uint32_t i = 0;
+    char *p = line;
+    while (p < line + len) { /* getline(ss, field, ','): a field ends at a comma or at the end */
+      char *q = p;
+      while (*q && *q != ',') ++q;
+      const char saved = *q;
+      *q = 0;
+      if (i < F) local_feature[(size_t)F * id + i] = (float)atof(p);
+      ++i;
+      if (!saved) break;
+      p = q + 1;
+    }
+    if (i != F) { /* the reference asserts i == size_0 */
+      rc = -3;
+      break;
+    }
+    long v = 0;
+    if (fscanf(fl, "%ld", &v) == 1) local_label[id] = v;
+  }
+  free(line);
+  fclose(ff);
+  fclose(fl);
+  if (rc) return rc;
+  static const char *names[3] = {"/train.csv", "/valid.csv", "/test.csv"};
+  for (int k = 0; k < 3; ++k) {
+    char path[4096];
+    snprintf(path, sizeof(path), "%s%s", dir_m, names[k]);
+    FILE *fm = fopen(path, "r");
+    if (!fm) return -1;
+    unsigned vtx = 0;
+    while (fscanf(fm, "%u", &vtx) == 1)
+      if (vtx < V) local_mask[vtx] = k;
+    fclose(fm);
+  }
+  return 0;
+}
+
+/* Binary edge list (EdgeUnit<Empty>, dep/gemini/type.hpp:99-106): file bytes / 8 records of
+ * {uint32 src, uint32 dst} (core/graph.hpp:1059-1060).  Returns the number of records read. */
+NTS_EXPORT uint64_t nts_oracle_read_edges(const char *path, uint32_t *src, uint32_t *dst, uint64_t capacity) {
+  FILE *f = fopen(path, "rb");
+  if (!f) return 0;
+  uint32_t rec[2];
+  uint64_t n = 0;
+  while (n < capacity && fread(rec, sizeof(uint32_t), 2, f) == 2) {
+    src[n] = rec[0];
+    dst[n] = rec[1];
+    ++n;
+  }
+  fclose(f);
+  return n;
 }
 
 NTS_EXPORT int nts_oracle_version(void) { return 1; }
