@@ -9,8 +9,10 @@ aggregate-then-transform order: layer-0 forward (F=602), layer-1 forward (F=128)
 by source over the CSR.  Inputs are resident in HBM before the timed region.
 
 Prints one JSON line: edges aggregated per second (4 * E edges per step), the roofline figure of
-the dominant kernel (the F=602 gather) from HIP events recorded around that kernel, and the CPU
-oracle timed on the host cores on a bounded sample of the same graph.
+the dominant kernel (the F=602 gather) from HIP events recorded around that kernel, and a CPU
+baseline timed on the host cores on a bounded sample of the same graph: the reference's own CPU
+operator where the reference-built program oracle/_ref/ref_fullgraph_cpu is present ("reference"),
+else the CPU oracle ("port").
 """
 import argparse
 import ctypes
@@ -26,6 +28,8 @@ if ROOT not in sys.path:
 V_REDDIT = 232_965
 E_REDDIT = 114_800_000
 F_IN, F_HID = 602, 128
+# The reference's own CPU operator, built from the reference tree where that is present (test infrastructure).
+REFERENCE_PROGRAM = os.path.join(ROOT, "oracle", "_ref", "ref_fullgraph_cpu")
 HBM_PEAK_GBS = 8000.0
 # Bytes per launch of the F=602 gather kernel that cross the L2 <-> fabric boundary, from rocprofv3
 # FETCH_SIZE (x1.986 calibration) + WRITE_SIZE at the default schedule
@@ -54,6 +58,8 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB row copy (identity gather) so that HBM byte counters can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the oracle sample")
+    ap.add_argument("--cpu-reference-edges", type=int, default=28_700_000,
+                    help="edges of the sample the reference's own CPU operator is timed on (0 = time the oracle instead)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -171,7 +177,10 @@ def main():
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
-        cpu_baseline = run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, args.cpu_seconds)
+        if args.cpu_reference_edges > 0 and os.path.exists(REFERENCE_PROGRAM):
+            cpu_baseline = run_reference_cpu_baseline(torch, chunk, x0, h1, V, min(E, args.cpu_reference_edges))
+        if cpu_baseline is None:
+            cpu_baseline = run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, args.cpu_seconds)
 
     out = {
         "metric": "edges aggregated/s (fwd+bwd)",
@@ -199,6 +208,49 @@ def main():
         "cpu_baseline": cpu_baseline,
     }
     print(json.dumps(out))
+
+
+def run_reference_cpu_baseline(torch, chunk, x0, h1, V, sample_edges):
+    """The reference's own CPU operator (ForwardCPUfuseOp behind oracle/_ref/ref_fullgraph_cpu, built
+    from the reference tree by oracle/build_ref.sh) on the edges of the lowest-numbered source
+    vertices of the same graph: its loader, partitioner and operator run unchanged on this host's
+    cores.  Returns None when the program fails, so that the caller can fall back to the oracle."""
+    import re
+    import shutil
+    import subprocess
+    import tempfile
+
+    tmp = tempfile.mkdtemp(prefix="nts_ref_")
+    try:
+        ro = chunk.row_offset_gpu.to(torch.int64)
+        pos = torch.arange(sample_edges, device=ro.device)
+        src = torch.searchsorted(ro, pos, right=True) - 1
+        dst = chunk.column_indices_gpu[:sample_edges].to(torch.int64)
+        torch.stack([src, dst], 1).to(torch.int32).cpu().numpy().tofile(os.path.join(tmp, "g.edge"))
+        del ro, pos, src, dst
+        x0.cpu().numpy().tofile(os.path.join(tmp, f"p.x{F_IN}"))
+        h1.cpu().numpy().tofile(os.path.join(tmp, f"p.x{F_HID}"))
+        r = subprocess.run([REFERENCE_PROGRAM, os.path.join(tmp, "g.edge"), str(V), f"{F_IN},{F_HID}", "1",
+                            os.path.join(tmp, "p"), "agg-cpu"], capture_output=True, text=True, timeout=240)
+        rows = re.findall(r"timing: V=\d+ E=(\d+) F=(\d+) forward_s=([0-9.]+) backward_s=([0-9.]+) threads=(\d+)", r.stdout)
+        if r.returncode != 0 or len(rows) != 2:
+            return None
+        total_s = sum(float(f) + float(b) for _, _, f, b, _ in rows)
+        edges = int(rows[0][0])
+        return {
+            "value": round(4 * edges / total_s, 1),
+            "unit": "edges/s",
+            "cores": int(rows[0][4]),
+            "kind": "reference",
+            "sample": f"the reference's ForwardCPUfuseOp (its own loader, partitioner and operator, built from the "
+                      f"reference sources) on the {edges} edges of the lowest-numbered source vertices of the same "
+                      f"graph, forward and backward at F={F_IN} and F={F_HID}, best of 3: "
+                      + ", ".join(f"F={w} fwd {float(f):.3f} s bwd {float(b):.3f} s" for _, w, f, b, _ in rows),
+        }
+    except (OSError, subprocess.SubprocessError):
+        return None
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
 
 
 def run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, target_s):

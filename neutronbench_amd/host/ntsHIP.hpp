@@ -102,9 +102,10 @@ inline void zero_buffer(float *buffer, int size) {
   NTS_VENEER_CHECK(nts_device_sync());
 }
 inline void CUDA_DEVICE_SYNCHRONIZE() { NTS_VENEER_CHECK(nts_device_sync()); }
-// The few raw runtime names that core/ calls outside cuda/ (core/ntsMiniBatchGraphOp.hpp:283,
-// core/coocsc.hpp:673-773).
+// The few raw runtime names that core/ and comm/ call outside cuda/ (core/ntsMiniBatchGraphOp.hpp:283,
+// core/coocsc.hpp:673-773, comm/network.cpp:53, 84).
 inline int cudaFree(void *p) { return nts_free_device(p); }
+inline int cudaFreeHost(void *p) { return nts_free_pinned(p); }
 inline int cudaStreamSynchronize(cudaStream_t s) { return nts_stream_sync(s); }
 
 // cudaMallocManaged as the data loader uses it (core/ntsDataloador.hpp:66-73): memory that both the

@@ -8,13 +8,19 @@
  * tree).  Arithmetic is fp32 with the reference's operation order; the file is compiled with
  * -ffp-contract=off so that "mul then add" stays two roundings unless a function says otherwise.
  *
- * Pinning status (what independent evidence each function is checked against lives in
- * tests/test_oracle_*.py):
- *   norm_degree, spmm (fwd/bwd), csr_from_csc, postprocess, layer weights, gathers, scatter /
- *   aggregate edge ops: pinned by closed forms, brute force and library routines.
- *   edge_softmax fwd: the reference calls libtorch's softmax (core/ntsSingleCPUGraphOp.hpp:310);
- *   the reference holds no test vector at that boundary -> parity unpinned against the reference
- *   itself, pinned against torch.softmax / scipy as a library identity.
+ * Pinning status (the independent evidence each function is checked against lives in
+ * tests/test_oracle_pins.py, tests/test_golden.py, tests/test_oracle_vs_reference_build.py,
+ * tests/test_reference_operators.py and tests/test_dataset_formats.py):
+ *   norm_degree, comp, spmm (fwd/bwd), build_chunk, scatter / aggregate edge ops, edge_softmax fwd/bwd:
+ *   pinned by closed forms, brute force and library routines, AND against the reference's own code
+ *   compiled from its tree (oracle/build_ref.sh): nts_comp / nts_norm_degree bit for bit, and the
+ *   operator classes ForwardCPUfuseOp (bit for bit, forward and backward), SingleCPUSrcDstScatterOp,
+ *   SingleCPUDstAggregateOp (bit for bit) and SingleEdgeSoftMax (to rounding: it calls libtorch's
+ *   softmax) run on graphs loaded by the reference's loader and partitioner.
+ *   csr_from_csc, postprocess, layer weights, init_co, gathers, cache split: the reference code for
+ *   these (core/coocsc.hpp, core/ntsSampler.hpp, core/ntsMiniBatchGraphOp.hpp) needs METIS headers
+ *   the tree does not carry and cannot be compiled; pinned by brute force and exact fixtures.
+ *   dataset readers: pinned by exact rational rounding of every token and by the file definitions.
  */
 #define _GNU_SOURCE /* getline */
 #include <math.h>

@@ -1,0 +1,247 @@
+// Driver around the REFERENCE's own full-graph operators, compiled from the reference tree where it
+// lies (see build_ref.sh).  TEST INFRASTRUCTURE ONLY: it exists so that tests can compare the oracle
+// and the HIP library with what the reference's code itself computes.
+//
+// It loads a binary edge file through the reference's loader (Graph::load_directed), builds the
+// reference's chunks (PartitionedGraph::GenerateAll with nts_norm_degree) and runs, on inputs read
+// from raw little-endian float32 files, the reference's operator classes unchanged:
+//   CPU  ForwardCPUfuseOp                  (core/ntsCPUFusedGraphOp.hpp)
+//        SingleCPUSrcDstScatterOp, SingleEdgeSoftMax, SingleCPUDstAggregateOp
+//                                          (core/ntsSingleCPUGraphOp.hpp)
+//   GPU  (only when built with CUDA_ENABLE=1 against the HIP veneer and libntship.so)
+//        ForwardSingleGPUfuseOp            (core/ntsSingleGPUFusedGraphOp.hpp)
+//        DistGPUScatterSrc, DistGPUScatterDst, DistGPUEdgeSoftMax, DistGPUAggregateDst
+//                                          (core/ntsDistGPUGraphOp.hpp)
+// and writes every result as a raw file <prefix>.<name>.
+//
+//   usage: ref_fullgraph <edge_file> <vertices> <F> <H> <prefix> <cpu|gpu|both|agg-cpu>
+//   agg-cpu runs ForwardCPUfuseOp only; <F> may be a comma-separated list, and for every width the
+//   input is <prefix>.x<F>.  Three timed repetitions per width, best forward and backward time
+//   printed: the CPU baseline of the aggregation benchmark.
+//   inputs:  <prefix>.x  [V, F]   vertex features, also used as the vertex-side gradient
+//            <prefix>.m  [E, H]   edge scores;  <prefix>.gm [E, H] their gradient
+//            <prefix>.e  [E, F]   edge messages;  <prefix>.g2 [E, 2F] gradient of the (src | dst) scatter
+#include "comm/logger.h"
+#include "core/PartitionedGraph.hpp"
+#include "core/graph.hpp"
+#include "core/ntsBaseOp.hpp"
+#include "core/ntsCPUFusedGraphOp.hpp"
+#include "core/ntsSingleCPUGraphOp.hpp"
+#if CUDA_ENABLE
+#include "core/ntsDistGPUGraphOp.hpp"
+#include "core/ntsSingleGPUFusedGraphOp.hpp"
+#endif
+
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <sstream>
+#include <string>
+#include <vector>
+
+static std::string g_prefix;
+
+static NtsVar read_matrix(const std::string &name, long rows, long cols) {
+  const std::string path = g_prefix + "." + name;
+  NtsVar t = torch::zeros({rows, cols}, torch::kFloat);
+  FILE *f = fopen(path.c_str(), "rb");
+  const size_t n = static_cast<size_t>(rows) * cols;
+  if (!f || fread(t.data_ptr<float>(), sizeof(float), n, f) != n) {
+    fprintf(stderr, "cannot read %ld x %ld floats from %s\n", rows, cols, path.c_str());
+    exit(2);
+  }
+  fclose(f);
+  return t;
+}
+
+static void write_raw(const std::string &name, const void *p, size_t bytes) {
+  const std::string path = g_prefix + "." + name;
+  FILE *f = fopen(path.c_str(), "wb");
+  if (!f || (bytes && fwrite(p, 1, bytes, f) != bytes)) {
+    fprintf(stderr, "cannot write %s\n", path.c_str());
+    exit(2);
+  }
+  fclose(f);
+}
+
+static void write_tensor(const std::string &name, const NtsVar &t_in) {
+  NtsVar t = t_in.detach().cpu().contiguous();
+  write_raw(name, t.data_ptr<float>(), static_cast<size_t>(t.numel()) * sizeof(float));
+}
+
+static double now() {
+  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+int main(int argc, char **argv) {
+  MPI_Instance mpi(&argc, &argv);
+  if (argc < 7) {
+    fprintf(stderr, "usage: %s edge_file vertices F H prefix cpu|gpu|both|agg-cpu\n", argv[0]);
+    return 2;
+  }
+  const std::string edge_file = argv[1];
+  const VertexId vertices = static_cast<VertexId>(std::stoul(argv[2]));
+  std::vector<int> widths;
+  {
+    std::stringstream ss(argv[3]);
+    std::string item;
+    while (std::getline(ss, item, ',')) widths.push_back(std::stoi(item));
+  }
+  const int F = widths.at(0);
+  const int H = std::stoi(argv[4]);
+  g_prefix = argv[5];
+  const std::string mode = argv[6];
+  const bool agg_only = mode == "agg-cpu";
+  const bool run_cpu = mode == "cpu" || mode == "both";
+  const bool run_gpu = mode == "gpu" || mode == "both";
+
+  Graph<Empty> *graph = new Graph<Empty>();
+  graph->config->vertices = vertices;
+  graph->config->edge_file = edge_file;
+  graph->config->layer_string = std::to_string(F) + "-" + std::to_string(F);
+  graph->replication_threshold = 0;
+  graph->load_directed(edge_file, vertices);
+  graph->generate_backward_structure();
+
+  VertexSubset *active = graph->alloc_vertex_subset();
+  active->fill();
+  graph->init_gnnctx(graph->config->layer_string);
+  graph->init_rtminfo();
+  graph->rtminfo->process_local = false;
+  graph->rtminfo->reduce_comm = false;
+  graph->rtminfo->copy_data = false;
+  graph->rtminfo->process_overlap = false;
+  graph->rtminfo->with_weight = true;
+  graph->rtminfo->lock_free = false;
+  graph->rtminfo->with_cuda = false;
+
+  // One CPU-side partitioned graph with the mirror index and whole-graph topology (dist = true), as
+  // GAT_GPU_DIST sets it up (toolkits/GAT_GPU_DIST.hpp:67-70): the CPU operators read its chunks, the
+  // DistGPU* operators upload its column_offset / row_indices / MirrorIndex themselves.
+  PartitionedGraph *pg = new PartitionedGraph(graph, active);
+  pg->GenerateAll([&](VertexId src, VertexId dst) { return nts::op::nts_norm_degree(graph, src, dst); }, CPU_T, true);
+  graph->init_communicatior();
+  const long V = vertices, E = pg->owned_edges;
+  printf("reference graph: V=%ld E=%ld mirrors=%u\n", V, E, pg->owned_mirrors);
+
+  if (agg_only) {
+    nts::op::ForwardCPUfuseOp op(pg, active);
+    for (int width : widths) {
+      NtsVar X = read_matrix("x" + std::to_string(width), V, width);
+      double best_f = 1e30, best_b = 1e30;
+      for (int rep = 0; rep < 3; ++rep) {
+        double t0 = now();
+        NtsVar Y = op.forward(X);
+        double t1 = now();
+        NtsVar G = op.backward(X);
+        double t2 = now();
+        best_f = std::min(best_f, t1 - t0);
+        best_b = std::min(best_b, t2 - t1);
+      }
+      printf("reference ForwardCPUfuseOp timing: V=%ld E=%ld F=%d forward_s=%.6f backward_s=%.6f threads=%d\n", V, E,
+             width, best_f, best_b, graph->threads);
+    }
+    return 0;
+  }
+
+  CSC_segment_pinned *chunk = pg->graph_chunks[0];
+  write_raw("column_offset", chunk->column_offset, (V + 1) * sizeof(VertexId));
+  write_raw("row_indices", chunk->row_indices, E * sizeof(VertexId));
+  write_raw("edge_weight_forward", chunk->edge_weight_forward, E * sizeof(ValueType));
+  write_raw("row_offset", chunk->row_offset, (V + 1) * sizeof(VertexId));
+  write_raw("column_indices", chunk->column_indices, E * sizeof(VertexId));
+  write_raw("edge_weight_backward", chunk->edge_weight_backward, E * sizeof(ValueType));
+  write_raw("mirror_index", pg->MirrorIndex, (V + 1) * sizeof(VertexId));
+
+  NtsVar X = read_matrix("x", V, F);
+  NtsVar M = read_matrix("m", E, H), GM = read_matrix("gm", E, H);
+  NtsVar Emsg = read_matrix("e", E, F), G2 = read_matrix("g2", E, 2 * F);
+  NtsVar M1 = M.slice(1, 0, 1).contiguous(), GM1 = GM.slice(1, 0, 1).contiguous();
+
+  if (run_cpu) {
+    {
+      nts::op::ForwardCPUfuseOp op(pg, active);
+      double t0 = now();
+      NtsVar Y = op.forward(X);
+      double t1 = now();
+      NtsVar G = op.backward(X);
+      double t2 = now();
+      write_tensor("cpu_fwd", Y);
+      write_tensor("cpu_bwd", G);
+      printf("reference ForwardCPUfuseOp: forward %.6f s backward %.6f s threads %d\n", t1 - t0, t2 - t1,
+             graph->threads);
+    }
+    {
+      nts::op::SingleCPUSrcDstScatterOp op(pg, active);
+      write_tensor("cpu_scatter", op.forward(X));
+      write_tensor("cpu_scatter_bwd", op.backward(G2));
+    }
+    {
+      nts::op::SingleEdgeSoftMax op(pg, active);
+      write_tensor("cpu_softmax", op.forward(M));
+      // The backward expression is only shape-correct for one column (d.t().mm(imr) is H x H).
+      nts::op::SingleEdgeSoftMax op1(pg, active);
+      NtsVar y1 = op1.forward(M1);
+      write_tensor("cpu_softmax1", y1);
+      write_tensor("cpu_softmax1_bwd", op1.backward(GM1));
+    }
+    {
+      nts::op::SingleCPUDstAggregateOp op(pg, active);
+      write_tensor("cpu_agg", op.forward(Emsg));
+      write_tensor("cpu_agg_bwd", op.backward(X));
+    }
+    printf("reference CPU operators done\n");
+  }
+#if CUDA_ENABLE
+  if (run_gpu) {
+    {
+      graph->rtminfo->with_cuda = true;
+      PartitionedGraph *pgg = new PartitionedGraph(graph, active);
+      pgg->GenerateAll([&](VertexId src, VertexId dst) { return nts::op::nts_norm_degree(graph, src, dst); }, GPU_T);
+      graph->init_message_buffer();
+      NtsVar Xg = X.cuda();
+      nts::op::ForwardSingleGPUfuseOp op(pgg, active);
+      write_tensor("gpu_fwd", op.forward(Xg));
+      write_tensor("gpu_bwd", op.backward(Xg));
+    }
+    {
+      // DistGPUScatterSrc reads rows of the mirror tensor: row MirrorIndex[v] holds vertex v, for
+      // every vertex with an outgoing edge (what DistGPUGetDepNbrOp delivers at one partition).
+      std::vector<long> mirror_vertices;
+      for (long v = 0; v < V; ++v)
+        if (pg->MirrorIndex[v + 1] != pg->MirrorIndex[v]) mirror_vertices.push_back(v);
+      NtsVar sel = torch::from_blob(mirror_vertices.data(), {static_cast<long>(mirror_vertices.size())}, torch::kLong);
+      NtsVar mirror = X.index_select(0, sel).cuda();
+      NtsVar Xg = X.cuda(), G2g = G2.cuda();
+      nts::op::DistGPUScatterSrc src_op(pg, active);
+      nts::op::DistGPUScatterDst dst_op(pg, active);
+      write_tensor("gpu_scatter_src", src_op.forward(mirror));
+      write_tensor("gpu_scatter_dst", dst_op.forward(Xg));
+      NtsVar gs = G2g.slice(1, 0, F).contiguous(), gd = G2g.slice(1, F, 2 * F).contiguous();
+      write_tensor("gpu_scatter_src_bwd", src_op.backward(gs));
+      write_tensor("gpu_scatter_dst_bwd", dst_op.backward(gd));
+    }
+    {
+      NtsVar Mg = M.cuda(), M1g = M1.cuda(), GM1g = GM1.cuda();
+      nts::op::DistGPUEdgeSoftMax op(pg, active);
+      write_tensor("gpu_softmax", op.forward(Mg));
+      nts::op::DistGPUEdgeSoftMax op1(pg, active);
+      write_tensor("gpu_softmax1", op1.forward(M1g));
+      write_tensor("gpu_softmax1_bwd", op1.backward(GM1g));
+    }
+    {
+      NtsVar Eg = Emsg.cuda(), Xg = X.cuda();
+      nts::op::DistGPUAggregateDst op(pg, active);
+      write_tensor("gpu_agg", op.forward(Eg));
+      write_tensor("gpu_agg_bwd", op.backward(Xg));
+    }
+    printf("reference GPU operators over libntship done\n");
+  }
+#else
+  if (run_gpu) {
+    fprintf(stderr, "this build has no GPU operators\n");
+    return 2;
+  }
+#endif
+  return 0;
+}

@@ -1,0 +1,57 @@
+"""Runs the reference-built operator programs oracle/_ref/ref_fullgraph_{cpu,gpu} (the reference's
+own loader, partitioner and operator classes behind oracle/ref_fullgraph_driver.cpp, built by
+oracle/build_ref.sh where the reference tree is present) on seeded inputs and returns every array
+they write.  Test infrastructure only."""
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PROGRAMS = {k: os.path.join(ROOT, "oracle", "_ref", f"ref_fullgraph_{k}") for k in ("cpu", "gpu")}
+
+
+def available(kind):
+    return os.path.exists(PROGRAMS[kind])
+
+
+def make_inputs(V, E, F, H, seed, skew=2.0):
+    rng = np.random.default_rng(seed)
+    src = np.minimum((rng.random(E) ** skew * V).astype(np.uint32), V - 1)
+    dst = np.minimum((rng.random(E) ** (skew + 1) * V).astype(np.uint32), V - 1)
+    return dict(src=src, dst=dst, x=rng.standard_normal((V, F)).astype(np.float32),
+                m=(3 * rng.standard_normal((E, H))).astype(np.float32),
+                gm=rng.standard_normal((E, H)).astype(np.float32),
+                e=rng.standard_normal((E, F)).astype(np.float32),
+                g2=rng.standard_normal((E, 2 * F)).astype(np.float32))
+
+
+def run(kind, mode, inputs, tmp_path, timeout=600):
+    """kind: which program ("cpu" / "gpu"); mode: "cpu", "gpu" or "both"."""
+    V, F = inputs["x"].shape
+    E, H = inputs["m"].shape
+    prefix = os.path.join(str(tmp_path), "ref")
+    np.stack([inputs["src"], inputs["dst"]], 1).astype(np.uint32).tofile(prefix + ".edge")
+    for k in ("x", "m", "gm", "e", "g2"):
+        inputs[k].tofile(prefix + "." + k)
+    r = subprocess.run([PROGRAMS[kind], prefix + ".edge", str(V), str(F), str(H), prefix, mode], capture_output=True,
+                       text=True, timeout=timeout)
+    assert r.returncode == 0, f"reference program failed ({r.returncode}):\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}"
+    out = {"stdout": r.stdout}
+    shapes = {"column_offset": (np.uint32, (V + 1,)), "row_indices": (np.uint32, (E,)),
+              "edge_weight_forward": (np.float32, (E,)), "row_offset": (np.uint32, (V + 1,)),
+              "column_indices": (np.uint32, (E,)), "edge_weight_backward": (np.float32, (E,)),
+              "mirror_index": (np.uint32, (V + 1,))}
+    for side in ("cpu", "gpu"):
+        shapes.update({f"{side}_fwd": (np.float32, (V, F)), f"{side}_bwd": (np.float32, (V, F)),
+                       f"{side}_softmax": (np.float32, (E, H)), f"{side}_softmax1": (np.float32, (E, 1)),
+                       f"{side}_softmax1_bwd": (np.float32, (E, 1)), f"{side}_agg": (np.float32, (V, F)),
+                       f"{side}_agg_bwd": (np.float32, (E, F))})
+    shapes.update({"cpu_scatter": (np.float32, (E, 2 * F)), "cpu_scatter_bwd": (np.float32, (V, F)),
+                   "gpu_scatter_src": (np.float32, (E, F)), "gpu_scatter_dst": (np.float32, (E, F)),
+                   "gpu_scatter_src_bwd": (np.float32, (-1, F)), "gpu_scatter_dst_bwd": (np.float32, (V, F))})
+    for name, (dtype, shape) in shapes.items():
+        path = prefix + "." + name
+        if os.path.exists(path):
+            out[name] = np.fromfile(path, dtype=dtype).reshape(shape)
+    return out
