@@ -17,6 +17,9 @@
 // per edge and element -- the order of the CPU operators (core/ntsMiniBatchGraphOp.hpp:154-240),
 // so unsplit rows reproduce an FMA-contracted CPU build bit for bit.
 #include <stdlib.h>
+#include <string.h>
+
+#include <rocprim/device/device_scan.hpp>
 
 #include <algorithm>
 #include <new>
@@ -102,7 +105,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
                                                         const uint32_t *__restrict__ indices, uint32_t index_base,
                                                         uint32_t n_items, uint32_t F, uint32_t col_base,
                                                         const Item *__restrict__ items, float *__restrict__ partial,
-                                                        int accumulate, HeadArgs heads) {
+                                                        int accumulate, HeadArgs heads, uint32_t row_edge_limit) {
   using V = typename Vec<VEC>::type;
   constexpr int U = unroll_for(NACC);
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -121,6 +124,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
     e0 = wave_first(offsets[item]);
     e1 = wave_first(offsets[item + 1]);
     slot = kNoSlot;
+    if (e1 - e0 > row_edge_limit) return;  // a long row: its pieces are separate work items
   }
 
   // Lanes past the end of the row (only possible in the last accumulator) read the row's last
@@ -248,7 +252,8 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
                                                          const uint32_t *__restrict__ offsets,
                                                          const uint32_t *__restrict__ indices, uint32_t index_base,
                                                          uint32_t n_items, uint32_t F, const Item *__restrict__ items,
-                                                         float *__restrict__ partial, int accumulate, HeadArgs heads) {
+                                                         float *__restrict__ partial, int accumulate, HeadArgs heads,
+                                                         uint32_t row_edge_limit) {
   using V = typename Vec<VEC>::type;
   constexpr int U = 4;
   const uint32_t gl = threadIdx.x & (G - 1);
@@ -267,6 +272,7 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
     e0 = offsets[item];
     e1 = offsets[item + 1];
     slot = kNoSlot;
+    if (e1 - e0 > row_edge_limit) return;  // a long row: its pieces are separate work items
   }
   const uint32_t col = gl * VEC;
   const bool live = col < F;
@@ -364,6 +370,7 @@ struct LaunchArgs {
   int accumulate;
   hipStream_t stream;
   HeadArgs heads = HeadArgs{nullptr, 0u, 0u};  // H == 0: one weight per edge
+  uint32_t row_edge_limit = 0xFFFFFFFFu;       // whole-row launches skip rows with more edges than this
 };
 
 // How the wave kernel hands neighbour pairs to its lanes: through a wave-private LDS tile (default)
@@ -384,7 +391,8 @@ void launch_wave(const LaunchArgs &a, uint32_t col_base) {
   const dim3 grid(blocks), block(kWavesPerBlock * kWave);
 #define NTS_LAUNCH_WAVE(LDS, HD)                                                                                       \
   hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, LDS, HD>), grid, block, 0, a.stream, a.in, a.out, a.w, a.offsets,     \
-                     a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate, a.heads)
+                     a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate, a.heads,     \
+                     a.row_edge_limit)
   if (a.heads.H) {
     if (lds_tile_enabled()) NTS_LAUNCH_WAVE(true, true); else NTS_LAUNCH_WAVE(false, true);
   } else {
@@ -399,10 +407,12 @@ void launch_group(const LaunchArgs &a) {
   const uint32_t blocks = ceil_div(a.n_items, per_block);
   if (a.heads.H)
     hipLaunchKernelGGL((spmm_group_kernel<G, VEC, true>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
-                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads);
+                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,
+                       a.row_edge_limit);
   else
     hipLaunchKernelGGL((spmm_group_kernel<G, VEC, false>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
-                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads);
+                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,
+                       a.row_edge_limit);
 }
 
 template <int VEC>
@@ -464,6 +474,138 @@ void launch_spmm(const LaunchArgs &a) {
   return launch_wave_vec<1>(a);
 }
 
+// ---- launches without a plan: hub rows are cut into pieces on the device ---------------------------
+//
+// A call that brings no plan still must not let one wavefront walk a 10^5-edge row alone.  For edge
+// counts where that can matter, the pieces are derived on the device in the same stream, without
+// any copy to the host: pieces[r] = ceil(deg/chunk) for rows longer than `chunk` (else 0), an
+// exclusive scan gives each long row its first partial slot, one thread per possible piece writes
+// the work item (binary search of the scan), whole-row wavefronts skip the long rows, the piece
+// wavefronts write partial sums and a last kernel adds each long row's partials in slot order.
+// The number of pieces is not known on the host, so grids and buffers are sized for its upper bound
+// E/chunk + min(rows, E/chunk); surplus work items are empty.  Scratch is stream-ordered
+// (hipMallocAsync / hipFreeAsync).
+
+constexpr uint32_t kAutoMinEdges = 1u << 16;  // below this a serial hub row costs less than the set-up
+constexpr uint32_t kAutoChunk = 1024;
+
+__global__ __launch_bounds__(256) void auto_count_kernel(uint32_t *__restrict__ pieces,
+                                                         const uint32_t *__restrict__ off, uint32_t rows,
+                                                         uint32_t chunk) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r > rows) return;
+  uint32_t n = 0;
+  if (r < rows) {
+    const uint32_t deg = off[r + 1] - off[r];
+    if (deg > chunk) n = (deg + chunk - 1) / chunk;
+  }
+  pieces[r] = n;  // pieces[rows] = 0, so that the scan's last entry is the total
+}
+
+__global__ __launch_bounds__(256) void auto_items_kernel(Item *__restrict__ items, const uint32_t *__restrict__ base,
+                                                         const uint32_t *__restrict__ off, uint32_t rows,
+                                                         uint32_t chunk, uint32_t p_max) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= p_max) return;
+  if (i >= base[rows]) {
+    items[i] = make_uint4(0u, 0u, 0u, i);  // empty item: writes zeros to its own unused slot
+    return;
+  }
+  const uint32_t r = owner_of(base, rows, i);  // the last row whose first slot is <= i is the long row itself
+  const uint32_t e0 = off[r] + (i - base[r]) * chunk;
+  items[i] = make_uint4(r, e0, min(off[r + 1], e0 + chunk), i);
+}
+
+// Block (x, y): if work item x is the first piece of its row, adds that row's partials in slot order
+// into out (256 columns per block, tile y).
+__global__ __launch_bounds__(256) void auto_reduce_kernel(float *__restrict__ out, const float *__restrict__ partial,
+                                                          const Item *__restrict__ items,
+                                                          const uint32_t *__restrict__ base, uint32_t F,
+                                                          int accumulate) {
+  const uint32_t i = blockIdx.x;
+  const uint32_t r = items[i].x;
+  if (base[r] != i) return;
+  const uint32_t n = base[r + 1] - i;
+  if (n == 0) return;
+  const uint32_t c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= F) return;
+  const float *src = partial + static_cast<size_t>(i) * F + c;
+  float a = src[0];
+  uint32_t k = 1;
+  for (; k + 8 <= n; k += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[static_cast<size_t>(k + u) * F];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a += v[u];
+  }
+  for (; k < n; ++k) a += src[static_cast<size_t>(k) * F];
+  float *dst = out + static_cast<size_t>(r) * F + c;
+  if (accumulate) a += *dst;
+  *dst = a;
+}
+
+inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
+
+// `a` describes the whole-row launch (a.n_items = rows, no items).
+int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
+  const uint32_t rows = a.n_items;
+  if (edges < kAutoMinEdges) {
+    launch_spmm(a);
+    return NTS_OK;
+  }
+  const uint32_t chunk = kAutoChunk;
+  const uint32_t by_edges = edges / chunk;
+  const uint32_t p_max = by_edges + (rows < by_edges ? rows : by_edges) + 1;
+  size_t scan_bytes = 0;
+  {
+    uint32_t *nul = nullptr;
+    NTS_HIP_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, nul, nul, 0u, static_cast<size_t>(rows) + 1,
+                                        rocprim::plus<uint32_t>(), a.stream, false));
+  }
+  const size_t n_off = up256((static_cast<size_t>(rows) + 1) * sizeof(uint32_t));
+  const size_t n_items_b = up256(static_cast<size_t>(p_max) * sizeof(Item));
+  const size_t n_partial = up256(static_cast<size_t>(p_max) * a.F * sizeof(float));
+  unsigned char *buf = nullptr;
+  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&buf), 2 * n_off + n_items_b + up256(scan_bytes) + n_partial,
+                             a.stream));
+  uint32_t *pieces = reinterpret_cast<uint32_t *>(buf);
+  uint32_t *base = reinterpret_cast<uint32_t *>(buf + n_off);
+  Item *items = reinterpret_cast<Item *>(buf + 2 * n_off);
+  void *scan_tmp = buf + 2 * n_off + n_items_b;
+  float *partial = reinterpret_cast<float *>(buf + 2 * n_off + n_items_b + up256(scan_bytes));
+  auto bail = [&](hipError_t err, const char *what) {
+    (void)hipFreeAsync(buf, a.stream);
+    return fail_hip(err, what);
+  };
+  hipLaunchKernelGGL(auto_count_kernel, dim3(ceil_div(static_cast<uint64_t>(rows) + 1, 256)), dim3(256), 0, a.stream,
+                     pieces, a.offsets, rows, chunk);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return bail(err, "auto_count_kernel");
+  err = rocprim::exclusive_scan(scan_tmp, scan_bytes, pieces, base, 0u, static_cast<size_t>(rows) + 1,
+                                rocprim::plus<uint32_t>(), a.stream, false);
+  if (err != hipSuccess) return bail(err, "spmm: scan of piece counts");
+  hipLaunchKernelGGL(auto_items_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, items, base, a.offsets, rows,
+                     chunk, p_max);
+  err = hipGetLastError();
+  if (err != hipSuccess) return bail(err, "auto_items_kernel");
+  // Pieces first (the heavy, uniform work), then the rows that fit one wavefront.
+  LaunchArgs pc = a;
+  pc.n_items = p_max;
+  pc.items = items;
+  pc.partial = partial;
+  launch_spmm(pc);
+  LaunchArgs whole = a;
+  whole.row_edge_limit = chunk;
+  launch_spmm(whole);
+  hipLaunchKernelGGL(auto_reduce_kernel, dim3(p_max, ceil_div(a.F, 256)), dim3(256), 0, a.stream, a.out, partial, items,
+                     base, a.F, a.accumulate);
+  err = hipGetLastError();
+  if (err != hipSuccess) return bail(err, "spmm: balanced launch");
+  NTS_HIP_TRY(hipFreeAsync(buf, a.stream));
+  return NTS_OK;
+}
+
 int check_common(const float *in, float *out, const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
                  uint32_t edges, uint32_t F, const char *who) {
   if (F == 0) return fail(NTS_ERR_INVALID, "spmm: feature width F is 0");
@@ -500,7 +642,7 @@ int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t 
   if (int rc = nts::check_common(in, out, offsets, indices, rows, edges, F, "nts_spmm_gather: null pointer")) return rc;
   if (rows == 0) return NTS_OK;
   nts::LaunchArgs a{in, out, w, offsets, indices, index_base, rows, F, nullptr, nullptr, accumulate, stream};
-  nts::launch_spmm(a);
+  if (int rc = nts::launch_spmm_balanced(a, edges)) return rc;
   NTS_LAUNCH_CHECK("nts_spmm_gather");
   return NTS_OK;
 }

@@ -134,6 +134,47 @@ def test_planned_split_rows(device, F, chunk):
     plan.close()
 
 
+@pytest.mark.parametrize("F", [16, 100, 128, 602])
+def test_planless_call_balances_hub_rows_on_the_device(device, F):
+    """nts_spmm_gather without a plan: above 65,536 edges rows longer than 1,024 edges are cut into
+    pieces on the device (partial sums + ordered second stage).  Short rows keep the sequential FMA
+    chain bit for bit; long rows match within the fp32 tolerance; accumulate still adds; two runs
+    give identical bits."""
+    print(f"case F={F}", flush=True)
+    rng = np.random.default_rng(F)
+    Vd, Vs = 3000, 5000
+    deg = rng.integers(0, 40, Vd)
+    deg[[5, 77, 1500, 2999]] = [60000, 1025, 1024, 20001]  # hubs, and both sides of the piece size
+    deg[100:110] = 0
+    co = np.zeros(Vd + 1, dtype=np.uint32)
+    co[1:] = np.cumsum(deg)
+    E = int(co[-1])
+    assert E >= 1 << 16
+    ri = rng.integers(0, Vs, E).astype(np.uint32)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    w = rng.random(E).astype(np.float32)
+    got = _run_planless(x, w, co, ri, Vd, F, device)
+    again = _run_planless(x, w, co, ri, Vd, F, device)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    scale = abs_term_scale(x, w, co, ri, Vd)
+    check(got, oracle.spmm(x, w, co, ri, Vd), scale)
+    short = deg <= 1024
+    ref_fma = oracle.spmm(x, w, co, ri, Vd, fused=True)
+    assert np.array_equal(got[short].view(np.uint32), ref_fma[short].view(np.uint32))
+    assert not got[100:110].any()
+    # exact value of the hub rows in fp64: the pieced sum must not be less accurate than the chain
+    for r in (5, 2999):
+        sl = slice(int(co[r]), int(co[r + 1]))
+        exact = (x[ri[sl]].astype(np.float64) * w[sl, None]).sum(0)
+        assert np.max(np.abs(got[r] - exact) / np.maximum(np.abs(exact), 1e-2 * scale[r])) <= TOL
+    init = rng.standard_normal((Vd, F)).astype(np.float32)
+    acc = _run_planless(x, w, co, ri, Vd, F, device, accumulate=1, out_init=init)
+    check(acc, ref_fma + init, scale + np.abs(init))
+    # unweighted
+    got_u = _run_planless(x, None, co, ri, Vd, F, device)
+    check(got_u, oracle.spmm(x, None, co, ri, Vd), abs_term_scale(x, None, co, ri, Vd))
+
+
 def test_invariants(device):
     """All-ones input with unit weights gives the degree; GCN weights on a k-regular ring average."""
     Vd = Vs = 128

@@ -10,7 +10,7 @@ import pytest
 
 import oracle
 import refops
-from util import check
+from util import abs_term_scale, check
 
 CASES = [(300, 4000, 19, 4, 1), (2000, 60000, 64, 1, 2), (5000, 40000, 7, 3, 3)]
 
@@ -85,9 +85,16 @@ def test_reference_gpu_operator_classes_over_the_library_match_its_cpu_operators
     inp = refops.make_inputs(V, E, F, H, seed)
     ref = refops.run("gpu", "both", inp, tmp_path)
     co, ri = ref["column_offset"], ref["row_indices"]
-    # aggregation: one wave walks a row's edges in order with fused multiply-adds, as nts_comp does
-    assert ref["gpu_fwd"].tobytes() == ref["cpu_fwd"].tobytes()
-    assert ref["gpu_bwd"].tobytes() == ref["cpu_bwd"].tobytes()
+    # aggregation: one wave walks a row's edges in order with fused multiply-adds, as nts_comp does ->
+    # bit-identical; rows of more than 1024 edges are summed in pieces (calls of >= 65,536 edges) ->
+    # tolerance for those
+    x = inp["x"]
+    for got, want, off, idx, w in ((ref["gpu_fwd"], ref["cpu_fwd"], co, ri, ref["edge_weight_forward"]),
+                                   (ref["gpu_bwd"], ref["cpu_bwd"], ref["row_offset"], ref["column_indices"],
+                                    ref["edge_weight_backward"])):
+        one_wave = np.diff(off.astype(np.int64)) <= (1024 if E >= 1 << 16 else E)
+        assert got[one_wave].tobytes() == want[one_wave].tobytes()
+        check(got, want, abs_term_scale(x, w, off, idx, V))
     # vertex -> edge copies
     assert ref["gpu_scatter_src"].tobytes() == ref["cpu_scatter"][:, :F].tobytes()
     assert ref["gpu_scatter_dst"].tobytes() == ref["cpu_scatter"][:, F:].tobytes()
