@@ -29,22 +29,41 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(V *__restrict__ out, c
   for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
 }
 
+// Cached gather: a row comes from the HBM cache when its id has a slot, else from the (mapped host)
+// table.  Blocks stride over the rows and count their hits locally; one integer atomic per block
+// adds the block's count (one atomic per hit row on a single address was measured at 1.3 ms of a
+// 1.9 ms launch for 337 k rows).
 template <typename V, int G>
 __global__ __launch_bounds__(256) void gather_rows_cached_kernel(V *__restrict__ out, const V *__restrict__ table,
                                                                  const V *__restrict__ cache,
                                                                  const uint32_t *__restrict__ row_ids,
                                                                  const uint32_t *__restrict__ hashmap, uint32_t n,
                                                                  uint32_t Fv, uint32_t *__restrict__ hits) {
-  const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) / G;
-  if (i >= n) return;
+  constexpr uint32_t kRowsPerBlock = 256 / G;
   const uint32_t gl = threadIdx.x & (G - 1);
-  const uint32_t g = row_ids[i];
-  const uint32_t slot = hashmap[g];
-  const bool hit = slot != kMiss;
-  const V *src = hit ? cache + static_cast<size_t>(slot) * Fv : table + static_cast<size_t>(g) * Fv;
-  V *dst = out + static_cast<size_t>(i) * Fv;
-  for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
-  if (hits && hit && gl == 0) atomicAdd(hits, 1u);  // integer count: order-independent
+  uint32_t my_hits = 0;
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / G; i < n;
+       i += static_cast<uint64_t>(gridDim.x) * kRowsPerBlock) {
+    const uint32_t g = row_ids[i];
+    const uint32_t slot = hashmap[g];
+    const bool hit = slot != kMiss;
+    const V *src = hit ? cache + static_cast<size_t>(slot) * Fv : table + static_cast<size_t>(g) * Fv;
+    V *dst = out + static_cast<size_t>(i) * Fv;
+    for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
+    my_hits += (hit && gl == 0) ? 1u : 0u;
+  }
+  if (!hits) return;  // uniform across the block
+  __shared__ uint32_t wave_hits[256 / kWave];
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) my_hits += __shfl_xor(my_hits, m, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) wave_hits[threadIdx.x / kWave] = my_hits;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t total = 0;
+#pragma unroll
+    for (int k = 0; k < 256 / kWave; ++k) total += wave_hits[k];
+    if (total) atomicAdd(hits, total);  // integer count: order-independent
+  }
 }
 
 __global__ __launch_bounds__(256) void gather_labels_kernel(int64_t *__restrict__ out,
@@ -86,8 +105,10 @@ template <typename V, int G>
 void launch_rows(const RowsArgs &a, uint32_t Fv) {
   const uint32_t per_block = 256 / G;
   const dim3 grid(ceil_div(a.n, per_block));
+  // The cached kernel strides: enough blocks to fill the chip several times over, no more.
+  const dim3 cached_grid(grid.x < 16384u ? grid.x : 16384u);
   if (a.cache)
-    hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), grid, dim3(256), 0, a.stream,
+    hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), cached_grid, dim3(256), 0, a.stream,
                        reinterpret_cast<V *>(a.out), reinterpret_cast<const V *>(a.table),
                        reinterpret_cast<const V *>(a.cache), a.row_ids, a.remap, a.n, Fv, a.hits);
   else
