@@ -15,7 +15,7 @@
 namespace nts {
 namespace {
 
-constexpr int kMaxFanout = 64;  // distinct picks are kept in a per-thread array of this size
+constexpr int kMaxFanout = 64;  // distinct picks are resolved inside one wavefront
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   z += 0x9E3779B97F4A7C15ull;
@@ -39,53 +39,70 @@ __global__ __launch_bounds__(256) void hop_counts_kernel(uint32_t *__restrict__ 
   counts[i] = (fanout < 0 || deg < static_cast<uint32_t>(fanout)) ? deg : static_cast<uint32_t>(fanout);
 }
 
-// One thread per destination.
+// True if `pred` holds on any lane of the caller's aligned group of G lanes (all of them active).
+template <int G>
+__device__ __forceinline__ bool group_any(bool pred) {
+  const uint64_t votes = __ballot(pred);
+  if (G == kWave) return votes != 0;
+  const uint32_t first = (threadIdx.x & (kWave - 1)) & ~static_cast<uint32_t>(G - 1);
+  return ((votes >> first) & ((1ull << G) - 1ull)) != 0;
+}
+
+// A group of G lanes per destination (G = power of two >= the fanout, at most one wavefront).
+//
+// Floyd's algorithm draws `take` distinct positions of [0, deg): for j = deg-take .. deg-1 it draws
+// t uniform in [0, j] and inserts t, or j when t is already in the set.  Lane l owns step
+// j_l = deg-take+l: every lane advances the destination's hash chain to its own step and draws its
+// t at the same time (the 64-bit modulo is the expensive part); the "already in the set" decisions,
+// which depend on the earlier steps, are then resolved in `take` rounds of cross-lane shuffles
+// without touching memory; finally every lane ranks its value among the group's (values are
+// distinct) and copies one neighbour, so the sample comes out in ascending position order and the
+// neighbour reads of a destination are one parallel access instead of a chain.
+template <int G>
 __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri_out,
                                                        const uint32_t *__restrict__ co,
                                                        const uint32_t *__restrict__ graph_co,
                                                        const uint32_t *__restrict__ graph_ri,
                                                        const uint32_t *__restrict__ dst, uint32_t n, int32_t fanout,
                                                        uint64_t seed) {
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
+  const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) / G;
+  if (i >= n) return;  // whole groups leave together
+  const uint32_t gl = threadIdx.x & (G - 1);
   const uint32_t d = dst[i];
   const uint32_t base = graph_co[d];
   const uint32_t deg = graph_co[d + 1] - base;
   const uint32_t out = co[i];
   const uint32_t take = co[i + 1] - out;
   if (take == deg) {  // full neighbourhood, in CSC order
-    for (uint32_t k = 0; k < deg; ++k) ri_out[out + k] = graph_ri[base + k];
+    for (uint32_t k = gl; k < deg; k += G) ri_out[out + k] = graph_ri[base + k];
     return;
   }
-  uint64_t state = mix64(seed ^ (static_cast<uint64_t>(i) << 32) ^ d);
-  if (take > kMaxFanout) {
+  const uint64_t state0 = mix64(seed ^ (static_cast<uint64_t>(i) << 32) ^ d);
+  if (take > kMaxFanout || take > G) {
     // Very large fanouts: a window of consecutive positions from a random start (distinct by
-    // construction), emitted in ascending position order.
-    const uint32_t start = static_cast<uint32_t>(state % deg);
-    const uint32_t wrap = start + take > deg ? start + take - deg : 0;  // positions [0, wrap) belong to the window
-    uint32_t k = 0;
-    for (uint32_t p = 0; p < wrap; ++p) ri_out[out + k++] = graph_ri[base + p];
-    for (uint32_t p = start; p < deg && k < take; ++p) ri_out[out + k++] = graph_ri[base + p];
+    // construction), emitted in ascending position order: [0, wrap) then [start, start + take - wrap).
+    const uint32_t start = static_cast<uint32_t>(state0 % deg);
+    const uint32_t wrap = start + take > deg ? start + take - deg : 0;
+    for (uint32_t k = gl; k < take; k += G) ri_out[out + k] = graph_ri[base + (k < wrap ? k : start + (k - wrap))];
     return;
   }
-  // Floyd's algorithm: `take` distinct values from [0, deg), kept sorted by insertion.
-  uint32_t pick[kMaxFanout];
-  uint32_t m = 0;
-  for (uint32_t j = deg - take; j < deg; ++j) {
-    state = mix64(state);
-    uint32_t t = static_cast<uint32_t>(state % (static_cast<uint64_t>(j) + 1));
-    bool present = false;
-    for (uint32_t q = 0; q < m; ++q) present = present || pick[q] == t;
-    if (present) t = j;  // j cannot be present yet: every earlier value is < j
-    uint32_t pos = m;
-    while (pos > 0 && pick[pos - 1] > t) {
-      pick[pos] = pick[pos - 1];
-      --pos;
-    }
-    pick[pos] = t;
-    ++m;
+  // Lane gl < take: step j = deg - take + gl, hash chain advanced gl + 1 times.
+  uint64_t state = state0;
+  for (uint32_t q = 0; q <= gl && q < take; ++q) state = mix64(state);
+  const uint32_t j = deg - take + gl;
+  const uint32_t t = gl < take ? static_cast<uint32_t>(state % (static_cast<uint64_t>(j) + 1)) : 0xFFFFFFFFu;
+  uint32_t v = 0xFFFFFFFFu;  // this lane's inserted value, set in round gl
+  for (uint32_t l = 0; l < take; ++l) {
+    const uint32_t tl = __shfl(t, l, G);
+    // lanes of earlier rounds that already hold tl (at most one); lanes >= l still hold the marker
+    const bool present = group_any<G>(v == tl);
+    if (gl == l) v = present ? j : tl;  // j cannot be present yet: every earlier value is < j
   }
-  for (uint32_t k = 0; k < take; ++k) ri_out[out + k] = graph_ri[base + pick[k]];
+  if (gl < take) {
+    uint32_t rank = 0;
+    for (uint32_t q = 0; q < take; ++q) rank += __shfl(v, q, G) < v ? 1u : 0u;
+    ri_out[out + rank] = graph_ri[base + v];
+  }
 }
 
 hipError_t scan_bytes(uint32_t n, size_t *bytes) {
@@ -136,8 +153,24 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
   if (n == 0) return NTS_OK;
   if (!ri_global || !co || !graph_co || !graph_ri || !dst)
     return fail(NTS_ERR_INVALID, "nts_sample_hop_neighbors: null pointer");
-  hipLaunchKernelGGL(hop_pick_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream, ri_global, co, graph_co, graph_ri,
-                     dst, n, fanout, seed);
+  // Lanes per destination: the fanout rounded up to a power of two (full neighbourhoods and
+  // fanouts above one wavefront are strided copies, for which a quarter wavefront serves well).
+  int g = 8;
+  if (fanout > 0 && fanout <= kMaxFanout)
+    while (g < fanout) g <<= 1;
+  else
+    g = 16;
+  const dim3 grid(ceil_div(static_cast<uint64_t>(n) * g, 256));
+#define NTS_LAUNCH_PICK(G)                                                                                      \
+  hipLaunchKernelGGL(hop_pick_kernel<G>, grid, dim3(256), 0, stream, ri_global, co, graph_co, graph_ri, dst, n, \
+                     fanout, seed)
+  switch (g) {
+    case 8: NTS_LAUNCH_PICK(8); break;
+    case 16: NTS_LAUNCH_PICK(16); break;
+    case 32: NTS_LAUNCH_PICK(32); break;
+    default: NTS_LAUNCH_PICK(64); break;
+  }
+#undef NTS_LAUNCH_PICK
   NTS_LAUNCH_CHECK("hop_pick_kernel");
   return NTS_OK;
 }
