@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, con
 
 constexpr uint32_t kNoLimit = 0xFFFFFFFFu;
 constexpr uint32_t kLongRowEdges = 1024;    // edges of a row above which the block kernel takes over
-constexpr uint32_t kLongRowValues = 4096;   // the same for softmax segments, in values (edges * heads)
+constexpr uint32_t kLongRowValues = 32768;  // the same for softmax segments, in values (edges * heads)
 constexpr uint32_t kLongMinVertices = 16384;  // vertex count below which the extra launches are not worth it
 constexpr int kLongBlock = 1024;
 
@@ -105,7 +105,24 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__
     float a[NF];
 #pragma unroll
     for (int t = 0; t < NF; ++t) a[t] = 0.f;
-    for (uint32_t k = e0; k < e1; ++k) {
+    // Eight edge rows are loaded before they are added, in order: the loads overlap, the order of
+    // the additions stays the edge order.
+    uint32_t k = e0;
+    for (; k + 8 <= e1; k += 8) {
+      V v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const uint32_t e = perm ? perm[k + u] : k + u;
+        v[u] = msg[static_cast<size_t>(e) * Fv + c];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float *vf = reinterpret_cast<const float *>(&v[u]);
+#pragma unroll
+        for (int t = 0; t < NF; ++t) a[t] += vf[t];
+      }
+    }
+    for (; k < e1; ++k) {
       const uint32_t e = perm ? perm[k] : k;
       const V v = msg[static_cast<size_t>(e) * Fv + c];
       const float *vf = reinterpret_cast<const float *>(&v);
@@ -156,7 +173,20 @@ __global__ __launch_bounds__(kLongBlock) void gather_edge_to_row_long_kernel(
       const uint32_t col = cb + c;
       float a = 0.f;
       if (col < F) {
-        for (uint32_t k = e0 + slice; k < e1; k += n_slices) {
+        // eight loads in flight, added in the slice's edge order
+        uint32_t k = e0 + slice;
+        for (; static_cast<uint64_t>(k) + 7ull * n_slices < e1; k += 8 * n_slices) {
+          float v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const uint32_t kk = k + u * n_slices;
+            const uint32_t e = perm ? perm[kk] : kk;
+            v[u] = msg[static_cast<size_t>(e) * F + col];
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) a += v[u];
+        }
+        for (; k < e1; k += n_slices) {
           const uint32_t e = perm ? perm[k] : k;
           a += msg[static_cast<size_t>(e) * F + col];
         }
@@ -192,117 +222,118 @@ __device__ __forceinline__ float head_reduce(float v, uint32_t H) {
 
 __device__ __forceinline__ float leaky(float s, float slope) { return s > 0.f ? s : s * slope; }
 
-// FUSED = false: y = softmax_seg(x).   FUSED = true: x is ignored and the score is
-// leaky_relu(el[ri[e],h] + er[d,h], slope); y first holds the raw score, then alpha.
-template <bool FUSED, bool POW2>
-__global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict__ y, const float *__restrict__ x,
-                                                               const float *__restrict__ el,
-                                                               const float *__restrict__ er,
-                                                               const uint32_t *__restrict__ co,
-                                                               const uint32_t *__restrict__ ri, uint32_t Vd,
-                                                               uint32_t H, float slope, uint32_t long_limit) {
-  const uint32_t d = wave_item();
-  if (d >= Vd) return;
-  const uint32_t lane = lane_id();
-  const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
-  if (e0 == e1) return;
-  if (static_cast<uint64_t>(e1 - e0) * H > long_limit) return;  // left to the block kernel
-  const size_t base = static_cast<size_t>(e0) * H;
-  const uint32_t n = (e1 - e0) * H;
-  float *ys = y + base;
-  const float *xs = FUSED ? nullptr : x + base;
+// Three kernels share a launch, by segment size n = degree * H (values):
+//   short   n <= 128, power-of-two H <= 16: a group of 16 lanes per destination, the segment held
+//           in registers -- one pass over memory, four destinations per wavefront in flight;
+//   wave    up to kLongRowValues (or any size when the block kernel is not used): one wavefront per
+//           destination; segments of at most 512 values are register-resident too, larger ones take
+//           the three passes (max, sum, write) / two passes (dot, write) over memory;
+//   block   longer segments (hub destinations), listed by collect_long_rows.
+// The short and the wave kernel stride over the destinations (a wavefront of the wave kernel looks
+// at 64 destinations at a time and visits only those that fall in its size class), so their launch
+// size does not grow with the vertex count.
 
-  if (POW2) {
-    const uint32_t h = lane & (H - 1);
-    float erv = 0.f;
-    if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
-    float mx = -INFINITY;
-    for (uint32_t i = lane; i < n; i += kWave) {
-      float s;
+constexpr int kShortG = 16;        // lanes per destination in the short kernel
+constexpr int kShortK = 8;         // values per lane held in registers there
+constexpr uint32_t kShortValues = kShortG * kShortK;
+constexpr int kWaveK = 8;          // values per lane the wave kernel can hold in registers
+constexpr uint32_t kWaveRegValues = kWave * kWaveK;
+
+// One strided pass over a segment with U loads in flight: positions first, first + stride, ...
+// below n; `load(i)` fetches, `use(i, v)` consumes, in ascending position order.
+template <int U, typename Load, typename Use>
+__device__ __forceinline__ void strided_pass(uint64_t first, uint64_t n, uint64_t stride, Load load, Use use) {
+  uint64_t i = first;
+  for (; i + (U - 1) * stride < n; i += U * stride) {
+    decltype(load(i)) v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = load(i + u * stride);
+#pragma unroll
+    for (int u = 0; u < U; ++u) use(i + u * stride, v[u]);
+  }
+  for (; i < n; i += stride) use(i, load(i));
+}
+
+// Reduction over the lanes of an aligned group of WIDTH lanes that share a head (lane mod H).
+template <int MODE, int WIDTH>  // 0 = max, 1 = sum
+__device__ __forceinline__ float head_reduce_w(float v, uint32_t H) {
+  for (uint32_t m = WIDTH / 2; m >= H; m >>= 1) {
+    const float o = __shfl_xor(v, m, WIDTH);
+    v = MODE == 0 ? fmaxf(v, o) : v + o;
+  }
+  return v;
+}
+
+// Register-resident forward of one segment by WIDTH lanes (lane index gl), K values per lane;
+// n <= WIDTH*K values, H a power of two <= WIDTH.
+template <bool FUSED, int WIDTH, int K>
+__device__ __forceinline__ void softmax_fwd_regs(float *__restrict__ ys, const float *__restrict__ xs,
+                                                 const float *__restrict__ el, const float *__restrict__ er,
+                                                 const uint32_t *__restrict__ ri, uint32_t d, uint32_t e0, uint32_t n,
+                                                 uint32_t H, float slope, uint32_t gl) {
+  const uint32_t h = gl & (H - 1);
+  float erv = 0.f;
+  if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+  float v[K];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const uint32_t i = gl + WIDTH * k;
+    v[k] = -INFINITY;
+    if (i < n) {
       if (FUSED) {
         const uint32_t src = ri[e0 + i / H];
-        s = leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
-        ys[i] = s;
+        v[k] = leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
       } else {
-        s = xs[i];
-      }
-      mx = fmaxf(mx, s);
-    }
-    mx = head_reduce<0>(mx, H);
-    float sum = 0.f;
-    for (uint32_t i = lane; i < n; i += kWave) {
-      const float s = FUSED ? ys[i] : xs[i];
-      sum += expf(s - mx);
-    }
-    sum = head_reduce<1>(sum, H);
-    for (uint32_t i = lane; i < n; i += kWave) {
-      const float s = FUSED ? ys[i] : xs[i];
-      ys[i] = expf(s - mx) / sum;
-    }
-  } else {
-    const uint32_t deg = e1 - e0;
-    for (uint32_t h = 0; h < H; ++h) {
-      float erv = 0.f;
-      if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
-      float mx = -INFINITY;
-      for (uint32_t k = lane; k < deg; k += kWave) {
-        float s;
-        if (FUSED) {
-          const uint32_t src = ri[e0 + k];
-          s = leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
-          ys[static_cast<size_t>(k) * H + h] = s;
-        } else {
-          s = xs[static_cast<size_t>(k) * H + h];
-        }
-        mx = fmaxf(mx, s);
-      }
-      mx = group_max<kWave>(mx);
-      float sum = 0.f;
-      for (uint32_t k = lane; k < deg; k += kWave) {
-        const float s = FUSED ? ys[static_cast<size_t>(k) * H + h] : xs[static_cast<size_t>(k) * H + h];
-        sum += expf(s - mx);
-      }
-      sum = group_sum<kWave>(sum);
-      for (uint32_t k = lane; k < deg; k += kWave) {
-        const float s = FUSED ? ys[static_cast<size_t>(k) * H + h] : xs[static_cast<size_t>(k) * H + h];
-        ys[static_cast<size_t>(k) * H + h] = expf(s - mx) / sum;
+        v[k] = xs[i];
       }
     }
+    mx = fmaxf(mx, v[k]);
+  }
+  mx = head_reduce_w<0, WIDTH>(mx, H);
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    v[k] = (gl + WIDTH * k < n) ? expf(v[k] - mx) : 0.f;
+    sum += v[k];
+  }
+  sum = head_reduce_w<1, WIDTH>(sum, H);
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const uint32_t i = gl + WIDTH * k;
+    if (i < n) ys[i] = v[k] / sum;
   }
 }
 
-// FUSED = false: gx = y * (gy - sum_seg gy*y).
-// FUSED = true : additionally multiplies by leaky_relu'(el[src]+er[d]) and writes
-//                ger[d,h] = sum_seg gx[e,h].
-template <bool FUSED, bool POW2>
-__global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict__ gx, float *__restrict__ ger,
-                                                               const float *__restrict__ gy,
-                                                               const float *__restrict__ y,
-                                                               const float *__restrict__ el,
-                                                               const float *__restrict__ er,
-                                                               const uint32_t *__restrict__ co,
-                                                               const uint32_t *__restrict__ ri, uint32_t Vd,
-                                                               uint32_t H, float slope, uint32_t long_limit) {
-  const uint32_t d = wave_item();
-  if (d >= Vd) return;
-  const uint32_t lane = lane_id();
-  const uint32_t e0 = wave_first(co[d]), e1 = wave_first(co[d + 1]);
-  if (static_cast<uint64_t>(e1 - e0) * H > long_limit) return;  // left to the block kernel
-  const size_t base = static_cast<size_t>(e0) * H;
-  const uint32_t n = (e1 - e0) * H;
-  const float *gys = gy + base;
-  const float *ys = y + base;
-  float *gxs = gx + base;
-
-  if (POW2) {
-    const uint32_t h = lane & (H - 1);
-    float dot = 0.f;
-    for (uint32_t i = lane; i < n; i += kWave) dot += gys[i] * ys[i];
-    dot = head_reduce<1>(dot, H);
-    float erv = 0.f, gsum = 0.f;
-    if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
-    for (uint32_t i = lane; i < n; i += kWave) {
-      float g = ys[i] * (gys[i] - dot);
+// Register-resident backward, same shape.  Writes ger[d, :] when FUSED (zeros for an empty segment).
+template <bool FUSED, int WIDTH, int K>
+__device__ __forceinline__ void softmax_bwd_regs(float *__restrict__ gxs, float *__restrict__ ger,
+                                                 const float *__restrict__ gys, const float *__restrict__ ys,
+                                                 const float *__restrict__ el, const float *__restrict__ er,
+                                                 const uint32_t *__restrict__ ri, uint32_t d, uint32_t e0, uint32_t n,
+                                                 uint32_t H, float slope, uint32_t gl) {
+  const uint32_t h = gl & (H - 1);
+  float yv[K], gv[K];
+  float dot = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const uint32_t i = gl + WIDTH * k;
+    yv[k] = 0.f;
+    gv[k] = 0.f;
+    if (i < n) {
+      yv[k] = ys[i];
+      gv[k] = gys[i];
+    }
+    dot += gv[k] * yv[k];
+  }
+  dot = head_reduce_w<1, WIDTH>(dot, H);
+  float erv = 0.f, gsum = 0.f;
+  if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const uint32_t i = gl + WIDTH * k;
+    if (i < n) {
+      float g = yv[k] * (gv[k] - dot);
       if (FUSED) {
         const uint32_t src = ri[e0 + i / H];
         const float pre = el[static_cast<size_t>(src) * H + h] + erv;
@@ -311,35 +342,238 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
       }
       gxs[i] = g;
     }
-    if (FUSED) {
-      gsum = head_reduce<1>(gsum, H);
-      if (lane < H) ger[static_cast<size_t>(d) * H + lane] = gsum;
+  }
+  if (FUSED) {
+    gsum = head_reduce_w<1, WIDTH>(gsum, H);
+    if (gl < H) ger[static_cast<size_t>(d) * H + gl] = gsum;
+  }
+}
+
+// Short segments (n <= kShortValues; power-of-two H <= kShortG): a group of kShortG lanes per
+// destination, striding over the destinations.  BWD selects the backward formula.
+template <bool FUSED, bool BWD>
+__global__ __launch_bounds__(256) void edge_softmax_short_kernel(float *__restrict__ out, float *__restrict__ ger,
+                                                                 const float *__restrict__ x_or_gy,
+                                                                 const float *__restrict__ y,
+                                                                 const float *__restrict__ el,
+                                                                 const float *__restrict__ er,
+                                                                 const uint32_t *__restrict__ co,
+                                                                 const uint32_t *__restrict__ ri, uint32_t Vd,
+                                                                 uint32_t H, float slope) {
+  const uint32_t gl = threadIdx.x & (kShortG - 1);
+  const uint64_t n_groups = static_cast<uint64_t>(gridDim.x) * (256 / kShortG);
+  for (uint64_t d64 = (static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x) / kShortG; d64 < Vd; d64 += n_groups) {
+    const uint32_t d = static_cast<uint32_t>(d64);
+    const uint32_t e0 = co[d], e1 = co[d + 1];
+    const uint64_t n64 = static_cast<uint64_t>(e1 - e0) * H;
+    if (n64 > kShortValues) continue;  // the whole group skips together
+    const uint32_t n = static_cast<uint32_t>(n64);
+    const size_t base = static_cast<size_t>(e0) * H;
+    if (BWD) {
+      softmax_bwd_regs<FUSED, kShortG, kShortK>(out + base, ger, x_or_gy + base, y + base, el, er, ri, d, e0, n, H,
+                                                slope, gl);
+    } else {
+      if (n == 0) continue;
+      softmax_fwd_regs<FUSED, kShortG, kShortK>(out + base, FUSED ? nullptr : x_or_gy + base, el, er, ri, d, e0, n, H,
+                                                slope, gl);
     }
-  } else {
-    const uint32_t deg = e1 - e0;
-    for (uint32_t h = 0; h < H; ++h) {
-      float dot = 0.f;
-      for (uint32_t k = lane; k < deg; k += kWave) {
-        const size_t i = static_cast<size_t>(k) * H + h;
-        dot += gys[i] * ys[i];
-      }
-      dot = group_sum<kWave>(dot);
-      float erv = 0.f, gsum = 0.f;
-      if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
-      for (uint32_t k = lane; k < deg; k += kWave) {
-        const size_t i = static_cast<size_t>(k) * H + h;
-        float g = ys[i] * (gys[i] - dot);
-        if (FUSED) {
-          const uint32_t src = ri[e0 + k];
-          const float pre = el[static_cast<size_t>(src) * H + h] + erv;
-          g *= pre > 0.f ? 1.f : slope;
-          gsum += g;
+  }
+}
+
+// The destinations of [base, base + 64) whose segment size lies in [min_values, max_values], as a
+// wave-uniform bit mask; every lane keeps the offsets of its own destination for the visit.
+__device__ __forceinline__ uint64_t wave_rows_in_class(const uint32_t *__restrict__ co, uint32_t Vd, uint64_t base,
+                                                       uint32_t H, uint32_t min_values, uint32_t max_values,
+                                                       uint32_t &my_e0, uint32_t &my_e1) {
+  const uint64_t d = base + lane_id();
+  my_e0 = 0;
+  my_e1 = 0;
+  bool mine = false;
+  if (d < Vd) {
+    my_e0 = co[d];
+    my_e1 = co[d + 1];
+    const uint64_t n = static_cast<uint64_t>(my_e1 - my_e0) * H;
+    mine = n >= min_values && n <= max_values;
+  }
+  return __ballot(mine);
+}
+
+// FUSED = false: y = softmax_seg(x).   FUSED = true: x is ignored and the score is
+// leaky_relu(el[ri[e],h] + er[d,h], slope); in the three-pass path y first holds the raw score, then
+// alpha.  Visits the destinations with min_values <= n <= max_values.
+template <bool FUSED, bool POW2>
+__global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict__ y, const float *__restrict__ x,
+                                                               const float *__restrict__ el,
+                                                               const float *__restrict__ er,
+                                                               const uint32_t *__restrict__ co,
+                                                               const uint32_t *__restrict__ ri, uint32_t Vd,
+                                                               uint32_t H, float slope, uint32_t min_values,
+                                                               uint32_t max_values) {
+  const uint32_t lane = lane_id();
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  for (uint64_t first = wave * kWave; first < Vd; first += n_waves * kWave) {
+    uint32_t my_e0, my_e1;
+    uint64_t todo = wave_rows_in_class(co, Vd, first, H, min_values < 1 ? 1 : min_values, max_values, my_e0, my_e1);
+    while (todo) {
+      const uint32_t j = static_cast<uint32_t>(__builtin_ctzll(todo));
+      todo &= todo - 1;
+      const uint32_t d = static_cast<uint32_t>(first) + j;
+      const uint32_t e0 = wave_read(my_e0, j), e1 = wave_read(my_e1, j);
+      const size_t base = static_cast<size_t>(e0) * H;
+      const uint32_t n = (e1 - e0) * H;
+      float *ys = y + base;
+      const float *xs = FUSED ? nullptr : x + base;
+
+      if (POW2) {
+        if (n <= kWaveRegValues) {
+          softmax_fwd_regs<FUSED, kWave, kWaveK>(ys, xs, el, er, ri, d, e0, n, H, slope, lane);
+          continue;
         }
-        gxs[i] = g;
+        const uint32_t h = lane & (H - 1);
+        float erv = 0.f;
+        if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+        float mx = -INFINITY;
+        strided_pass<8>(lane, n, kWave,
+                        [&](uint64_t i) -> float {
+                          if (!FUSED) return xs[i];
+                          const uint32_t src = ri[e0 + i / H];
+                          return leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
+                        },
+                        [&](uint64_t i, float sc) {
+                          if (FUSED) ys[i] = sc;
+                          mx = fmaxf(mx, sc);
+                        });
+        mx = head_reduce<0>(mx, H);
+        float sum = 0.f;
+        strided_pass<8>(lane, n, kWave, [&](uint64_t i) -> float { return FUSED ? ys[i] : xs[i]; },
+                        [&](uint64_t, float sc) { sum += expf(sc - mx); });
+        sum = head_reduce<1>(sum, H);
+        strided_pass<8>(lane, n, kWave, [&](uint64_t i) -> float { return FUSED ? ys[i] : xs[i]; },
+                        [&](uint64_t i, float sc) { ys[i] = expf(sc - mx) / sum; });
+      } else {
+        const uint32_t deg = e1 - e0;
+        for (uint32_t h = 0; h < H; ++h) {
+          float erv = 0.f;
+          if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+          float mx = -INFINITY;
+          for (uint32_t k = lane; k < deg; k += kWave) {
+            float sc;
+            if (FUSED) {
+              const uint32_t src = ri[e0 + k];
+              sc = leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
+              ys[static_cast<size_t>(k) * H + h] = sc;
+            } else {
+              sc = xs[static_cast<size_t>(k) * H + h];
+            }
+            mx = fmaxf(mx, sc);
+          }
+          mx = group_max<kWave>(mx);
+          float sum = 0.f;
+          for (uint32_t k = lane; k < deg; k += kWave) {
+            const float sc = FUSED ? ys[static_cast<size_t>(k) * H + h] : xs[static_cast<size_t>(k) * H + h];
+            sum += expf(sc - mx);
+          }
+          sum = group_sum<kWave>(sum);
+          for (uint32_t k = lane; k < deg; k += kWave) {
+            const float sc = FUSED ? ys[static_cast<size_t>(k) * H + h] : xs[static_cast<size_t>(k) * H + h];
+            ys[static_cast<size_t>(k) * H + h] = expf(sc - mx) / sum;
+          }
+        }
       }
-      if (FUSED) {
-        gsum = group_sum<kWave>(gsum);
-        if (lane == 0) ger[static_cast<size_t>(d) * H + h] = gsum;
+    }
+  }
+}
+
+// FUSED = false: gx = y * (gy - sum_seg gy*y).
+// FUSED = true : additionally multiplies by leaky_relu'(el[src]+er[d]) and writes
+//                ger[d,h] = sum_seg gx[e,h].
+// Visits the destinations with min_values <= n <= max_values (empty segments included when
+// min_values is 0, so that ger is written for every destination).
+template <bool FUSED, bool POW2>
+__global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict__ gx, float *__restrict__ ger,
+                                                               const float *__restrict__ gy,
+                                                               const float *__restrict__ y,
+                                                               const float *__restrict__ el,
+                                                               const float *__restrict__ er,
+                                                               const uint32_t *__restrict__ co,
+                                                               const uint32_t *__restrict__ ri, uint32_t Vd,
+                                                               uint32_t H, float slope, uint32_t min_values,
+                                                               uint32_t max_values) {
+  const uint32_t lane = lane_id();
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  for (uint64_t first = wave * kWave; first < Vd; first += n_waves * kWave) {
+    uint32_t my_e0, my_e1;
+    uint64_t todo = wave_rows_in_class(co, Vd, first, H, min_values, max_values, my_e0, my_e1);
+    while (todo) {
+      const uint32_t j = static_cast<uint32_t>(__builtin_ctzll(todo));
+      todo &= todo - 1;
+      const uint32_t d = static_cast<uint32_t>(first) + j;
+      const uint32_t e0 = wave_read(my_e0, j), e1 = wave_read(my_e1, j);
+      const size_t base = static_cast<size_t>(e0) * H;
+      const uint32_t n = (e1 - e0) * H;
+      const float *gys = gy + base;
+      const float *ys = y + base;
+      float *gxs = gx + base;
+
+      if (POW2) {
+        if (n <= kWaveRegValues) {
+          softmax_bwd_regs<FUSED, kWave, kWaveK>(gxs, ger, gys, ys, el, er, ri, d, e0, n, H, slope, lane);
+          continue;
+        }
+        const uint32_t h = lane & (H - 1);
+        float dot = 0.f;
+        strided_pass<8>(lane, n, kWave, [&](uint64_t i) -> float2 { return make_float2(gys[i], ys[i]); },
+                        [&](uint64_t, float2 v) { dot += v.x * v.y; });
+        dot = head_reduce<1>(dot, H);
+        float erv = 0.f, gsum = 0.f;
+        if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+        strided_pass<8>(lane, n, kWave,
+                        [&](uint64_t i) -> float4 {
+                          float pre = 1.f;
+                          if (FUSED) pre = el[static_cast<size_t>(ri[e0 + i / H]) * H + h] + erv;
+                          return make_float4(gys[i], ys[i], pre, 0.f);
+                        },
+                        [&](uint64_t i, float4 v) {
+                          float g = v.y * (v.x - dot);
+                          if (FUSED) {
+                            g *= v.z > 0.f ? 1.f : slope;
+                            gsum += g;
+                          }
+                          gxs[i] = g;
+                        });
+        if (FUSED) {
+          gsum = head_reduce<1>(gsum, H);
+          if (lane < H) ger[static_cast<size_t>(d) * H + lane] = gsum;
+        }
+      } else {
+        const uint32_t deg = e1 - e0;
+        for (uint32_t h = 0; h < H; ++h) {
+          float dot = 0.f;
+          for (uint32_t k = lane; k < deg; k += kWave) {
+            const size_t i = static_cast<size_t>(k) * H + h;
+            dot += gys[i] * ys[i];
+          }
+          dot = group_sum<kWave>(dot);
+          float erv = 0.f, gsum = 0.f;
+          if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+          for (uint32_t k = lane; k < deg; k += kWave) {
+            const size_t i = static_cast<size_t>(k) * H + h;
+            float g = ys[i] * (gys[i] - dot);
+            if (FUSED) {
+              const uint32_t src = ri[e0 + k];
+              const float pre = el[static_cast<size_t>(src) * H + h] + erv;
+              g *= pre > 0.f ? 1.f : slope;
+              gsum += g;
+            }
+            gxs[i] = g;
+          }
+          if (FUSED) {
+            gsum = group_sum<kWave>(gsum);
+            if (lane == 0) ger[static_cast<size_t>(d) * H + h] = gsum;
+          }
+        }
       }
     }
   }
@@ -380,22 +614,23 @@ __global__ __launch_bounds__(kLongBlock) void edge_softmax_fwd_long_kernel(
     float erv = 0.f;
     if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
     float mx = -INFINITY;
-    for (size_t j = threadIdx.x; j < n; j += kLongBlock) {
-      float sc;
-      if (FUSED) {
-        const uint32_t src = ri[e0 + j / H];
-        sc = leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
-        ys[j] = sc;
-      } else {
-        sc = xs[j];
-      }
-      mx = fmaxf(mx, sc);
-    }
+    strided_pass<8>(threadIdx.x, n, kLongBlock,
+                    [&](uint64_t j) -> float {
+                      if (!FUSED) return xs[j];
+                      const uint32_t src = ri[e0 + j / H];
+                      return leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
+                    },
+                    [&](uint64_t j, float sc) {
+                      if (FUSED) ys[j] = sc;
+                      mx = fmaxf(mx, sc);
+                    });
     mx = block_head_reduce<0>(mx, H, red);
     float sum = 0.f;
-    for (size_t j = threadIdx.x; j < n; j += kLongBlock) sum += expf((FUSED ? ys[j] : xs[j]) - mx);
+    strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
+                    [&](uint64_t, float sc) { sum += expf(sc - mx); });
     sum = block_head_reduce<1>(sum, H, red);
-    for (size_t j = threadIdx.x; j < n; j += kLongBlock) ys[j] = expf((FUSED ? ys[j] : xs[j]) - mx) / sum;
+    strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
+                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) / sum; });
   }
 }
 
@@ -417,20 +652,25 @@ __global__ __launch_bounds__(kLongBlock) void edge_softmax_bwd_long_kernel(
     const float *ys = y + base;
     float *gxs = gx + base;
     float dot = 0.f;
-    for (size_t j = threadIdx.x; j < n; j += kLongBlock) dot += gys[j] * ys[j];
+    strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float2 { return make_float2(gys[j], ys[j]); },
+                    [&](uint64_t, float2 v) { dot += v.x * v.y; });
     dot = block_head_reduce<1>(dot, H, red);
     float erv = 0.f, gsum = 0.f;
     if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
-    for (size_t j = threadIdx.x; j < n; j += kLongBlock) {
-      float g = ys[j] * (gys[j] - dot);
-      if (FUSED) {
-        const uint32_t src = ri[e0 + j / H];
-        const float pre = el[static_cast<size_t>(src) * H + h] + erv;
-        g *= pre > 0.f ? 1.f : slope;
-        gsum += g;
-      }
-      gxs[j] = g;
-    }
+    strided_pass<8>(threadIdx.x, n, kLongBlock,
+                    [&](uint64_t j) -> float4 {
+                      float pre = 1.f;
+                      if (FUSED) pre = el[static_cast<size_t>(ri[e0 + j / H]) * H + h] + erv;
+                      return make_float4(gys[j], ys[j], pre, 0.f);
+                    },
+                    [&](uint64_t j, float4 v) {
+                      float g = v.y * (v.x - dot);
+                      if (FUSED) {
+                        g *= v.z > 0.f ? 1.f : slope;
+                        gsum += g;
+                      }
+                      gxs[j] = g;
+                    });
     if (FUSED) {
       gsum = block_head_reduce<1>(gsum, H, red);
       if (threadIdx.x < H) ger[static_cast<size_t>(d) * H + threadIdx.x] = gsum;
@@ -659,12 +899,28 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   LongRows lr;
   if (pow2)
     if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, stream)) return rc;
-  const uint32_t limit = lr.list ? kLongRowValues : kNoLimit;
-  const dim3 grid = wave_grid(Vd), block = wave_block();
+  const uint32_t max_values = lr.list ? kLongRowValues : kNoLimit;
+  const bool use_short = pow2 && H <= static_cast<uint32_t>(kShortG);
+  const uint32_t min_values = use_short ? kShortValues + 1 : 0u;
+  // Both strided kernels: enough wavefronts to fill the chip several times, never more than the work.
+  const dim3 block(256);
+  const uint32_t short_blocks = ceil_div(static_cast<uint64_t>(Vd) * kShortG, 256);
+  const dim3 short_grid(short_blocks < 16384u ? short_blocks : 16384u);
+  const uint32_t wave_blocks = ceil_div(Vd, 4);  // at most one destination per wavefront
+  const dim3 grid(wave_blocks < 8192u ? wave_blocks : 8192u);
+  if (use_short) {
+#define NTS_SHORT(FU, BW)                                                                                          \
+  hipLaunchKernelGGL((edge_softmax_short_kernel<FU, BW>), short_grid, block, 0, stream, out, ger, x_or_gy, y, el, er, \
+                     co, ri, Vd, H, slope)
+    if (fused) { if (backward) NTS_SHORT(true, true); else NTS_SHORT(true, false); }
+    else       { if (backward) NTS_SHORT(false, true); else NTS_SHORT(false, false); }
+#undef NTS_SHORT
+    NTS_LAUNCH_CHECK(who);
+  }
   if (!backward) {
 #define NTS_FWD(FU, P2)                                                                                          \
   hipLaunchKernelGGL((edge_softmax_fwd_kernel<FU, P2>), grid, block, 0, stream, out, x_or_gy, el, er, co, ri, Vd, H, \
-                     slope, limit)
+                     slope, min_values, max_values)
     if (fused) { if (pow2) NTS_FWD(true, true); else NTS_FWD(true, false); }
     else       { if (pow2) NTS_FWD(false, true); else NTS_FWD(false, false); }
 #undef NTS_FWD
@@ -681,7 +937,7 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   } else {
 #define NTS_BWD(FU, P2)                                                                                           \
   hipLaunchKernelGGL((edge_softmax_bwd_kernel<FU, P2>), grid, block, 0, stream, out, ger, x_or_gy, y, el, er, co, ri, \
-                     Vd, H, slope, limit)
+                     Vd, H, slope, min_values, max_values)
     if (fused) { if (pow2) NTS_BWD(true, true); else NTS_BWD(true, false); }
     else       { if (pow2) NTS_BWD(false, true); else NTS_BWD(false, false); }
 #undef NTS_BWD

@@ -203,11 +203,16 @@ def test_fused_gat_layer(device, H, Fh):
 
 @pytest.mark.parametrize("H", [1, 4, 3])
 def test_long_segments_softmax_and_attention(device, H):
-    """Vertex counts at which the library hands hub segments (more than 4096 values) to its block
-    kernels: edge softmax and fused attention, forward and backward, still match the oracle."""
+    """Vertex counts at which the library hands hub segments (more than 32,768 values) to its block
+    kernels: edge softmax and fused attention, forward and backward, still match the oracle.  A second
+    hub of 9,000 edges stays on the wave kernel's multi-pass path."""
     print(f"case H={H}", flush=True)
     Vd, Vs = 17000, 2500
-    co, ri = random_block(Vd, Vs, 3, seed=300 + H, hub=7000, dup=True)
+    co, ri = random_block(Vd, Vs, 3, seed=300 + H, hub=40000, dup=True)
+    deg = np.diff(co.astype(np.int64))
+    deg[Vd // 2] = 9000
+    co = np.concatenate([[0], np.cumsum(deg)]).astype(np.uint32)
+    ri = np.random.default_rng(17 + H).integers(0, Vs, int(co[-1])).astype(np.uint32)
     co, ri = co.copy(), ri.copy()
     E = ri.size
     rng = np.random.default_rng(H)
