@@ -240,10 +240,11 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
  * toolkits/GAT_CPU.hpp:196-201):
  *   out[r, h*Fh + f] (+)= sum_{e in [offsets[r], offsets[r+1])} alpha[eid(e), h] * in[indices[e], h*Fh + f]
  * eid(e) = e when perm is NULL (forward over CSC) or perm[e] (backward over CSR, alpha kept in
- * CSC edge order). */
+ * CSC edge order).  `edges` = offsets[rows]; as in nts_spmm_gather, calls of 65,536 edges or more
+ * cut rows of more than 1,024 edges into pieces on the device. */
 int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
                           const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
-                          uint32_t H, uint32_t Fh, int accumulate, nts_stream_t stream);
+                          uint32_t edges, uint32_t H, uint32_t Fh, int accumulate, nts_stream_t stream);
 /* The same through a schedule built by nts_spmm_plan_create[_slabs] for `offsets` (full-graph GAT:
  * hub rows are split and the sum order of split rows is the plan's). */
 int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *alpha,

@@ -67,7 +67,7 @@ SIGNATURES = {
     "nts_edge_softmax_bwd": [_vp, _vp, _vp, _vp, _u32, _u32, _vp],
     "nts_gat_attention_fwd": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp],
     "nts_gat_attention_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp],
-    "nts_spmm_gather_heads": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _int, _vp],
+    "nts_spmm_gather_heads": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
     "nts_spmm_gather_heads_planned": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _int, _vp],
     "nts_sddmm_heads": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp],
     "nts_gather_rows_f32": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],

@@ -831,14 +831,14 @@ int check_heads(const float *alpha, uint32_t H, uint32_t Fh, const char *who) {
 }  // namespace
 
 int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
-                          const uint32_t *offsets, const uint32_t *indices, uint32_t rows, uint32_t H, uint32_t Fh,
-                          int accumulate, nts_stream_t stream) {
+                          const uint32_t *offsets, const uint32_t *indices, uint32_t rows, uint32_t edges, uint32_t H,
+                          uint32_t Fh, int accumulate, nts_stream_t stream) {
   if (int rc = check_heads(alpha, H, Fh, "nts_spmm_gather_heads: bad H / Fh / alpha")) return rc;
   if (rows == 0) return NTS_OK;
   if (!in || !out || !offsets || !indices) return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_heads: null pointer");
   nts::LaunchArgs a{in, out, alpha, offsets, indices, 0u, rows, H * Fh, nullptr, nullptr, accumulate, stream};
   a.heads = nts::HeadArgs{perm, H, Fh};
-  nts::launch_spmm(a);
+  if (int rc = nts::launch_spmm_balanced(a, edges)) return rc;
   NTS_LAUNCH_CHECK("nts_spmm_gather_heads");
   return NTS_OK;
 }

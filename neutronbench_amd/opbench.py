@@ -77,7 +77,8 @@ def main():
     out = torch.empty_like(h)
     heads_bytes = E * (4 * F + 4 + 4 * H) + V * 4 * F + 4 * (V + 1)
     report("nts_spmm_gather_heads", lambda: call("nts_spmm_gather_heads", ptr(h), ptr(out), ptr(y), 0, ptr(co32),
-                                                  ptr(ri32), V, H, Fh, 0, s), heads_bytes, whole + f", F'={F}, no plan")
+                                                  ptr(ri32), V, E, H, Fh, 0, s), heads_bytes,
+           whole + f", F'={F}, no plan: hub rows cut on the device")
     plan = SpmmPlan(co32, V, E, 512, indices=ri32, n_index=V, n_slabs=32)
     plan.reserve(F)
     report("nts_spmm_gather_heads_planned",

@@ -220,7 +220,7 @@ class GATAggregateOp:
         out = torch.empty(sg.v_size, x.shape[1], dtype=torch.float32, device=x.device)
         stream = torch.cuda.current_stream(x.device).cuda_stream
         call("nts_spmm_gather_heads", ptr(x), ptr(out), ptr(alpha), 0, ptr(sg.dev_c_o()), ptr(sg.dev_r_i()), sg.v_size,
-             self.H, Fh, 0, stream)
+             sg.e_size, self.H, Fh, 0, stream)
         self.x, self.alpha = x, alpha
         return out
 
@@ -232,7 +232,7 @@ class GATAggregateOp:
         stream = torch.cuda.current_stream(dev).cuda_stream
         gx = torch.empty(sg.src_size, g_out.shape[1], dtype=torch.float32, device=dev)
         call("nts_spmm_gather_heads", ptr(g_out), ptr(gx), ptr(self.alpha), ptr(sg.dev_csr_to_csc), ptr(sg.dev_r_o()),
-             ptr(sg.dev_c_i()), sg.src_size, self.H, Fh, 0, stream)
+             ptr(sg.dev_c_i()), sg.src_size, sg.e_size, self.H, Fh, 0, stream)
         self.galpha = torch.empty(sg.e_size, self.H, dtype=torch.float32, device=dev)
         call("nts_sddmm_heads", ptr(self.galpha), ptr(self.x), ptr(g_out), ptr(sg.dev_c_o()), ptr(sg.dev_r_i()),
              sg.v_size, self.H, Fh, stream)

@@ -9,7 +9,7 @@ import torch
 import oracle
 from gpu_util import dev, stream
 from neutronbench_amd.abi import call, ptr
-from util import check, brute_csr, random_block, rel_err
+from util import abs_term_scale, check, brute_csr, random_block, rel_err
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -171,13 +171,13 @@ def test_fused_gat_layer(device, H, Fh):
     call("nts_gat_attention_fwd", ptr(alpha), ptr(del_), ptr(der), ptr(dco), ptr(dri), Vd, H, 0.2, s)
     check(alpha.cpu().numpy(), alpha_ref, scale=1.0, floor=1e-6)
     out = torch.full((Vd, F), float("nan"), device=device)
-    call("nts_spmm_gather_heads", ptr(dhs), ptr(out), ptr(alpha), 0, ptr(dco), ptr(dri), Vd, H, Fh, 0, s)
+    call("nts_spmm_gather_heads", ptr(dhs), ptr(out), ptr(alpha), 0, ptr(dco), ptr(dri), Vd, ri.size, H, Fh, 0, s)
     a_exp = np.repeat(alpha_ref, Fh, axis=1)
     scale_out = oracle.aggregate_dst(np.abs(msg) * a_exp, co)
     check(out.cpu().numpy(), out_ref, scale=scale_out)
     # backward of the aggregation: gradient of the features over the CSR, gradient of alpha per edge
     ghs = torch.full((Vs, F), float("nan"), device=device)
-    call("nts_spmm_gather_heads", ptr(dgout), ptr(ghs), ptr(alpha), ptr(dperm), ptr(dro), ptr(dci), Vs, H, Fh, 0, s)
+    call("nts_spmm_gather_heads", ptr(dgout), ptr(ghs), ptr(alpha), ptr(dperm), ptr(dro), ptr(dci), Vs, ri.size, H, Fh, 0, s)
     scale_g = oracle.gather_to_src(np.abs(g_eout) * a_exp, co, ri, Vs)
     check(ghs.cpu().numpy(), ghs_ref, scale=scale_g)
     galpha = torch.full((E, H), float("nan"), device=device)
@@ -283,3 +283,36 @@ def test_long_rows_edge_sums(device, F):
     outs_ = dev(init, device)
     call("nts_gather_edge_to_src", ptr(outs_), ptr(dem), ptr(dro), ptr(dperm), Vs, F, 1, stream())
     check(outs_.cpu().numpy(), want_s + init, scale=sc_s + np.abs(init))
+
+
+def test_heads_aggregation_without_a_plan_cuts_hub_rows(device):
+    """nts_spmm_gather_heads at >= 65,536 edges with a 30,000-edge hub, over the CSC (perm NULL) and
+    over the CSR with alpha kept in CSC order (perm = csr_to_csc): per head it is the weighted
+    aggregation with that head's alpha column as the edge weight."""
+    H, Fh = 4, 8
+    F = H * Fh
+    Vd, Vs = 4000, 3000
+    co, ri = random_block(Vd, Vs, 12, seed=91, hub=30000, dup=True)
+    E = ri.size
+    assert E >= 1 << 16
+    rng = np.random.default_rng(92)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    g = rng.standard_normal((Vd, F)).astype(np.float32)
+    alpha = rng.random((E, H)).astype(np.float32)
+    ro, ci, perm = brute_csr(co, ri, Vs)
+    s = stream()
+    dco, dri, dro, dci, dperm = (dev(a, device) for a in (co, ri, ro, ci, perm))
+    dx, dg, dalpha = dev(x, device), dev(g, device), dev(alpha, device)
+    out = torch.full((Vd, F), float("nan"), device=device)
+    call("nts_spmm_gather_heads", ptr(dx), ptr(out), ptr(dalpha), 0, ptr(dco), ptr(dri), Vd, E, H, Fh, 0, s)
+    gx = torch.full((Vs, F), float("nan"), device=device)
+    call("nts_spmm_gather_heads", ptr(dg), ptr(gx), ptr(dalpha), ptr(dperm), ptr(dro), ptr(dci), Vs, E, H, Fh, 0, s)
+    torch.cuda.synchronize()
+    out, gx = out.cpu().numpy(), gx.cpu().numpy()
+    for h in range(H):
+        sl = slice(h * Fh, (h + 1) * Fh)
+        w = np.ascontiguousarray(alpha[:, h])
+        xs, gs = np.ascontiguousarray(x[:, sl]), np.ascontiguousarray(g[:, sl])
+        check(out[:, sl], oracle.spmm(xs, w, co, ri, Vd), abs_term_scale(xs, w, co, ri, Vd))
+        wb = np.ascontiguousarray(w[perm])
+        check(gx[:, sl], oracle.spmm(gs, wb, ro, ci, Vs), abs_term_scale(gs, wb, ro, ci, Vs))
