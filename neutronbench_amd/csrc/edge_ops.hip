@@ -85,6 +85,7 @@ __global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, con
 
 constexpr uint32_t kNoLimit = 0xFFFFFFFFu;
 constexpr uint32_t kLongRowEdges = 1024;    // edges of a row above which the block kernel takes over
+constexpr uint64_t kGiantRowEdges = 16384;  // edges of a row above which it is cut into pieces for several blocks
 constexpr uint32_t kLongRowValues = 32768;  // the same for softmax segments, in values (edges * heads)
 constexpr uint32_t kLongMinVertices = 16384;  // vertex count below which the extra launches are not worth it
 constexpr int kLongBlock = 1024;
@@ -144,62 +145,163 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__
   }
 }
 
-// list[0 .. *count) = rows r with (off[r+1] - off[r]) * width > limit (any order).
+// Giant rows: a row so long that one block working through it alone would outlast the rest of the
+// launch (a 300,000-edge hub next to 10^4 rows of a few thousand edges) is cut into pieces that
+// separate blocks reduce, and a last kernel combines the pieces in order.  The caller's argument
+// lists carry no edge count, so everything is sized by fixed capacities and decided on the device:
+// up to kGiantCap rows are listed (further ones simply stay with the one-block-per-row kernel), and
+// the piece length is chosen so that the listed rows need at most kPieceCap pieces.
+constexpr uint32_t kGiantCap = 1024;
+constexpr uint32_t kPieceCap = 8192;
+constexpr uint32_t kGiantMinPiece = 4096;  // edges
+
+// hdr: [0] giant rows seen (may exceed kGiantCap until the plan kernel clamps it), [1] pieces,
+//      [2] edges per piece, [4..5] edges of the listed giant rows (64-bit).
+// list[0 .. *count) = rows r with (off[r+1] - off[r]) * width > limit that are not listed as giant
+// (any order); giant_rows[0 .. min(hdr[0], kGiantCap)) = rows above giant_limit values.
 __global__ __launch_bounds__(256) void collect_long_rows_kernel(uint32_t *__restrict__ list,
                                                                 uint32_t *__restrict__ count,
+                                                                uint32_t *__restrict__ giant_rows,
+                                                                uint32_t *__restrict__ hdr,
                                                                 const uint32_t *__restrict__ off, uint32_t rows,
-                                                                uint32_t width, uint32_t limit) {
+                                                                uint32_t width, uint32_t limit,
+                                                                uint64_t giant_limit) {
   const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
   if (r >= rows) return;
-  if (static_cast<uint64_t>(off[r + 1] - off[r]) * width > limit) list[atomicAdd(count, 1u)] = r;
+  const uint32_t deg = off[r + 1] - off[r];
+  const uint64_t n = static_cast<uint64_t>(deg) * width;
+  if (n > giant_limit) {
+    const uint32_t gi = atomicAdd(&hdr[0], 1u);
+    if (gi < kGiantCap) {
+      giant_rows[gi] = r;
+      atomicAdd(reinterpret_cast<unsigned long long *>(hdr + 4), static_cast<unsigned long long>(deg));
+      return;
+    }
+  }
+  if (n > limit) list[atomicAdd(count, 1u)] = r;
 }
 
-// One 1024-thread block per listed row.  Columns are taken in tiles of `tile` (a power of two
-// <= 1024); thread t owns column t % tile of slice t / tile, a slice adds every (1024/tile)-th edge
-// of the row in ascending order, and slice 0 then adds the slices' sums in slice order.
+// One block: fixes the piece length, gives every listed giant row its first piece (a serial prefix
+// over at most kGiantCap rows) and writes the piece table (list position, row, first edge, end).
+__global__ __launch_bounds__(256) void giant_plan_kernel(uint32_t *__restrict__ hdr,
+                                                         const uint32_t *__restrict__ giant_rows,
+                                                         uint32_t *__restrict__ first, uint4 *__restrict__ pieces,
+                                                         const uint32_t *__restrict__ off) {
+  __shared__ uint32_t n_sh, len_sh;
+  if (threadIdx.x == 0) {
+    const uint32_t n = hdr[0] < kGiantCap ? hdr[0] : kGiantCap;
+    const unsigned long long edges = *reinterpret_cast<const unsigned long long *>(hdr + 4);
+    unsigned long long len = (edges + (kPieceCap - kGiantCap) - 1) / (kPieceCap - kGiantCap);
+    if (len < kGiantMinPiece) len = kGiantMinPiece;
+    uint32_t p = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+      first[i] = p;
+      const uint32_t r = giant_rows[i];
+      p += static_cast<uint32_t>((off[r + 1] - off[r] + len - 1) / len);
+    }
+    first[n] = p;
+    hdr[0] = n;
+    hdr[1] = p;
+    hdr[2] = static_cast<uint32_t>(len);
+    n_sh = n;
+    len_sh = static_cast<uint32_t>(len);
+  }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < n_sh; i += blockDim.x) {
+    const uint32_t r = giant_rows[i];
+    const uint32_t e1 = off[r + 1];
+    uint32_t p = first[i];
+    for (uint64_t k = off[r]; k < e1; k += len_sh, ++p)
+      pieces[p] = make_uint4(i, r, static_cast<uint32_t>(k), static_cast<uint32_t>(k + len_sh < e1 ? k + len_sh : e1));
+  }
+}
+
+// Sum of the edge rows [e0, e1) by one 1024-thread block, added into dst[0 .. F).  Columns are taken
+// in tiles of `tile` (a power of two <= 1024); thread t owns column t % tile of slice t / tile, a
+// slice adds every (1024/tile)-th edge of the range in ascending order (eight loads in flight), and
+// slice 0 then adds the slices' sums in slice order.
+__device__ __forceinline__ void block_sum_edge_rows(float *__restrict__ dst, const float *__restrict__ msg,
+                                                    const uint32_t *__restrict__ perm, uint32_t e0, uint32_t e1,
+                                                    uint32_t F, uint32_t tile, int accumulate, float *part) {
+  const uint32_t c = threadIdx.x & (tile - 1);
+  const uint32_t slice = threadIdx.x / tile;
+  const uint32_t n_slices = kLongBlock / tile;
+  for (uint32_t cb = 0; cb < F; cb += tile) {
+    const uint32_t col = cb + c;
+    float a = 0.f;
+    if (col < F) {
+      uint32_t k = e0 + slice;
+      for (; static_cast<uint64_t>(k) + 7ull * n_slices < e1; k += 8 * n_slices) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const uint32_t kk = k + u * n_slices;
+          const uint32_t e = perm ? perm[kk] : kk;
+          v[u] = msg[static_cast<size_t>(e) * F + col];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a += v[u];
+      }
+      for (; k < e1; k += n_slices) {
+        const uint32_t e = perm ? perm[k] : k;
+        a += msg[static_cast<size_t>(e) * F + col];
+      }
+    }
+    part[threadIdx.x] = a;
+    __syncthreads();
+    if (slice == 0 && col < F) {
+      float total = part[c];
+      for (uint32_t sidx = 1; sidx < n_slices; ++sidx) total += part[sidx * tile + c];
+      dst[col] = accumulate ? dst[col] + total : total;
+    }
+    __syncthreads();
+  }
+}
+
+// One 1024-thread block per listed long row.
 __global__ __launch_bounds__(kLongBlock) void gather_edge_to_row_long_kernel(
     float *__restrict__ out, const float *__restrict__ msg, const uint32_t *__restrict__ off,
     const uint32_t *__restrict__ perm, const uint32_t *__restrict__ list, const uint32_t *__restrict__ count,
     uint32_t F, uint32_t tile, int accumulate) {
   __shared__ float part[kLongBlock];
   const uint32_t n_rows = *count;
-  const uint32_t c = threadIdx.x & (tile - 1);
-  const uint32_t slice = threadIdx.x / tile;
-  const uint32_t n_slices = kLongBlock / tile;
   for (uint32_t i = blockIdx.x; i < n_rows; i += gridDim.x) {
     const uint32_t r = list[i];
-    const uint32_t e0 = off[r], e1 = off[r + 1];
-    for (uint32_t cb = 0; cb < F; cb += tile) {
-      const uint32_t col = cb + c;
+    block_sum_edge_rows(out + static_cast<size_t>(r) * F, msg, perm, off[r], off[r + 1], F, tile, accumulate, part);
+  }
+}
+
+// One block per piece of a giant row: partial[piece, :] = sum of the piece's edge rows.
+__global__ __launch_bounds__(kLongBlock) void giant_sum_pieces_kernel(float *__restrict__ partial,
+                                                                      const float *__restrict__ msg,
+                                                                      const uint32_t *__restrict__ perm,
+                                                                      const uint32_t *__restrict__ hdr,
+                                                                      const uint4 *__restrict__ pieces, uint32_t F,
+                                                                      uint32_t tile) {
+  __shared__ float part[kLongBlock];
+  const uint32_t n_pieces = hdr[1];
+  for (uint32_t p = blockIdx.x; p < n_pieces; p += gridDim.x) {
+    const uint4 pc = pieces[p];
+    block_sum_edge_rows(partial + static_cast<size_t>(p) * F, msg, perm, pc.z, pc.w, F, tile, 0, part);
+  }
+}
+
+// out[row, :] (+)= the row's piece sums, added in piece order.
+__global__ __launch_bounds__(256) void giant_sum_combine_kernel(float *__restrict__ out,
+                                                                const float *__restrict__ partial,
+                                                                const uint32_t *__restrict__ hdr,
+                                                                const uint32_t *__restrict__ giant_rows,
+                                                                const uint32_t *__restrict__ first, uint32_t F,
+                                                                int accumulate) {
+  const uint32_t n = hdr[0];
+  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
+    const uint32_t r = giant_rows[i];
+    const uint32_t p0 = first[i], p1 = first[i + 1];
+    for (uint32_t c = threadIdx.x; c < F; c += blockDim.x) {
       float a = 0.f;
-      if (col < F) {
-        // eight loads in flight, added in the slice's edge order
-        uint32_t k = e0 + slice;
-        for (; static_cast<uint64_t>(k) + 7ull * n_slices < e1; k += 8 * n_slices) {
-          float v[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const uint32_t kk = k + u * n_slices;
-            const uint32_t e = perm ? perm[kk] : kk;
-            v[u] = msg[static_cast<size_t>(e) * F + col];
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u) a += v[u];
-        }
-        for (; k < e1; k += n_slices) {
-          const uint32_t e = perm ? perm[k] : k;
-          a += msg[static_cast<size_t>(e) * F + col];
-        }
-      }
-      part[threadIdx.x] = a;
-      __syncthreads();
-      if (slice == 0 && col < F) {
-        float total = part[c];
-        for (uint32_t sidx = 1; sidx < n_slices; ++sidx) total += part[sidx * tile + c];
-        float *p = out + static_cast<size_t>(r) * F + col;
-        *p = accumulate ? *p + total : total;
-      }
-      __syncthreads();
+      for (uint32_t p = p0; p < p1; ++p) a += partial[static_cast<size_t>(p) * F + c];
+      float *dst = out + static_cast<size_t>(r) * F + c;
+      *dst = accumulate ? *dst + a : a;
     }
   }
 }
@@ -819,30 +921,47 @@ int edge_copy_impl(float *msg, const float *feat, const uint32_t *ri, const uint
   return NTS_OK;
 }
 
-// Scratch of the long-row path: list[rows] followed by the counter, in stream-ordered memory.
+// Scratch of the long-row path in one stream-ordered allocation: list[rows], its counter, and the
+// tables of the giant rows (header, row list, first-piece prefix, piece table).
 struct LongRows {
   uint32_t *list = nullptr;
   uint32_t *count = nullptr;
+  uint32_t *hdr = nullptr;
+  uint32_t *giant_rows = nullptr;
+  uint32_t *first = nullptr;
+  uint4 *pieces = nullptr;
 };
 
 // Collects the rows whose segment holds more than `limit` values (edges * width) when the vertex
-// count makes hubs likely; returns with lr.list == nullptr when the long path is not used.
+// count makes hubs likely, the ones above `giant_limit` values separately (with their piece table);
+// returns with lr.list == nullptr when the long path is not used.
 int collect_long_rows(LongRows &lr, const uint32_t *off, uint32_t rows, uint32_t width, uint32_t limit,
-                      hipStream_t stream) {
+                      uint64_t giant_limit, hipStream_t stream) {
   if (rows < kLongMinVertices) return NTS_OK;
-  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&lr.list), (static_cast<size_t>(rows) + 1) * sizeof(uint32_t),
+  const size_t list_bytes = (static_cast<size_t>(rows) + 1 + 7) / 8 * 8 * sizeof(uint32_t);  // list + counter, 32-byte multiple
+  const size_t small_bytes = (8 + kGiantCap + kGiantCap + 8) * sizeof(uint32_t);             // hdr, rows, first
+  unsigned char *buf = nullptr;
+  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&buf), list_bytes + small_bytes + kPieceCap * sizeof(uint4),
                              stream));
+  lr.list = reinterpret_cast<uint32_t *>(buf);
   lr.count = lr.list + rows;
+  lr.hdr = reinterpret_cast<uint32_t *>(buf + list_bytes);
+  lr.giant_rows = lr.hdr + 8;
+  lr.first = lr.giant_rows + kGiantCap;
+  lr.pieces = reinterpret_cast<uint4 *>(buf + list_bytes + small_bytes);
   if (int rc = nts_memset_zero(lr.count, sizeof(uint32_t), stream)) return rc;
-  hipLaunchKernelGGL(collect_long_rows_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, stream, lr.list, lr.count, off,
-                     rows, width, limit);
+  if (int rc = nts_memset_zero(lr.hdr, 8 * sizeof(uint32_t), stream)) return rc;
+  hipLaunchKernelGGL(collect_long_rows_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, stream, lr.list, lr.count,
+                     lr.giant_rows, lr.hdr, off, rows, width, limit, giant_limit);
   NTS_LAUNCH_CHECK("collect_long_rows_kernel");
+  hipLaunchKernelGGL(giant_plan_kernel, dim3(1), dim3(256), 0, stream, lr.hdr, lr.giant_rows, lr.first, lr.pieces, off);
+  NTS_LAUNCH_CHECK("giant_plan_kernel");
   return NTS_OK;
 }
 
 int release_long_rows(LongRows &lr, hipStream_t stream) {
   if (lr.list) NTS_HIP_TRY(hipFreeAsync(lr.list, stream));
-  lr.list = lr.count = nullptr;
+  lr = LongRows();
   return NTS_OK;
 }
 
@@ -872,7 +991,7 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
   if (rows == 0) return NTS_OK;
   if (!out || !msg || !off) return fail(NTS_ERR_INVALID, who);
   LongRows lr;
-  if (int rc = collect_long_rows(lr, off, rows, 1u, kLongRowEdges, stream)) return rc;
+  if (int rc = collect_long_rows(lr, off, rows, 1u, kLongRowEdges, kGiantRowEdges, stream)) return rc;
   const uint32_t limit = lr.list ? kLongRowEdges : kNoLimit;
   if (F % 4 == 0 && aligned_to(out, 16) && aligned_to(msg, 16))
     launch_gather_rows(reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, rows, F / 4,
@@ -886,6 +1005,17 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
     hipLaunchKernelGGL(gather_edge_to_row_long_kernel, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, msg, off,
                        perm, lr.list, lr.count, F, tile, accumulate);
     NTS_LAUNCH_CHECK(who);
+    // Giant rows: pieces by separate blocks into stream-ordered scratch, then the ordered combine.
+    float *partial = nullptr;
+    NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&partial), static_cast<size_t>(kPieceCap) * F * sizeof(float),
+                               stream));
+    hipLaunchKernelGGL(giant_sum_pieces_kernel, dim3(kLongGrid), dim3(kLongBlock), 0, stream, partial, msg, perm, lr.hdr,
+                       lr.pieces, F, tile);
+    hipLaunchKernelGGL(giant_sum_combine_kernel, dim3(kGiantCap / 4), dim3(256), 0, stream, out, partial, lr.hdr,
+                       lr.giant_rows, lr.first, F, accumulate);
+    const hipError_t launch_err = hipGetLastError();
+    NTS_HIP_TRY(hipFreeAsync(partial, stream));
+    if (launch_err != hipSuccess) return fail_hip(launch_err, who);
   }
   return release_long_rows(lr, stream);
 }
@@ -898,7 +1028,7 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   const bool pow2 = is_pow2(H) && H <= kWave;
   LongRows lr;
   if (pow2)
-    if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, stream)) return rc;
+    if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, ~0ull, stream)) return rc;
   const uint32_t max_values = lr.list ? kLongRowValues : kNoLimit;
   const bool use_short = pow2 && H <= static_cast<uint32_t>(kShortG);
   const uint32_t min_values = use_short ? kShortValues + 1 : 0u;

@@ -254,13 +254,18 @@ def test_long_segments_softmax_and_attention(device, H):
 
 @pytest.mark.parametrize("F", [1, 4, 33, 128, 1100])
 def test_long_rows_edge_sums(device, F):
-    """Edge -> vertex sums with hub rows beyond 1024 edges (block kernel: slices added in a fixed
-    order): within tolerance of the oracle's edge-order sum, bit-reproducible, accumulate honoured."""
+    """Edge -> vertex sums with hub rows: beyond 1,024 edges one block per row (slices added in a fixed
+    order), beyond 16,384 edges pieces by several blocks combined in order.  Within tolerance of the
+    oracle's edge-order sum, bit-reproducible, accumulate honoured."""
     print(f"case F={F}", flush=True)
     Vd, Vs = 17000, 20000
-    co, ri = random_block(Vd, Vs, 2, seed=400 + F, hub=5000, dup=True)
-    ri[int(co[1]):int(co[2])] = 7  # make source 7 a hub of the transposed structure as well
-    ri[:3000] = 7
+    rng0 = np.random.default_rng(400 + F)
+    deg = rng0.poisson(2, Vd).astype(np.int64)
+    deg[0], deg[1], deg[2] = 40000, 5000, 16385  # giant, long, just giant
+    co = np.concatenate([[0], np.cumsum(deg)]).astype(np.uint32)
+    ri = rng0.integers(0, Vs, int(co[-1])).astype(np.uint32)
+    ri[:20000] = 7         # source 7: a giant row of the transposed structure
+    ri[41000:44000] = 9    # source 9: a long one
     ro, ci, perm = brute_csr(co, ri, Vs)
     E = ri.size
     rng = np.random.default_rng(F)
