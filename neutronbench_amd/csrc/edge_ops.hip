@@ -85,6 +85,7 @@ __global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, con
 
 constexpr uint32_t kNoLimit = 0xFFFFFFFFu;
 constexpr uint32_t kLongRowEdges = 1024;    // edges of a row above which the block kernel takes over
+constexpr uint64_t kGiantValues = 131072;   // softmax segments above this many values are cut into pieces
 constexpr uint64_t kGiantRowEdges = 16384;  // edges of a row above which it is cut into pieces for several blocks
 constexpr uint32_t kLongRowValues = 32768;  // the same for softmax segments, in values (edges * heads)
 constexpr uint32_t kLongMinVertices = 16384;  // vertex count below which the extra launches are not worth it
@@ -780,6 +781,172 @@ __global__ __launch_bounds__(kLongBlock) void edge_softmax_bwd_long_kernel(
   }
 }
 
+// ---- giant segments of the softmax operators ----------------------------------------------------
+//
+// A piece of a giant destination is reduced by one block; per-head results of the pieces are
+// combined in piece order.  Forward uses the online form: a piece keeps (m_p, s_p = sum exp(x - m_p));
+// the destination's maximum is max_p m_p and its sum is sum_p s_p * exp(m_p - m).
+// stats[piece, 0..H) / [H..2H) and rowstat[giant row, 0..H) / [H..2H) hold the two values per head.
+
+template <bool FUSED>
+__global__ __launch_bounds__(kLongBlock) void giant_softmax_stats_kernel(
+    float *__restrict__ stats, float *__restrict__ y, const float *__restrict__ x, const float *__restrict__ el,
+    const float *__restrict__ er, const uint32_t *__restrict__ ri, const uint32_t *__restrict__ hdr,
+    const uint4 *__restrict__ pieces, uint32_t H, float slope) {
+  __shared__ float red[kLongBlock / kWave][kWave];
+  const uint32_t n_pieces = hdr[1];
+  const uint32_t h = threadIdx.x & (H - 1);
+  for (uint32_t p = blockIdx.x; p < n_pieces; p += gridDim.x) {
+    const uint4 pc = pieces[p];
+    const uint32_t d = pc.y, e0 = pc.z;
+    const size_t base = static_cast<size_t>(e0) * H;
+    const uint64_t n = static_cast<uint64_t>(pc.w - e0) * H;
+    float *ys = y + base;
+    const float *xs = FUSED ? nullptr : x + base;
+    float erv = 0.f;
+    if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+    float mx = -INFINITY;
+    strided_pass<8>(threadIdx.x, n, kLongBlock,
+                    [&](uint64_t j) -> float {
+                      if (!FUSED) return xs[j];
+                      const uint32_t src = ri[e0 + j / H];
+                      return leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
+                    },
+                    [&](uint64_t j, float sc) {
+                      if (FUSED) ys[j] = sc;
+                      mx = fmaxf(mx, sc);
+                    });
+    mx = block_head_reduce<0>(mx, H, red);
+    float sum = 0.f;
+    strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
+                    [&](uint64_t, float sc) { sum += expf(sc - mx); });
+    sum = block_head_reduce<1>(sum, H, red);
+    if (threadIdx.x < H) {
+      stats[static_cast<size_t>(p) * 2 * H + threadIdx.x] = mx;
+      stats[static_cast<size_t>(p) * 2 * H + H + threadIdx.x] = sum;
+    }
+  }
+}
+
+// MODE 0: online-softmax combine of (m_p, s_p).  MODE 1: plain sum of stats[piece, 0..H) in piece
+// order; the result goes to rowstat[giant row, 0..H) or, when `to_rows` is set, to to_rows[row, 0..H)
+// (the per-destination gradient sum of the fused backward).
+template <int MODE>
+__global__ __launch_bounds__(64) void giant_softmax_combine_kernel(float *__restrict__ rowstat,
+                                                                   float *__restrict__ to_rows,
+                                                                   const float *__restrict__ stats,
+                                                                   const uint32_t *__restrict__ hdr,
+                                                                   const uint32_t *__restrict__ giant_rows,
+                                                                   const uint32_t *__restrict__ first, uint32_t H) {
+  const uint32_t n = hdr[0];
+  const uint32_t h = threadIdx.x;
+  if (h >= H) return;
+  const uint32_t width = MODE == 0 ? 2 * H : H;
+  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
+    const uint32_t p0 = first[i], p1 = first[i + 1];
+    if (MODE == 0) {
+      float m = -INFINITY;
+      for (uint32_t p = p0; p < p1; ++p) m = fmaxf(m, stats[static_cast<size_t>(p) * width + h]);
+      float sum = 0.f;
+      for (uint32_t p = p0; p < p1; ++p)
+        sum += stats[static_cast<size_t>(p) * width + H + h] * expf(stats[static_cast<size_t>(p) * width + h] - m);
+      rowstat[static_cast<size_t>(i) * 2 * H + h] = m;
+      rowstat[static_cast<size_t>(i) * 2 * H + H + h] = sum;
+    } else {
+      float sum = 0.f;
+      for (uint32_t p = p0; p < p1; ++p) sum += stats[static_cast<size_t>(p) * width + h];
+      if (to_rows) to_rows[static_cast<size_t>(giant_rows[i]) * H + h] = sum;
+      else rowstat[static_cast<size_t>(i) * 2 * H + h] = sum;
+    }
+  }
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(kLongBlock) void giant_softmax_apply_kernel(float *__restrict__ y,
+                                                                         const float *__restrict__ x,
+                                                                         const float *__restrict__ rowstat,
+                                                                         const uint32_t *__restrict__ hdr,
+                                                                         const uint4 *__restrict__ pieces,
+                                                                         uint32_t H) {
+  const uint32_t n_pieces = hdr[1];
+  const uint32_t h = threadIdx.x & (H - 1);
+  for (uint32_t p = blockIdx.x; p < n_pieces; p += gridDim.x) {
+    const uint4 pc = pieces[p];
+    const size_t base = static_cast<size_t>(pc.z) * H;
+    const uint64_t n = static_cast<uint64_t>(pc.w - pc.z) * H;
+    const float mx = rowstat[static_cast<size_t>(pc.x) * 2 * H + h];
+    const float sum = rowstat[static_cast<size_t>(pc.x) * 2 * H + H + h];
+    float *ys = y + base;
+    const float *xs = FUSED ? ys : x + base;  // the fused forward left the raw score in y
+    strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return xs[j]; },
+                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) / sum; });
+  }
+}
+
+// Backward, first stage: stats[piece, h] = sum over the piece of gy * y.
+__global__ __launch_bounds__(kLongBlock) void giant_softmax_dot_kernel(float *__restrict__ stats,
+                                                                       const float *__restrict__ gy,
+                                                                       const float *__restrict__ y,
+                                                                       const uint32_t *__restrict__ hdr,
+                                                                       const uint4 *__restrict__ pieces, uint32_t H) {
+  __shared__ float red[kLongBlock / kWave][kWave];
+  const uint32_t n_pieces = hdr[1];
+  for (uint32_t p = blockIdx.x; p < n_pieces; p += gridDim.x) {
+    const uint4 pc = pieces[p];
+    const size_t base = static_cast<size_t>(pc.z) * H;
+    const uint64_t n = static_cast<uint64_t>(pc.w - pc.z) * H;
+    const float *gys = gy + base;
+    const float *ys = y + base;
+    float dot = 0.f;
+    strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float2 { return make_float2(gys[j], ys[j]); },
+                    [&](uint64_t, float2 v) { dot += v.x * v.y; });
+    dot = block_head_reduce<1>(dot, H, red);
+    if (threadIdx.x < H) stats[static_cast<size_t>(p) * H + threadIdx.x] = dot;
+  }
+}
+
+// Backward, last stage: gx over the piece; with FUSED also stats[piece, h] = sum of the piece's gx.
+template <bool FUSED>
+__global__ __launch_bounds__(kLongBlock) void giant_softmax_bwd_apply_kernel(
+    float *__restrict__ gx, float *__restrict__ stats, const float *__restrict__ gy, const float *__restrict__ y,
+    const float *__restrict__ el, const float *__restrict__ er, const uint32_t *__restrict__ ri,
+    const float *__restrict__ rowstat, const uint32_t *__restrict__ hdr, const uint4 *__restrict__ pieces, uint32_t H,
+    float slope) {
+  __shared__ float red[kLongBlock / kWave][kWave];
+  const uint32_t n_pieces = hdr[1];
+  const uint32_t h = threadIdx.x & (H - 1);
+  for (uint32_t p = blockIdx.x; p < n_pieces; p += gridDim.x) {
+    const uint4 pc = pieces[p];
+    const uint32_t d = pc.y, e0 = pc.z;
+    const size_t base = static_cast<size_t>(e0) * H;
+    const uint64_t n = static_cast<uint64_t>(pc.w - e0) * H;
+    const float *gys = gy + base;
+    const float *ys = y + base;
+    float *gxs = gx + base;
+    const float dot = rowstat[static_cast<size_t>(pc.x) * 2 * H + h];
+    float erv = 0.f, gsum = 0.f;
+    if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
+    strided_pass<8>(threadIdx.x, n, kLongBlock,
+                    [&](uint64_t j) -> float4 {
+                      float pre = 1.f;
+                      if (FUSED) pre = el[static_cast<size_t>(ri[e0 + j / H]) * H + h] + erv;
+                      return make_float4(gys[j], ys[j], pre, 0.f);
+                    },
+                    [&](uint64_t j, float4 v) {
+                      float g = v.y * (v.x - dot);
+                      if (FUSED) {
+                        g *= v.z > 0.f ? 1.f : slope;
+                        gsum += g;
+                      }
+                      gxs[j] = g;
+                    });
+    if (FUSED) {
+      gsum = block_head_reduce<1>(gsum, H, red);
+      if (threadIdx.x < H) stats[static_cast<size_t>(p) * H + threadIdx.x] = gsum;
+    }
+  }
+}
+
 // ---- gradient of the attention-weighted aggregation with respect to alpha ----------------------
 //
 // galpha[e,h] = < in[ri[e], h-th slice], gout[d, h-th slice] > for e in CSC(d).  Edge-parallel like
@@ -1028,7 +1195,7 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   const bool pow2 = is_pow2(H) && H <= kWave;
   LongRows lr;
   if (pow2)
-    if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, ~0ull, stream)) return rc;
+    if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, kGiantValues, stream)) return rc;
   const uint32_t max_values = lr.list ? kLongRowValues : kNoLimit;
   const bool use_short = pow2 && H <= static_cast<uint32_t>(kShortG);
   const uint32_t min_values = use_short ? kShortValues + 1 : 0u;
@@ -1081,6 +1248,46 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
                            x_or_gy, y, el, er, co, ri, lr.list, lr.count, H, slope);
       NTS_LAUNCH_CHECK(who);
     }
+  }
+  if (lr.list) {
+    // Giant segments: per-piece statistics, ordered combine, apply (see the kernels above).
+    float *stats = nullptr;
+    const size_t stats_floats = static_cast<size_t>(kPieceCap) * 2 * H, row_floats = static_cast<size_t>(kGiantCap) * 2 * H;
+    NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&stats), (stats_floats + row_floats) * sizeof(float), stream));
+    float *rowstat = stats + stats_floats;
+    const dim3 pgrid(kLongGrid), pblock(kLongBlock), cgrid(kGiantCap / 4), cblock(64);
+    if (!backward) {
+      if (fused)
+        hipLaunchKernelGGL(giant_softmax_stats_kernel<true>, pgrid, pblock, 0, stream, stats, out, x_or_gy, el, er, ri,
+                           lr.hdr, lr.pieces, H, slope);
+      else
+        hipLaunchKernelGGL(giant_softmax_stats_kernel<false>, pgrid, pblock, 0, stream, stats, out, x_or_gy, el, er, ri,
+                           lr.hdr, lr.pieces, H, slope);
+      hipLaunchKernelGGL(giant_softmax_combine_kernel<0>, cgrid, cblock, 0, stream, rowstat,
+                         static_cast<float *>(nullptr), stats, lr.hdr, lr.giant_rows, lr.first, H);
+      if (fused)
+        hipLaunchKernelGGL(giant_softmax_apply_kernel<true>, pgrid, pblock, 0, stream, out, x_or_gy, rowstat, lr.hdr,
+                           lr.pieces, H);
+      else
+        hipLaunchKernelGGL(giant_softmax_apply_kernel<false>, pgrid, pblock, 0, stream, out, x_or_gy, rowstat, lr.hdr,
+                           lr.pieces, H);
+    } else {
+      hipLaunchKernelGGL(giant_softmax_dot_kernel, pgrid, pblock, 0, stream, stats, x_or_gy, y, lr.hdr, lr.pieces, H);
+      hipLaunchKernelGGL(giant_softmax_combine_kernel<1>, cgrid, cblock, 0, stream, rowstat,
+                         static_cast<float *>(nullptr), stats, lr.hdr, lr.giant_rows, lr.first, H);
+      if (fused) {
+        hipLaunchKernelGGL(giant_softmax_bwd_apply_kernel<true>, pgrid, pblock, 0, stream, out, stats, x_or_gy, y, el, er,
+                           ri, rowstat, lr.hdr, lr.pieces, H, slope);
+        hipLaunchKernelGGL(giant_softmax_combine_kernel<1>, cgrid, cblock, 0, stream, rowstat, ger, stats, lr.hdr,
+                           lr.giant_rows, lr.first, H);
+      } else {
+        hipLaunchKernelGGL(giant_softmax_bwd_apply_kernel<false>, pgrid, pblock, 0, stream, out, stats, x_or_gy, y, el, er,
+                           ri, rowstat, lr.hdr, lr.pieces, H, slope);
+      }
+    }
+    const hipError_t launch_err = hipGetLastError();
+    NTS_HIP_TRY(hipFreeAsync(stats, stream));
+    if (launch_err != hipSuccess) return fail_hip(launch_err, who);
   }
   return release_long_rows(lr, stream);
 }
