@@ -17,9 +17,12 @@
  *   operator classes ForwardCPUfuseOp (bit for bit, forward and backward), SingleCPUSrcDstScatterOp,
  *   SingleCPUDstAggregateOp (bit for bit) and SingleEdgeSoftMax (to rounding: it calls libtorch's
  *   softmax) run on graphs loaded by the reference's loader and partitioner.
- *   csr_from_csc, postprocess, layer weights, init_co, gathers, cache split: the reference code for
- *   these (core/coocsc.hpp, core/ntsSampler.hpp, core/ntsMiniBatchGraphOp.hpp) needs METIS headers
- *   the tree does not carry and cannot be compiled; pinned by brute force and exact fixtures.
+ *   postprocess, csr_from_csc, layer weights: additionally against the reference's sampCSC itself
+ *   (core/coocsc.hpp compiles against the HIP veneer; postprocessing, generate_csr_from_csc,
+ *   update_degree, compute_weight_forward / backward run on sampled lists made by the tests), bit for bit.
+ *   init_co, gathers, cache split: the reference code for these (core/ntsSampler.hpp,
+ *   core/ntsMiniBatchGraphOp.hpp) needs METIS headers the tree does not carry and cannot be
+ *   compiled; pinned by brute force and exact fixtures.
  *   dataset readers: pinned by exact rational rounding of every token and by the file definitions.
  */
 #define _GNU_SOURCE /* getline */

@@ -18,6 +18,12 @@
 //   agg-cpu runs ForwardCPUfuseOp only; <F> may be a comma-separated list, and for every width the
 //   input is <prefix>.x<F>.  Three timed repetitions per width, best forward and backward time
 //   printed: the CPU baseline of the aggregation benchmark.
+//   samp (GPU build only, but makes no device call): <H> is a number of sampled layers; for layer k
+//   the files <prefix>.l<k>.dst [Vd], .co [Vd+1], .ri [E] (uint32; ri = GLOBAL source ids of the
+//   sampled edges) are run through the reference's sampCSC (core/coocsc.hpp): postprocessing,
+//   generate_csr_from_csc, update_degree, compute_weight_forward / backward, and the resulting
+//   source, row_indices (local), row_offset, column_indices and both weight arrays are written as
+//   <prefix>.l<k>.<name>.
 //   inputs:  <prefix>.x  [V, F]   vertex features, also used as the vertex-side gradient
 //            <prefix>.m  [E, H]   edge scores;  <prefix>.gm [E, H] their gradient
 //            <prefix>.e  [E, F]   edge messages;  <prefix>.g2 [E, 2F] gradient of the (src | dst) scatter
@@ -28,6 +34,7 @@
 #include "core/ntsCPUFusedGraphOp.hpp"
 #include "core/ntsSingleCPUGraphOp.hpp"
 #if CUDA_ENABLE
+#include "core/coocsc.hpp"
 #include "core/ntsDistGPUGraphOp.hpp"
 #include "core/ntsSingleGPUFusedGraphOp.hpp"
 #endif
@@ -69,6 +76,53 @@ static void write_tensor(const std::string &name, const NtsVar &t_in) {
   write_raw(name, t.data_ptr<float>(), static_cast<size_t>(t.numel()) * sizeof(float));
 }
 
+static std::vector<VertexId> read_ids(const std::string &name) {
+  const std::string path = g_prefix + "." + name;
+  FILE *f = fopen(path.c_str(), "rb");
+  if (!f) {
+    fprintf(stderr, "cannot open %s\n", path.c_str());
+    exit(2);
+  }
+  fseek(f, 0, SEEK_END);
+  const size_t n = static_cast<size_t>(ftell(f)) / sizeof(VertexId);
+  fseek(f, 0, SEEK_SET);
+  std::vector<VertexId> v(n);
+  if (n && fread(v.data(), sizeof(VertexId), n, f) != n) exit(2);
+  fclose(f);
+  return v;
+}
+
+#if CUDA_ENABLE
+// The reference's per-layer construction steps of Sampler::sample_one after the neighbour pick
+// (core/ntsSampler.hpp:1006-1106), on sampled lists handed in by the caller.
+static void run_sampled_layers(Graph<Empty> *graph, int layers) {
+  VertexId *node_idx = new VertexId[graph->vertices];
+  for (int k = 0; k < layers; ++k) {
+    const std::string tag = "l" + std::to_string(k) + ".";
+    std::vector<VertexId> dst = read_ids(tag + "dst"), co = read_ids(tag + "co"), ri = read_ids(tag + "ri");
+    // Never destroyed: ~sampCSC frees device pointers its constructors leave uninitialised.
+    sampCSC *sg = new sampCSC(static_cast<VertexId>(dst.size()), static_cast<VertexId>(ri.size()));
+    sg->dst() = dst;
+    sg->c_o() = co;
+    sg->r_i() = ri;
+    Bitmap bits(graph->vertices);
+    for (VertexId g : ri) bits.set_bit(g);
+    sg->postprocessing(&bits, node_idx);
+    sg->generate_csr_from_csc();
+    sg->update_degree(graph);
+    sg->compute_weight_forward(graph);
+    sg->compute_weight_backward(graph);
+    write_raw(tag + "source", sg->src().data(), sg->src().size() * sizeof(VertexId));
+    write_raw(tag + "row_indices", sg->r_i().data(), sg->r_i().size() * sizeof(VertexId));
+    write_raw(tag + "row_offset", sg->r_o().data(), sg->r_o().size() * sizeof(VertexId));
+    write_raw(tag + "column_indices", sg->c_i().data(), sg->c_i().size() * sizeof(VertexId));
+    write_raw(tag + "edge_weight_forward", sg->edge_weight_forward.data(), sg->edge_weight_forward.size() * sizeof(ValueType));
+    write_raw(tag + "edge_weight_backward", sg->edge_weight_backward.data(), sg->edge_weight_backward.size() * sizeof(ValueType));
+  }
+  printf("reference sampCSC construction done for %d layers\n", layers);
+}
+#endif
+
 static double now() {
   return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
@@ -102,6 +156,13 @@ int main(int argc, char **argv) {
   graph->replication_threshold = 0;
   graph->load_directed(edge_file, vertices);
   graph->generate_backward_structure();
+
+#if CUDA_ENABLE
+  if (mode == "samp") {
+    run_sampled_layers(graph, H);
+    return 0;
+  }
+#endif
 
   VertexSubset *active = graph->alloc_vertex_subset();
   active->fill();

@@ -55,3 +55,26 @@ def run(kind, mode, inputs, tmp_path, timeout=600):
         if os.path.exists(path):
             out[name] = np.fromfile(path, dtype=dtype).reshape(shape)
     return out
+
+
+def run_sampled_layers(graph_src, graph_dst, V, layers, tmp_path, timeout=600):
+    """layers: list of dicts with dst [Vd], co [Vd+1], ri [E] (global source ids), uint32.  Runs the
+    reference's sampCSC construction (the GPU-variant program; this mode makes no device call) and
+    returns, per layer, source / row_indices / row_offset / column_indices / both weight arrays."""
+    prefix = os.path.join(str(tmp_path), "samp")
+    np.stack([graph_src, graph_dst], 1).astype(np.uint32).tofile(prefix + ".edge")
+    for k, layer in enumerate(layers):
+        for name in ("dst", "co", "ri"):
+            np.ascontiguousarray(layer[name], dtype=np.uint32).tofile(f"{prefix}.l{k}.{name}")
+    r = subprocess.run([PROGRAMS["gpu"], prefix + ".edge", str(V), "4", str(len(layers)), prefix, "samp"],
+                       capture_output=True, text=True, timeout=timeout)
+    assert r.returncode == 0, f"reference program failed ({r.returncode}):\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}"
+    out = []
+    for k in range(len(layers)):
+        d = {}
+        for name, dtype in (("source", np.uint32), ("row_indices", np.uint32), ("row_offset", np.uint32),
+                            ("column_indices", np.uint32), ("edge_weight_forward", np.float32),
+                            ("edge_weight_backward", np.float32)):
+            d[name] = np.fromfile(f"{prefix}.l{k}.{name}", dtype=dtype)
+        out.append(d)
+    return out

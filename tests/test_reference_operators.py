@@ -137,3 +137,41 @@ def test_reference_gpu_operator_classes_over_the_library_match_its_cpu_operators
     check(ref["gpu_softmax1_bwd"], exact(y_gpu).astype(np.float32), scale)
     small = (deg <= 1024)[seg]
     check(ref["gpu_softmax1_bwd"][small], ref["cpu_softmax1_bwd"][small], scale[small])
+
+
+@pytest.mark.skipif(not refops.available("gpu"), reason="reference-built program with sampCSC not present")
+@pytest.mark.parametrize("V,E,batch,fanouts,seed", [(500, 6000, 40, [3, 5], 1), (20000, 300000, 512, [10, 25], 2),
+                                                    (3000, 90000, 200, [5, 10, 15], 3)])
+def test_oracle_matches_the_reference_sampled_layer_construction(tmp_path, V, E, batch, fanouts, seed):
+    """sampCSC::postprocessing, generate_csr_from_csc, update_degree and compute_weight_forward /
+    backward of the reference itself (core/coocsc.hpp:136-450), run on sampled lists made here, against
+    the oracle's restatements: every array bit for bit."""
+    rng = np.random.default_rng(seed)
+    gsrc = rng.integers(0, V, E).astype(np.uint32)
+    gdst = np.minimum((rng.random(E) ** 2 * V).astype(np.uint32), V - 1)
+    order = np.argsort(gdst, kind="stable")
+    csc_src = gsrc[order]
+    gco = np.concatenate([[0], np.cumsum(np.bincount(gdst, minlength=V))]).astype(np.int64)
+    layers = []
+    dst = rng.choice(V, batch, replace=False).astype(np.uint32)
+    for fan in fanouts:
+        co, picks = [0], []
+        for d in dst:
+            nb = csc_src[gco[d]:gco[d + 1]]
+            take = nb if nb.size <= fan else nb[np.sort(rng.choice(nb.size, fan, replace=False))]
+            picks.append(take)
+            co.append(co[-1] + take.size)
+        ri = np.concatenate(picks).astype(np.uint32) if picks else np.zeros(0, np.uint32)
+        layers.append(dict(dst=dst, co=np.array(co, dtype=np.uint32), ri=ri))
+        dst = np.unique(ri)  # the next hop's destinations are this hop's sources (ascending ids)
+    ref = refops.run_sampled_layers(gsrc, gdst, V, layers, tmp_path)
+    for layer, want in zip(layers, ref):
+        local, source, n_src = oracle.postprocess(layer["ri"], V)
+        assert n_src == want["source"].size
+        assert np.array_equal(source, want["source"]) and np.array_equal(local, want["row_indices"])
+        ro, ci = oracle.csr_from_csc(layer["co"], local, n_src)
+        assert np.array_equal(ro, want["row_offset"]) and np.array_equal(ci, want["column_indices"])
+        outd, ind = np.ones(V, np.uint32), np.ones(V, np.uint32)
+        ewf, ewb = oracle.layer_weights(layer["co"], local, ro, ci, source, layer["dst"], outd, ind)
+        assert ewf.tobytes() == want["edge_weight_forward"].tobytes()
+        assert ewb.tobytes() == want["edge_weight_backward"].tobytes()
