@@ -23,7 +23,8 @@
  *   init_co, gathers, cache split: the reference code for these (core/ntsSampler.hpp,
  *   core/ntsMiniBatchGraphOp.hpp) needs METIS headers the tree does not carry and cannot be
  *   compiled; pinned by brute force and exact fixtures.
- *   dataset readers: pinned by exact rational rounding of every token and by the file definitions.
+ *   dataset readers: pinned by exact rational rounding of every token and by the file definitions, and
+ *   against the reference's GNNDatum::readFeature_Label_Mask itself (GPU test: its tables are pinned memory).
  */
 #define _GNU_SOURCE /* getline */
 #include <math.h>

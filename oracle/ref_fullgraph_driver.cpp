@@ -24,6 +24,10 @@
 //   generate_csr_from_csc, update_degree, compute_weight_forward / backward, and the resulting
 //   source, row_indices (local), row_offset, column_indices and both weight arrays are written as
 //   <prefix>.l<k>.<name>.
+//   data (GPU build only; allocates the feature table in pinned memory, so it needs the device):
+//   GNNDatum::readFeature_Label_Mask (core/ntsDataloador.hpp:264-395) on <prefix>.feat / .label /
+//   .mask with F features and <H> classes; writes local_feature, local_label, local_mask,
+//   global_label, global_mask as <prefix>.<name>.
 //   inputs:  <prefix>.x  [V, F]   vertex features, also used as the vertex-side gradient
 //            <prefix>.m  [E, H]   edge scores;  <prefix>.gm [E, H] their gradient
 //            <prefix>.e  [E, F]   edge messages;  <prefix>.g2 [E, 2F] gradient of the (src | dst) scatter
@@ -35,6 +39,7 @@
 #include "core/ntsSingleCPUGraphOp.hpp"
 #if CUDA_ENABLE
 #include "core/coocsc.hpp"
+#include "core/ntsDataloador.hpp"
 #include "core/ntsDistGPUGraphOp.hpp"
 #include "core/ntsSingleGPUFusedGraphOp.hpp"
 #endif
@@ -160,6 +165,21 @@ int main(int argc, char **argv) {
 #if CUDA_ENABLE
   if (mode == "samp") {
     run_sampled_layers(graph, H);
+    return 0;
+  }
+  if (mode == "data") {
+    graph->config->classes = H;
+    graph->config->mode = "zerocopy";
+    graph->init_gnnctx(graph->config->layer_string);
+    GNNDatum *datum = new GNNDatum(graph->gnnctx, graph);
+    datum->readFeature_Label_Mask(g_prefix + ".feat", g_prefix + ".label", g_prefix + ".mask");
+    const size_t V = vertices, width = H > 1 ? H : 1;
+    write_raw("local_feature", datum->local_feature, V * F * sizeof(ValueType));
+    write_raw("local_label", datum->local_label, V * width * sizeof(long));
+    write_raw("global_label", datum->global_label, V * width * sizeof(long));
+    write_raw("local_mask", datum->local_mask, V * sizeof(int));
+    write_raw("global_mask", datum->global_mask, V * sizeof(int));
+    printf("reference GNNDatum::readFeature_Label_Mask done\n");
     return 0;
   }
 #endif

@@ -78,3 +78,17 @@ def run_sampled_layers(graph_src, graph_dst, V, layers, tmp_path, timeout=600):
             d[name] = np.fromfile(f"{prefix}.l{k}.{name}", dtype=dtype)
         out.append(d)
     return out
+
+
+def run_data_loader(V, F, classes, files_prefix, timeout=300):
+    """Runs the reference's GNNDatum::readFeature_Label_Mask (GPU-variant program: its feature table
+    lives in pinned memory) on <files_prefix>.feat / .label / .mask; needs <files_prefix>.edge."""
+    r = subprocess.run([PROGRAMS["gpu"], files_prefix + ".edge", str(V), str(F), str(classes), files_prefix, "data"],
+                       capture_output=True, text=True, timeout=timeout)
+    assert r.returncode == 0, f"reference program failed ({r.returncode}):\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}"
+    width = classes if classes > 1 else 1
+    return dict(local_feature=np.fromfile(files_prefix + ".local_feature", dtype=np.float32).reshape(V, F),
+                local_label=np.fromfile(files_prefix + ".local_label", dtype=np.int64).reshape(V * width),
+                global_label=np.fromfile(files_prefix + ".global_label", dtype=np.int64).reshape(V * width),
+                local_mask=np.fromfile(files_prefix + ".local_mask", dtype=np.int32),
+                global_mask=np.fromfile(files_prefix + ".global_mask", dtype=np.int32))

@@ -147,3 +147,45 @@ def test_chunk_from_edges_full_size_properties(device):
     ind = (co[1:] - co[:-1]).cpu().numpy()
     want = np.array([oracle.norm_degree(int(outd[s]), int(ind[d])) for s, d in zip(ri, d_of)], dtype=np.float32)
     assert chunk.edge_weight_forward_gpu[idx].cpu().numpy().tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("classes,fmt,sep,shuffled", [(1, "%.4f", " ", False), (1, "%.9g", "\t", True),
+                                                      (12, "%.6e", " ", True)])
+def test_readers_match_the_reference_data_loader(device, tmp_path, classes, fmt, sep, shuffled):
+    """The reference's own GNNDatum::readFeature_Label_Mask (built from its tree, run as a program)
+    on the same files: the library's reader and the oracle's restatement give the same five tables
+    bit for bit."""
+    import refops
+
+    if not refops.available("gpu"):
+        pytest.skip("reference-built program not present")
+    rng = np.random.default_rng(31 + classes)
+    V, F = 1500, 23
+    prefix = str(tmp_path / "d")
+    np.stack([rng.integers(0, V, 4000), rng.integers(0, V, 4000)], 1).astype(np.uint32).tofile(prefix + ".edge")
+    ids = rng.permutation(V) if shuffled else np.arange(V)
+    x = (rng.standard_normal((V, F)) * 10.0 ** rng.integers(-3, 4, (V, 1))).astype(np.float32)
+    with open(prefix + ".feat", "w") as f:
+        for i in ids:
+            f.write(str(int(i)) + sep + sep.join(fmt % v for v in x[i]) + "\n")
+    with open(prefix + ".label", "w") as f:
+        for i in ids:
+            if classes > 1:
+                idx = rng.choice(classes, rng.integers(0, 4), replace=False)
+                f.write(f"{i} {len(idx)} " + " ".join(map(str, idx)) + "\n")
+            else:
+                f.write(f"{i} {rng.integers(0, 40)}\n")
+    words = rng.choice(["train", "val", "eval", "test", "other"], V)
+    with open(prefix + ".mask", "w") as f:
+        for i in ids:
+            f.write(f"{i} {words[i]}\n")
+    ref = refops.run_data_loader(V, F, classes, prefix)
+    o = oracle.read_feature_label_mask(prefix + ".feat", prefix + ".label", prefix + ".mask", V, F, classes)
+    lib = dataset.GNNDatum(V, F, classes, pinned=True)
+    lib.readFeature_Label_Mask(prefix + ".feat", prefix + ".label", prefix + ".mask")
+    assert np.array_equal(ref["local_feature"].view(np.uint32), o["local_feature"].view(np.uint32))
+    assert np.array_equal(ref["local_feature"].view(np.uint32), lib.local_feature.view(np.uint32))
+    for k in ("local_label", "global_label", "local_mask", "global_mask"):
+        assert np.array_equal(ref[k], o[k]), k
+        assert np.array_equal(ref[k], getattr(lib, k)), k
+    lib.close()
