@@ -18,6 +18,9 @@
 //   agg-cpu runs ForwardCPUfuseOp only; <F> may be a comma-separated list, and for every width the
 //   input is <prefix>.x<F>.  Three timed repetitions per width, best forward and backward time
 //   printed: the CPU baseline of the aggregation benchmark.
+//   agg-gpu (GPU build only): ForwardSingleGPUfuseOp only, on the reference's GPU chunk
+//   (GenerateAll(GPU_T) + CopyGraphToDevice), same width list and inputs as agg-cpu; prints the best
+//   wall time of forward and backward (each call ends with the operator's own stream synchronisation).
 //   samp (GPU build only, but makes no device call): <H> is a number of sampled layers; for layer k
 //   the files <prefix>.l<k>.dst [Vd], .co [Vd+1], .ri [E] (uint32; ri = GLOBAL source ids of the
 //   sampled edges) are run through the reference's sampCSC (core/coocsc.hpp): postprocessing,
@@ -163,6 +166,39 @@ int main(int argc, char **argv) {
   graph->generate_backward_structure();
 
 #if CUDA_ENABLE
+  if (mode == "agg-gpu") {
+    VertexSubset *all = graph->alloc_vertex_subset();
+    all->fill();
+    graph->init_gnnctx(graph->config->layer_string);
+    graph->init_rtminfo();
+    graph->rtminfo->with_weight = true;
+    graph->rtminfo->with_cuda = true;
+    graph->rtminfo->copy_data = false;
+    graph->rtminfo->process_local = false;
+    graph->rtminfo->reduce_comm = false;
+    graph->rtminfo->process_overlap = false;
+    graph->rtminfo->lock_free = false;
+    PartitionedGraph *pgg = new PartitionedGraph(graph, all);
+    pgg->GenerateAll([&](VertexId src, VertexId dst) { return nts::op::nts_norm_degree(graph, src, dst); }, GPU_T);
+    graph->init_message_buffer();
+    nts::op::ForwardSingleGPUfuseOp op(pgg, all);
+    for (int width : widths) {
+      NtsVar X = read_matrix("x" + std::to_string(width), vertices, width).cuda();
+      double best_f = 1e30, best_b = 1e30;
+      for (int rep = 0; rep < 5; ++rep) {
+        double t0 = now();
+        NtsVar Y = op.forward(X);
+        double t1 = now();
+        NtsVar G = op.backward(X);
+        double t2 = now();
+        best_f = std::min(best_f, t1 - t0);
+        best_b = std::min(best_b, t2 - t1);
+      }
+      printf("reference ForwardSingleGPUfuseOp over libntship timing: V=%u E=%u F=%d forward_s=%.6f backward_s=%.6f\n",
+             vertices, pgg->owned_edges, width, best_f, best_b);
+    }
+    return 0;
+  }
   if (mode == "samp") {
     run_sampled_layers(graph, H);
     return 0;
