@@ -146,6 +146,103 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__
   }
 }
 
+// The same sums for rows that fit one group (Fv <= G), with the rows of a wavefront handed out
+// dynamically: a wavefront takes 64 consecutive rows, reads their offsets with one coalesced load,
+// and its 64/G groups then pull rows from that set one after the other -- a group that finishes a
+// short row takes the next pending one instead of idling until the longest row of a fixed
+// assignment is done.  Every group adds its row's edge rows in order (eight loads in flight), so
+// the result does not depend on which group happened to take which row.
+template <typename V, int G>
+__global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__restrict__ out,
+                                                                          const V *__restrict__ msg,
+                                                                          const uint32_t *__restrict__ off,
+                                                                          const uint32_t *__restrict__ perm,
+                                                                          uint32_t rows, uint32_t Fv, int accumulate,
+                                                                          uint32_t long_limit) {
+  constexpr int NF = sizeof(V) / 4;
+  const uint32_t lane = lane_id();
+  const uint32_t gl = lane & (G - 1), grp = lane / G;
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  const bool col_live = gl < Fv;
+  for (uint64_t base = wave * kWave; base < rows; base += n_waves * kWave) {
+    uint32_t my_e0 = 0, my_e1 = 0;
+    bool mine = false;
+    if (base + lane < rows) {
+      my_e0 = off[base + lane];
+      my_e1 = off[base + lane + 1];
+      mine = my_e1 - my_e0 <= long_limit;  // longer rows belong to the block kernels
+    }
+    uint64_t pending = __ballot(mine);  // rows of this set not handed out yet (wave-uniform)
+    bool have = false;
+    uint32_t row = 0, k = 0, e1 = 0;
+    float a[NF];
+    while (true) {
+      // Groups without a row take the lowest pending rows, in group order.
+      const uint64_t need_mask = __ballot(!have && gl == 0);
+      bool took = false;
+      if (!have) {
+        const uint32_t rank = __popcll(need_mask & ((1ull << (grp * G)) - 1ull));
+        uint64_t m = pending;
+        for (uint32_t t = 0; t < rank && m; ++t) m &= m - 1;
+        if (m) {
+          row = static_cast<uint32_t>(__builtin_ctzll(m));
+          took = true;
+        }
+      }
+      const uint32_t from = took ? row : lane;
+      const uint32_t new_e0 = __shfl(my_e0, from, kWave), new_e1 = __shfl(my_e1, from, kWave);
+      if (took) {
+        have = true;
+        k = new_e0;
+        e1 = new_e1;
+#pragma unroll
+        for (int t = 0; t < NF; ++t) a[t] = 0.f;
+      }
+      for (uint32_t t = __popcll(need_mask); t > 0 && pending; --t) pending &= pending - 1;  // handed out
+      if (!__ballot(have)) break;
+      if (have) {
+        // up to eight edge rows of this group's row, loaded together, added in order
+        V v[8];
+        const uint32_t n = e1 - k < 8u ? e1 - k : 8u;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (static_cast<uint32_t>(u) < n && col_live) {
+            const uint32_t e = perm ? perm[k + u] : k + u;
+            v[u] = msg[static_cast<size_t>(e) * Fv + gl];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (static_cast<uint32_t>(u) < n && col_live) {
+            const float *vf = reinterpret_cast<const float *>(&v[u]);
+#pragma unroll
+            for (int t = 0; t < NF; ++t) a[t] += vf[t];
+          }
+        }
+        k += n;
+        if (k >= e1) {
+          if (col_live) {
+            V *p = out + (base + row) * Fv + gl;
+            if (accumulate) {
+              const V o = *p;
+              const float *of = reinterpret_cast<const float *>(&o);
+#pragma unroll
+              for (int t = 0; t < NF; ++t) a[t] += of[t];
+            }
+            V res;
+            float *rf = reinterpret_cast<float *>(&res);
+#pragma unroll
+            for (int t = 0; t < NF; ++t) rf[t] = a[t];
+            *p = res;
+          }
+          have = false;
+        }
+      }
+    }
+  }
+}
+
 // Giant rows: a row so long that one block working through it alone would outlast the rest of the
 // launch (a 300,000-edge hub next to 10^4 rows of a few thousand edges) is cut into pieces that
 // separate blocks reduce, and a last kernel combines the pieces in order.  The caller's argument
@@ -1137,6 +1234,25 @@ constexpr unsigned kLongGrid = 512;  // blocks of the long-row kernels; they str
 template <typename V>
 void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_t *perm, uint32_t rows, uint32_t Fv,
                         int accumulate, uint32_t limit, hipStream_t stream) {
+  if (Fv <= 64 && rows >= 4096) {
+    // One group covers a row: wavefronts hand their 64 rows out dynamically (strided launch).
+    const uint32_t blocks = ceil_div(rows, 4 * kWave);  // at most 64 rows per wavefront
+    const dim3 grid(blocks < 8192u ? blocks : 8192u);
+#define NTS_BALANCED(GG)                                                                                           \
+  hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG>), grid, dim3(256), 0, stream, out, msg, off, perm, \
+                     rows, Fv, accumulate, limit)
+    switch (lanes_for(Fv)) {
+      case 1: NTS_BALANCED(1); break;
+      case 2: NTS_BALANCED(2); break;
+      case 4: NTS_BALANCED(4); break;
+      case 8: NTS_BALANCED(8); break;
+      case 16: NTS_BALANCED(16); break;
+      case 32: NTS_BALANCED(32); break;
+      default: NTS_BALANCED(64); break;
+    }
+#undef NTS_BALANCED
+    return;
+  }
 #define NTS_GATHER(GG)                                                                                          \
   hipLaunchKernelGGL((gather_edge_to_row_kernel<V, GG>), dim3(ceil_div(static_cast<uint64_t>(rows) * GG, 256)),  \
                      dim3(256), 0, stream, out, msg, off, perm, rows, Fv, accumulate, limit)
