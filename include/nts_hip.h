@@ -121,8 +121,8 @@ int nts_event_elapsed_ms(float *ms, nts_event_t start, nts_event_t stop);
  * leave long rows to one wavefront: rows of more than 1,024 edges are cut into 1,024-edge pieces on
  * the device (no copy to the host), the pieces write partial sums and a second stage adds them in
  * order -- still deterministic, but a long row's sum is then associated piece by piece.  That path
- * takes stream-ordered scratch (hipMallocAsync, (E/1024 + min(rows, E/1024) + 1) * (F * 4 + 16) bytes
- * plus 8 bytes per row, released with hipFreeAsync); a caller that must not allocate, or that runs
+ * takes stream-ordered scratch (hipMallocAsync, about (E/1024 + min(rows, E/1024) + 1) * (F * 4 + 48)
+ * bytes plus 8 bytes per row, released with hipFreeAsync); a caller that must not allocate, or that runs
  * the same structure many times, uses a plan (below), which also orders the pieces for the L2. */
 int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t *offsets,
                     const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,

@@ -19,7 +19,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
 
 #include <algorithm>
 #include <new>
@@ -502,18 +504,32 @@ __global__ __launch_bounds__(256) void auto_count_kernel(uint32_t *__restrict__ 
   pieces[r] = n;  // pieces[rows] = 0, so that the scan's last entry is the total
 }
 
-__global__ __launch_bounds__(256) void auto_items_kernel(Item *__restrict__ items, const uint32_t *__restrict__ base,
-                                                         const uint32_t *__restrict__ off, uint32_t rows,
-                                                         uint32_t chunk, uint32_t p_max) {
+// Also writes keys[i] = the gather index of the piece's first edge (0xFFFFFFFF for an empty item):
+// the pieces are then issued in ascending key order, so that wavefronts resident at the same time
+// gather from nearby source rows (with sorted adjacency a piece covers a narrow index range).
+__global__ __launch_bounds__(256) void auto_items_kernel(Item *__restrict__ items, uint32_t *__restrict__ keys,
+                                                         const uint32_t *__restrict__ base,
+                                                         const uint32_t *__restrict__ off,
+                                                         const uint32_t *__restrict__ indices, uint32_t index_base,
+                                                         uint32_t rows, uint32_t chunk, uint32_t p_max) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= p_max) return;
   if (i >= base[rows]) {
     items[i] = make_uint4(0u, 0u, 0u, i);  // empty item: writes zeros to its own unused slot
+    keys[i] = 0xFFFFFFFFu;
     return;
   }
   const uint32_t r = owner_of(base, rows, i);  // the last row whose first slot is <= i is the long row itself
   const uint32_t e0 = off[r] + (i - base[r]) * chunk;
   items[i] = make_uint4(r, e0, min(off[r + 1], e0 + chunk), i);
+  keys[i] = indices[e0] - index_base;
+}
+
+__global__ __launch_bounds__(256) void auto_order_items_kernel(Item *__restrict__ ordered,
+                                                               const Item *__restrict__ items,
+                                                               const uint32_t *__restrict__ order, uint32_t p_max) {
+  const uint32_t j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j < p_max) ordered[j] = items[order[j]];
 }
 
 // Block (x, y): if work item x is the first piece of its row, adds that row's partials in slot order
@@ -557,23 +573,37 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
   const uint32_t chunk = kAutoChunk;
   const uint32_t by_edges = edges / chunk;
   const uint32_t p_max = by_edges + (rows < by_edges ? rows : by_edges) + 1;
-  size_t scan_bytes = 0;
+  size_t scan_bytes = 0, sort_bytes = 0;
   {
     uint32_t *nul = nullptr;
     NTS_HIP_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, nul, nul, 0u, static_cast<size_t>(rows) + 1,
                                         rocprim::plus<uint32_t>(), a.stream, false));
+    NTS_HIP_TRY(rocprim::radix_sort_pairs(nullptr, sort_bytes, nul, nul, rocprim::counting_iterator<uint32_t>(0u), nul,
+                                          p_max, 0u, 32u, a.stream, false));
   }
+  const size_t tmp_bytes = up256(scan_bytes > sort_bytes ? scan_bytes : sort_bytes);
   const size_t n_off = up256((static_cast<size_t>(rows) + 1) * sizeof(uint32_t));
   const size_t n_items_b = up256(static_cast<size_t>(p_max) * sizeof(Item));
+  const size_t n_keys_b = up256(static_cast<size_t>(p_max) * sizeof(uint32_t));
   const size_t n_partial = up256(static_cast<size_t>(p_max) * a.F * sizeof(float));
   unsigned char *buf = nullptr;
-  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&buf), 2 * n_off + n_items_b + up256(scan_bytes) + n_partial,
-                             a.stream));
-  uint32_t *pieces = reinterpret_cast<uint32_t *>(buf);
-  uint32_t *base = reinterpret_cast<uint32_t *>(buf + n_off);
-  Item *items = reinterpret_cast<Item *>(buf + 2 * n_off);
-  void *scan_tmp = buf + 2 * n_off + n_items_b;
-  float *partial = reinterpret_cast<float *>(buf + 2 * n_off + n_items_b + up256(scan_bytes));
+  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&buf),
+                             2 * n_off + 2 * n_items_b + 3 * n_keys_b + tmp_bytes + n_partial, a.stream));
+  unsigned char *cursor = buf;
+  auto take = [&cursor](size_t bytes) {
+    unsigned char *p = cursor;
+    cursor += bytes;
+    return p;
+  };
+  uint32_t *pieces = reinterpret_cast<uint32_t *>(take(n_off));
+  uint32_t *base = reinterpret_cast<uint32_t *>(take(n_off));
+  Item *items = reinterpret_cast<Item *>(take(n_items_b));
+  Item *ordered = reinterpret_cast<Item *>(take(n_items_b));
+  uint32_t *keys = reinterpret_cast<uint32_t *>(take(n_keys_b));
+  uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(take(n_keys_b));
+  uint32_t *order = reinterpret_cast<uint32_t *>(take(n_keys_b));
+  void *tmp = take(tmp_bytes);
+  float *partial = reinterpret_cast<float *>(take(n_partial));
   auto bail = [&](hipError_t err, const char *what) {
     (void)hipFreeAsync(buf, a.stream);
     return fail_hip(err, what);
@@ -582,17 +612,24 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
                      pieces, a.offsets, rows, chunk);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return bail(err, "auto_count_kernel");
-  err = rocprim::exclusive_scan(scan_tmp, scan_bytes, pieces, base, 0u, static_cast<size_t>(rows) + 1,
+  err = rocprim::exclusive_scan(tmp, scan_bytes, pieces, base, 0u, static_cast<size_t>(rows) + 1,
                                 rocprim::plus<uint32_t>(), a.stream, false);
   if (err != hipSuccess) return bail(err, "spmm: scan of piece counts");
-  hipLaunchKernelGGL(auto_items_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, items, base, a.offsets, rows,
-                     chunk, p_max);
+  hipLaunchKernelGGL(auto_items_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, items, keys, base, a.offsets,
+                     a.indices, a.index_base, rows, chunk, p_max);
   err = hipGetLastError();
   if (err != hipSuccess) return bail(err, "auto_items_kernel");
+  err = rocprim::radix_sort_pairs(tmp, sort_bytes, keys, keys_sorted, rocprim::counting_iterator<uint32_t>(0u), order,
+                                  p_max, 0u, 32u, a.stream, false);
+  if (err != hipSuccess) return bail(err, "spmm: ordering of the pieces");
+  hipLaunchKernelGGL(auto_order_items_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, ordered, items, order,
+                     p_max);
+  err = hipGetLastError();
+  if (err != hipSuccess) return bail(err, "auto_order_items_kernel");
   // Pieces first (the heavy, uniform work), then the rows that fit one wavefront.
   LaunchArgs pc = a;
   pc.n_items = p_max;
-  pc.items = items;
+  pc.items = ordered;
   pc.partial = partial;
   launch_spmm(pc);
   LaunchArgs whole = a;
