@@ -14,6 +14,9 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <map>
+#include <mutex>
+
 #include "nts_hip.h"
 
 typedef uint32_t VertexId_CUDA;
@@ -38,6 +41,132 @@ enum weight_type { NULL_TYPE, SCALA_TYPE, TENSOR_TYPE };
     }                                                                                      \
   } while (0)
 
+// ---- aggregation schedules for static graphs, kept behind the reference's call signatures --------
+//
+// The reference calls Gather_By_Dst_From_Src / Gather_By_Src_From_Dst with bare device pointers.
+// For a whole-graph chunk those arrays never change after CopyGraphToDevice, and a schedule built
+// once (nts_spmm_plan_create_slabs) makes every later pass about 1.5x faster than the per-call
+// balancing of nts_spmm_gather.  The veneer can tell a static structure from a per-batch one because
+// every write the tree makes to device memory it allocated goes through the helpers of this header:
+// each allocation made here is a region with a generation number that every upload, zeroing or
+// kernel output into it advances.  A call whose offsets and indices both lie in such regions, names
+// its source range, has at least 2^22 edges and repeats with unchanged generations for the third
+// time gets a schedule (built once, blocking); any later write to either region, or freeing it,
+// drops the schedule.  Mini-batch layers are re-uploaded every batch and never qualify.
+// NTS_VENEER_PLAN_CACHE=0 in the environment switches the mechanism off.
+namespace nts_veneer {
+
+struct Region {
+  size_t bytes;
+  unsigned long long generation;
+};
+struct CachedPlan {
+  nts_spmm_plan_t *plan;
+  const void *indices;
+  uint32_t rows, edges, n_index, index_base;
+  unsigned long long gen_offsets, gen_indices;
+  int seen;
+  nts_stream_t stream;  // a schedule's scratch serves one stream at a time: other streams go without
+};
+struct State {
+  std::mutex mu;
+  std::map<uintptr_t, Region> regions;
+  std::map<uintptr_t, CachedPlan> plans;  // keyed by the offsets pointer
+  unsigned long long clock = 1;
+  long plans_built = 0;
+  long planned_calls = 0;
+  int enabled = -1;
+};
+inline State &state() {
+  static State s;
+  return s;
+}
+const uint32_t kPlanMinEdges = 1u << 22;
+
+inline std::map<uintptr_t, Region>::iterator region_of(State &st, const void *p) {
+  const uintptr_t a = (uintptr_t)p;
+  std::map<uintptr_t, Region>::iterator it = st.regions.upper_bound(a);
+  if (it == st.regions.begin()) return st.regions.end();
+  --it;
+  return a < it->first + it->second.bytes ? it : st.regions.end();
+}
+inline void note_alloc(void *p, size_t bytes) {
+  if (!p) return;
+  State &st = state();
+  std::lock_guard<std::mutex> lock(st.mu);
+  Region r = {bytes, st.clock++};
+  st.regions[(uintptr_t)p] = r;
+}
+inline void drop_plans_touching(State &st, uintptr_t base, size_t bytes) {
+  for (std::map<uintptr_t, CachedPlan>::iterator it = st.plans.begin(); it != st.plans.end();) {
+    const uintptr_t o = it->first, i = (uintptr_t)it->second.indices;
+    if ((o >= base && o < base + bytes) || (i >= base && i < base + bytes)) {
+      if (it->second.plan) nts_spmm_plan_destroy(it->second.plan);
+      it = st.plans.erase(it);
+    } else {
+      ++it;
+    }
+  }
+}
+inline void note_free(void *p) {
+  if (!p) return;
+  State &st = state();
+  std::lock_guard<std::mutex> lock(st.mu);
+  std::map<uintptr_t, Region>::iterator it = st.regions.find((uintptr_t)p);
+  if (it == st.regions.end()) return;
+  drop_plans_touching(st, it->first, it->second.bytes);
+  st.regions.erase(it);
+}
+// A write into device memory at p (an upload, a zeroing, a kernel output).
+inline void note_write(const void *p) {
+  if (!p) return;
+  State &st = state();
+  std::lock_guard<std::mutex> lock(st.mu);
+  std::map<uintptr_t, Region>::iterator it = region_of(st, p);
+  if (it != st.regions.end()) it->second.generation = st.clock++;
+}
+// The schedule for this (offsets, indices) pair if the structure has proved static, else NULL.
+inline nts_spmm_plan_t *plan_for(const uint32_t *offsets, const uint32_t *indices, uint32_t index_base,
+                                 uint32_t n_index, uint32_t rows, uint32_t edges, nts_stream_t stream) {
+  if (edges < kPlanMinEdges || n_index == 0) return NULL;
+  State &st = state();
+  std::lock_guard<std::mutex> lock(st.mu);
+  if (st.enabled < 0) {
+    const char *e = getenv("NTS_VENEER_PLAN_CACHE");
+    st.enabled = (e && e[0] == '0') ? 0 : 1;
+  }
+  if (!st.enabled) return NULL;
+  std::map<uintptr_t, Region>::iterator ro = region_of(st, offsets), ri = region_of(st, indices);
+  if (ro == st.regions.end() || ri == st.regions.end()) return NULL;
+  CachedPlan &c = st.plans[(uintptr_t)offsets];
+  const bool same = c.indices == indices && c.rows == rows && c.edges == edges && c.n_index == n_index &&
+                    c.index_base == index_base && c.gen_offsets == ro->second.generation &&
+                    c.gen_indices == ri->second.generation;
+  if (!same) {
+    if (c.plan) nts_spmm_plan_destroy(c.plan);
+    CachedPlan fresh = {NULL, indices, rows, edges, n_index, index_base, ro->second.generation, ri->second.generation, 1,
+                        stream};
+    c = fresh;
+    return NULL;
+  }
+  if (c.stream != stream) return NULL;
+  if (!c.plan) {
+    if (++c.seen < 3) return NULL;
+    if (nts_spmm_plan_create_slabs(&c.plan, offsets, indices, index_base, n_index, rows, edges, 0, 0, stream) != NTS_OK) {
+      c.plan = NULL;
+      c.seen = -1000000;  // do not try again for this structure
+      return NULL;
+    }
+    ++st.plans_built;
+  }
+  ++st.planned_calls;
+  return c.plan;
+}
+inline long plans_built() { return state().plans_built; }
+inline long planned_calls() { return state().planned_calls; }
+
+}  // namespace nts_veneer
+
 // ---- allocation and copies ---------------------------------------------------------------------
 
 inline void *cudaMallocPinned(long size_of_bytes) {
@@ -53,58 +182,85 @@ inline void *getDevicePointer(void *host_data_to_device) {
 inline void *cudaMallocGPU(long size_of_bytes) {
   void *p = NULL;
   NTS_VENEER_CHECK(nts_malloc_device(&p, (size_t)size_of_bytes));
+  nts_veneer::note_alloc(p, (size_t)size_of_bytes);
   return p;
 }
 inline void ntsFreeHost(void *buffer) { NTS_VENEER_CHECK(nts_free_pinned(buffer)); }
-inline void FreeBuffer(float *buffer) { NTS_VENEER_CHECK(nts_free_device(buffer)); }
-inline void FreeEdge(VertexId_CUDA *buffer) { NTS_VENEER_CHECK(nts_free_device(buffer)); }
-inline void FreeBufferAsync(float *buffer, cudaStream_t cs) { NTS_VENEER_CHECK(nts_free_device_async(buffer, cs)); }
-inline void FreeEdgeAsync(VertexId_CUDA *buffer, cudaStream_t cs) { NTS_VENEER_CHECK(nts_free_device_async(buffer, cs)); }
+inline void FreeBuffer(float *buffer) {
+  nts_veneer::note_free(buffer);
+  NTS_VENEER_CHECK(nts_free_device(buffer));
+}
+inline void FreeEdge(VertexId_CUDA *buffer) {
+  nts_veneer::note_free(buffer);
+  NTS_VENEER_CHECK(nts_free_device(buffer));
+}
+inline void FreeBufferAsync(float *buffer, cudaStream_t cs) {
+  nts_veneer::note_free(buffer);
+  NTS_VENEER_CHECK(nts_free_device_async(buffer, cs));
+}
+inline void FreeEdgeAsync(VertexId_CUDA *buffer, cudaStream_t cs) {
+  nts_veneer::note_free(buffer);
+  NTS_VENEER_CHECK(nts_free_device_async(buffer, cs));
+}
 template <typename T>
 inline void free_gpu_data(T *data) {
+  nts_veneer::note_free(data);
   NTS_VENEER_CHECK(nts_free_device(data));
 }
 template <typename T>
 inline void alloc_gpu_data(T **input, int size) {
   NTS_VENEER_CHECK(nts_malloc_device((void **)input, sizeof(T) * (size_t)size));
+  nts_veneer::note_alloc(*input, sizeof(T) * (size_t)size);
 }
 inline void allocate_gpu_buffer(float **input, int size) {
   NTS_VENEER_CHECK(nts_malloc_device((void **)input, sizeof(float) * (size_t)size));
+  nts_veneer::note_alloc(*input, sizeof(float) * (size_t)size);
 }
 inline void allocate_gpu_edge(VertexId_CUDA **input, int size) {
   NTS_VENEER_CHECK(nts_malloc_device((void **)input, sizeof(VertexId_CUDA) * (size_t)size));
+  nts_veneer::note_alloc(*input, sizeof(VertexId_CUDA) * (size_t)size);
 }
 inline void allocate_gpu_buffer_async(float **input, int size, cudaStream_t cs) {
   NTS_VENEER_CHECK(nts_malloc_device_async((void **)input, sizeof(float) * (size_t)size, cs));
+  nts_veneer::note_alloc(*input, sizeof(float) * (size_t)size);
 }
 inline void allocate_gpu_edge_async(VertexId_CUDA **input, int size, cudaStream_t cs) {
   NTS_VENEER_CHECK(nts_malloc_device_async((void **)input, sizeof(VertexId_CUDA) * (size_t)size, cs));
+  nts_veneer::note_alloc(*input, sizeof(VertexId_CUDA) * (size_t)size);
 }
 inline void move_result_out(float *output, float *input, int src, int dst, int feature_size, bool sync = true) {
   NTS_VENEER_CHECK(nts_memcpy_d2h(output, input, (size_t)(dst - src) * feature_size * sizeof(float), sync));
 }
 inline void move_data_in(float *d_pointer, float *h_pointer, int start, int end, int feature_size, bool sync = true) {
+  nts_veneer::note_write(d_pointer);
   NTS_VENEER_CHECK(nts_memcpy_h2d(d_pointer, h_pointer, (size_t)(end - start) * feature_size * sizeof(float), sync));
 }
 inline void move_edge_in(VertexId_CUDA *d_pointer, VertexId_CUDA *h_pointer, VertexId_CUDA start, VertexId_CUDA end,
                          int feature_size, bool sync = true) {
+  nts_veneer::note_write(d_pointer);
   NTS_VENEER_CHECK(
       nts_memcpy_h2d(d_pointer, h_pointer, (size_t)(end - start) * feature_size * sizeof(VertexId_CUDA), sync));
 }
 inline void move_bytes_in(void *d_pointer, void *h_pointer, long bytes, bool sync = true) {
+  nts_veneer::note_write(d_pointer);
   NTS_VENEER_CHECK(nts_memcpy_h2d(d_pointer, h_pointer, (size_t)bytes, sync));
 }
 inline void move_bytes_in_async(void *d_pointer, void *h_pointer, long bytes, cudaStream_t cs) {
+  nts_veneer::note_write(d_pointer);
   NTS_VENEER_CHECK(nts_memcpy_h2d_async(d_pointer, h_pointer, (size_t)bytes, cs));
 }
 inline void zero_buffer(float *buffer, int size) {
+  nts_veneer::note_write(buffer);
   NTS_VENEER_CHECK(nts_memset_zero(buffer, sizeof(float) * (size_t)size, (cudaStream_t)0));
   NTS_VENEER_CHECK(nts_device_sync());
 }
 inline void CUDA_DEVICE_SYNCHRONIZE() { NTS_VENEER_CHECK(nts_device_sync()); }
 // The few raw runtime names that core/ and comm/ call outside cuda/ (core/ntsMiniBatchGraphOp.hpp:283,
 // core/coocsc.hpp:673-773, comm/network.cpp:53, 84).
-inline int cudaFree(void *p) { return nts_free_device(p); }
+inline int cudaFree(void *p) {
+  nts_veneer::note_free(p);
+  return nts_free_device(p);
+}
 inline int cudaFreeHost(void *p) { return nts_free_pinned(p); }
 inline int cudaStreamSynchronize(cudaStream_t s) { return nts_stream_sync(s); }
 
@@ -189,12 +345,14 @@ class Cuda_Stream {
   void move_data_in(float *d_pointer, float *h_pointer, VertexId_CUDA start, VertexId_CUDA end, int feature_size,
                     bool sync = true) {
     (void)sync;
+    nts_veneer::note_write(d_pointer);
     NTS_VENEER_CHECK(
         nts_memcpy_h2d_async(d_pointer, h_pointer, (size_t)(end - start) * feature_size * sizeof(float), stream));
   }
   void move_edge_in(VertexId_CUDA *d_pointer, VertexId_CUDA *h_pointer, VertexId_CUDA start, VertexId_CUDA end,
                     int feature_size, bool sync = true) {
     (void)sync;
+    nts_veneer::note_write(d_pointer);
     NTS_VENEER_CHECK(nts_memcpy_h2d_async(d_pointer, h_pointer,
                                           (size_t)(end - start) * feature_size * sizeof(VertexId_CUDA), stream));
   }
@@ -206,10 +364,17 @@ class Cuda_Stream {
                               VertexId_CUDA dst_start, VertexId_CUDA dst_end, VertexId_CUDA edges,
                               VertexId_CUDA batch_size, VertexId_CUDA feature_size, bool with_weight = false,
                               bool tensor_weight = false) {
-    (void)src_end; (void)dst_start; (void)dst_end;
+    (void)dst_start; (void)dst_end;
     reject_tensor_weight(with_weight && tensor_weight);
-    NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_forward : NULL, column_offset, row_indices,
-                                     src_start, batch_size, edges, feature_size, 1, stream));
+    nts_veneer::note_write(output);
+    nts_spmm_plan_t *plan = nts_veneer::plan_for(column_offset, row_indices, src_start,
+                                                  src_end > src_start ? src_end - src_start : 0, batch_size, edges, stream);
+    if (plan)
+      NTS_VENEER_CHECK(nts_spmm_gather_planned(plan, input, output, with_weight ? weight_forward : NULL, column_offset,
+                                               row_indices, src_start, feature_size, 1, stream));
+    else
+      NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_forward : NULL, column_offset, row_indices,
+                                       src_start, batch_size, edges, feature_size, 1, stream));
   }
   void Gather_By_Dst_From_Src_Optim(float *input, float *output, float *weight_forward, VertexId_CUDA *row_indices,
                                     VertexId_CUDA *column_offset, VertexId_CUDA src_start, VertexId_CUDA src_end,
@@ -224,10 +389,17 @@ class Cuda_Stream {
                               VertexId_CUDA dst_start, VertexId_CUDA dst_end, VertexId_CUDA edges,
                               VertexId_CUDA batch_size, VertexId_CUDA feature_size, bool with_weight = false,
                               bool tensor_weight = false) {
-    (void)src_start; (void)src_end; (void)dst_end;
+    (void)src_start; (void)src_end;
     reject_tensor_weight(with_weight && tensor_weight);
-    NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_backward : NULL, row_offset, column_indices,
-                                     dst_start, batch_size, edges, feature_size, 1, stream));
+    nts_veneer::note_write(output);
+    nts_spmm_plan_t *plan = nts_veneer::plan_for(row_offset, column_indices, dst_start,
+                                                  dst_end > dst_start ? dst_end - dst_start : 0, batch_size, edges, stream);
+    if (plan)
+      NTS_VENEER_CHECK(nts_spmm_gather_planned(plan, input, output, with_weight ? weight_backward : NULL, row_offset,
+                                               column_indices, dst_start, feature_size, 1, stream));
+    else
+      NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_backward : NULL, row_offset, column_indices,
+                                       dst_start, batch_size, edges, feature_size, 1, stream));
   }
   void Gather_By_Src_From_Dst_Optim(float *input, float *output, float *weight_backward, VertexId_CUDA *row_offset,
                                     VertexId_CUDA *column_indices, VertexId_CUDA src_start, VertexId_CUDA src_end,
@@ -246,6 +418,7 @@ class Cuda_Stream {
       printf("tensor_weight Scatter_Grad_Back_To_Weight not implemented\n");
       exit(0);
     }
+    nts_veneer::note_write(message_grad);
     NTS_VENEER_CHECK(nts_scatter_grad_to_edge(message_grad, input, column_offset, batch_size, feature_size, stream));
   }
 
@@ -253,23 +426,27 @@ class Cuda_Stream {
   void Scatter_Src_Mirror_to_Msg(float *message, float *src_mirror_feature, VertexId_CUDA *row_indices,
                                  VertexId_CUDA *column_offset, VertexId_CUDA *mirror_index, VertexId_CUDA batch_size,
                                  VertexId_CUDA feature_size) {
+    nts_veneer::note_write(message);
     NTS_VENEER_CHECK(nts_scatter_src_to_edge(message, src_mirror_feature, row_indices, column_offset, mirror_index,
                                              batch_size, feature_size, stream));
   }
   void Scatter_Dst_to_Msg(float *message, float *dst_feature, VertexId_CUDA *row_indices,
                           VertexId_CUDA *column_offset, VertexId_CUDA batch_size, VertexId_CUDA feature_size) {
     (void)row_indices;
+    nts_veneer::note_write(message);
     NTS_VENEER_CHECK(nts_scatter_dst_to_edge(message, dst_feature, column_offset, batch_size, feature_size, stream));
   }
   void Gather_Msg_to_Dst(float *dst_feature, float *message, VertexId_CUDA *row_indices, VertexId_CUDA *column_offset,
                          VertexId_CUDA batch_size, VertexId_CUDA feature_size) {
     (void)row_indices;
+    nts_veneer::note_write(dst_feature);
     NTS_VENEER_CHECK(nts_gather_edge_to_dst(dst_feature, message, column_offset, batch_size, feature_size, 1, stream));
   }
   // Reference argument list; deterministic, but sorts the edges by target row on every call.
   void Gather_Msg_To_Src_Mirror(float *src_mirror_feature, float *message, VertexId_CUDA *row_indices,
                                 VertexId_CUDA *column_offset, VertexId_CUDA *mirror_index, VertexId_CUDA batch_size,
                                 VertexId_CUDA feature_size) {
+    nts_veneer::note_write(src_mirror_feature);
     NTS_VENEER_CHECK(nts_gather_edge_to_src_unsorted(src_mirror_feature, message, row_indices, column_offset,
                                                      mirror_index, batch_size, feature_size, stream));
   }
@@ -277,6 +454,7 @@ class Cuda_Stream {
   // (row_offset [src_size+1], csr_to_csc [E]) instead of (row_indices, column_offset, mirror_index).
   void Gather_Msg_To_Src(float *src_feature, float *message, VertexId_CUDA *row_offset, VertexId_CUDA *csr_to_csc,
                          VertexId_CUDA src_size, VertexId_CUDA feature_size) {
+    nts_veneer::note_write(src_feature);
     NTS_VENEER_CHECK(nts_gather_edge_to_src(src_feature, message, row_offset, csr_to_csc, src_size, feature_size, 1,
                                             stream));
   }
@@ -284,6 +462,7 @@ class Cuda_Stream {
                                   VertexId_CUDA *column_offset, VertexId_CUDA batch_size,
                                   VertexId_CUDA feature_size) {
     (void)row_indices;
+    nts_veneer::note_write(msg_output);
     NTS_VENEER_CHECK(nts_edge_softmax_fwd(msg_output, msg_input, column_offset, batch_size, feature_size, stream));
     if (msg_cached && msg_cached != msg_output) {
       // The edge count is only known on the device: copy column_offset[batch_size] back once.
@@ -298,6 +477,7 @@ class Cuda_Stream {
                                    VertexId_CUDA *row_indices, VertexId_CUDA *column_offset, VertexId_CUDA batch_size,
                                    VertexId_CUDA feature_size) {
     (void)row_indices;
+    nts_veneer::note_write(msg_input_grad);
     NTS_VENEER_CHECK(nts_edge_softmax_bwd(msg_input_grad, msg_output_grad, msg_cached, column_offset, batch_size,
                                           feature_size, stream));
   }
@@ -324,6 +504,7 @@ class Cuda_Stream {
   // Mini-batch assembly; like the reference these return with the result complete.
   void zero_copy_feature_move_gpu(float *dev_feature, float *pinned_host_feature, VertexId_CUDA *src_vertex,
                                   VertexId_CUDA feature_size, VertexId_CUDA vertex_size) {
+    nts_veneer::note_write(dev_feature);
     NTS_VENEER_CHECK(nts_gather_rows_f32(dev_feature, pinned_host_feature, src_vertex, NULL, NULL, vertex_size,
                                          feature_size, stream));
     CUDA_DEVICE_SYNCHRONIZE();
@@ -331,6 +512,7 @@ class Cuda_Stream {
   void zero_copy_feature_move_gpu_cache(float *dev_feature, float *host_pinned_feature, VertexId_CUDA *src_vertex,
                                         VertexId_CUDA feature_size, VertexId_CUDA vertex_size,
                                         VertexId_CUDA *local_idx) {
+    nts_veneer::note_write(dev_feature);
     NTS_VENEER_CHECK(nts_gather_rows_f32(dev_feature, host_pinned_feature, src_vertex, local_idx, NULL, vertex_size,
                                          feature_size, stream));
     CUDA_DEVICE_SYNCHRONIZE();
@@ -338,18 +520,21 @@ class Cuda_Stream {
   void gather_feature_from_gpu_cache(float *dev_feature, float *dev_cache_feature, VertexId_CUDA *src_vertex,
                                      VertexId_CUDA feature_size, VertexId_CUDA vertex_size,
                                      VertexId_CUDA *local_idx_cache, VertexId_CUDA *cache_node_hashmap) {
+    nts_veneer::note_write(dev_feature);
     NTS_VENEER_CHECK(nts_gather_rows_f32(dev_feature, dev_cache_feature, src_vertex, local_idx_cache,
                                          cache_node_hashmap, vertex_size, feature_size, stream));
     CUDA_DEVICE_SYNCHRONIZE();
   }
   void global_copy_label_move_gpu(long *dev_label, long *global_dev_label, VertexId_CUDA *dst_vertex,
                                   VertexId_CUDA vertex_size) {
+    nts_veneer::note_write(dev_label);
     NTS_VENEER_CHECK(nts_gather_labels_i64((int64_t *)dev_label, (const int64_t *)global_dev_label, dst_vertex,
                                            vertex_size, 1, stream));
     CUDA_DEVICE_SYNCHRONIZE();
   }
   void global_copy_mulilabel_move_gpu(long *dev_label, long *global_dev_label, VertexId_CUDA *dst_vertex,
                                       VertexId_CUDA vertex_size, VertexId_CUDA label_size) {
+    nts_veneer::note_write(dev_label);
     NTS_VENEER_CHECK(nts_gather_labels_i64((int64_t *)dev_label, (const int64_t *)global_dev_label, dst_vertex,
                                            vertex_size, label_size, stream));
     CUDA_DEVICE_SYNCHRONIZE();
