@@ -27,6 +27,12 @@
 //   generate_csr_from_csc, update_degree, compute_weight_forward / backward, and the resulting
 //   source, row_indices (local), row_offset, column_indices and both weight arrays are written as
 //   <prefix>.l<k>.<name>.
+//   mini (GPU build only): the sampled layers of `samp`, held one after the other in a single sampCSC
+//   object as the reference's sampler re-uses it, are mirrored on the device by the reference's own
+//   alloc_dev_array_async / copy_data_to_device_async / copy_ewf/ewb_to_device_async (grow-only
+//   device arrays, core/coocsc.hpp:673-773) and aggregated forward and backward with the calls of
+//   SingleGPUSampleGraphOp (core/ntsMiniBatchGraphOp.hpp:288-375) on <prefix>.l<k>.x [src_size, F] and
+//   <prefix>.l<k>.g [v_size, F]; writes <prefix>.l<k>.fwd and .bwd next to the arrays of `samp`.
 //   data (GPU build only; allocates the feature table in pinned memory, so it needs the device):
 //   GNNDatum::readFeature_Label_Mask (core/ntsDataloador.hpp:264-395) on <prefix>.feat / .label /
 //   .mask with F features and <H> classes; writes local_feature, local_label, local_mask,
@@ -103,13 +109,17 @@ static std::vector<VertexId> read_ids(const std::string &name) {
 #if CUDA_ENABLE
 // The reference's per-layer construction steps of Sampler::sample_one after the neighbour pick
 // (core/ntsSampler.hpp:1006-1106), on sampled lists handed in by the caller.
-static void run_sampled_layers(Graph<Empty> *graph, int layers) {
+static void run_sampled_layers(Graph<Empty> *graph, int layers, bool on_device, int F) {
   VertexId *node_idx = new VertexId[graph->vertices];
+  // Never destroyed: ~sampCSC frees device pointers its constructors leave uninitialised.
+  sampCSC *shared = new sampCSC();
+  Cuda_Stream *cs = on_device ? new Cuda_Stream() : nullptr;
   for (int k = 0; k < layers; ++k) {
     const std::string tag = "l" + std::to_string(k) + ".";
     std::vector<VertexId> dst = read_ids(tag + "dst"), co = read_ids(tag + "co"), ri = read_ids(tag + "ri");
-    // Never destroyed: ~sampCSC frees device pointers its constructors leave uninitialised.
-    sampCSC *sg = new sampCSC(static_cast<VertexId>(dst.size()), static_cast<VertexId>(ri.size()));
+    sampCSC *sg = on_device ? shared : new sampCSC(static_cast<VertexId>(dst.size()), static_cast<VertexId>(ri.size()));
+    sg->update_vertices(static_cast<VertexId>(dst.size()));
+    sg->update_edges(static_cast<VertexId>(ri.size()));
     sg->dst() = dst;
     sg->c_o() = co;
     sg->r_i() = ri;
@@ -126,6 +136,23 @@ static void run_sampled_layers(Graph<Empty> *graph, int layers) {
     write_raw(tag + "column_indices", sg->c_i().data(), sg->c_i().size() * sizeof(VertexId));
     write_raw(tag + "edge_weight_forward", sg->edge_weight_forward.data(), sg->edge_weight_forward.size() * sizeof(ValueType));
     write_raw(tag + "edge_weight_backward", sg->edge_weight_backward.data(), sg->edge_weight_backward.size() * sizeof(ValueType));
+    if (on_device) {
+      sg->alloc_dev_array_async(cs->stream);
+      sg->copy_data_to_device_async(cs->stream);
+      sg->copy_ewf_to_device_async(cs->stream);
+      sg->copy_ewb_to_device_async(cs->stream);
+      const long Vd = sg->v_size, Vs = sg->src_size;
+      NtsVar x = read_matrix(tag + "x", Vs, F).cuda(), g = read_matrix(tag + "g", Vd, F).cuda();
+      NtsVar y = torch::zeros({Vd, (long)F}, x.options()), gx = torch::zeros({Vs, (long)F}, x.options());
+      torch::cuda::synchronize();
+      cs->Gather_By_Dst_From_Src(x.data_ptr<float>(), y.data_ptr<float>(), sg->dev_ewf(), sg->dev_r_i(), sg->dev_c_o(), 0, 0,
+                                 0, 0, sg->e_size, sg->v_size, F, true, false);
+      cs->Gather_By_Src_From_Dst(g.data_ptr<float>(), gx.data_ptr<float>(), sg->dev_ewb(), sg->dev_r_o(), sg->dev_c_i(), 0,
+                                 0, 0, 0, sg->e_size, sg->src_size, F, true, false);
+      cs->CUDA_DEVICE_SYNCHRONIZE();
+      write_tensor(tag + "fwd", y);
+      write_tensor(tag + "bwd", gx);
+    }
   }
   printf("reference sampCSC construction done for %d layers\n", layers);
 }
@@ -199,8 +226,8 @@ int main(int argc, char **argv) {
     }
     return 0;
   }
-  if (mode == "samp") {
-    run_sampled_layers(graph, H);
+  if (mode == "samp" || mode == "mini") {
+    run_sampled_layers(graph, H, mode == "mini", F);
     return 0;
   }
   if (mode == "data") {

@@ -57,17 +57,23 @@ def run(kind, mode, inputs, tmp_path, timeout=600):
     return out
 
 
-def run_sampled_layers(graph_src, graph_dst, V, layers, tmp_path, timeout=600):
+def run_sampled_layers(graph_src, graph_dst, V, layers, tmp_path, timeout=600, device_F=0):
     """layers: list of dicts with dst [Vd], co [Vd+1], ri [E] (global source ids), uint32.  Runs the
     reference's sampCSC construction (the GPU-variant program; this mode makes no device call) and
-    returns, per layer, source / row_indices / row_offset / column_indices / both weight arrays."""
+    returns, per layer, source / row_indices / row_offset / column_indices / both weight arrays.
+    With device_F > 0 (needs the GPU) every layer also carries x [src_size, F] and g [Vd, F]; the
+    layers are then mirrored on the device by the reference's own sampCSC code and aggregated with
+    the calls of SingleGPUSampleGraphOp, and "fwd" / "bwd" are returned as well."""
     prefix = os.path.join(str(tmp_path), "samp")
     np.stack([graph_src, graph_dst], 1).astype(np.uint32).tofile(prefix + ".edge")
     for k, layer in enumerate(layers):
         for name in ("dst", "co", "ri"):
             np.ascontiguousarray(layer[name], dtype=np.uint32).tofile(f"{prefix}.l{k}.{name}")
-    r = subprocess.run([PROGRAMS["gpu"], prefix + ".edge", str(V), "4", str(len(layers)), prefix, "samp"],
-                       capture_output=True, text=True, timeout=timeout)
+        if device_F:
+            for name in ("x", "g"):
+                np.ascontiguousarray(layer[name], dtype=np.float32).tofile(f"{prefix}.l{k}.{name}")
+    r = subprocess.run([PROGRAMS["gpu"], prefix + ".edge", str(V), str(device_F or 4), str(len(layers)), prefix,
+                        "mini" if device_F else "samp"], capture_output=True, text=True, timeout=timeout)
     assert r.returncode == 0, f"reference program failed ({r.returncode}):\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}"
     out = []
     for k in range(len(layers)):
@@ -76,6 +82,9 @@ def run_sampled_layers(graph_src, graph_dst, V, layers, tmp_path, timeout=600):
                             ("column_indices", np.uint32), ("edge_weight_forward", np.float32),
                             ("edge_weight_backward", np.float32)):
             d[name] = np.fromfile(f"{prefix}.l{k}.{name}", dtype=dtype)
+        if device_F:
+            d["fwd"] = np.fromfile(f"{prefix}.l{k}.fwd", dtype=np.float32).reshape(-1, device_F)
+            d["bwd"] = np.fromfile(f"{prefix}.l{k}.bwd", dtype=np.float32).reshape(-1, device_F)
         out.append(d)
     return out
 

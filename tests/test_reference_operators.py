@@ -146,6 +146,22 @@ def test_oracle_matches_the_reference_sampled_layer_construction(tmp_path, V, E,
     """sampCSC::postprocessing, generate_csr_from_csc, update_degree and compute_weight_forward /
     backward of the reference itself (core/coocsc.hpp:136-450), run on sampled lists made here, against
     the oracle's restatements: every array bit for bit."""
+    _sampled_layers_case(tmp_path, V, E, batch, fanouts, seed, device_F=0)
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not refops.available("gpu"), reason="reference-built program with sampCSC not present")
+@pytest.mark.parametrize("V,E,batch,fanouts,seed", [(20000, 300000, 512, [10, 25], 2), (3000, 90000, 200, [15, 10, 5], 3)])
+def test_reference_sampled_layers_on_the_device_match_the_oracle(tmp_path, V, E, batch, fanouts, seed):
+    """The reference's sampCSC mirrors each layer on the device itself (grow-only arrays re-used from
+    layer to layer, asynchronous copies: core/coocsc.hpp:673-773) through the veneer's allocator and
+    copies, and the layer is aggregated forward and backward with the calls of SingleGPUSampleGraphOp
+    (core/ntsMiniBatchGraphOp.hpp:288-375).  Results against the oracle's fused aggregation on the
+    reference's own arrays: rows of at most 1,024 edges bit for bit, the rest within tolerance."""
+    _sampled_layers_case(tmp_path, V, E, batch, fanouts, seed, device_F=24)
+
+
+def _sampled_layers_case(tmp_path, V, E, batch, fanouts, seed, device_F):
     rng = np.random.default_rng(seed)
     gsrc = rng.integers(0, V, E).astype(np.uint32)
     gdst = np.minimum((rng.random(E) ** 2 * V).astype(np.uint32), V - 1)
@@ -164,7 +180,10 @@ def test_oracle_matches_the_reference_sampled_layer_construction(tmp_path, V, E,
         ri = np.concatenate(picks).astype(np.uint32) if picks else np.zeros(0, np.uint32)
         layers.append(dict(dst=dst, co=np.array(co, dtype=np.uint32), ri=ri))
         dst = np.unique(ri)  # the next hop's destinations are this hop's sources (ascending ids)
-    ref = refops.run_sampled_layers(gsrc, gdst, V, layers, tmp_path)
+        if device_F:
+            layers[-1]["x"] = rng.standard_normal((dst.size, device_F)).astype(np.float32)
+            layers[-1]["g"] = rng.standard_normal((layers[-1]["dst"].size, device_F)).astype(np.float32)
+    ref = refops.run_sampled_layers(gsrc, gdst, V, layers, tmp_path, device_F=device_F)
     for layer, want in zip(layers, ref):
         local, source, n_src = oracle.postprocess(layer["ri"], V)
         assert n_src == want["source"].size
@@ -175,3 +194,11 @@ def test_oracle_matches_the_reference_sampled_layer_construction(tmp_path, V, E,
         ewf, ewb = oracle.layer_weights(layer["co"], local, ro, ci, source, layer["dst"], outd, ind)
         assert ewf.tobytes() == want["edge_weight_forward"].tobytes()
         assert ewb.tobytes() == want["edge_weight_backward"].tobytes()
+        if device_F:
+            Vd = layer["dst"].size
+            for got, x, w, off, idx, rows in ((want["fwd"], layer["x"], ewf, layer["co"], local, Vd),
+                                              (want["bwd"], layer["g"], ewb, ro, ci, n_src)):
+                expect = oracle.spmm(x, w, off, idx, rows, fused=True)
+                one_wave = np.diff(off.astype(np.int64)) <= (1024 if idx.size >= 1 << 16 else idx.size)
+                assert got[one_wave].tobytes() == expect[one_wave].tobytes()
+                check(got, expect, abs_term_scale(x, w, off, idx, rows))
