@@ -307,6 +307,50 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
                              const uint32_t *graph_ri, const uint32_t *dst, uint32_t n, int32_t fanout,
                              uint64_t seed, nts_stream_t stream);
 
+/* All layers of one mini-batch in one stream-ordered sequence, with no host step between the hops:
+ * for every hop init_dst, init_co, the neighbour pick, sampCSC::postprocessing,
+ * generate_csr_from_csc, update_degree and compute_weight_forward / backward (Sampler::sample_one,
+ * core/ntsSampler.hpp:843-1106; core/coocsc.hpp:136-450).  The reference sizes each hop's arrays on
+ * the host from the previous hop's result and copies eight arrays per layer to the device
+ * (core/coocsc.hpp:737-773); here the arrays live in one caller-provided device arena laid out for
+ * the largest batch, the kernels read the live counts from the device, and the host learns the
+ * layer shapes from ONE read-back per batch.  Every array equals what the per-hop entry points
+ * above give with seeds seed, seed + 1, ... for hops 0, 1, ... (hop 0 = the batch's own hop).
+ *
+ *   fanouts[h]   fanout of hop h, hop 0 first (the output-side hop); < 0 = whole neighbourhood, in
+ *                which case the batch must not repeat a vertex
+ *   arena        nts_batch_builder_arena_bytes(...) bytes of 256-byte-aligned device memory, owned by
+ *                the caller, in use until nts_batch_builder_destroy; graph_co / graph_ri likewise
+ *   nts_batch_builder_sample  enqueues everything on `stream` and returns; n <= max_batch
+ *   nts_batch_builder_layers  waits for that batch and fills layers[0 .. hops): index 0 is the
+ *                input-side layer (its `source` indexes the feature gather), index hops-1 the
+ *                layer whose `destination` is the batch -- the order of SampledSubgraph::sampled_sgs.
+ *                Pointers address the arena and stay valid until the next nts_batch_builder_sample
+ *                on the same builder; a pipeline that samples batch k+1 while batch k trains uses
+ *                one builder per stage in flight, as the reference uses one SampledSubgraph each. */
+typedef struct nts_batch_builder nts_batch_builder_t;
+typedef struct nts_sampled_layer {
+  uint32_t v_size, e_size, src_size, reserved; /* destinations, edges, distinct sources */
+  uint32_t *destination;                       /* [v_size]   global ids                        */
+  uint32_t *source;                            /* [src_size] global ids, ascending             */
+  uint32_t *column_offset;                     /* [v_size+1]                                   */
+  uint32_t *row_indices;                       /* [e_size]   LOCAL source index                */
+  uint32_t *row_offset;                        /* [src_size+1]                                 */
+  uint32_t *column_indices;                    /* [e_size]   local destination index           */
+  uint32_t *csr_to_csc;                        /* [e_size]   CSC position of CSR edge k, or NULL */
+  float *edge_weight_forward;                  /* [e_size]   CSC order                         */
+  float *edge_weight_backward;                 /* [e_size]   CSR order                         */
+} nts_sampled_layer_t;
+size_t nts_batch_builder_arena_bytes(uint32_t V, uint32_t graph_edges, const int32_t *fanouts, uint32_t hops,
+                                     uint32_t max_batch, int want_perm);
+int nts_batch_builder_create(nts_batch_builder_t **builder, const uint32_t *graph_co, const uint32_t *graph_ri,
+                             uint32_t V, uint32_t graph_edges, const int32_t *fanouts, uint32_t hops,
+                             uint32_t max_batch, int want_perm, void *arena, size_t arena_bytes);
+int nts_batch_builder_sample(nts_batch_builder_t *builder, const uint32_t *batch_ids, uint32_t n, uint64_t seed,
+                             nts_stream_t stream);
+int nts_batch_builder_layers(nts_batch_builder_t *builder, nts_sampled_layer_t *layers);
+int nts_batch_builder_destroy(nts_batch_builder_t *builder);
+
 /* sampCSC::postprocessing (core/coocsc.hpp:338-424): the sampled edges' GLOBAL source ids
  * (values < V) are marked in a bitmap; `source` receives the set bits in ascending order (the
  * distinct sampled sources), *n_source (device) their count, and local[e] the position of

@@ -76,6 +76,12 @@ SIGNATURES = {
     "nts_sample_hop_work_bytes": [_u32],
     "nts_sample_hop_offsets": [_vp, _vp, _vp, _u32, ctypes.c_int32, _vp, _vp],
     "nts_sample_hop_neighbors": [_vp, _vp, _vp, _vp, _vp, _u32, ctypes.c_int32, ctypes.c_uint64, _vp],
+    "nts_batch_builder_arena_bytes": [_u32, _u32, ctypes.POINTER(ctypes.c_int32), _u32, _u32, _int],
+    "nts_batch_builder_create": [ctypes.POINTER(_vp), _vp, _vp, _u32, _u32, ctypes.POINTER(ctypes.c_int32), _u32, _u32,
+                                 _int, _vp, _sz],
+    "nts_batch_builder_sample": [_vp, _vp, _u32, _u64, _vp],
+    "nts_batch_builder_layers": [_vp, _vp],
+    "nts_batch_builder_destroy": [_vp],
     "nts_relabel_sources_work_bytes": [_u32],
     "nts_relabel_sources": [_vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp],
     "nts_csr_from_csc_work_bytes": [_u32, _u32, _u32],
@@ -94,10 +100,18 @@ SIGNATURES = {
 }
 _RESTYPES = {"nts_last_error": ctypes.c_char_p, "nts_csr_from_csc_work_bytes": _sz,
              "nts_relabel_sources_work_bytes": _sz, "nts_sample_hop_work_bytes": _sz,
-             "nts_chunk_from_edges_work_bytes": _sz}
+             "nts_chunk_from_edges_work_bytes": _sz, "nts_batch_builder_arena_bytes": _sz}
 # Entry points whose int result is a value, not a status.
 _NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
-              "nts_sample_hop_work_bytes", "nts_chunk_from_edges_work_bytes"}
+              "nts_sample_hop_work_bytes", "nts_chunk_from_edges_work_bytes", "nts_batch_builder_arena_bytes"}
+
+
+class SampledLayerDesc(ctypes.Structure):
+    """nts_sampled_layer_t of include/nts_hip.h."""
+    _fields_ = [("v_size", _u32), ("e_size", _u32), ("src_size", _u32), ("reserved", _u32),
+                ("destination", _vp), ("source", _vp), ("column_offset", _vp), ("row_indices", _vp),
+                ("row_offset", _vp), ("column_indices", _vp), ("csr_to_csc", _vp),
+                ("edge_weight_forward", _vp), ("edge_weight_backward", _vp)]
 
 
 class NtsError(RuntimeError):

@@ -5,8 +5,8 @@ import ctypes
 
 import torch
 
-from .abi import call, ptr
-from .layout import as_u32
+from .abi import SampledLayerDesc, call, ptr
+from .layout import SampledLayer, as_u32
 from .stream import CudaStream
 
 
@@ -104,5 +104,98 @@ def sample_hop(graph_co, graph_ri, dst, fanout, seed):
     call("nts_sample_hop_offsets", ptr(co), ptr(graph_co), ptr(dst), n, fanout, base, stream)
     E = int(co[-1].item()) & 0xFFFFFFFF  # one read-back: sizes the edge array
     ri = torch.empty(E, dtype=torch.int32, device=device)
-    call("nts_sample_hop_neighbors", ptr(ri), ptr(co), ptr(graph_co), ptr(graph_ri), ptr(dst), n, fanout, seed, stream)
+    if E:
+        call("nts_sample_hop_neighbors", ptr(ri), ptr(co), ptr(graph_co), ptr(graph_ri), ptr(dst), n, fanout, seed,
+             stream)
     return co, ri
+
+
+class DevArray:
+    """A typed range of device memory inside a larger torch allocation: what `ptr()` and the
+    operators need (address, device, element count) without creating a tensor per array and batch."""
+    __slots__ = ("owner", "address", "count", "dtype")
+
+    def __init__(self, owner, address, count, dtype):
+        self.owner, self.address, self.count, self.dtype = owner, address, count, dtype
+
+    def data_ptr(self):
+        return self.address
+
+    def numel(self):
+        return self.count
+
+    @property
+    def device(self):
+        return self.owner.device
+
+    def tensor(self):
+        start = self.address - self.owner.data_ptr()
+        return self.owner[start:start + 4 * self.count].view(self.dtype)
+
+    def cpu(self):
+        return self.tensor().cpu()
+
+
+class BatchBuilder:
+    """All layers of a mini-batch built on the device without a host step between the hops
+    (nts_batch_builder_*): the whole of Sampler::sample_one's construction for every hop
+    (core/ntsSampler.hpp:843-1106), one read-back of the layer shapes per batch.
+
+    graph_co / graph_ri: int32 device tensors (uint32 bit patterns) of the whole graph's CSC;
+    fanouts: hop 0 (the batch's own hop) first.  The layers returned by `sample` are views into
+    this object's arena: they are overwritten by the next `sample`."""
+
+    def __init__(self, graph_co, graph_ri, fanouts, max_batch, want_perm=False):
+        self.device = graph_co.device
+        self.graph_co, self.graph_ri = graph_co, graph_ri
+        self.hops = len(fanouts)
+        V, E = graph_co.numel() - 1, graph_ri.numel()
+        fan = (ctypes.c_int32 * self.hops)(*fanouts)
+        nbytes = call("nts_batch_builder_arena_bytes", V, E, fan, self.hops, max_batch, int(want_perm))
+        if nbytes == 0:
+            raise ValueError("nts_batch_builder_arena_bytes: unsupported configuration")
+        self.arena = torch.empty(nbytes + 256, dtype=torch.uint8, device=self.device)
+        self._skew = (-self.arena.data_ptr()) % 256
+        handle = ctypes.c_void_p()
+        call("nts_batch_builder_create", ctypes.byref(handle), ptr(graph_co), ptr(graph_ri), V, E, fan, self.hops,
+             max_batch, int(want_perm), self.arena.data_ptr() + self._skew, nbytes)
+        self.handle = handle.value
+        self._desc = (SampledLayerDesc * self.hops)()
+
+    def _array(self, address, count, dtype):
+        return DevArray(self.arena, address, count, dtype) if address else None
+
+    def sample(self, batch_ids, seed):
+        """batch_ids: int32 device tensor.  Returns the SampledLayer list, input-side layer first;
+        the arrays are DevArray ranges of the arena (`.tensor()` gives a torch view)."""
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        call("nts_batch_builder_sample", self.handle, ptr(batch_ids), batch_ids.numel(), seed, stream)
+        call("nts_batch_builder_layers", self.handle, ctypes.addressof(self._desc))
+        layers = []
+        i32, f32 = torch.int32, torch.float32
+        for d in self._desc:
+            layer = SampledLayer()
+            Vd, E, Vs = d.v_size, d.e_size, d.src_size
+            layer.v_size, layer.e_size, layer.src_size = Vd, E, Vs
+            layer.dev_destination = self._array(d.destination, Vd, i32)
+            layer.dev_source = self._array(d.source, Vs, i32)
+            layer.dev_column_offset = self._array(d.column_offset, Vd + 1, i32)
+            layer.dev_row_indices = self._array(d.row_indices, E, i32)
+            layer.dev_row_offset = self._array(d.row_offset, Vs + 1, i32)
+            layer.dev_column_indices = self._array(d.column_indices, E, i32)
+            layer.dev_csr_to_csc = self._array(d.csr_to_csc, E, i32)
+            layer.dev_edge_weight_forward = self._array(d.edge_weight_forward, E, f32)
+            layer.dev_edge_weight_backward = self._array(d.edge_weight_backward, E, f32)
+            layers.append(layer)
+        return layers
+
+    def close(self):
+        if self.handle:
+            call("nts_batch_builder_destroy", self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -33,6 +33,52 @@ inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintp
 
 inline uint32_t ceil_div(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
 
+// A count that kernels need: known on the host (`n` null, value = `cap`), or produced earlier in the
+// same stream and read on the device -- the word `*n`, or `off[*n]` when `off` is set (an offsets
+// array indexed by a live row count, i.e. an edge total).  Device values are clamped to the
+// capacities the host sized grids and buffers for, so a kernel never indexes past them.
+struct DevCount {
+  uint32_t cap;
+  const uint32_t *n;
+  const uint32_t *off;
+  uint32_t n_cap;
+#if defined(__HIPCC__)
+  __device__ __forceinline__ uint32_t get() const {
+    if (!n) return cap;
+    uint32_t v = *n;
+    if (off) v = off[v < n_cap ? v : n_cap];
+    return v < cap ? v : cap;
+  }
+#endif
+};
+inline DevCount host_count(uint32_t v) { return DevCount{v, nullptr, nullptr, 0}; }
+inline DevCount device_count(const uint32_t *n, uint32_t cap) { return DevCount{cap, n, nullptr, 0}; }
+inline DevCount device_edge_count(const uint32_t *off, const uint32_t *n, uint32_t n_cap, uint32_t cap) {
+  return DevCount{cap, n, off, n_cap};
+}
+
+// Steps of a sampled layer's construction with sizes that may live on the device (sampler.hip,
+// layout.hip); the C entry points pass host counts, the batch builder device counts.
+int hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, DevCount n, int32_t fanout, void *scan_tmp,
+                size_t scan_tmp_bytes, hipStream_t stream);
+int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co, const uint32_t *graph_ri,
+                  const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, uint64_t seed, uint32_t *mark_bits,
+                  hipStream_t stream);
+size_t hop_scan_bytes(uint32_t n);
+// fill_to > E: local[E .. fill_to) = fill_value (padding for a sort over a fixed capacity);
+// n_source_copy / e_out (nullable) receive the source count again / the edge count.  marked: the
+// bitmap at the start of `work` already holds the ids' bits (hop_neighbors wrote them).
+int relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *n_source_copy, uint32_t *local,
+                    const uint32_t *global_ids, DevCount E, uint32_t fill_to, uint32_t fill_value, uint32_t *e_out,
+                    uint32_t V, void *work, bool marked, hipStream_t stream);
+// Sorts sort_n keys of key_bits bits (sort_n = E.cap, padded entries sort last).
+int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, DevCount Vd,
+                 DevCount Vs, DevCount E, uint32_t sort_n, unsigned key_bits, void *work, hipStream_t stream);
+size_t csr_from_csc_bytes(uint32_t sort_n);
+int gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t *ri, const uint32_t *ro,
+                     const uint32_t *ci, DevCount Vd, DevCount Vs, uint32_t *clear, uint32_t clear_words,
+                     hipStream_t stream);
+
 #if defined(__HIPCC__)
 // Value of `v` held by wavefront lane `lane` (lane must be wave-uniform); result is an SGPR.
 __device__ __forceinline__ uint32_t wave_read(uint32_t v, uint32_t lane) {

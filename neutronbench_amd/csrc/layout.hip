@@ -7,6 +7,7 @@
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
+#include <rocprim/iterator/transform_iterator.hpp>
 
 #include "common.hpp"
 
@@ -15,11 +16,11 @@ namespace {
 
 // ro[s] = number of sorted keys < s, for s in [0, Vs]; keys ascending, E of them.
 __global__ __launch_bounds__(256) void offsets_from_sorted_kernel(uint32_t *__restrict__ ro,
-                                                                  const uint32_t *__restrict__ keys, uint32_t Vs,
-                                                                  uint32_t E) {
+                                                                  const uint32_t *__restrict__ keys, DevCount Vs,
+                                                                  DevCount E) {
   const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
-  if (s > Vs) return;
-  uint32_t lo = 0, hi = E;  // first position whose key >= s
+  if (s > Vs.get()) return;
+  uint32_t lo = 0, hi = E.get();  // first position whose key >= s
   while (lo < hi) {
     const uint32_t mid = lo + (hi - lo) / 2;
     if (keys[mid] < s) lo = mid + 1; else hi = mid;
@@ -27,12 +28,24 @@ __global__ __launch_bounds__(256) void offsets_from_sorted_kernel(uint32_t *__re
   ro[s] = lo;
 }
 
-// ci[k] = destination that owns CSC edge perm[k].
-__global__ __launch_bounds__(256) void dst_of_perm_kernel(uint32_t *__restrict__ ci, const uint32_t *__restrict__ perm,
-                                                          const uint32_t *__restrict__ co, uint32_t Vd, uint32_t E) {
-  const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= E) return;
-  ci[k] = owner_of(co, Vd, perm[k]);
+// Both halves of the transposed structure from the sorted (source, CSC edge id) pairs in one launch:
+// thread t writes ro[t] (as above) when t <= Vs, and ci[t] = the destination that owns CSC edge
+// perm[t] when t < E.  perm may alias ci: each thread reads its own element before writing it.
+__global__ __launch_bounds__(256) void csr_finish_kernel(uint32_t *__restrict__ ro, uint32_t *ci,
+                                                         const uint32_t *__restrict__ keys, const uint32_t *perm,
+                                                         const uint32_t *__restrict__ co, DevCount Vd, DevCount Vs,
+                                                         DevCount edges) {
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t E = edges.get();
+  if (t <= Vs.get()) {
+    uint32_t lo = 0, hi = E;
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      if (keys[mid] < t) lo = mid + 1; else hi = mid;
+    }
+    ro[t] = lo;
+  }
+  if (t < E) ci[t] = owner_of(co, Vd.get(), perm[t]);
 }
 
 // 1 / ((float)sqrt((double)out_deg) * (float)sqrt((double)in_deg)) with every step rounded to
@@ -43,16 +56,30 @@ __device__ __forceinline__ float norm_weight(uint32_t out_deg, uint32_t in_deg) 
   return __fdiv_rn(1.0f, __fmul_rn(a, b));
 }
 
-// which = 0: CSC edges e, owner = destination, other end = ri[e] (a source).
-// which = 1: CSR edges k, owner = source, other end = ci[k] (a destination).
-// The edge count is read on the device (own_off[n_own]); threads stride over the edges.
-__global__ __launch_bounds__(256) void edge_weights_kernel(float *__restrict__ wout,
-                                                           const uint32_t *__restrict__ own_off, uint32_t n_own,
-                                                           const uint32_t *__restrict__ other_idx,
-                                                           const uint32_t *__restrict__ other_off, int which) {
-  const uint32_t E = own_off[n_own];
+// blockIdx.y (+ first) = 0: CSC edges e, owner = destination, other end = ri[e] (a source)   -> ewf
+//                        1: CSR edges k, owner = source, other end = ci[k] (a destination)    -> ewb
+// The edge count is read on the device (own_off[n_own]); threads stride over the edges.  `clear`
+// (nullable): `clear_words` words zeroed on the side for the caller's next step.
+__global__ __launch_bounds__(256) void edge_weights_kernel(float *__restrict__ ewf, float *__restrict__ ewb,
+                                                           const uint32_t *__restrict__ co,
+                                                           const uint32_t *__restrict__ ri,
+                                                           const uint32_t *__restrict__ ro,
+                                                           const uint32_t *__restrict__ ci, DevCount Vd, DevCount Vs,
+                                                           int first, uint32_t *__restrict__ clear,
+                                                           uint32_t clear_words) {
+  const int which = first + static_cast<int>(blockIdx.y);
   const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
-  for (uint64_t e = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; e < E; e += stride) {
+  const uint64_t start = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (clear && blockIdx.y == 0)
+    for (uint64_t w = start; w < clear_words; w += stride) clear[w] = 0;
+  const uint32_t *own_off = which == 0 ? co : ro;
+  const uint32_t *other_off = which == 0 ? ro : co;
+  const uint32_t *other_idx = which == 0 ? ri : ci;
+  float *wout = which == 0 ? ewf : ewb;
+  if (!wout) return;
+  const uint32_t n_own = which == 0 ? Vd.get() : Vs.get();
+  const uint32_t E = own_off[n_own];
+  for (uint64_t e = start; e < E; e += stride) {
     const uint32_t o = owner_of(own_off, n_own, static_cast<uint32_t>(e));
     const uint32_t own_deg = own_off[o + 1] - own_off[o];
     const uint32_t t = other_idx[e];
@@ -92,41 +119,55 @@ __global__ __launch_bounds__(256) void add_runs_kernel(float *__restrict__ out, 
 // ---- sampled-source relabelling (bitmap of sampled global ids -> sorted list + local ids) --------
 
 __global__ __launch_bounds__(256) void mark_bits_kernel(uint32_t *__restrict__ bits, const uint32_t *__restrict__ ids,
-                                                        uint32_t E) {
+                                                        DevCount E) {
   const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= E) return;
+  if (e >= E.get()) return;
   const uint32_t g = ids[e];
   atomicOr(&bits[g >> 5], 1u << (g & 31));  // integer OR: the result does not depend on the order
 }
 
-__global__ __launch_bounds__(256) void popcount_words_kernel(uint32_t *__restrict__ counts,
-                                                             const uint32_t *__restrict__ bits, uint32_t words) {
-  const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
-  if (w < words) counts[w] = __popc(bits[w]);
-}
+struct WordPopcount {
+  const uint32_t *bits;
+  __device__ uint32_t operator()(uint32_t w) const { return __popc(bits[w]); }
+};
+using PopcountIterator = rocprim::transform_iterator<rocprim::counting_iterator<uint32_t>, WordPopcount, uint32_t>;
 
-// source[prefix[w] + rank] = 32*w + bit for every set bit, ascending; the last word also stores the total.
-__global__ __launch_bounds__(256) void expand_bits_kernel(uint32_t *__restrict__ source,
-                                                          uint32_t *__restrict__ n_source,
-                                                          const uint32_t *__restrict__ bits,
-                                                          const uint32_t *__restrict__ prefix, uint32_t words) {
-  const uint32_t w = blockIdx.x * blockDim.x + threadIdx.x;
-  if (w >= words) return;
-  uint32_t word = bits[w];
-  uint32_t pos = prefix[w];
-  if (w + 1 == words) *n_source = pos + __popc(word);
-  while (word) {
-    const uint32_t b = __ffs(word) - 1;
-    source[pos++] = (w << 5) + b;
-    word &= word - 1;
+// Two independent uses of the bitmap and its per-word prefix in one launch.
+// Threads [0, words): source[prefix[w] + rank] = 32*w + bit for every set bit of word w, ascending;
+//   the last word also stores the total (twice when n_source_copy is set).
+// Threads words + e: local[e] = rank of ids[e] among the set bits, for e < E; local[e] = fill_value
+//   for E <= e < fill_to (padding for a sort over a fixed capacity); e_out (nullable) receives E.
+__global__ __launch_bounds__(256) void expand_relabel_kernel(uint32_t *__restrict__ source,
+                                                             uint32_t *__restrict__ n_source,
+                                                             uint32_t *__restrict__ n_source_copy,
+                                                             uint32_t *__restrict__ local,
+                                                             const uint32_t *__restrict__ ids,
+                                                             const uint32_t *__restrict__ bits,
+                                                             const uint32_t *__restrict__ prefix, uint32_t words,
+                                                             DevCount edges, uint32_t fill_to, uint32_t fill_value,
+                                                             uint32_t *__restrict__ e_out) {
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < words) {
+    uint32_t word = bits[t];
+    uint32_t pos = prefix[t];
+    if (t + 1 == words) {
+      *n_source = pos + __popc(word);
+      if (n_source_copy) *n_source_copy = pos + __popc(word);
+    }
+    while (word) {
+      const uint32_t b = __ffs(word) - 1;
+      source[pos++] = (t << 5) + b;
+      word &= word - 1;
+    }
+    return;
   }
-}
-
-__global__ __launch_bounds__(256) void relabel_kernel(uint32_t *__restrict__ local, const uint32_t *__restrict__ ids,
-                                                      const uint32_t *__restrict__ bits,
-                                                      const uint32_t *__restrict__ prefix, uint32_t E) {
-  const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= E) return;
+  const uint32_t e = t - words;
+  const uint32_t E = edges.get();
+  if (e == 0 && e_out) *e_out = E;
+  if (e >= E) {
+    if (e < fill_to) local[e] = fill_value;
+    return;
+  }
   const uint32_t g = ids[e];
   const uint32_t w = g >> 5;
   local[e] = prefix[w] + __popc(bits[w] & ((1u << (g & 31)) - 1u));
@@ -135,7 +176,8 @@ __global__ __launch_bounds__(256) void relabel_kernel(uint32_t *__restrict__ loc
 hipError_t scan_temp_bytes(uint32_t words, size_t *bytes) {
   size_t tmp = 0;
   uint32_t *nul = nullptr;
-  hipError_t err = rocprim::exclusive_scan(nullptr, tmp, nul, nul, 0u, words ? words : 1u, rocprim::plus<uint32_t>(),
+  PopcountIterator in(rocprim::counting_iterator<uint32_t>(0u), WordPopcount{nullptr});
+  hipError_t err = rocprim::exclusive_scan(nullptr, tmp, in, nul, 0u, words ? words : 1u, rocprim::plus<uint32_t>(),
                                            static_cast<hipStream_t>(nullptr), false);
   *bytes = tmp;
   return err;
@@ -153,8 +195,9 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 hipError_t sort_temp_bytes(uint32_t E, size_t *bytes) {
   size_t tmp = 0;
   uint32_t *nul = nullptr;
-  hipError_t err = rocprim::radix_sort_pairs(nullptr, tmp, nul, nul, rocprim::counting_iterator<uint32_t>(0u), nul,
-                                             E ? E : 1u, 0u, 32u, static_cast<hipStream_t>(nullptr), false);
+  hipError_t err = rocprim::radix_sort_pairs(nullptr, tmp, nul, nul,
+                                                              rocprim::counting_iterator<uint32_t>(0u), nul, E ? E : 1u,
+                                                              0u, 32u, static_cast<hipStream_t>(nullptr), false);
   *bytes = tmp;
   return err;
 }
@@ -179,6 +222,78 @@ hipError_t sort_pairs_temp_bytes(uint32_t E, size_t *bytes) {
 }
 
 }  // namespace
+
+size_t csr_from_csc_bytes(uint32_t sort_n) {
+  size_t tmp = 0;
+  if (sort_temp_bytes(sort_n, &tmp) != hipSuccess) return 0;
+  return align_up(static_cast<size_t>(sort_n) * sizeof(uint32_t), 256) + align_up(tmp, 256) + 256;
+}
+
+int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, DevCount Vd,
+                 DevCount Vs, DevCount E, uint32_t sort_n, unsigned key_bits, void *work, hipStream_t stream) {
+  unsigned char *w = static_cast<unsigned char *>(work);
+  uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(w);
+  size_t keys_bytes = align_up(static_cast<size_t>(sort_n) * sizeof(uint32_t), 256);
+  // Without a caller buffer for perm, ci doubles as the sorted edge-id array and is rewritten in
+  // place by a second pass (each thread reads its own element before writing it).
+  uint32_t *perm_out = perm ? perm : ci;
+  size_t tmp = 0;
+  NTS_HIP_TRY(sort_temp_bytes(sort_n, &tmp));
+  // Stable LSD radix sort of (local source, CSC edge id): edge ids stay ascending within a source,
+  // which is exactly the order the host counting sort produces.
+  NTS_HIP_TRY(rocprim::radix_sort_pairs(w + keys_bytes, tmp, ri, keys_sorted,
+                                                         rocprim::counting_iterator<uint32_t>(0u), perm_out, sort_n,
+                                                         0u, key_bits, stream, false));
+  const uint64_t span = static_cast<uint64_t>(Vs.cap) + 1 > E.cap ? static_cast<uint64_t>(Vs.cap) + 1 : E.cap;
+  hipLaunchKernelGGL(csr_finish_kernel, dim3(ceil_div(span, 256)), dim3(256), 0, stream, ro, ci, keys_sorted, perm_out,
+                     co, Vd, Vs, E);
+  NTS_LAUNCH_CHECK("csr_finish_kernel");
+  return NTS_OK;
+}
+
+int relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *n_source_copy, uint32_t *local,
+                    const uint32_t *global_ids, DevCount E, uint32_t fill_to, uint32_t fill_value, uint32_t *e_out,
+                    uint32_t V, void *work, bool marked, hipStream_t stream) {
+  const uint32_t words = (V + 31) / 32;
+  const size_t arr = align_up(static_cast<size_t>(words) * sizeof(uint32_t), 256);
+  unsigned char *w = static_cast<unsigned char *>(work);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(w);
+  uint32_t *prefix = reinterpret_cast<uint32_t *>(w + arr);
+  size_t tmp = 0;
+  NTS_HIP_TRY(scan_temp_bytes(words, &tmp));
+  if (!marked) {
+    if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
+    hipLaunchKernelGGL(mark_bits_kernel, dim3(ceil_div(E.cap, 256)), dim3(256), 0, stream, bits, global_ids, E);
+    NTS_LAUNCH_CHECK("mark_bits_kernel");
+  }
+  PopcountIterator counts(rocprim::counting_iterator<uint32_t>(0u), WordPopcount{bits});
+  NTS_HIP_TRY(rocprim::exclusive_scan(w + 2 * arr, tmp, counts, prefix, 0u, words, rocprim::plus<uint32_t>(), stream,
+                                      false));
+  const uint64_t span = static_cast<uint64_t>(words) + (fill_to > E.cap ? fill_to : E.cap);
+  hipLaunchKernelGGL(expand_relabel_kernel, dim3(ceil_div(span, 256)), dim3(256), 0, stream, source, n_source,
+                     n_source_copy, local, global_ids, bits, prefix, words, E, fill_to, fill_value, e_out);
+  NTS_LAUNCH_CHECK("expand_relabel_kernel");
+  return NTS_OK;
+}
+
+int gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t *ri, const uint32_t *ro,
+                     const uint32_t *ci, DevCount Vd, DevCount Vs, uint32_t *clear, uint32_t clear_words,
+                     hipStream_t stream) {
+  // The edge count lives on the device: the grid is sized from the vertex counts and the kernel
+  // strides over co[Vd] edges, so the call neither needs the count nor synchronises.  Forward and
+  // backward weights share one launch (grid.y).
+  uint64_t blocks = (static_cast<uint64_t>(Vd.cap > Vs.cap ? Vd.cap : Vs.cap) * 32 + 255) / 256;
+  if (blocks < 64) blocks = 64;
+  if (blocks > 8192) blocks = 8192;
+  if (!ewf && !ewb && !clear) return NTS_OK;
+  const int first = ewf ? 0 : 1;
+  const unsigned passes = (ewf && ewb) ? 2u : 1u;
+  hipLaunchKernelGGL(edge_weights_kernel, dim3(static_cast<unsigned>(blocks), passes), dim3(256), 0, stream, ewf, ewb, co,
+                     ri, ro, ci, Vd, Vs, first, clear, clear_words);
+  NTS_LAUNCH_CHECK("edge_weights_kernel");
+  return NTS_OK;
+}
+
 }  // namespace nts
 
 using namespace nts;
@@ -188,9 +303,7 @@ extern "C" {
 size_t nts_csr_from_csc_work_bytes(uint32_t Vd, uint32_t Vs, uint32_t E) {
   (void)Vd;
   (void)Vs;
-  size_t tmp = 0;
-  if (sort_temp_bytes(E, &tmp) != hipSuccess) return 0;
-  return align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256) + align_up(tmp, 256) + 256;
+  return csr_from_csc_bytes(E);
 }
 
 int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, uint32_t Vd,
@@ -201,25 +314,7 @@ int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t 
   }
   if (!ci || !co || !ri || !work) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: null pointer");
   if (!aligned_to(work, 256)) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: work must be 256-byte aligned");
-  unsigned char *w = static_cast<unsigned char *>(work);
-  uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(w);
-  size_t keys_bytes = align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256);
-  // Without a caller buffer for perm, ci doubles as the sorted edge-id array and is rewritten in
-  // place by a second pass (each thread reads its own element before writing it).
-  uint32_t *perm_out = perm ? perm : ci;
-  size_t tmp = 0;
-  NTS_HIP_TRY(sort_temp_bytes(E, &tmp));
-  // Stable LSD radix sort of (local source, CSC edge id): edge ids stay ascending within a source,
-  // which is exactly the order the host counting sort produces.
-  NTS_HIP_TRY(rocprim::radix_sort_pairs(w + keys_bytes, tmp, ri, keys_sorted,
-                                        rocprim::counting_iterator<uint32_t>(0u), perm_out, E, 0u, bits_for(Vs),
-                                        stream, false));
-  hipLaunchKernelGGL(offsets_from_sorted_kernel, dim3(ceil_div(static_cast<uint64_t>(Vs) + 1, 256)), dim3(256), 0,
-                     stream, ro, keys_sorted, Vs, E);
-  NTS_LAUNCH_CHECK("offsets_from_sorted_kernel");
-  hipLaunchKernelGGL(dst_of_perm_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, ci, perm_out, co, Vd, E);
-  NTS_LAUNCH_CHECK("dst_of_perm_kernel");
-  return NTS_OK;
+  return csr_from_csc(ro, ci, perm, co, ri, host_count(Vd), host_count(Vs), host_count(E), E, bits_for(Vs), work, stream);
 }
 
 size_t nts_chunk_from_edges_work_bytes(uint32_t V, uint32_t E) {
@@ -255,12 +350,12 @@ int nts_chunk_from_edges(uint32_t *co, uint32_t *ri, float *ewf, uint32_t *ro, u
   // The edge list ordered by source, file order kept inside a source (stable sort): the CSR rows.
   NTS_HIP_TRY(rocprim::radix_sort_pairs(tmp_ptr, tmp, a, c, b, ci, E, 0u, bits, stream, false));
   hipLaunchKernelGGL(offsets_from_sorted_kernel, dim3(ceil_div(static_cast<uint64_t>(V) + 1, 256)), dim3(256), 0,
-                     stream, ro, c, V, E);
+                     stream, ro, c, host_count(V), host_count(E));
   NTS_LAUNCH_CHECK("offsets_from_sorted_kernel(ro)");
   // That list re-ordered by destination, again stable: the CSC rows (sources ascending inside a row).
   NTS_HIP_TRY(rocprim::radix_sort_pairs(tmp_ptr, tmp, ci, a, c, ri, E, 0u, bits, stream, false));
   hipLaunchKernelGGL(offsets_from_sorted_kernel, dim3(ceil_div(static_cast<uint64_t>(V) + 1, 256)), dim3(256), 0,
-                     stream, co, a, V, E);
+                     stream, co, a, host_count(V), host_count(E));
   NTS_LAUNCH_CHECK("offsets_from_sorted_kernel(co)");
   if (ewf || ewb) return nts_gcn_edge_weights(ewf, ewb, co, ri, ro, ci, V, V, stream);
   return NTS_OK;
@@ -279,27 +374,8 @@ int nts_relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *local, c
   if (E == 0 || V == 0) return nts_memset_zero(n_source, sizeof(uint32_t), stream);
   if (!source || !local || !global_ids || !work) return fail(NTS_ERR_INVALID, "nts_relabel_sources: null pointer");
   if (!aligned_to(work, 256)) return fail(NTS_ERR_INVALID, "nts_relabel_sources: work must be 256-byte aligned");
-  const uint32_t words = (V + 31) / 32;
-  const size_t arr = align_up(static_cast<size_t>(words) * sizeof(uint32_t), 256);
-  unsigned char *w = static_cast<unsigned char *>(work);
-  uint32_t *bits = reinterpret_cast<uint32_t *>(w);
-  uint32_t *counts = reinterpret_cast<uint32_t *>(w + arr);
-  uint32_t *prefix = reinterpret_cast<uint32_t *>(w + 2 * arr);
-  size_t tmp = 0;
-  NTS_HIP_TRY(scan_temp_bytes(words, &tmp));
-  if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
-  hipLaunchKernelGGL(mark_bits_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, bits, global_ids, E);
-  NTS_LAUNCH_CHECK("mark_bits_kernel");
-  hipLaunchKernelGGL(popcount_words_kernel, dim3(ceil_div(words, 256)), dim3(256), 0, stream, counts, bits, words);
-  NTS_LAUNCH_CHECK("popcount_words_kernel");
-  NTS_HIP_TRY(rocprim::exclusive_scan(w + 3 * arr, tmp, counts, prefix, 0u, words, rocprim::plus<uint32_t>(), stream,
-                                      false));
-  hipLaunchKernelGGL(expand_bits_kernel, dim3(ceil_div(words, 256)), dim3(256), 0, stream, source, n_source, bits,
-                     prefix, words);
-  NTS_LAUNCH_CHECK("expand_bits_kernel");
-  hipLaunchKernelGGL(relabel_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, local, global_ids, bits, prefix, E);
-  NTS_LAUNCH_CHECK("relabel_kernel");
-  return NTS_OK;
+  return relabel_sources(source, n_source, nullptr, local, global_ids, host_count(E), 0, 0, nullptr, V, work, false,
+                         stream);
 }
 
 int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t *ri, const uint32_t *co,
@@ -322,8 +398,9 @@ int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t
   hipLaunchKernelGGL(target_keys_kernel, dim3(ceil_div(E, 256)), dim3(256), 0, stream, keys, ri, mirror, E);
   hipError_t err = hipGetLastError();
   if (err == hipSuccess)
-    err = rocprim::radix_sort_pairs(work + 3 * arr, tmp, keys, keys_sorted, rocprim::counting_iterator<uint32_t>(0u),
-                                    perm, E, 0u, 32u, stream, false);
+    err = rocprim::radix_sort_pairs(work + 3 * arr, tmp, keys, keys_sorted,
+                                                     rocprim::counting_iterator<uint32_t>(0u), perm, E, 0u, 32u, stream,
+                                                     false);
   if (err == hipSuccess) {
     hipLaunchKernelGGL(add_runs_kernel, dim3(ceil_div(E, 4)), dim3(256), 0, stream, out, msg, keys_sorted, perm, E, F);
     err = hipGetLastError();
@@ -338,23 +415,9 @@ int nts_gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint3
                          const uint32_t *ci, uint32_t Vd, uint32_t Vs, nts_stream_t stream) {
   if (!co || !ro) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null offsets");
   if (Vd == 0 || Vs == 0) return NTS_OK;
-  // The edge count lives on the device: the grid is sized from the vertex counts and the kernel
-  // strides over co[Vd] edges, so the call neither needs the count nor synchronises.
-  uint64_t blocks = (static_cast<uint64_t>(Vd > Vs ? Vd : Vs) * 32 + 255) / 256;
-  if (blocks < 64) blocks = 64;
-  if (blocks > 8192) blocks = 8192;
-  const dim3 grid(static_cast<unsigned>(blocks));
-  if (ewf) {
-    if (!ri) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ri");
-    hipLaunchKernelGGL(edge_weights_kernel, grid, dim3(256), 0, stream, ewf, co, Vd, ri, ro, 0);
-    NTS_LAUNCH_CHECK("edge_weights_kernel(fwd)");
-  }
-  if (ewb) {
-    if (!ci) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ci");
-    hipLaunchKernelGGL(edge_weights_kernel, grid, dim3(256), 0, stream, ewb, ro, Vs, ci, co, 1);
-    NTS_LAUNCH_CHECK("edge_weights_kernel(bwd)");
-  }
-  return NTS_OK;
+  if (ewf && !ri) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ri");
+  if (ewb && !ci) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ci");
+  return gcn_edge_weights(ewf, ewb, co, ri, ro, ci, host_count(Vd), host_count(Vs), nullptr, 0, stream);
 }
 
 }  // extern "C"

@@ -9,6 +9,8 @@
 // ascending position order, which keeps source ids ascending inside a destination for graphs with
 // sorted adjacency.  Results depend only on the arguments: the same seed gives the same sample.
 #include <rocprim/device/device_scan.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
+#include <rocprim/iterator/transform_iterator.hpp>
 
 #include "common.hpp"
 
@@ -24,20 +26,21 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   return z ^ (z >> 31);
 }
 
-__global__ __launch_bounds__(256) void hop_counts_kernel(uint32_t *__restrict__ counts,
-                                                         const uint32_t *__restrict__ graph_co,
-                                                         const uint32_t *__restrict__ dst, uint32_t n,
-                                                         int32_t fanout) {
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i > n) return;
-  if (i == n) {
-    counts[n] = 0;  // the exclusive scan turns this last slot into the edge total
-    return;
+// min(in-degree, fanout) of destination slot i; 0 from the live count on, so that an exclusive scan
+// over cap + 1 slots leaves the edge total in every slot from the live count up.
+struct HopCount {
+  const uint32_t *graph_co;
+  const uint32_t *dst;
+  DevCount n;
+  int32_t fanout;
+  __device__ uint32_t operator()(uint32_t i) const {
+    if (i >= n.get()) return 0;
+    const uint32_t d = dst[i];
+    const uint32_t deg = graph_co[d + 1] - graph_co[d];
+    return (fanout < 0 || deg < static_cast<uint32_t>(fanout)) ? deg : static_cast<uint32_t>(fanout);
   }
-  const uint32_t d = dst[i];
-  const uint32_t deg = graph_co[d + 1] - graph_co[d];
-  counts[i] = (fanout < 0 || deg < static_cast<uint32_t>(fanout)) ? deg : static_cast<uint32_t>(fanout);
-}
+};
+using HopCountIterator = rocprim::transform_iterator<rocprim::counting_iterator<uint32_t>, HopCount, uint32_t>;
 
 // True if `pred` holds on any lane of the caller's aligned group of G lanes (all of them active).
 template <int G>
@@ -46,6 +49,14 @@ __device__ __forceinline__ bool group_any(bool pred) {
   if (G == kWave) return votes != 0;
   const uint32_t first = (threadIdx.x & (kWave - 1)) & ~static_cast<uint32_t>(G - 1);
   return ((votes >> first) & ((1ull << G) - 1ull)) != 0;
+}
+
+// Stores one sampled source id; with `mark` also sets its bit in the bitmap of sampled sources
+// (integer OR: the result does not depend on the order), which saves the relabelling a pass.
+__device__ __forceinline__ void emit(uint32_t *__restrict__ ri_out, uint32_t *__restrict__ mark, uint32_t pos,
+                                     uint32_t g) {
+  ri_out[pos] = g;
+  if (mark) atomicOr(&mark[g >> 5], 1u << (g & 31));
 }
 
 // A group of G lanes per destination (G = power of two >= the fanout, at most one wavefront).
@@ -63,18 +74,20 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
                                                        const uint32_t *__restrict__ co,
                                                        const uint32_t *__restrict__ graph_co,
                                                        const uint32_t *__restrict__ graph_ri,
-                                                       const uint32_t *__restrict__ dst, uint32_t n, int32_t fanout,
-                                                       uint64_t seed) {
+                                                       const uint32_t *__restrict__ dst, DevCount n,
+                                                       uint32_t edge_cap, int32_t fanout, uint64_t seed,
+                                                       uint32_t *__restrict__ mark) {
   const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) / G;
-  if (i >= n) return;  // whole groups leave together
+  if (i >= n.get()) return;  // whole groups leave together
   const uint32_t gl = threadIdx.x & (G - 1);
   const uint32_t d = dst[i];
   const uint32_t base = graph_co[d];
   const uint32_t deg = graph_co[d + 1] - base;
   const uint32_t out = co[i];
   const uint32_t take = co[i + 1] - out;
+  if (co[i + 1] > edge_cap) return;  // never past the edge array (a full-neighbourhood batch that repeats vertices)
   if (take == deg) {  // full neighbourhood, in CSC order
-    for (uint32_t k = gl; k < deg; k += G) ri_out[out + k] = graph_ri[base + k];
+    for (uint32_t k = gl; k < deg; k += G) emit(ri_out, mark, out + k, graph_ri[base + k]);
     return;
   }
   const uint64_t state0 = mix64(seed ^ (static_cast<uint64_t>(i) << 32) ^ d);
@@ -83,7 +96,8 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
     // construction), emitted in ascending position order: [0, wrap) then [start, start + take - wrap).
     const uint32_t start = static_cast<uint32_t>(state0 % deg);
     const uint32_t wrap = start + take > deg ? start + take - deg : 0;
-    for (uint32_t k = gl; k < take; k += G) ri_out[out + k] = graph_ri[base + (k < wrap ? k : start + (k - wrap))];
+    for (uint32_t k = gl; k < take; k += G)
+      emit(ri_out, mark, out + k, graph_ri[base + (k < wrap ? k : start + (k - wrap))]);
     return;
   }
   // Lane gl < take: step j = deg - take + gl, hash chain advanced gl + 1 times.
@@ -101,14 +115,15 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
   if (gl < take) {
     uint32_t rank = 0;
     for (uint32_t q = 0; q < take; ++q) rank += __shfl(v, q, G) < v ? 1u : 0u;
-    ri_out[out + rank] = graph_ri[base + v];
+    emit(ri_out, mark, out + rank, graph_ri[base + v]);
   }
 }
 
 hipError_t scan_bytes(uint32_t n, size_t *bytes) {
   size_t tmp = 0;
   uint32_t *nul = nullptr;
-  hipError_t err = rocprim::exclusive_scan(nullptr, tmp, nul, nul, 0u, n ? n : 1u, rocprim::plus<uint32_t>(),
+  HopCountIterator in(rocprim::counting_iterator<uint32_t>(0u), HopCount{nullptr, nullptr, host_count(0), 0});
+  hipError_t err = rocprim::exclusive_scan(nullptr, tmp, in, nul, 0u, n ? n : 1u, rocprim::plus<uint32_t>(),
                                            static_cast<hipStream_t>(nullptr), false);
   *bytes = tmp;
   return err;
@@ -117,42 +132,24 @@ hipError_t scan_bytes(uint32_t n, size_t *bytes) {
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
-}  // namespace nts
 
-using namespace nts;
-
-extern "C" {
-
-size_t nts_sample_hop_work_bytes(uint32_t n) {
+size_t hop_scan_bytes(uint32_t n) {
   size_t tmp = 0;
-  if (scan_bytes(n + 1, &tmp) != hipSuccess) return 0;
-  return align_up((static_cast<size_t>(n) + 1) * sizeof(uint32_t), 256) + align_up(tmp, 256) + 256;
+  return scan_bytes(n + 1, &tmp) == hipSuccess ? tmp : 0;
 }
 
-int nts_sample_hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, uint32_t n, int32_t fanout,
-                           void *work, nts_stream_t stream) {
-  if (!co) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: null co");
-  if (n == 0) return nts_memset_zero(co, sizeof(uint32_t), stream);
-  if (!graph_co || !dst || !work) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: null pointer");
-  if (!aligned_to(work, 256)) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: work must be 256-byte aligned");
-  unsigned char *w = static_cast<unsigned char *>(work);
-  uint32_t *counts = reinterpret_cast<uint32_t *>(w);
-  const size_t arr = align_up((static_cast<size_t>(n) + 1) * sizeof(uint32_t), 256);
-  size_t tmp = 0;
-  NTS_HIP_TRY(scan_bytes(n + 1, &tmp));
-  hipLaunchKernelGGL(hop_counts_kernel, dim3(ceil_div(static_cast<uint64_t>(n) + 1, 256)), dim3(256), 0, stream, counts,
-                     graph_co, dst, n, fanout);
-  NTS_LAUNCH_CHECK("hop_counts_kernel");
-  NTS_HIP_TRY(rocprim::exclusive_scan(w + arr, tmp, counts, co, 0u, n + 1, rocprim::plus<uint32_t>(), stream, false));
+int hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, DevCount n, int32_t fanout, void *scan_tmp,
+                size_t scan_tmp_bytes, hipStream_t stream) {
+  // One scan whose input is computed on the fly; slot n.cap (count 0) receives the edge total.
+  HopCountIterator in(rocprim::counting_iterator<uint32_t>(0u), HopCount{graph_co, dst, n, fanout});
+  NTS_HIP_TRY(rocprim::exclusive_scan(scan_tmp, scan_tmp_bytes, in, co, 0u, n.cap + 1, rocprim::plus<uint32_t>(), stream,
+                                      false));
   return NTS_OK;
 }
 
-int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co,
-                             const uint32_t *graph_ri, const uint32_t *dst, uint32_t n, int32_t fanout, uint64_t seed,
-                             nts_stream_t stream) {
-  if (n == 0) return NTS_OK;
-  if (!ri_global || !co || !graph_co || !graph_ri || !dst)
-    return fail(NTS_ERR_INVALID, "nts_sample_hop_neighbors: null pointer");
+int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co, const uint32_t *graph_ri,
+                  const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, uint64_t seed, uint32_t *mark_bits,
+                  hipStream_t stream) {
   // Lanes per destination: the fanout rounded up to a power of two (full neighbourhoods and
   // fanouts above one wavefront are strided copies, for which a quarter wavefront serves well).
   int g = 8;
@@ -160,10 +157,10 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
     while (g < fanout) g <<= 1;
   else
     g = 16;
-  const dim3 grid(ceil_div(static_cast<uint64_t>(n) * g, 256));
+  const dim3 grid(ceil_div(static_cast<uint64_t>(n.cap) * g, 256));
 #define NTS_LAUNCH_PICK(G)                                                                                      \
   hipLaunchKernelGGL(hop_pick_kernel<G>, grid, dim3(256), 0, stream, ri_global, co, graph_co, graph_ri, dst, n, \
-                     fanout, seed)
+                     edge_cap, fanout, seed, mark_bits)
   switch (g) {
     case 8: NTS_LAUNCH_PICK(8); break;
     case 16: NTS_LAUNCH_PICK(16); break;
@@ -173,6 +170,39 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
 #undef NTS_LAUNCH_PICK
   NTS_LAUNCH_CHECK("hop_pick_kernel");
   return NTS_OK;
+}
+
+}  // namespace nts
+
+using namespace nts;
+
+extern "C" {
+
+size_t nts_sample_hop_work_bytes(uint32_t n) {
+  size_t tmp = 0;
+  if (scan_bytes(n + 1, &tmp) != hipSuccess) return 0;
+  return align_up(tmp, 256) + 256;
+}
+
+int nts_sample_hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, uint32_t n, int32_t fanout,
+                           void *work, nts_stream_t stream) {
+  if (!co) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: null co");
+  if (n == 0) return nts_memset_zero(co, sizeof(uint32_t), stream);
+  if (!graph_co || !dst || !work) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: null pointer");
+  if (!aligned_to(work, 256)) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: work must be 256-byte aligned");
+  size_t tmp = 0;
+  NTS_HIP_TRY(scan_bytes(n + 1, &tmp));
+  return hop_offsets(co, graph_co, dst, host_count(n), fanout, work, tmp, stream);
+}
+
+int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co,
+                             const uint32_t *graph_ri, const uint32_t *dst, uint32_t n, int32_t fanout, uint64_t seed,
+                             nts_stream_t stream) {
+  if (n == 0) return NTS_OK;
+  if (!ri_global || !co || !graph_co || !graph_ri || !dst)
+    return fail(NTS_ERR_INVALID, "nts_sample_hop_neighbors: null pointer");
+  return hop_neighbors(ri_global, co, graph_co, graph_ri, dst, host_count(n), 0xFFFFFFFFu, fanout, seed, nullptr,
+                       stream);
 }
 
 }  // extern "C"

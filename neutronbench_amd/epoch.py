@@ -10,7 +10,10 @@ Configurations (BASELINE.json configs 2, 4, 5):
             top 20 % out-degree nodes, fanout [15,10,5], batch 6,000, 196,615 train nodes
   gat       same graph, fanout [10,10], batch 4,096, 4 heads x 32, fused attention + aggregation fwd+bwd
 Everything goes through the C ABI: neighbour sampling of each hop, relabelling, CSR construction,
-weights, gathers, aggregation (--sampler harness uses the torch sampler of the test harness instead).  Stages are separated by
+weights, gathers, aggregation.  --sampler builder (default) builds all layers of a batch in one
+stream-ordered sequence with one read-back (nts_batch_builder_*; "sample" then holds sampling and
+structure together); --sampler library goes hop by hop through the per-step entry points;
+--sampler harness uses the torch sampler of the test harness instead.  Stages are separated by
 stream synchronisation, as every reference operator synchronises its stream.
 """
 import argparse
@@ -20,7 +23,7 @@ import time
 import torch
 
 from . import synth
-from .batch import FeatureCache, MappedHostTable, load_feature_gpu_cache, load_label_gpu, sample_hop
+from .batch import BatchBuilder, FeatureCache, MappedHostTable, load_feature_gpu_cache, load_label_gpu, sample_hop
 from .layout import SampledLayer, as_u32
 from .ops import GATAggregateOp, GATAttentionOp, SingleGPUSampleGraphOp
 from .stream import CudaStream
@@ -44,7 +47,7 @@ class Timer:
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
-def run(name, scale=1.0, max_batches=0, sampler="library"):
+def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2):
     cfg = dict(CONFIGS[name])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
@@ -66,14 +69,27 @@ def run(name, scale=1.0, max_batches=0, sampler="library"):
     if max_batches:
         n_batches = min(n_batches, max_batches)
     edges_total, hits_total, rows_total = 0, 0, 0
-    torch.cuda.synchronize()
+    builder = BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0) if sampler == "builder" else None
+    train32 = as_u32(train_nodes)
+    # The first batches load every kernel's code and grow the allocator's pools; they are run once
+    # untimed, then the epoch starts over from its first batch.
+    n_warm = min(warmup_batches, n_batches)
     t_epoch = time.perf_counter()
-    for b in range(n_batches):
+    for step, b in enumerate(list(range(n_warm)) + list(range(n_batches))):
+        if step == n_warm:
+            torch.cuda.synchronize()
+            tm.t.clear()
+            edges_total, hits_total, rows_total = 0, 0, 0
+            t_epoch = time.perf_counter()
         batch = train_nodes[b * cfg["batch"]:(b + 1) * cfg["batch"]]
         # -- sample (harness) + structure (library) -------------------------------------------
         layers = []
         dst_ids = batch
-        for hop, fan in enumerate(cfg["fanout"]):
+        if builder is not None:
+            t0 = time.perf_counter()
+            layers = builder.sample(train32[b * cfg["batch"]:(b + 1) * cfg["batch"]], 1000 * b)[::-1]
+            tm.add("sample", t0)
+        for hop, fan in enumerate(cfg["fanout"] if builder is None else []):
             t0 = time.perf_counter()
             if sampler == "library":
                 dst32 = dst_ids if dst_ids.dtype == torch.int32 else as_u32(dst_ids)
@@ -144,9 +160,10 @@ def run(name, scale=1.0, max_batches=0, sampler="library"):
     table.close()
     out = {
         "config": name, "scale": scale, "vertices": V, "edges": E, "batches": n_batches, "batch_size": cfg["batch"],
+        "warmup_batches": n_warm,
         "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
-        "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler == "library"), 4),
+        "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
         "sampler": sampler, "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
     }
@@ -159,6 +176,7 @@ if __name__ == "__main__":
     ap.add_argument("--config", choices=sorted(CONFIGS), required=True)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--max-batches", type=int, default=0)
-    ap.add_argument("--sampler", choices=["library", "harness"], default="library")
+    ap.add_argument("--sampler", choices=["builder", "library", "harness"], default="builder")
+    ap.add_argument("--warmup-batches", type=int, default=2, help="untimed batches before the epoch starts")
     a = ap.parse_args()
-    run(a.config, a.scale, a.max_batches, a.sampler)
+    run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches)

@@ -1,0 +1,153 @@
+"""Whole-batch construction on the device (nts_batch_builder_*) against the per-hop entry points and
+the CPU oracle: every array of every layer, bit for bit."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import host_u32
+from neutronbench_amd import abi, synth
+from neutronbench_amd.abi import call, ptr
+from neutronbench_amd.batch import BatchBuilder, sample_hop
+from neutronbench_amd.layout import SampledLayer, as_u32
+
+pytestmark = pytest.mark.gpu
+
+
+def graph(V, E, seed, device):
+    src, dst = synth.rmat_edges(V, E, seed=seed, device=device, sort=True)
+    co, ri = synth.build_csc(src, dst, V)
+    return as_u32(co), as_u32(ri)
+
+
+def per_hop_layers(gco, gri, batch, fanouts, seed, V):
+    """The same batch through the per-hop entry points (a read-back after every step)."""
+    layers, dst = [], batch
+    for h, fan in enumerate(fanouts):
+        co, ri = sample_hop(gco, gri, dst, fan, seed + h)
+        layers.append(SampledLayer.from_device_hop(co, ri, dst, V, want_perm=True))
+        dst = layers[-1].dev_source
+    return layers[::-1]
+
+
+ARRAYS = ("dev_destination", "dev_source", "dev_column_offset", "dev_row_indices", "dev_row_offset",
+          "dev_column_indices", "dev_csr_to_csc", "dev_edge_weight_forward", "dev_edge_weight_backward")
+
+
+def assert_same_layers(got, want):
+    assert len(got) == len(want)
+    for k, (a, b) in enumerate(zip(got, want)):
+        assert (a.v_size, a.e_size, a.src_size) == (b.v_size, b.e_size, b.src_size), f"layer {k}"
+        for name in ARRAYS:
+            x, y = getattr(a, name), getattr(b, name)
+            assert x.numel() == y.numel(), f"layer {k} {name}"
+            assert x.cpu().numpy().tobytes() == y.cpu().numpy().tobytes(), f"layer {k} {name}"
+
+
+@pytest.mark.parametrize("V,E,batch,fanouts,seed", [
+    (30000, 600000, 1024, [10, 25], 1),          # the Arxiv-shaped configuration's hops
+    (50000, 2000000, 3000, [5, 10, 15], 2),      # Products-shaped hops
+    (4000, 30000, 500, [3, 2, 2, 2], 3),         # more hops than layers of the configurations, sparse graph
+    (2000, 400000, 64, [64, 100], 4),            # fanout of a whole wavefront and the window pick above it
+    (3000, 40000, 700, [-1, 4], 5),              # whole neighbourhoods first
+])
+def test_builder_equals_the_per_hop_entry_points(device, V, E, batch, fanouts, seed):
+    gco, gri = graph(V, E, seed, device)
+    ids = as_u32(synth.permutation(V, seed + 10, device)[:batch])
+    builder = BatchBuilder(gco, gri, fanouts, batch, want_perm=True)
+    got = builder.sample(ids, 1000 * seed)
+    want = per_hop_layers(gco, gri, ids, fanouts, 1000 * seed, V)
+    assert_same_layers(got, want)
+    assert got[-1].dev_destination.cpu().numpy().tobytes() == ids.cpu().numpy().tobytes()
+    builder.close()
+
+
+def test_builder_layers_equal_the_oracle_construction(device):
+    """Directly against the restated host algorithms (postprocessing, generate_csr_from_csc,
+    update_degree + compute_weight_*) on the sampled lists the builder picked."""
+    V, E, batch, fanouts = 20000, 500000, 800, [6, 12]
+    gco, gri = graph(V, E, 21, device)
+    ids = as_u32(synth.permutation(V, 22, device)[:batch])
+    builder = BatchBuilder(gco, gri, fanouts, batch)
+    layers = builder.sample(ids, 5)
+    gco_h, gri_h = host_u32(gco), host_u32(gri)
+    dst = host_u32(ids)
+    for hop, layer in enumerate(layers[::-1]):
+        co = host_u32(layer.dev_column_offset)
+        assert np.array_equal(co, oracle.init_co(gco_h, dst, fanouts[hop]))
+        local, source = host_u32(layer.dev_row_indices), host_u32(layer.dev_source)
+        glob = source[local]
+        for i in range(0, dst.size, 37):  # sampled sources are in-neighbours of their destination
+            seg = gri_h[gco_h[dst[i]]:gco_h[dst[i] + 1]]
+            assert np.isin(glob[co[i]:co[i + 1]], seg).all()
+        want_local, want_source, n = oracle.postprocess(glob, V)
+        assert n == layer.src_size and np.array_equal(source, want_source) and np.array_equal(local, want_local)
+        ro, ci = oracle.csr_from_csc(co, local, n)
+        assert np.array_equal(host_u32(layer.dev_row_offset), ro)
+        assert np.array_equal(host_u32(layer.dev_column_indices), ci)
+        outd, ind = np.ones(V, np.uint32), np.ones(V, np.uint32)
+        ewf, ewb = oracle.layer_weights(co, local, ro, ci, source, dst, outd, ind)
+        assert layer.dev_ewf().cpu().numpy().tobytes() == ewf.tobytes()
+        assert layer.dev_ewb().cpu().numpy().tobytes() == ewb.tobytes()
+        assert layer.dev_csr_to_csc is None
+        dst = source
+    builder.close()
+
+
+def test_builder_reused_over_batches_of_changing_size(device):
+    """One builder, batches large -> tiny -> empty -> one vertex -> large: nothing of an earlier
+    batch shows in a later one (the arena keeps stale data beyond the live counts)."""
+    V, E, fanouts = 20000, 300000, [8, 8]
+    gco, gri = graph(V, E, 31, device)
+    # a few isolated vertices: no in-edges
+    deg = host_u32(gco)[1:] - host_u32(gco)[:-1]
+    isolated = np.nonzero(deg == 0)[0][:5]
+    perm = synth.permutation(V, 32, device)
+    builder = BatchBuilder(gco, gri, fanouts, 2048, want_perm=True)
+    batches = [perm[:2048], perm[100:103], perm[:0], perm[7:8], perm[2048:4096]]
+    if isolated.size:
+        batches.insert(2, torch.from_numpy(isolated.astype(np.int64)).to(device))
+    for k, ids64 in enumerate(batches):
+        ids = as_u32(ids64)
+        got = builder.sample(ids, 40 + k)
+        if ids.numel() == 0:
+            assert all((l.v_size, l.e_size, l.src_size) == (0, 0, 0) for l in got)
+            assert all(host_u32(l.dev_column_offset).tolist() == [0] and host_u32(l.dev_row_offset).tolist() == [0]
+                       for l in got)
+            continue
+        want = per_hop_layers(gco, gri, ids, fanouts, 40 + k, V)
+        assert_same_layers(got, want)
+    builder.close()
+
+
+def test_builder_rejects_what_it_cannot_hold(device):
+    gco, gri = graph(1000, 8000, 41, device)
+    V, E = 1000, 8000
+    fan = (ctypes.c_int32 * 2)(4, 4)
+    assert call("nts_batch_builder_arena_bytes", V, E, fan, 0, 16, 0) == 0
+    assert call("nts_batch_builder_arena_bytes", V, E, fan, 9, 16, 0) == 0
+    assert call("nts_batch_builder_arena_bytes", V, E, fan, 2, 0, 0) == 0
+    need = call("nts_batch_builder_arena_bytes", V, E, fan, 2, 16, 0)
+    arena = torch.empty(need + 256, dtype=torch.uint8, device=device)
+    base = (arena.data_ptr() + 255) // 256 * 256
+    handle = ctypes.c_void_p()
+    args = (ptr(gco), ptr(gri), V, E, fan, 2, 16, 0)
+    assert abi.status("nts_batch_builder_create", ctypes.byref(handle), *args, base, need - 1) == abi.NTS_ERR_INVALID
+    assert "arena" in abi.last_error()
+    assert abi.status("nts_batch_builder_create", ctypes.byref(handle), *args, base + 4, need) == abi.NTS_ERR_INVALID
+    zero = (ctypes.c_int32 * 2)(4, 0)
+    assert abi.status("nts_batch_builder_create", ctypes.byref(handle), ptr(gco), ptr(gri), V, E, zero, 2, 16, 0, base,
+                      need) == abi.NTS_ERR_INVALID
+    call("nts_batch_builder_create", ctypes.byref(handle), *args, base, need)
+    desc = (abi.SampledLayerDesc * 2)()
+    assert abi.status("nts_batch_builder_layers", handle.value, ctypes.addressof(desc)) == abi.NTS_ERR_INVALID
+    ids = torch.arange(17, dtype=torch.int32, device=device)
+    s = torch.cuda.current_stream().cuda_stream
+    assert abi.status("nts_batch_builder_sample", handle.value, ptr(ids), 17, 1, s) == abi.NTS_ERR_INVALID
+    assert "max_batch" in abi.last_error()
+    call("nts_batch_builder_sample", handle.value, ptr(ids), 16, 1, s)
+    call("nts_batch_builder_layers", handle.value, ctypes.addressof(desc))
+    assert desc[1].v_size == 16 and desc[0].v_size == desc[1].src_size
+    call("nts_batch_builder_destroy", handle.value)
