@@ -1050,7 +1050,9 @@ __global__ __launch_bounds__(kLongBlock) void giant_softmax_bwd_apply_kernel(
 // the copies: 64 consecutive edges per wave step, (source, owner) looked up per lane.
 
 // Fast path: G = (H*Fh)/VEC lanes cover one edge's row (G a power of two <= 64), the Fh/VEC lanes of
-// a head add their products with an xor butterfly; 64/G edges per step.
+// a head add their products with an xor butterfly.  A wave step takes 64 consecutive edges and each
+// of the 64/G lane groups G consecutive ones of them, so a group's destination changes rarely and
+// its gout row stays in registers until it does: one gathered row per edge instead of two.
 template <int VEC>
 __global__ __launch_bounds__(256) void sddmm_edge_kernel(float *__restrict__ galpha, const float *__restrict__ in,
                                                          const float *__restrict__ gout,
@@ -1061,9 +1063,11 @@ __global__ __launch_bounds__(256) void sddmm_edge_kernel(float *__restrict__ gal
   const uint32_t F = H * Fh;
   const uint32_t lane = lane_id();
   const uint32_t gl = lane & (G - 1), grp = lane / G;
-  const uint32_t edges_per_step = kWave / G;
   const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  uint32_t d_held = 0xFFFFFFFFu;
+  float4 y4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  float y1 = 0.f;
   for (uint64_t base = wave * kWave; base < E; base += n_waves * kWave) {
     const uint64_t e = base + lane;
     uint32_t src = 0, own = 0;
@@ -1071,26 +1075,41 @@ __global__ __launch_bounds__(256) void sddmm_edge_kernel(float *__restrict__ gal
       src = ri[e];
       own = owner_of(co, Vd, static_cast<uint32_t>(e));
     }
-    for (uint32_t j = 0; j < G; ++j) {
-      const uint32_t holder = j * edges_per_step + grp;
-      const uint32_t s = __shfl(src, holder, kWave);
-      const uint32_t d = __shfl(own, holder, kWave);
-      const uint64_t ee = base + holder;
-      const bool valid = ee < E;
-      float p = 0.f;
-      if (valid) {
-        const float *a = in + static_cast<size_t>(s) * F + gl * VEC;
-        const float *b = gout + static_cast<size_t>(d) * F + gl * VEC;
-        if (VEC == 4) {
-          const float4 x = *reinterpret_cast<const float4 *>(a);
-          const float4 y = *reinterpret_cast<const float4 *>(b);
-          p = fmaf(x.w, y.w, fmaf(x.z, y.z, fmaf(x.y, y.y, x.x * y.x)));
-        } else {
-          p = a[0] * b[0];
+    // Four edges at a time: their gathered rows are requested before the first is used.
+    constexpr uint32_t U = 4;
+    for (uint32_t j0 = 0; j0 < G; j0 += U) {
+      uint32_t d[U];
+      bool valid[U];
+      float4 x4[U];
+      float x1[U];
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u) {
+        const uint32_t holder = grp * G + j0 + u;
+        const uint32_t s = __shfl(src, holder & (kWave - 1), kWave);
+        d[u] = __shfl(own, holder & (kWave - 1), kWave);
+        valid[u] = j0 + u < G && base + holder < E;
+        x4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        x1[u] = 0.f;
+        if (valid[u]) {
+          const float *a = in + static_cast<size_t>(s) * F + gl * VEC;
+          if (VEC == 4) x4[u] = *reinterpret_cast<const float4 *>(a); else x1[u] = a[0];
         }
       }
-      for (uint32_t m = lanes_per_head / 2; m >= 1; m >>= 1) p += __shfl_xor(p, m, kWave);
-      if (valid && (gl & (lanes_per_head - 1)) == 0) galpha[ee * H + gl / lanes_per_head] = p;
+#pragma unroll
+      for (uint32_t u = 0; u < U; ++u) {
+        float p = 0.f;
+        if (valid[u]) {
+          if (d[u] != d_held) {
+            const float *b = gout + static_cast<size_t>(d[u]) * F + gl * VEC;
+            if (VEC == 4) y4 = *reinterpret_cast<const float4 *>(b); else y1 = b[0];
+            d_held = d[u];
+          }
+          p = VEC == 4 ? fmaf(x4[u].w, y4.w, fmaf(x4[u].z, y4.z, fmaf(x4[u].y, y4.y, x4[u].x * y4.x))) : x1[u] * y1;
+        }
+        for (uint32_t m = lanes_per_head / 2; m >= 1; m >>= 1) p += __shfl_xor(p, m, kWave);
+        if (valid[u] && (gl & (lanes_per_head - 1)) == 0)
+          galpha[(base + grp * G + j0 + u) * H + gl / lanes_per_head] = p;
+      }
     }
   }
 }
