@@ -188,6 +188,122 @@ int main() {
     FreeEdge(dco); FreeEdge(dri); FreeBuffer(dxb); FreeBuffer(doutb);
   }
 
+  // A whole mini-batch built on the device (nts_batch_builder_*), the way Sampler::sample_one's
+  // replacement calls it, with whole neighbourhoods (fanout -1) so that plain host loops give the
+  // expected layers; then the layer is aggregated through Cuda_Stream as SingleGPUSampleGraphOp does.
+  {
+    const VertexId_CUDA Vg = 400;
+    std::vector<VertexId_CUDA> gco(Vg + 1, 0), gri;
+    for (VertexId_CUDA d = 0; d < Vg; ++d) {
+      std::vector<VertexId_CUDA> nb;
+      const uint32_t deg = next() % 7;  // some vertices have no in-edge
+      for (uint32_t k = 0; k < deg; ++k) nb.push_back(next() % Vg);
+      std::sort(nb.begin(), nb.end());
+      gri.insert(gri.end(), nb.begin(), nb.end());
+      gco[d + 1] = (VertexId_CUDA)gri.size();
+    }
+    const VertexId_CUDA Eg = (VertexId_CUDA)gri.size();
+    VertexId_CUDA *dgco = (VertexId_CUDA *)cudaMallocGPU((Vg + 1) * sizeof(VertexId_CUDA));
+    VertexId_CUDA *dgri = (VertexId_CUDA *)cudaMallocGPU(Eg * sizeof(VertexId_CUDA));
+    move_bytes_in(dgco, gco.data(), (Vg + 1) * sizeof(VertexId_CUDA));
+    move_bytes_in(dgri, gri.data(), Eg * sizeof(VertexId_CUDA));
+    const int32_t fanouts[2] = {-1, -1};
+    const uint32_t hops = 2, max_batch = 32;
+    const size_t bytes = nts_batch_builder_arena_bytes(Vg, Eg, fanouts, hops, max_batch, 0);
+    EXPECT(bytes > 0);
+    void *arena = cudaMallocGPU(bytes);
+    nts_batch_builder_t *builder = NULL;
+    NTS_VENEER_CHECK(nts_batch_builder_create(&builder, dgco, dgri, Vg, Eg, fanouts, hops, max_batch, 0, arena, bytes));
+    std::vector<VertexId_CUDA> batch;
+    for (VertexId_CUDA v = 3; batch.size() < 20; v += 17) batch.push_back(v % Vg);  // distinct ids
+    VertexId_CUDA *dbatch_ids = (VertexId_CUDA *)cudaMallocGPU(batch.size() * sizeof(VertexId_CUDA));
+    move_bytes_in(dbatch_ids, batch.data(), batch.size() * sizeof(VertexId_CUDA));
+    for (int rep = 0; rep < 2; ++rep) {  // the second batch re-uses the arena
+      NTS_VENEER_CHECK(nts_batch_builder_sample(builder, dbatch_ids, (uint32_t)batch.size(), 7 + rep, cs.stream));
+      nts_sampled_layer_t L[2];
+      NTS_VENEER_CHECK(nts_batch_builder_layers(builder, L));
+      std::vector<VertexId_CUDA> dst = batch;
+      for (int hop = 0; hop < 2; ++hop) {
+        const nts_sampled_layer_t &l = L[1 - hop];  // L[0] is the input-side layer
+        // expected: all in-neighbours of every destination, sources = sorted distinct ids
+        std::vector<VertexId_CUDA> eco(dst.size() + 1, 0), eglob;
+        for (size_t i = 0; i < dst.size(); ++i) {
+          eglob.insert(eglob.end(), gri.begin() + gco[dst[i]], gri.begin() + gco[dst[i] + 1]);
+          eco[i + 1] = (VertexId_CUDA)eglob.size();
+        }
+        std::vector<VertexId_CUDA> esrc = eglob;
+        std::sort(esrc.begin(), esrc.end());
+        esrc.erase(std::unique(esrc.begin(), esrc.end()), esrc.end());
+        EXPECT(l.v_size == dst.size() && l.e_size == eglob.size() && l.src_size == esrc.size());
+        if (l.v_size != dst.size() || l.e_size != eglob.size() || l.src_size != esrc.size()) break;
+        std::vector<VertexId_CUDA> gotco(l.v_size + 1), gotri(l.e_size), gotsrc(l.src_size), gotro(l.src_size + 1),
+            gotci(l.e_size), gotdst(l.v_size);
+        std::vector<float> gotwf(l.e_size), gotwb(l.e_size);
+        NTS_VENEER_CHECK(nts_memcpy_d2h(gotco.data(), l.column_offset, gotco.size() * 4, 1));
+        NTS_VENEER_CHECK(nts_memcpy_d2h(gotdst.data(), l.destination, gotdst.size() * 4, 1));
+        if (l.e_size) {
+          NTS_VENEER_CHECK(nts_memcpy_d2h(gotri.data(), l.row_indices, gotri.size() * 4, 1));
+          NTS_VENEER_CHECK(nts_memcpy_d2h(gotsrc.data(), l.source, gotsrc.size() * 4, 1));
+          NTS_VENEER_CHECK(nts_memcpy_d2h(gotci.data(), l.column_indices, gotci.size() * 4, 1));
+          NTS_VENEER_CHECK(nts_memcpy_d2h(gotwf.data(), l.edge_weight_forward, gotwf.size() * 4, 1));
+          NTS_VENEER_CHECK(nts_memcpy_d2h(gotwb.data(), l.edge_weight_backward, gotwb.size() * 4, 1));
+        }
+        NTS_VENEER_CHECK(nts_memcpy_d2h(gotro.data(), l.row_offset, gotro.size() * 4, 1));
+        EXPECT(gotco == eco && gotsrc == esrc && gotdst == dst);
+        bool ok = true;
+        std::vector<VertexId_CUDA> outdeg(esrc.size(), 0);
+        for (size_t e = 0; e < eglob.size(); ++e) {
+          ok = ok && gotri[e] < esrc.size() && esrc[gotri[e]] == eglob[e];
+          if (ok) ++outdeg[gotri[e]];
+        }
+        EXPECT(ok);
+        for (size_t s2 = 0; ok && s2 < esrc.size(); ++s2) ok = gotro[s2 + 1] - gotro[s2] == outdeg[s2];
+        EXPECT(ok && gotro[0] == 0);
+        // CSR rows list the destinations of a source in ascending edge order; weights follow
+        // nts_norm_degree on the layer's own degrees
+        for (size_t s2 = 0; ok && s2 < esrc.size(); ++s2) {
+          VertexId_CUDA k = gotro[s2];
+          for (size_t i = 0; i < dst.size(); ++i)
+            for (VertexId_CUDA e = eco[i]; e < eco[i + 1]; ++e)
+              if (gotri[e] == s2) {
+                ok = ok && gotci[k] == i;
+                const float wgt = 1.0f / ((float)sqrt((double)outdeg[s2]) * (float)sqrt((double)(eco[i + 1] - eco[i])));
+                ok = ok && gotwb[k] == wgt && gotwf[e] == wgt;
+                ++k;
+              }
+          ok = ok && k == gotro[s2 + 1];
+        }
+        EXPECT(ok);
+        // aggregate the layer as SingleGPUSampleGraphOp::forward does
+        if (l.e_size) {
+          const VertexId_CUDA Fl = 24;
+          std::vector<float> xl((size_t)l.src_size * Fl), want((size_t)l.v_size * Fl, 0.f), have(want.size());
+          for (auto &v : xl) v = (float)(next() % 2001) / 1000.f - 1.f;
+          for (size_t i = 0; i < dst.size(); ++i)
+            for (VertexId_CUDA e = eco[i]; e < eco[i + 1]; ++e)
+              for (VertexId_CUDA f = 0; f < Fl; ++f)
+                want[i * Fl + f] = fmaf(xl[(size_t)gotri[e] * Fl + f], gotwf[e], want[i * Fl + f]);
+          float *dxl, *dyl;
+          allocate_gpu_buffer(&dxl, (int)xl.size());
+          allocate_gpu_buffer(&dyl, (int)want.size());
+          move_data_in(dxl, xl.data(), 0, l.src_size, Fl);
+          zero_buffer(dyl, (int)want.size());
+          cs.Gather_By_Dst_From_Src(dxl, dyl, l.edge_weight_forward, l.row_indices, l.column_offset, 0, 0, 0, 0, l.e_size,
+                                    l.v_size, Fl, true, false);
+          cs.CUDA_DEVICE_SYNCHRONIZE();
+          move_result_out(have.data(), dyl, 0, l.v_size, Fl);
+          EXPECT(memcmp(have.data(), want.data(), want.size() * sizeof(float)) == 0);
+          FreeBuffer(dxl); FreeBuffer(dyl);
+        }
+        dst = esrc;
+      }
+      std::reverse(batch.begin(), batch.end());  // another order of the same ids for the second batch
+      move_bytes_in(dbatch_ids, batch.data(), batch.size() * sizeof(VertexId_CUDA));
+    }
+    NTS_VENEER_CHECK(nts_batch_builder_destroy(builder));
+    FreeEdge(dgco); FreeEdge(dgri); FreeEdge(dbatch_ids); FreeEdge((VertexId_CUDA *)arena);
+  }
+
   csc.release();
   FreeBuffer(dx); FreeBuffer(dw); FreeBuffer(dout); FreeBuffer(dbatch); FreeBuffer(dlog); FreeBuffer(dalpha);
   FreeBuffer(dcache); FreeEdge(dids); free_gpu_data(dlab); free_gpu_data(dlab_out); ntsFreeHost(pinned);
