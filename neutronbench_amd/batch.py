@@ -168,8 +168,18 @@ class BatchBuilder:
     def sample(self, batch_ids, seed):
         """batch_ids: int32 device tensor.  Returns the SampledLayer list, input-side layer first;
         the arrays are DevArray ranges of the arena (`.tensor()` gives a torch view)."""
-        stream = torch.cuda.current_stream(self.device).cuda_stream
+        self.enqueue(batch_ids, seed)
+        return self.collect()
+
+    def enqueue(self, batch_ids, seed, stream=None):
+        """Starts building a batch on `stream` (a raw stream handle; default: torch's current one)
+        and returns at once; `collect` waits for it.  batch_ids must stay alive until then."""
+        if stream is None:
+            stream = torch.cuda.current_stream(self.device).cuda_stream
         call("nts_batch_builder_sample", self.handle, ptr(batch_ids), batch_ids.numel(), seed, stream)
+
+    def collect(self):
+        """Waits for the batch started by `enqueue`; the layers are complete when this returns."""
         call("nts_batch_builder_layers", self.handle, ctypes.addressof(self._desc))
         layers = []
         i32, f32 = torch.int32, torch.float32

@@ -14,7 +14,8 @@ weights, gathers, aggregation.  --sampler builder (default) builds all layers of
 stream-ordered sequence with one read-back (nts_batch_builder_*; "sample" then holds sampling and
 structure together); --sampler library goes hop by hop through the per-step entry points;
 --sampler harness uses the torch sampler of the test harness instead.  Stages are separated by
-stream synchronisation, as every reference operator synchronises its stream.
+stream synchronisation, as every reference operator synchronises its stream.  --pipeline 2 samples
+the next batch on a second stream while the current one is gathered and aggregated.
 """
 import argparse
 import json
@@ -43,11 +44,13 @@ class Timer:
         self.t = {}
 
     def add(self, key, t0):
-        torch.cuda.synchronize()
+        # Only the stream the stages run on: a device-wide wait would also wait for the next batch
+        # being sampled on the second stream of the pipelined mode.
+        torch.cuda.current_stream().synchronize()
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
-def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2):
+def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1):
     cfg = dict(CONFIGS[name])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
@@ -75,7 +78,22 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2):
     # untimed, then the epoch starts over from its first batch.
     n_warm = min(warmup_batches, n_batches)
     t_epoch = time.perf_counter()
-    for step, b in enumerate(list(range(n_warm)) + list(range(n_batches))):
+    sequence = list(range(n_warm)) + list(range(n_batches))
+    # pipeline = 2 (the reference's PIPELINES mode, toolkits/GCN_GPU_NEIGHBOR.hpp:1350-1363, with two
+    # stages in flight): the next batch is sampled on a second stream, by a second builder, while
+    # this one is gathered and aggregated.
+    pipelined = builder is not None and pipeline > 1
+    if pipelined:
+        builders = [builder, BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0)]
+        side_stream = torch.cuda.Stream(device=dev)
+
+        def start_sampling(step):
+            b = sequence[step]
+            builders[step % 2].enqueue(train32[b * cfg["batch"]:(b + 1) * cfg["batch"]], 1000 * b,
+                                       side_stream.cuda_stream)
+        torch.cuda.synchronize()
+        start_sampling(0)
+    for step, b in enumerate(sequence):
         if step == n_warm:
             torch.cuda.synchronize()
             tm.t.clear()
@@ -85,7 +103,13 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2):
         # -- sample (harness) + structure (library) -------------------------------------------
         layers = []
         dst_ids = batch
-        if builder is not None:
+        if pipelined:
+            t0 = time.perf_counter()
+            layers = builders[step % 2].collect()[::-1]
+            if step + 1 < len(sequence):
+                start_sampling(step + 1)
+            tm.t["sample_wait"] = tm.t.get("sample_wait", 0.0) + time.perf_counter() - t0
+        elif builder is not None:
             t0 = time.perf_counter()
             layers = builder.sample(train32[b * cfg["batch"]:(b + 1) * cfg["batch"]], 1000 * b)[::-1]
             tm.add("sample", t0)
@@ -164,7 +188,7 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2):
         "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
         "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
-        "sampler": sampler, "sampled_edges": edges_total, "gathered_rows": rows_total,
+        "sampler": sampler, "pipeline": 2 if pipelined else 1, "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
     }
     print(json.dumps(out))
@@ -178,5 +202,7 @@ if __name__ == "__main__":
     ap.add_argument("--max-batches", type=int, default=0)
     ap.add_argument("--sampler", choices=["builder", "library", "harness"], default="builder")
     ap.add_argument("--warmup-batches", type=int, default=2, help="untimed batches before the epoch starts")
+    ap.add_argument("--pipeline", type=int, default=1, choices=[1, 2],
+                    help="2: the next batch is sampled on a second stream while this one is gathered and aggregated")
     a = ap.parse_args()
-    run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches)
+    run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline)
