@@ -327,7 +327,10 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
  *                layer whose `destination` is the batch -- the order of SampledSubgraph::sampled_sgs.
  *                Pointers address the arena and stay valid until the next nts_batch_builder_sample
  *                on the same builder; a pipeline that samples batch k+1 while batch k trains uses
- *                one builder per stage in flight, as the reference uses one SampledSubgraph each. */
+ *                one builder per stage in flight, as the reference uses one SampledSubgraph each.
+ * Calls on one builder must not overlap: consecutive nts_batch_builder_sample calls go to the same
+ * stream, or the earlier batch is waited for first (nts_batch_builder_layers does).  The sequence
+ * contains a device-to-host copy and an event record and is not meant for HIP-graph capture. */
 typedef struct nts_batch_builder nts_batch_builder_t;
 typedef struct nts_sampled_layer {
   uint32_t v_size, e_size, src_size, reserved; /* destinations, edges, distinct sources */

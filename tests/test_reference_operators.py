@@ -10,7 +10,7 @@ import pytest
 
 import oracle
 import refops
-from util import abs_term_scale, check
+from util import abs_term_scale, check, planless_piece_edges
 
 CASES = [(300, 4000, 19, 4, 1), (2000, 60000, 64, 1, 2), (5000, 40000, 7, 3, 3)]
 
@@ -86,13 +86,13 @@ def test_reference_gpu_operator_classes_over_the_library_match_its_cpu_operators
     ref = refops.run("gpu", "both", inp, tmp_path)
     co, ri = ref["column_offset"], ref["row_indices"]
     # aggregation: one wave walks a row's edges in order with fused multiply-adds, as nts_comp does ->
-    # bit-identical; rows of more than 1024 edges are summed in pieces (calls of >= 65,536 edges) ->
+    # bit-identical; rows longer than the piece length are summed in pieces (calls of >= 65,536 edges) ->
     # tolerance for those
     x = inp["x"]
     for got, want, off, idx, w in ((ref["gpu_fwd"], ref["cpu_fwd"], co, ri, ref["edge_weight_forward"]),
                                    (ref["gpu_bwd"], ref["cpu_bwd"], ref["row_offset"], ref["column_indices"],
                                     ref["edge_weight_backward"])):
-        one_wave = np.diff(off.astype(np.int64)) <= (1024 if E >= 1 << 16 else E)
+        one_wave = np.diff(off.astype(np.int64)) <= (planless_piece_edges(E) or E)
         assert got[one_wave].tobytes() == want[one_wave].tobytes()
         check(got, want, abs_term_scale(x, w, off, idx, V))
     # vertex -> edge copies
@@ -157,7 +157,7 @@ def test_reference_sampled_layers_on_the_device_match_the_oracle(tmp_path, V, E,
     layer to layer, asynchronous copies: core/coocsc.hpp:673-773) through the veneer's allocator and
     copies, and the layer is aggregated forward and backward with the calls of SingleGPUSampleGraphOp
     (core/ntsMiniBatchGraphOp.hpp:288-375).  Results against the oracle's fused aggregation on the
-    reference's own arrays: rows of at most 1,024 edges bit for bit, the rest within tolerance."""
+    reference's own arrays: rows of at most one piece bit for bit, the rest within tolerance."""
     _sampled_layers_case(tmp_path, V, E, batch, fanouts, seed, device_F=24)
 
 
@@ -199,6 +199,6 @@ def _sampled_layers_case(tmp_path, V, E, batch, fanouts, seed, device_F):
             for got, x, w, off, idx, rows in ((want["fwd"], layer["x"], ewf, layer["co"], local, Vd),
                                               (want["bwd"], layer["g"], ewb, ro, ci, n_src)):
                 expect = oracle.spmm(x, w, off, idx, rows, fused=True)
-                one_wave = np.diff(off.astype(np.int64)) <= (1024 if idx.size >= 1 << 16 else idx.size)
+                one_wave = np.diff(off.astype(np.int64)) <= (planless_piece_edges(idx.size) or idx.size)
                 assert got[one_wave].tobytes() == expect[one_wave].tobytes()
                 check(got, expect, abs_term_scale(x, w, off, idx, rows))

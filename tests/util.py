@@ -26,6 +26,13 @@ def random_block(Vd, Vs, mean_deg, seed, hub=0, dup=False, empty_frac=0.1):
     return co.astype(np.uint32), ri.astype(np.uint32)
 
 
+def planless_piece_edges(E):
+    """Rows of a plan-less aggregation call (nts_spmm_gather, nts_spmm_gather_heads) with at most
+    this many edges are summed as one sequential chain, in edge order; longer rows are summed in
+    pieces.  None = no row is cut (calls below 65,536 edges)."""
+    return 1024 if E >= 1 << 16 else None
+
+
 def brute_csr(co, ri, Vs):
     """Transposed structure by a stable sort of (source, edge id): (ro, ci, perm)."""
     Vd = co.size - 1
