@@ -42,6 +42,13 @@ enum nts_status {
 const char *nts_last_error(void);
 /* ABI version: bumped when a signature changes. */
 int nts_abi_version(void);
+/* Profiler ranges.  With NTS_TRACE_RANGES=1 in the environment (read when the first traced entry
+ * point runs) the compute, layout, sampling and reader entry points below push a rocTX range named
+ * after themselves on entry and pop it on return, so that `rocprofv3 --marker-trace --kernel-trace`
+ * attributes kernels to calls; the rocTX library is loaded at run time only then.  The reference
+ * brackets its stages with wall-clock accumulators instead (toolkits/GCN_GPU_NEIGHBOR.hpp:617-705).
+ * nts_trace_ranges_emitted: ranges pushed so far by this process (0 when ranges are off). */
+long nts_trace_ranges_emitted(void);
 
 /* ---------------------------------------------------------------------------------------------
  * Memory, copies, streams

@@ -27,6 +27,7 @@ _str = ctypes.c_char_p
 SIGNATURES = {
     "nts_last_error": [],
     "nts_abi_version": [],
+    "nts_trace_ranges_emitted": [],
     "nts_malloc_device": [ctypes.POINTER(_vp), _sz],
     "nts_free_device": [_vp],
     "nts_malloc_device_async": [ctypes.POINTER(_vp), _sz, _vp],
@@ -100,9 +101,10 @@ SIGNATURES = {
 }
 _RESTYPES = {"nts_last_error": ctypes.c_char_p, "nts_csr_from_csc_work_bytes": _sz,
              "nts_relabel_sources_work_bytes": _sz, "nts_sample_hop_work_bytes": _sz,
-             "nts_chunk_from_edges_work_bytes": _sz, "nts_batch_builder_arena_bytes": _sz}
+             "nts_chunk_from_edges_work_bytes": _sz, "nts_batch_builder_arena_bytes": _sz,
+             "nts_trace_ranges_emitted": ctypes.c_long}
 # Entry points whose int result is a value, not a status.
-_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
+_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_trace_ranges_emitted", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
               "nts_sample_hop_work_bytes", "nts_chunk_from_edges_work_bytes", "nts_batch_builder_arena_bytes"}
 
 

@@ -126,6 +126,7 @@ size_t nts_batch_builder_arena_bytes(uint32_t V, uint32_t graph_edges, const int
 int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co, const uint32_t *graph_ri, uint32_t V,
                              uint32_t graph_edges, const int32_t *fanouts, uint32_t hops, uint32_t max_batch,
                              int want_perm, void *arena, size_t arena_bytes) {
+  NTS_TRACE_RANGE("nts_batch_builder_create");
   if (!out) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: null out");
   *out = nullptr;
   if (!graph_co || !graph_ri || !fanouts || !arena) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: null pointer");
@@ -167,6 +168,7 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
 }
 
 int nts_batch_builder_destroy(nts_batch_builder_t *b) {
+  NTS_TRACE_RANGE("nts_batch_builder_destroy");
   if (!b) return NTS_OK;
   hipError_t e1 = hipEventDestroy(b->done);
   hipError_t e2 = hipHostFree(b->host_sizes);
@@ -178,6 +180,7 @@ int nts_batch_builder_destroy(nts_batch_builder_t *b) {
 
 int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, uint32_t n, uint64_t seed,
                              nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_batch_builder_sample");
   if (!b) return fail(NTS_ERR_INVALID, "nts_batch_builder_sample: null builder");
   if (n > b->max_batch) return fail(NTS_ERR_INVALID, "nts_batch_builder_sample: batch larger than max_batch");
   if (n && !batch_ids) return fail(NTS_ERR_INVALID, "nts_batch_builder_sample: null batch_ids");
@@ -234,6 +237,7 @@ int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, 
 }
 
 int nts_batch_builder_layers(nts_batch_builder_t *b, nts_sampled_layer_t *layers) {
+  NTS_TRACE_RANGE("nts_batch_builder_layers");
   if (!b || !layers) return fail(NTS_ERR_INVALID, "nts_batch_builder_layers: null pointer");
   if (!b->pending) return fail(NTS_ERR_INVALID, "nts_batch_builder_layers: no batch has been sampled");
   NTS_HIP_TRY(hipEventSynchronize(b->done));

@@ -29,6 +29,33 @@ int fail_hip(hipError_t err, const char *what);
     if (nts_err__ != hipSuccess) return ::nts::fail_hip(nts_err__, name); \
   } while (0)
 
+// Named ranges around the entry points for a profiler's marker trace (rocTX).  Off unless the
+// environment has NTS_TRACE_RANGES=1 when the first entry point runs; then the rocTX library is
+// loaded at run time (the library itself does not link against it) and every traced entry point
+// pushes its name on entry and pops it on return.
+struct TraceApi {
+  int (*push)(const char *);
+  int (*pop)();
+};
+const TraceApi *trace_api();  // NULL when ranges are off or the rocTX library is not there
+void count_trace_range();
+long trace_ranges_emitted();
+struct TraceRange {
+  explicit TraceRange(const char *name) : api(trace_api()) {
+    if (api) {
+      api->push(name);
+      count_trace_range();
+    }
+  }
+  ~TraceRange() {
+    if (api) api->pop();
+  }
+  TraceRange(const TraceRange &) = delete;
+  TraceRange &operator=(const TraceRange &) = delete;
+  const TraceApi *api;
+};
+#define NTS_TRACE_RANGE(name) ::nts::TraceRange nts_trace_range__(name)
+
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 inline uint32_t ceil_div(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }

@@ -197,6 +197,7 @@ using namespace nts;
 extern "C" {
 
 int nts_edge_file_count(const char *path, uint64_t *edges) {
+  NTS_TRACE_RANGE("nts_edge_file_count");
   if (!path || !edges) return fail(NTS_ERR_INVALID, "nts_edge_file_count: null argument");
   struct stat st;
   if (stat(path, &st) != 0) return fail(NTS_ERR_INVALID, (std::string("nts_edge_file_count: cannot stat ") + path).c_str());
@@ -205,6 +206,7 @@ int nts_edge_file_count(const char *path, uint64_t *edges) {
 }
 
 int nts_edge_file_read(const char *path, uint32_t *pairs, uint64_t first, uint64_t n, uint32_t *max_id) {
+  NTS_TRACE_RANGE("nts_edge_file_read");
   if (!path || (!pairs && n)) return fail(NTS_ERR_INVALID, "nts_edge_file_read: null argument");
   const int fd = open(path, O_RDONLY);
   if (fd < 0) return fail(NTS_ERR_INVALID, (std::string("nts_edge_file_read: cannot open ") + path).c_str());
@@ -302,6 +304,7 @@ static int feature_text_read(const char *path, float *table, std::vector<uint32_
 }
 
 int nts_feature_csv_read(const char *path, float *table, uint32_t V, uint32_t F, int threads) {
+  NTS_TRACE_RANGE("nts_feature_csv_read");
   if (!table || F == 0) return fail(NTS_ERR_INVALID, "nts_feature_csv_read: null table or F is 0");
   MappedFile f;
   if (int rc = f.open_path(path, "nts_feature_csv_read")) return rc;
@@ -457,6 +460,7 @@ static int mask_text_read(const char *path, int32_t *mask, const uint32_t *recor
 int nts_read_feature_label_mask(const char *path_f, const char *path_l, const char *path_m, uint32_t V, uint32_t F,
                                 uint32_t classes, float *local_feature, int64_t *local_label, int32_t *local_mask,
                                 int64_t *global_label, int32_t *global_mask, int threads) {
+  NTS_TRACE_RANGE("nts_read_feature_label_mask");
   std::vector<uint32_t> ids;
   if (int rc = feature_text_read(path_f, local_feature, ids, V, F, threads)) return rc;
   if (local_label)
@@ -471,6 +475,7 @@ int nts_read_feature_label_mask(const char *path_f, const char *path_l, const ch
 }
 
 int nts_int_list_text_read(const char *path, int64_t *out, uint64_t capacity, uint64_t *count) {
+  NTS_TRACE_RANGE("nts_int_list_text_read");
   if (!count) return fail(NTS_ERR_INVALID, "nts_int_list_text_read: null count");
   MappedFile f;
   if (int rc = f.open_path(path, "nts_int_list_text_read")) return rc;
@@ -492,6 +497,7 @@ int nts_int_list_text_read(const char *path, int64_t *out, uint64_t capacity, ui
 }
 
 int nts_table_bin_write(const char *path, const void *data, uint64_t rows, uint64_t cols, uint32_t elem_bytes) {
+  NTS_TRACE_RANGE("nts_table_bin_write");
   if (!path || (!data && rows * cols)) return fail(NTS_ERR_INVALID, "nts_table_bin_write: null argument");
   const int fd = open(path, O_WRONLY | O_CREAT | O_TRUNC, 0644);
   if (fd < 0) return fail(NTS_ERR_INVALID, (std::string("nts_table_bin_write: cannot create ") + path).c_str());
@@ -519,6 +525,7 @@ int nts_table_bin_write(const char *path, const void *data, uint64_t rows, uint6
 }
 
 int nts_table_bin_info(const char *path, uint64_t *rows, uint64_t *cols, uint32_t *elem_bytes) {
+  NTS_TRACE_RANGE("nts_table_bin_info");
   if (!path) return fail(NTS_ERR_INVALID, "nts_table_bin_info: null path");
   const int fd = open(path, O_RDONLY);
   if (fd < 0) return fail(NTS_ERR_INVALID, (std::string("nts_table_bin_info: cannot open ") + path).c_str());
@@ -538,6 +545,7 @@ int nts_table_bin_info(const char *path, uint64_t *rows, uint64_t *cols, uint32_
 }
 
 int nts_table_bin_read(const char *path, void *out, uint64_t row_begin, uint64_t rows) {
+  NTS_TRACE_RANGE("nts_table_bin_read");
   uint64_t R, C;
   uint32_t eb;
   if (int rc = nts_table_bin_info(path, &R, &C, &eb)) return rc;

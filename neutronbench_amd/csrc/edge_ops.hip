@@ -1432,34 +1432,40 @@ extern "C" {
 
 int nts_scatter_src_to_edge(float *msg, const float *feat, const uint32_t *ri, const uint32_t *co,
                             const uint32_t *mirror, uint32_t Vd, uint32_t F, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_scatter_src_to_edge");
   return edge_copy_impl(msg, feat, ri, co, mirror, Vd, F, kFromSrc, stream, "nts_scatter_src_to_edge: bad argument");
 }
 
 int nts_scatter_dst_to_edge(float *msg, const float *feat, const uint32_t *co, uint32_t Vd, uint32_t F,
                             nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_scatter_dst_to_edge");
   return edge_copy_impl(msg, feat, nullptr, co, nullptr, Vd, F, kFromDst, stream,
                         "nts_scatter_dst_to_edge: bad argument");
 }
 
 int nts_scatter_grad_to_edge(float *msg_grad, const float *gout, const uint32_t *co, uint32_t Vd, uint32_t F,
                              nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_scatter_grad_to_edge");
   return edge_copy_impl(msg_grad, gout, nullptr, co, nullptr, Vd, F, kAddFromDst, stream,
                         "nts_scatter_grad_to_edge: bad argument");
 }
 
 int nts_gather_edge_to_dst(float *out, const float *msg, const uint32_t *co, uint32_t Vd, uint32_t F, int accumulate,
                            nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gather_edge_to_dst");
   return gather_edge_impl(out, msg, co, nullptr, Vd, F, accumulate, stream, "nts_gather_edge_to_dst: bad argument");
 }
 
 int nts_gather_edge_to_src(float *out, const float *msg, const uint32_t *ro, const uint32_t *perm, uint32_t Vs,
                            uint32_t F, int accumulate, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gather_edge_to_src");
   if (Vs != 0 && !perm) return fail(NTS_ERR_INVALID, "nts_gather_edge_to_src: null perm");
   return gather_edge_impl(out, msg, ro, perm, Vs, F, accumulate, stream, "nts_gather_edge_to_src: bad argument");
 }
 
 int nts_edge_softmax_fwd(float *y, const float *x, const uint32_t *co, uint32_t Vd, uint32_t H,
                          nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_edge_softmax_fwd");
   if (H == 0) return fail(NTS_ERR_INVALID, "nts_edge_softmax_fwd: H is 0");
   if (Vd == 0) return NTS_OK;
   if (!y || !x || !co) return fail(NTS_ERR_INVALID, "nts_edge_softmax_fwd: null pointer");
@@ -1469,6 +1475,7 @@ int nts_edge_softmax_fwd(float *y, const float *x, const uint32_t *co, uint32_t 
 
 int nts_edge_softmax_bwd(float *gx, const float *gy, const float *y, const uint32_t *co, uint32_t Vd, uint32_t H,
                          nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_edge_softmax_bwd");
   if (H == 0) return fail(NTS_ERR_INVALID, "nts_edge_softmax_bwd: H is 0");
   if (Vd == 0) return NTS_OK;
   if (!gx || !gy || !y || !co) return fail(NTS_ERR_INVALID, "nts_edge_softmax_bwd: null pointer");
@@ -1478,6 +1485,7 @@ int nts_edge_softmax_bwd(float *gx, const float *gy, const float *y, const uint3
 
 int nts_gat_attention_fwd(float *alpha, const float *el, const float *er, const uint32_t *co, const uint32_t *ri,
                           uint32_t Vd, uint32_t H, float slope, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gat_attention_fwd");
   if (H == 0) return fail(NTS_ERR_INVALID, "nts_gat_attention_fwd: H is 0");
   if (Vd == 0) return NTS_OK;
   if (!alpha || !el || !er || !co || !ri) return fail(NTS_ERR_INVALID, "nts_gat_attention_fwd: null pointer");
@@ -1488,6 +1496,7 @@ int nts_gat_attention_fwd(float *alpha, const float *el, const float *er, const 
 int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const float *alpha, const float *el,
                           const float *er, const uint32_t *co, const uint32_t *ri, uint32_t Vd, uint32_t H,
                           float slope, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gat_attention_bwd");
   if (H == 0) return fail(NTS_ERR_INVALID, "nts_gat_attention_bwd: H is 0");
   if (Vd == 0) return NTS_OK;
   if (!gs || !ger || !galpha || !alpha || !el || !er || !co || !ri)
@@ -1498,6 +1507,7 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
 
 int nts_sddmm_heads(float *galpha, const float *in, const float *gout, const uint32_t *co, const uint32_t *ri,
                     uint32_t Vd, uint32_t H, uint32_t Fh, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_sddmm_heads");
   if (H == 0 || Fh == 0) return fail(NTS_ERR_INVALID, "nts_sddmm_heads: H or Fh is 0");
   if (static_cast<uint64_t>(H) * Fh > 0xFFFFFFFFull) return fail(NTS_ERR_INVALID, "nts_sddmm_heads: H*Fh overflows");
   if (Vd == 0) return NTS_OK;

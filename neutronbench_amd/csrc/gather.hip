@@ -144,6 +144,7 @@ extern "C" {
 
 int nts_gather_rows_f32(float *out, const float *table, const uint32_t *row_ids, const uint32_t *sel,
                         const uint32_t *remap, uint32_t n, uint32_t F, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gather_rows_f32");
   if (F == 0) return fail(NTS_ERR_INVALID, "nts_gather_rows_f32: F is 0");
   if (n == 0) return NTS_OK;
   if (!out || !table || !row_ids) return fail(NTS_ERR_INVALID, "nts_gather_rows_f32: null pointer");
@@ -156,6 +157,7 @@ int nts_gather_rows_f32(float *out, const float *table, const uint32_t *row_ids,
 int nts_gather_rows_cached_f32(float *out, const float *table, const float *cache, const uint32_t *row_ids,
                                const uint32_t *hashmap, uint32_t n, uint32_t F, uint32_t *hits,
                                nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gather_rows_cached_f32");
   if (F == 0) return fail(NTS_ERR_INVALID, "nts_gather_rows_cached_f32: F is 0");
   if (hits) {
     hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, stream, hits);
@@ -172,6 +174,7 @@ int nts_gather_rows_cached_f32(float *out, const float *table, const float *cach
 
 int nts_gather_labels_i64(int64_t *out, const int64_t *table, const uint32_t *ids, uint32_t n, uint32_t classes,
                           nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gather_labels_i64");
   if (classes == 0) return fail(NTS_ERR_INVALID, "nts_gather_labels_i64: classes is 0");
   if (n == 0) return NTS_OK;
   if (!out || !table || !ids) return fail(NTS_ERR_INVALID, "nts_gather_labels_i64: null pointer");

@@ -308,6 +308,7 @@ size_t nts_csr_from_csc_work_bytes(uint32_t Vd, uint32_t Vs, uint32_t E) {
 
 int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, uint32_t Vd,
                      uint32_t Vs, uint32_t E, void *work, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_csr_from_csc");
   if (!ro) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: null ro");
   if (E == 0) {
     return nts_memset_zero(ro, (static_cast<size_t>(Vs) + 1) * sizeof(uint32_t), stream);
@@ -326,6 +327,7 @@ size_t nts_chunk_from_edges_work_bytes(uint32_t V, uint32_t E) {
 
 int nts_chunk_from_edges(uint32_t *co, uint32_t *ri, float *ewf, uint32_t *ro, uint32_t *ci, float *ewb,
                          const uint32_t *pairs, uint32_t E, uint32_t V, void *work, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_chunk_from_edges");
   if (!co || !ro) return fail(NTS_ERR_INVALID, "nts_chunk_from_edges: null offsets");
   if (E == 0) {
     if (int rc = nts_memset_zero(co, (static_cast<size_t>(V) + 1) * sizeof(uint32_t), stream)) return rc;
@@ -370,6 +372,7 @@ size_t nts_relabel_sources_work_bytes(uint32_t V) {
 
 int nts_relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *local, const uint32_t *global_ids, uint32_t E,
                         uint32_t V, void *work, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_relabel_sources");
   if (!n_source) return fail(NTS_ERR_INVALID, "nts_relabel_sources: null n_source");
   if (E == 0 || V == 0) return nts_memset_zero(n_source, sizeof(uint32_t), stream);
   if (!source || !local || !global_ids || !work) return fail(NTS_ERR_INVALID, "nts_relabel_sources: null pointer");
@@ -380,6 +383,7 @@ int nts_relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *local, c
 
 int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t *ri, const uint32_t *co,
                                     const uint32_t *mirror, uint32_t Vd, uint32_t F, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gather_edge_to_src_unsorted");
   if (F == 0) return fail(NTS_ERR_INVALID, "nts_gather_edge_to_src_unsorted: F is 0");
   if (Vd == 0) return NTS_OK;
   if (!out || !msg || !ri || !co) return fail(NTS_ERR_INVALID, "nts_gather_edge_to_src_unsorted: null pointer");
@@ -413,6 +417,7 @@ int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t
 
 int nts_gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t *ri, const uint32_t *ro,
                          const uint32_t *ci, uint32_t Vd, uint32_t Vs, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gcn_edge_weights");
   if (!co || !ro) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null offsets");
   if (Vd == 0 || Vs == 0) return NTS_OK;
   if (ewf && !ri) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ri");

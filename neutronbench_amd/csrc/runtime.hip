@@ -2,6 +2,11 @@
 // Cuda_Stream plumbing of cuda/ntsCUDAGraphOP.cu:23-119, 476-653 and utils/cuda_memory.hpp).
 #include <string.h>
 
+#include <dlfcn.h>
+#include <stdlib.h>
+
+#include <atomic>
+
 #include "common.hpp"
 
 namespace nts {
@@ -33,6 +38,28 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned char *p, size_t
 }
 
 }  // namespace
+namespace {
+std::atomic<long> g_trace_ranges{0};
+}
+
+const TraceApi *trace_api() {
+  static const TraceApi *api = []() -> const TraceApi * {
+    const char *e = getenv("NTS_TRACE_RANGES");
+    if (!e || e[0] != '1') return nullptr;
+    void *lib = dlopen("librocprofiler-sdk-roctx.so", RTLD_NOW | RTLD_GLOBAL);
+    if (!lib) lib = dlopen("libroctx64.so", RTLD_NOW | RTLD_GLOBAL);
+    if (!lib) return nullptr;
+    static TraceApi found;
+    found.push = reinterpret_cast<int (*)(const char *)>(dlsym(lib, "roctxRangePushA"));
+    found.pop = reinterpret_cast<int (*)()>(dlsym(lib, "roctxRangePop"));
+    return (found.push && found.pop) ? &found : nullptr;
+  }();
+  return api;
+}
+
+void count_trace_range() { g_trace_ranges.fetch_add(1, std::memory_order_relaxed); }
+long trace_ranges_emitted() { return g_trace_ranges.load(std::memory_order_relaxed); }
+
 }  // namespace nts
 
 using nts::fail;
@@ -40,6 +67,7 @@ using nts::fail;
 extern "C" {
 
 const char *nts_last_error(void) { return nts::g_last_error; }
+long nts_trace_ranges_emitted(void) { return nts::trace_ranges_emitted(); }
 
 int nts_abi_version(void) { return 1; }
 

@@ -186,6 +186,7 @@ size_t nts_sample_hop_work_bytes(uint32_t n) {
 
 int nts_sample_hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, uint32_t n, int32_t fanout,
                            void *work, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_sample_hop_offsets");
   if (!co) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: null co");
   if (n == 0) return nts_memset_zero(co, sizeof(uint32_t), stream);
   if (!graph_co || !dst || !work) return fail(NTS_ERR_INVALID, "nts_sample_hop_offsets: null pointer");
@@ -198,6 +199,7 @@ int nts_sample_hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_
 int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co,
                              const uint32_t *graph_ri, const uint32_t *dst, uint32_t n, int32_t fanout, uint64_t seed,
                              nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_sample_hop_neighbors");
   if (n == 0) return NTS_OK;
   if (!ri_global || !co || !graph_co || !graph_ri || !dst)
     return fail(NTS_ERR_INVALID, "nts_sample_hop_neighbors: null pointer");

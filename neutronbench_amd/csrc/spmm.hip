@@ -676,6 +676,7 @@ extern "C" {
 int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t *offsets, const uint32_t *indices,
                     uint32_t index_base, uint32_t rows, uint32_t edges, uint32_t F, int accumulate,
                     nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_gather");
   if (int rc = nts::check_common(in, out, offsets, indices, rows, edges, F, "nts_spmm_gather: null pointer")) return rc;
   if (rows == 0) return NTS_OK;
   nts::LaunchArgs a{in, out, w, offsets, indices, index_base, rows, F, nullptr, nullptr, accumulate, stream};
@@ -795,6 +796,7 @@ int read_offsets(std::vector<uint32_t> &off, const uint32_t *offsets, uint32_t r
 
 int nts_spmm_plan_create(nts_spmm_plan_t **plan_out, const uint32_t *offsets, uint32_t rows, uint32_t edges,
                          uint32_t chunk_edges, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_plan_create");
   if (!plan_out) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null out-pointer");
   *plan_out = nullptr;
   if (rows != 0 && !offsets) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create: null offsets");
@@ -806,6 +808,7 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan_out, const uint32_t *offsets, ui
 int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan_out, const uint32_t *offsets, const uint32_t *indices,
                                uint32_t index_base, uint32_t n_index, uint32_t rows, uint32_t edges,
                                uint32_t chunk_edges, uint32_t n_slabs, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_plan_create_slabs");
   if (!plan_out) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create_slabs: null out-pointer");
   *plan_out = nullptr;
   if (rows != 0 && !offsets) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create_slabs: null offsets");
@@ -824,6 +827,7 @@ int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan_out, const uint32_t *offse
 }
 
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {
+  NTS_TRACE_RANGE("nts_spmm_plan_destroy");
   if (!plan) return NTS_OK;
   hipError_t e1 = plan->items ? hipFree(plan->items) : hipSuccess;
   hipError_t e2 = plan->splits ? hipFree(plan->splits) : hipSuccess;
@@ -836,6 +840,7 @@ int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {
 }
 
 int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows, uint32_t *partials) {
+  NTS_TRACE_RANGE("nts_spmm_plan_info");
   if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_info: null plan");
   if (items) *items = plan->n_items;
   if (split_rows) *split_rows = plan->n_splits;
@@ -844,6 +849,7 @@ int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *s
 }
 
 int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F) {
+  NTS_TRACE_RANGE("nts_spmm_plan_reserve");
   if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_reserve: null plan");
   if (plan->n_partials == 0 || F <= plan->partial_F) return NTS_OK;
   // The old buffer may still be read by work queued earlier: hipFree waits for the device.
@@ -870,6 +876,7 @@ int check_heads(const float *alpha, uint32_t H, uint32_t Fh, const char *who) {
 int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
                           const uint32_t *offsets, const uint32_t *indices, uint32_t rows, uint32_t edges, uint32_t H,
                           uint32_t Fh, int accumulate, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_gather_heads");
   if (int rc = check_heads(alpha, H, Fh, "nts_spmm_gather_heads: bad H / Fh / alpha")) return rc;
   if (rows == 0) return NTS_OK;
   if (!in || !out || !offsets || !indices) return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_heads: null pointer");
@@ -883,6 +890,7 @@ int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const
 int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *alpha,
                                   const uint32_t *perm, const uint32_t *offsets, const uint32_t *indices, uint32_t H,
                                   uint32_t Fh, int accumulate, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_gather_heads_planned");
   if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_heads_planned: null plan");
   if (offsets != plan->offsets)
     return nts::fail(NTS_ERR_INVALID,
@@ -908,6 +916,7 @@ int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float 
 }
 
 int nts_spmm_plan_set_events(nts_spmm_plan_t *plan, nts_event_t start, nts_event_t stop) {
+  NTS_TRACE_RANGE("nts_spmm_plan_set_events");
   if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_set_events: null plan");
   if ((start == nullptr) != (stop == nullptr))
     return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_set_events: pass both events or neither");
@@ -919,6 +928,7 @@ int nts_spmm_plan_set_events(nts_spmm_plan_t *plan, nts_event_t start, nts_event
 int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *w,
                             const uint32_t *offsets, const uint32_t *indices, uint32_t index_base, uint32_t F,
                             int accumulate, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_gather_planned");
   if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_planned: null plan");
   if (offsets != plan->offsets)
     return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_planned: offsets differ from the array the plan was built from");
