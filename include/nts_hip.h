@@ -149,8 +149,11 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan, const uint32_t *offsets, uint32
  * so that concurrently running wavefronts gather from the same range of source rows (each XCD's
  * L2 then holds that range's hot rows).  n_slabs = 0 and chunk_edges = 0 select the defaults (32
  * ranges, 512 edges, tuned on a 114.8 M-edge power-law graph at F = 602); rows whose indices do
- * not ascend are split by edge count as above.  Results differ from nts_spmm_plan_create only in
- * where split rows are cut. */
+ * not ascend are split by edge count as above.  With 8 or more ranges, ascending rows of more
+ * than chunk_edges / 4 edges are cut as well, at the boundaries of n_slabs / 4 four-times-wider
+ * ranges (their pieces run next to the long rows' pieces of the same sources); such a row stays
+ * whole when all its edges fall into one wide range.  Results differ from nts_spmm_plan_create only
+ * in which rows are cut and where; rows of at most chunk_edges / 4 edges are never cut. */
 int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan, const uint32_t *offsets, const uint32_t *indices,
                                uint32_t index_base, uint32_t n_index, uint32_t rows, uint32_t edges,
                                uint32_t chunk_edges, uint32_t n_slabs, nts_stream_t stream);

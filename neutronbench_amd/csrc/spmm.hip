@@ -708,9 +708,52 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
   std::vector<uint32_t> bucket(static_cast<size_t>(chunk) + 2, 0u);
   const bool slabbed = n_slabs > 1 && idx != nullptr && n_index > 0;
   const uint64_t slab_width = slabbed ? (static_cast<uint64_t>(n_index) + n_slabs - 1) / n_slabs : 0;
+  // Second tier: rows of chunk/4 .. chunk edges are too short for the fine ranges (their pieces
+  // would be a handful of edges each, and every piece costs a partial row), but cut at a quarter as
+  // many, four times wider ranges their pieces still run next to the long rows' pieces of the same
+  // sources.  A row whose edges all fall into one wide range stays whole.
+  constexpr uint32_t kWide = 4;  // fine ranges per wide range
+  constexpr uint32_t kDiv = 4;   // rows above chunk / kDiv edges take part
+  const uint32_t n_coarse = slabbed && n_slabs >= 2 * kWide ? n_slabs / kWide : 0;
+  const bool tier2 = n_coarse > 0;
+  std::vector<uint8_t> was_cut(tier2 ? rows : 0, 0);
   for (uint32_t r = 0; r < rows; ++r) {
     const uint32_t b = off[r], e = off[r + 1], deg = e - b;
     if (deg <= chunk) {
+      if (tier2 && deg > chunk / kDiv) {
+        bool ascending = true;
+        for (uint32_t k = b + 1; k < e && ascending; ++k) ascending = idx[k - 1] <= idx[k];
+        if (ascending) {
+          uint32_t cuts[64];
+          uint32_t n_cuts = 0, cut = b;
+          const uint64_t wide = slab_width * kWide;
+          const uint32_t ranges = n_coarse < 63 ? n_coarse : 63;
+          for (uint32_t c = 0; c < ranges && cut < e; ++c) {
+            const uint64_t hi = (c + 1) * wide;
+            const uint32_t stop =
+                c + 1 == ranges ? e
+                                : static_cast<uint32_t>(std::lower_bound(idx + cut, idx + e, hi,
+                                                                         [](uint32_t v, uint64_t lim) { return v < lim; }) -
+                                                        idx);
+            if (stop > cut) {
+              cuts[n_cuts++] = c;
+              cuts[n_cuts++] = stop;
+            }
+            cut = stop;
+          }
+          if (n_cuts > 2) {
+            const uint32_t first = n_partials;
+            uint32_t from = b;
+            for (uint32_t q = 0; q < n_cuts; q += 2) {
+              pieces.push_back(Piece{cuts[q] * kWide, r, from, cuts[q + 1], n_partials++});
+              from = cuts[q + 1];
+            }
+            splits.push_back(make_uint4(r, first, n_partials - first, 0u));
+            was_cut[r] = 1;
+            continue;
+          }
+        }
+      }
       ++bucket[chunk - deg + 1];  // descending degree
       continue;
     }
@@ -749,7 +792,8 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
   items.resize(base + bucket.back());
   for (uint32_t r = 0; r < rows; ++r) {
     const uint32_t deg = off[r + 1] - off[r];
-    if (deg <= chunk) items[base + bucket[chunk - deg]++] = make_uint4(r, off[r], off[r + 1], nts::kNoSlot);
+    if (deg <= chunk && !(tier2 && was_cut[r]))
+      items[base + bucket[chunk - deg]++] = make_uint4(r, off[r], off[r + 1], nts::kNoSlot);
   }
 
   nts_spmm_plan *p = new (std::nothrow) nts_spmm_plan();

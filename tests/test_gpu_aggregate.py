@@ -228,7 +228,7 @@ def test_empty_and_error_paths(device):
 
 
 @pytest.mark.parametrize("F,chunk,slabs,sorted_rows", [(128, 64, 4, True), (602, 100, 8, True), (41, 32, 16, True),
-                                                       (100, 64, 8, False), (16, 16, 3, True)])
+                                                       (100, 64, 8, False), (16, 16, 3, True), (64, 48, 32, True)])
 def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
     """Source-range ("slab") schedule: same results as the oracle to tolerance, bit-reproducible, and
     rows whose indices do not ascend fall back to edge-count chunks."""
@@ -245,12 +245,22 @@ def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
     plan = SpmmPlan(dco, Vd, ri.size, chunk, dri, Vs, slabs)
     info = plan.info()
     deg = np.diff(co.astype(np.int64))
-    assert info["split_rows"] == int((deg > chunk).sum())
+    # With 8 or more source ranges, sorted rows of more than chunk/4 edges are cut as well, at a
+    # quarter as many (wider) ranges, unless all their edges fall into one of those.
+    second_tier = sorted_rows and slabs >= 8
+    whole_up_to = chunk // 4 if second_tier else chunk
+    long_rows = int((deg > chunk).sum())
     plain = int(np.ceil(deg[deg > chunk] / chunk).sum())
-    if sorted_rows:
-        assert plain <= info["partials"] <= plain + info["split_rows"] * slabs
+    if second_tier:
+        medium = int(((deg > whole_up_to) & (deg <= chunk)).sum())
+        assert long_rows <= info["split_rows"] <= long_rows + medium
+        assert plain <= info["partials"] <= plain + long_rows * slabs + medium * (slabs // 4)
     else:
-        assert info["partials"] == plain
+        assert info["split_rows"] == long_rows
+        if sorted_rows:
+            assert plain <= info["partials"] <= plain + info["split_rows"] * slabs
+        else:
+            assert info["partials"] == plain
     outs = []
     for _ in range(2):
         out = torch.full((Vd, F), float("nan"), device=device)
@@ -259,7 +269,7 @@ def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
         outs.append(out.cpu().numpy())
     check(outs[0], oracle.spmm(x, w, co, ri, Vd), abs_term_scale(x, w, co, ri, Vd))
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
-    keep = deg <= chunk
+    keep = deg <= whole_up_to
     assert np.array_equal(outs[0][keep].view(np.uint32), oracle.spmm(x, w, co, ri, Vd, fused=True)[keep].view(np.uint32))
     plan.close()
 
