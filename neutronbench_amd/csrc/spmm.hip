@@ -707,72 +707,72 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
   uint32_t n_partials = 0;
   std::vector<uint32_t> bucket(static_cast<size_t>(chunk) + 2, 0u);
   const bool slabbed = n_slabs > 1 && idx != nullptr && n_index > 0;
-  const uint64_t slab_width = slabbed ? (static_cast<uint64_t>(n_index) + n_slabs - 1) / n_slabs : 0;
-  // Second tier: rows of chunk/4 .. chunk edges are too short for the fine ranges (their pieces
-  // would be a handful of edges each, and every piece costs a partial row), but cut at a quarter as
-  // many, four times wider ranges their pieces still run next to the long rows' pieces of the same
-  // sources.  A row whose edges all fall into one wide range stays whole.
-  constexpr uint32_t kWide = 4;  // fine ranges per wide range
-  constexpr uint32_t kDiv = 4;   // rows above chunk / kDiv edges take part
-  const uint32_t n_coarse = slabbed && n_slabs >= 2 * kWide ? n_slabs / kWide : 0;
-  const bool tier2 = n_coarse > 0;
-  std::vector<uint8_t> was_cut(tier2 ? rows : 0, 0);
+  // Source ranges come in two widths and a row is cut at the width that suits its length: every
+  // piece costs one partial row (written, then read by the second stage), so shorter rows get
+  // fewer, wider ranges.
+  //   more than chunk edges        n_slabs ranges
+  //   more than chunk / 4 edges    n_slabs / 4 ranges; a row whose edges all fall into one of them stays whole
+  // A piece is issued with the first narrow range it covers, so that wavefronts resident at the
+  // same time gather from the same part of the source rows whatever the width of their ranges.
+  // (Twice or four times as many, narrower ranges for rows above 2,048 .. 16,384 edges were
+  // measured as well: no gain on the 114.8 M-edge power-law graph.)
+  const uint32_t fine = slabbed ? n_slabs : 1;
+  const uint64_t fine_width = slabbed ? (static_cast<uint64_t>(n_index) + fine - 1) / fine : 0;
+  const uint32_t wide_ranges = slabbed && n_slabs >= 8 ? n_slabs / 4 : 0;
+  std::vector<uint8_t> was_cut(wide_ranges ? rows : 0, 0);
+  std::vector<uint32_t> stops;  // (narrow range id, end edge) of the non-empty ranges of one row
+  // Cuts edges [b, e) of a row with ascending indices at `ranges` equal ranges; ranges divides fine.
+  auto range_stops = [&](uint32_t b, uint32_t e, uint32_t ranges) {
+    stops.clear();
+    const uint32_t per = fine / ranges;
+    uint32_t cut = b;
+    for (uint32_t c = 0; c < ranges && cut < e; ++c) {
+      const uint64_t hi = static_cast<uint64_t>(c + 1) * per * fine_width;  // first index of the next range
+      const uint32_t stop =
+          c + 1 == ranges ? e
+                          : static_cast<uint32_t>(std::lower_bound(idx + cut, idx + e, hi,
+                                                                   [](uint32_t v, uint64_t lim) { return v < lim; }) -
+                                                  idx);
+      if (stop > cut) {
+        stops.push_back(c * per);
+        stops.push_back(stop);
+      }
+      cut = stop;
+    }
+  };
+  auto is_ascending = [&](uint32_t b, uint32_t e) {
+    for (uint32_t k = b + 1; k < e; ++k)
+      if (idx[k - 1] > idx[k]) return false;
+    return true;
+  };
   for (uint32_t r = 0; r < rows; ++r) {
     const uint32_t b = off[r], e = off[r + 1], deg = e - b;
     if (deg <= chunk) {
-      if (tier2 && deg > chunk / kDiv) {
-        bool ascending = true;
-        for (uint32_t k = b + 1; k < e && ascending; ++k) ascending = idx[k - 1] <= idx[k];
-        if (ascending) {
-          uint32_t cuts[64];
-          uint32_t n_cuts = 0, cut = b;
-          const uint64_t wide = slab_width * kWide;
-          const uint32_t ranges = n_coarse < 63 ? n_coarse : 63;
-          for (uint32_t c = 0; c < ranges && cut < e; ++c) {
-            const uint64_t hi = (c + 1) * wide;
-            const uint32_t stop =
-                c + 1 == ranges ? e
-                                : static_cast<uint32_t>(std::lower_bound(idx + cut, idx + e, hi,
-                                                                         [](uint32_t v, uint64_t lim) { return v < lim; }) -
-                                                        idx);
-            if (stop > cut) {
-              cuts[n_cuts++] = c;
-              cuts[n_cuts++] = stop;
-            }
-            cut = stop;
+      if (wide_ranges && deg > chunk / 4 && is_ascending(b, e)) {
+        range_stops(b, e, wide_ranges);
+        if (stops.size() > 2) {
+          const uint32_t first = n_partials;
+          uint32_t from = b;
+          for (size_t q = 0; q < stops.size(); q += 2) {
+            pieces.push_back(Piece{stops[q], r, from, stops[q + 1], n_partials++});
+            from = stops[q + 1];
           }
-          if (n_cuts > 2) {
-            const uint32_t first = n_partials;
-            uint32_t from = b;
-            for (uint32_t q = 0; q < n_cuts; q += 2) {
-              pieces.push_back(Piece{cuts[q] * kWide, r, from, cuts[q + 1], n_partials++});
-              from = cuts[q + 1];
-            }
-            splits.push_back(make_uint4(r, first, n_partials - first, 0u));
-            was_cut[r] = 1;
-            continue;
-          }
+          splits.push_back(make_uint4(r, first, n_partials - first, 0u));
+          was_cut[r] = 1;
+          continue;
         }
       }
       ++bucket[chunk - deg + 1];  // descending degree
       continue;
     }
     const uint32_t first = n_partials;
-    bool ascending = slabbed;
-    if (slabbed)
-      for (uint32_t k = b + 1; k < e && ascending; ++k) ascending = idx[k - 1] <= idx[k];
-    if (ascending) {
-      uint32_t cut = b;
-      for (uint32_t sl = 0; sl < n_slabs && cut < e; ++sl) {
-        const uint64_t hi = (sl + 1) * slab_width;  // first index value of the next slab
-        const uint32_t stop =
-            sl + 1 == n_slabs ? e
-                              : static_cast<uint32_t>(std::lower_bound(idx + cut, idx + e, hi,
-                                                                       [](uint32_t v, uint64_t lim) { return v < lim; }) -
-                                                      idx);
-        for (uint32_t k = cut; k < stop; k += chunk)
-          pieces.push_back(Piece{sl, r, k, std::min(stop, k + chunk), n_partials++});
-        cut = stop;
+    if (slabbed && is_ascending(b, e)) {
+      range_stops(b, e, n_slabs);
+      uint32_t from = b;
+      for (size_t q = 0; q < stops.size(); q += 2) {
+        for (uint32_t k = from; k < stops[q + 1]; k += chunk)
+          pieces.push_back(Piece{stops[q], r, k, std::min(stops[q + 1], k + chunk), n_partials++});
+        from = stops[q + 1];
       }
     } else {
       for (uint32_t k = b; k < e; k += chunk) pieces.push_back(Piece{0u, r, k, std::min(e, k + chunk), n_partials++});
@@ -792,7 +792,7 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
   items.resize(base + bucket.back());
   for (uint32_t r = 0; r < rows; ++r) {
     const uint32_t deg = off[r + 1] - off[r];
-    if (deg <= chunk && !(tier2 && was_cut[r]))
+    if (deg <= chunk && !(wide_ranges && was_cut[r]))
       items[base + bucket[chunk - deg]++] = make_uint4(r, off[r], off[r + 1], nts::kNoSlot);
   }
 
