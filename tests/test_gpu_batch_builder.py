@@ -151,3 +151,30 @@ def test_builder_rejects_what_it_cannot_hold(device):
     call("nts_batch_builder_layers", handle.value, ctypes.addressof(desc))
     assert desc[1].v_size == 16 and desc[0].v_size == desc[1].src_size
     call("nts_batch_builder_destroy", handle.value)
+
+
+def test_two_builders_on_two_streams_overlap_without_interference(device):
+    """The pipelined use: batch k+1 is built by a second builder on a second stream while batch k's
+    layers are still being read.  Each batch equals what a lone builder gives for it."""
+    V, E, fanouts, batch = 40000, 900000, [10, 15], 2000
+    gco, gri = graph(V, E, 51, device)
+    perm = as_u32(synth.permutation(V, 52, device))
+    lone = BatchBuilder(gco, gri, fanouts, batch, want_perm=True)
+    want = []
+    for k in range(6):
+        layers = lone.sample(perm[k * batch:(k + 1) * batch], 90 + k)
+        want.append([{name: getattr(l, name).cpu().numpy().copy() for name in ARRAYS} for l in layers])
+    lone.close()
+    builders = [BatchBuilder(gco, gri, fanouts, batch, want_perm=True) for _ in range(2)]
+    streams = [torch.cuda.Stream(device=device) for _ in range(2)]
+    torch.cuda.synchronize()
+    builders[0].enqueue(perm[0:batch], 90, streams[0].cuda_stream)
+    for k in range(6):
+        if k + 1 < 6:  # start the next batch before this one is collected
+            builders[(k + 1) % 2].enqueue(perm[(k + 1) * batch:(k + 2) * batch], 91 + k, streams[(k + 1) % 2].cuda_stream)
+        layers = builders[k % 2].collect()
+        for l, expect in zip(layers, want[k]):
+            for name in ARRAYS:
+                assert getattr(l, name).cpu().numpy().tobytes() == expect[name].tobytes(), f"batch {k} {name}"
+    for b in builders:
+        b.close()
