@@ -49,6 +49,15 @@ int nts_abi_version(void);
  * brackets its stages with wall-clock accumulators instead (toolkits/GCN_GPU_NEIGHBOR.hpp:617-705).
  * nts_trace_ranges_emitted: ranges pushed so far by this process (0 when ranges are off). */
 long nts_trace_ranges_emitted(void);
+/* Scratch memory.  A few entry points need device memory beyond their arguments (stated with each
+ * of them: calls of nts_spmm_gather / nts_spmm_gather_heads that cut hub rows, the lists of hub rows
+ * of the edge operators, nts_gather_edge_to_src_unsorted).  It is allocated and freed in stream
+ * order from a memory pool of the library's own, one per device, which keeps freed blocks for the
+ * next call instead of returning them to the driver at every synchronisation: the pool holds on to
+ * the largest scratch any call has needed (the reference allocates such buffers with cudaMalloc per
+ * call, cuda/ntsCUDAGraphOP.cu:595-653).  nts_scratch_trim returns the current device's unused
+ * scratch to the driver; work queued earlier is not affected. */
+int nts_scratch_trim(void);
 
 /* ---------------------------------------------------------------------------------------------
  * Memory, copies, streams
@@ -125,11 +134,12 @@ int nts_event_elapsed_ms(float *ms, nts_event_t start, nts_event_t stop);
  *               reference's semantics on a pre-zeroed output
  * Works without any preprocessing; one wavefront (or a sub-wavefront group for narrow F) per row,
  * its edges added in order with one fused multiply-add each.  Calls of 65,536 edges or more do not
- * leave long rows to one wavefront: rows of more than 1,024 edges are cut into 1,024-edge pieces on
- * the device (no copy to the host), the pieces write partial sums and a second stage adds them in
- * order -- still deterministic, but a long row's sum is then associated piece by piece.  That path
- * takes stream-ordered scratch (hipMallocAsync, about (E/1024 + min(rows, E/1024) + 1) * (F * 4 + 48)
- * bytes plus 8 bytes per row, released with hipFreeAsync); a caller that must not allocate, or that runs
+ * leave long rows to one wavefront: rows of more than P edges are cut into P-edge pieces on the
+ * device (no copy to the host), the pieces write partial sums and a second stage adds them in
+ * order -- still deterministic, but a long row's sum is then associated piece by piece.  P = 1,024
+ * edges, 256 for calls below 2^22 edges (sampled layers).  That path takes stream-ordered scratch
+ * (hipMallocAsync, about (E/P + min(rows, E/P) + 1) * (F * 4 + 48) bytes plus 8 bytes per row,
+ * released with hipFreeAsync); a caller that must not allocate, or that runs
  * the same structure many times, uses a plan (below), which also orders the pieces for the L2. */
 int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t *offsets,
                     const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
@@ -251,7 +261,7 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
  *   out[r, h*Fh + f] (+)= sum_{e in [offsets[r], offsets[r+1])} alpha[eid(e), h] * in[indices[e], h*Fh + f]
  * eid(e) = e when perm is NULL (forward over CSC) or perm[e] (backward over CSR, alpha kept in
  * CSC edge order).  `edges` = offsets[rows]; as in nts_spmm_gather, calls of 65,536 edges or more
- * cut rows of more than 1,024 edges into pieces on the device. */
+ * cut long rows into pieces on the device (same piece length). */
 int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
                           const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
                           uint32_t edges, uint32_t H, uint32_t Fh, int accumulate, nts_stream_t stream);

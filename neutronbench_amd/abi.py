@@ -28,6 +28,7 @@ SIGNATURES = {
     "nts_last_error": [],
     "nts_abi_version": [],
     "nts_trace_ranges_emitted": [],
+    "nts_scratch_trim": [],
     "nts_malloc_device": [ctypes.POINTER(_vp), _sz],
     "nts_free_device": [_vp],
     "nts_malloc_device_async": [ctypes.POINTER(_vp), _sz, _vp],

@@ -56,6 +56,15 @@ struct TraceRange {
 };
 #define NTS_TRACE_RANGE(name) ::nts::TraceRange nts_trace_range__(name)
 
+// Stream-ordered scratch of the entry points that need device memory beyond their arguments
+// (lists of hub rows, partial sums of calls without a plan).  It comes from a memory pool of the
+// library's own, one per device, that keeps freed blocks instead of handing them back to the
+// driver at every synchronisation (the default pool's behaviour, which makes each call pay for a
+// fresh allocation): the pool holds on to the largest scratch any call has needed.
+hipError_t scratch_alloc(void **ptr, size_t bytes, hipStream_t stream);
+hipError_t scratch_free(void *ptr, hipStream_t stream);
+hipError_t scratch_trim();  // gives the current device's unused scratch back to the driver
+
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 inline uint32_t ceil_div(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }

@@ -1224,7 +1224,7 @@ int collect_long_rows(LongRows &lr, const uint32_t *off, uint32_t rows, uint32_t
   const size_t list_bytes = (static_cast<size_t>(rows) + 1 + 7) / 8 * 8 * sizeof(uint32_t);  // list + counter, 32-byte multiple
   const size_t small_bytes = (8 + kGiantCap + kGiantCap + 8) * sizeof(uint32_t);             // hdr, rows, first
   unsigned char *buf = nullptr;
-  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&buf), list_bytes + small_bytes + kPieceCap * sizeof(uint4),
+  NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&buf), list_bytes + small_bytes + kPieceCap * sizeof(uint4),
                              stream));
   lr.list = reinterpret_cast<uint32_t *>(buf);
   lr.count = lr.list + rows;
@@ -1243,7 +1243,7 @@ int collect_long_rows(LongRows &lr, const uint32_t *off, uint32_t rows, uint32_t
 }
 
 int release_long_rows(LongRows &lr, hipStream_t stream) {
-  if (lr.list) NTS_HIP_TRY(hipFreeAsync(lr.list, stream));
+  if (lr.list) NTS_HIP_TRY(scratch_free(lr.list, stream));
   lr = LongRows();
   return NTS_OK;
 }
@@ -1309,14 +1309,14 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
     NTS_LAUNCH_CHECK(who);
     // Giant rows: pieces by separate blocks into stream-ordered scratch, then the ordered combine.
     float *partial = nullptr;
-    NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&partial), static_cast<size_t>(kPieceCap) * F * sizeof(float),
+    NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&partial), static_cast<size_t>(kPieceCap) * F * sizeof(float),
                                stream));
     hipLaunchKernelGGL(giant_sum_pieces_kernel, dim3(kLongGrid), dim3(kLongBlock), 0, stream, partial, msg, perm, lr.hdr,
                        lr.pieces, F, tile);
     hipLaunchKernelGGL(giant_sum_combine_kernel, dim3(kGiantCap / 4), dim3(256), 0, stream, out, partial, lr.hdr,
                        lr.giant_rows, lr.first, F, accumulate);
     const hipError_t launch_err = hipGetLastError();
-    NTS_HIP_TRY(hipFreeAsync(partial, stream));
+    NTS_HIP_TRY(scratch_free(partial, stream));
     if (launch_err != hipSuccess) return fail_hip(launch_err, who);
   }
   return release_long_rows(lr, stream);
@@ -1388,7 +1388,7 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
     // Giant segments: per-piece statistics, ordered combine, apply (see the kernels above).
     float *stats = nullptr;
     const size_t stats_floats = static_cast<size_t>(kPieceCap) * 2 * H, row_floats = static_cast<size_t>(kGiantCap) * 2 * H;
-    NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&stats), (stats_floats + row_floats) * sizeof(float), stream));
+    NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&stats), (stats_floats + row_floats) * sizeof(float), stream));
     float *rowstat = stats + stats_floats;
     const dim3 pgrid(kLongGrid), pblock(kLongBlock), cgrid(kGiantCap / 4), cblock(64);
     if (!backward) {
@@ -1421,7 +1421,7 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
       }
     }
     const hipError_t launch_err = hipGetLastError();
-    NTS_HIP_TRY(hipFreeAsync(stats, stream));
+    NTS_HIP_TRY(scratch_free(stats, stream));
     if (launch_err != hipSuccess) return fail_hip(launch_err, who);
   }
   return release_long_rows(lr, stream);

@@ -395,7 +395,7 @@ int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t
   NTS_HIP_TRY(sort_temp_bytes(E, &tmp));
   const size_t arr = align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256);
   unsigned char *work = nullptr;
-  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&work), 3 * arr + align_up(tmp, 256), stream));
+  NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&work), 3 * arr + align_up(tmp, 256), stream));
   uint32_t *keys = reinterpret_cast<uint32_t *>(work);
   uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(work + arr);
   uint32_t *perm = reinterpret_cast<uint32_t *>(work + 2 * arr);
@@ -409,7 +409,7 @@ int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t
     hipLaunchKernelGGL(add_runs_kernel, dim3(ceil_div(E, 4)), dim3(256), 0, stream, out, msg, keys_sorted, perm, E, F);
     err = hipGetLastError();
   }
-  hipError_t ferr = hipFreeAsync(work, stream);
+  hipError_t ferr = scratch_free(work, stream);
   if (err != hipSuccess) return fail_hip(err, "nts_gather_edge_to_src_unsorted");
   if (ferr != hipSuccess) return fail_hip(ferr, "nts_gather_edge_to_src_unsorted: hipFreeAsync");
   return NTS_OK;

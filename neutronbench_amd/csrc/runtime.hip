@@ -6,6 +6,7 @@
 #include <stdlib.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -57,6 +58,57 @@ const TraceApi *trace_api() {
   return api;
 }
 
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_pool_mutex;
+hipMemPool_t g_scratch_pool[kMaxDevices] = {};
+
+hipError_t scratch_pool(hipMemPool_t *pool) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  if (!g_scratch_pool[dev]) {
+    hipMemPoolProps props = {};
+    props.allocType = hipMemAllocationTypePinned;
+    props.handleTypes = hipMemHandleTypeNone;
+    props.location.type = hipMemLocationTypeDevice;
+    props.location.id = dev;
+    hipMemPool_t created = nullptr;
+    err = hipMemPoolCreate(&created, &props);
+    if (err != hipSuccess) return err;
+    uint64_t keep = UINT64_MAX;  // never trim at synchronisation points
+    err = hipMemPoolSetAttribute(created, hipMemPoolAttrReleaseThreshold, &keep);
+    if (err != hipSuccess) {
+      (void)hipMemPoolDestroy(created);
+      return err;
+    }
+    g_scratch_pool[dev] = created;
+  }
+  *pool = g_scratch_pool[dev];
+  return hipSuccess;
+}
+}  // namespace
+
+hipError_t scratch_alloc(void **ptr, size_t bytes, hipStream_t stream) {
+  hipMemPool_t pool = nullptr;
+  hipError_t err = scratch_pool(&pool);
+  if (err != hipSuccess) return err;
+  return hipMallocFromPoolAsync(ptr, bytes, pool, stream);
+}
+
+hipError_t scratch_free(void *ptr, hipStream_t stream) { return hipFreeAsync(ptr, stream); }
+
+hipError_t scratch_trim() {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  return g_scratch_pool[dev] ? hipMemPoolTrimTo(g_scratch_pool[dev], 0) : hipSuccess;
+}
+
 void count_trace_range() { g_trace_ranges.fetch_add(1, std::memory_order_relaxed); }
 long trace_ranges_emitted() { return g_trace_ranges.load(std::memory_order_relaxed); }
 
@@ -68,6 +120,10 @@ extern "C" {
 
 const char *nts_last_error(void) { return nts::g_last_error; }
 long nts_trace_ranges_emitted(void) { return nts::trace_ranges_emitted(); }
+int nts_scratch_trim(void) {
+  hipError_t err = nts::scratch_trim();
+  return err == hipSuccess ? NTS_OK : nts::fail_hip(err, "nts_scratch_trim");
+}
 
 int nts_abi_version(void) { return 1; }
 

@@ -480,7 +480,8 @@ void launch_spmm(const LaunchArgs &a) {
 //
 // A call that brings no plan still must not let one wavefront walk a 10^5-edge row alone.  For edge
 // counts where that can matter, the pieces are derived on the device in the same stream, without
-// any copy to the host: pieces[r] = ceil(deg/chunk) for rows longer than `chunk` (else 0), an
+// any copy to the host: pieces[r] = ceil(deg/chunk) for rows longer than `chunk` (else 0; chunk =
+// 1,024 edges, 256 for calls below 2^22 edges), an
 // exclusive scan gives each long row its first partial slot, one thread per possible piece writes
 // the work item (binary search of the scan), whole-row wavefronts skip the long rows, the piece
 // wavefronts write partial sums and a last kernel adds each long row's partials in slot order.
@@ -490,6 +491,11 @@ void launch_spmm(const LaunchArgs &a) {
 
 constexpr uint32_t kAutoMinEdges = 1u << 16;  // below this a serial hub row costs less than the set-up
 constexpr uint32_t kAutoChunk = 1024;
+// Calls below this many edges (sampled layers) use shorter pieces -- a few thousand 1,024-edge
+// chains leave most of the GPU idle -- and skip the ordering of the pieces by source: their source
+// rows fit the caches anyway and every launch saved counts at this size.
+constexpr uint32_t kAutoLargeEdges = 1u << 22;
+constexpr uint32_t kAutoSmallChunk = 256;
 
 __global__ __launch_bounds__(256) void auto_count_kernel(uint32_t *__restrict__ pieces,
                                                          const uint32_t *__restrict__ off, uint32_t rows,
@@ -570,7 +576,8 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
     launch_spmm(a);
     return NTS_OK;
   }
-  const uint32_t chunk = kAutoChunk;
+  const bool large = edges >= kAutoLargeEdges;
+  const uint32_t chunk = large ? kAutoChunk : kAutoSmallChunk;
   const uint32_t by_edges = edges / chunk;
   const uint32_t p_max = by_edges + (rows < by_edges ? rows : by_edges) + 1;
   size_t scan_bytes = 0, sort_bytes = 0;
@@ -587,7 +594,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
   const size_t n_keys_b = up256(static_cast<size_t>(p_max) * sizeof(uint32_t));
   const size_t n_partial = up256(static_cast<size_t>(p_max) * a.F * sizeof(float));
   unsigned char *buf = nullptr;
-  NTS_HIP_TRY(hipMallocAsync(reinterpret_cast<void **>(&buf),
+  NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&buf),
                              2 * n_off + 2 * n_items_b + 3 * n_keys_b + tmp_bytes + n_partial, a.stream));
   unsigned char *cursor = buf;
   auto take = [&cursor](size_t bytes) {
@@ -605,7 +612,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
   void *tmp = take(tmp_bytes);
   float *partial = reinterpret_cast<float *>(take(n_partial));
   auto bail = [&](hipError_t err, const char *what) {
-    (void)hipFreeAsync(buf, a.stream);
+    (void)scratch_free(buf, a.stream);
     return fail_hip(err, what);
   };
   hipLaunchKernelGGL(auto_count_kernel, dim3(ceil_div(static_cast<uint64_t>(rows) + 1, 256)), dim3(256), 0, a.stream,
@@ -619,17 +626,19 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
                      a.indices, a.index_base, rows, chunk, p_max);
   err = hipGetLastError();
   if (err != hipSuccess) return bail(err, "auto_items_kernel");
-  err = rocprim::radix_sort_pairs(tmp, sort_bytes, keys, keys_sorted, rocprim::counting_iterator<uint32_t>(0u), order,
-                                  p_max, 0u, 32u, a.stream, false);
-  if (err != hipSuccess) return bail(err, "spmm: ordering of the pieces");
-  hipLaunchKernelGGL(auto_order_items_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, ordered, items, order,
-                     p_max);
-  err = hipGetLastError();
-  if (err != hipSuccess) return bail(err, "auto_order_items_kernel");
+  if (large) {
+    err = rocprim::radix_sort_pairs(tmp, sort_bytes, keys, keys_sorted, rocprim::counting_iterator<uint32_t>(0u), order,
+                                    p_max, 0u, 32u, a.stream, false);
+    if (err != hipSuccess) return bail(err, "spmm: ordering of the pieces");
+    hipLaunchKernelGGL(auto_order_items_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, ordered, items,
+                       order, p_max);
+    err = hipGetLastError();
+    if (err != hipSuccess) return bail(err, "auto_order_items_kernel");
+  }
   // Pieces first (the heavy, uniform work), then the rows that fit one wavefront.
   LaunchArgs pc = a;
   pc.n_items = p_max;
-  pc.items = ordered;
+  pc.items = large ? ordered : items;
   pc.partial = partial;
   launch_spmm(pc);
   LaunchArgs whole = a;
@@ -639,7 +648,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
                      base, a.F, a.accumulate);
   err = hipGetLastError();
   if (err != hipSuccess) return bail(err, "spmm: balanced launch");
-  NTS_HIP_TRY(hipFreeAsync(buf, a.stream));
+  NTS_HIP_TRY(scratch_free(buf, a.stream));
   return NTS_OK;
 }
 

@@ -134,12 +134,12 @@ def test_planned_split_rows(device, F, chunk):
     plan.close()
 
 
-@pytest.mark.parametrize("F,hubs,piece", [(16, (60000, 20001), 1024), (100, (60000, 20001), 1024),
-                                          (128, (60000, 20001), 1024), (602, (60000, 20001), 1024),
+@pytest.mark.parametrize("F,hubs,piece", [(16, (60000, 20001), 256), (100, (60000, 20001), 256),
+                                          (128, (60000, 20001), 256), (602, (60000, 20001), 256),
                                           (100, (3000000, 2000000), 1024)])    # rows of millions of edges
 def test_planless_call_balances_hub_rows_on_the_device(device, F, hubs, piece):
-    """nts_spmm_gather without a plan: above 65,536 edges rows longer than 1,024 edges are cut into
-    pieces on the device (partial sums + ordered second stage).  Short rows keep the sequential FMA chain bit for
+    """nts_spmm_gather without a plan: above 65,536 edges rows longer than 1,024 edges (256 below
+    2^22 edges) are cut into pieces on the device (partial sums + ordered second stage).  Short rows keep the sequential FMA chain bit for
     bit; long rows match within the fp32 tolerance; accumulate still adds; two runs give identical
     bits."""
     print(f"case F={F} hubs={hubs}", flush=True)
@@ -288,3 +288,25 @@ def test_register_broadcast_variant_in_a_fresh_process(device):
                         "-k", "forward_matches_oracle or planned_split_rows or cache_aware", "--timeout", "120",
                         "--timeout-method", "thread"], env=env, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-1500:]
+
+
+def test_scratch_pool_is_kept_between_calls_and_can_be_trimmed(device):
+    """Calls that cut hub rows take their scratch from the library's own pool: it is kept after the
+    call (the next call does not pay for a fresh allocation) and nts_scratch_trim hands it back."""
+    rng = np.random.default_rng(7)
+    Vd, Vs, F = 2000, 3000, 256
+    deg = rng.integers(0, 30, Vd)
+    deg[3] = 3_000_000  # about 11,700 pieces of 256 edges -> ~24 MB of partial sums
+    co = np.zeros(Vd + 1, dtype=np.uint32)
+    co[1:] = np.cumsum(deg)
+    ri = rng.integers(0, Vs, int(co[-1])).astype(np.uint32)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    call("nts_scratch_trim")
+    first = _run_planless(x, None, co, ri, Vd, F, device)  # synchronises before it returns
+    held = torch.cuda.mem_get_info()[0]
+    call("nts_scratch_trim")
+    released = torch.cuda.mem_get_info()[0] - held
+    assert released >= 8 << 20, released  # the pool still had the partial-sum scratch, and gave it back
+    again = _run_planless(x, None, co, ri, Vd, F, device)
+    assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+    call("nts_scratch_trim")
