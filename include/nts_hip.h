@@ -138,9 +138,10 @@ int nts_event_elapsed_ms(float *ms, nts_event_t start, nts_event_t stop);
  * device (no copy to the host), the pieces write partial sums and a second stage adds them in
  * order -- still deterministic, but a long row's sum is then associated piece by piece.  P = 1,024
  * edges, 256 for calls below 2^22 edges (sampled layers).  That path takes stream-ordered scratch
- * (hipMallocAsync, about (E/P + min(rows, E/P) + 1) * (F * 4 + 48) bytes plus 8 bytes per row,
- * released with hipFreeAsync); a caller that must not allocate, or that runs
- * the same structure many times, uses a plan (below), which also orders the pieces for the L2. */
+ * from the library's pool (see nts_scratch_trim; about (E/P + min(rows, E/P) + 1) * (F * 4 + 48)
+ * bytes plus 8 bytes per row, released in stream order before the call returns); a caller that
+ * must not allocate, or that runs the same structure many times, uses a plan (below), which also
+ * orders the pieces for the L2. */
 int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t *offsets,
                     const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
                     uint32_t F, int accumulate, nts_stream_t stream);
