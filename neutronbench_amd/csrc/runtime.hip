@@ -93,8 +93,10 @@ hipError_t scratch_pool(hipMemPool_t *pool) {
 
 hipError_t scratch_alloc(void **ptr, size_t bytes, hipStream_t stream) {
   hipMemPool_t pool = nullptr;
-  hipError_t err = scratch_pool(&pool);
-  if (err != hipSuccess) return err;
+  if (scratch_pool(&pool) != hipSuccess) {
+    (void)hipGetLastError();                   // a device without pool support: the device's default pool
+    return hipMallocAsync(ptr, bytes, stream);
+  }
   return hipMallocFromPoolAsync(ptr, bytes, pool, stream);
 }
 
