@@ -43,7 +43,7 @@ bool plan_layout(Layout *L, uint32_t V, uint32_t graph_edges, const int32_t *fan
   L->sizes = take((hops + 1) * kSizeWords * sizeof(uint32_t));
   L->dst0 = take(static_cast<size_t>(max_batch) * sizeof(uint32_t));
   uint32_t vd = max_batch < V ? max_batch : V;
-  uint32_t e_max = 0, vd_max = 0;
+  uint32_t e_max = 0;
   for (uint32_t h = 0; h < hops; ++h) {
     HopLayout &H = L->hop[h];
     const int32_t fan = fanouts[h];
@@ -66,14 +66,21 @@ bool plan_layout(Layout *L, uint32_t V, uint32_t graph_edges, const int32_t *fan
     H.ewf = take(eb);
     H.ewb = take(eb);
     if (H.e_cap > e_max) e_max = H.e_cap;
-    if (H.vd_cap > vd_max) vd_max = H.vd_cap;
     vd = H.vs_cap;
   }
   L->ri_global = take(static_cast<size_t>(e_max) * sizeof(uint32_t));
   L->relabel_bytes = nts_relabel_sources_work_bytes(V);
-  L->csr_bytes = csr_from_csc_bytes(e_max);
-  L->scan_bytes = hop_scan_bytes(vd_max);
-  if (!L->relabel_bytes || !L->csr_bytes || !L->scan_bytes) return false;
+  // The sort and scan scratch is shared by the hops: the largest any of them asks for (a library
+  // routine may pick another algorithm, with other needs, for a smaller input).
+  L->csr_bytes = 0;
+  L->scan_bytes = 0;
+  for (uint32_t h = 0; h < hops; ++h) {
+    const size_t c = csr_from_csc_bytes(L->hop[h].e_cap), sc = hop_scan_bytes(L->hop[h].vd_cap);
+    if (!c || !sc) return false;
+    if (c > L->csr_bytes) L->csr_bytes = c;
+    if (sc > L->scan_bytes) L->scan_bytes = sc;
+  }
+  if (!L->relabel_bytes) return false;
   L->relabel_work = take(L->relabel_bytes);
   L->csr_work = take(L->csr_bytes);
   L->scan_work = take(L->scan_bytes);
