@@ -168,6 +168,15 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan, const uint32_t *offsets, uint32
 int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan, const uint32_t *offsets, const uint32_t *indices,
                                uint32_t index_base, uint32_t n_index, uint32_t rows, uint32_t edges,
                                uint32_t chunk_edges, uint32_t n_slabs, nts_stream_t stream);
+/* The schedule the two calls above would build, computed from HOST copies of the arrays and
+ * returned instead of uploaded (no device needed; indices_host NULL = nts_spmm_plan_create's
+ * schedule, chunk_edges / n_slabs 0 = that call's defaults).  items_out (nullable) receives up to
+ * items_cap items of four words each, in issue order: (row, first edge, end edge, partial-sum slot
+ * or 0xFFFFFFFF for a row that is summed whole).  For tests and for inspecting a schedule. */
+int nts_spmm_plan_schedule_host(const uint32_t *offsets_host, const uint32_t *indices_host, uint32_t n_index,
+                                uint32_t rows, uint32_t chunk_edges, uint32_t n_slabs, uint32_t *items_out,
+                                uint64_t items_cap, uint32_t *n_items, uint32_t *n_split_rows,
+                                uint32_t *n_partials);
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan);
 /* Number of work items, split rows and partial-sum slots of a plan (for tests and reports). */
 int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows,

@@ -55,6 +55,8 @@ SIGNATURES = {
     "nts_spmm_gather": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
     "nts_spmm_plan_create": [ctypes.POINTER(_vp), _vp, _u32, _u32, _u32, _vp],
     "nts_spmm_plan_create_slabs": [ctypes.POINTER(_vp), _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _vp],
+    "nts_spmm_plan_schedule_host": [_vp, _vp, _u32, _u32, _u32, _u32, _vp, _u64, ctypes.POINTER(_u32),
+                                    ctypes.POINTER(_u32), ctypes.POINTER(_u32)],
     "nts_spmm_plan_destroy": [_vp],
     "nts_spmm_plan_info": [_vp, ctypes.POINTER(_u32), ctypes.POINTER(_u32), ctypes.POINTER(_u32)],
     "nts_spmm_plan_reserve": [_vp, _u32],

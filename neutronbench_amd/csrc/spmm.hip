@@ -708,11 +708,17 @@ struct Piece {
 // gather from the same 1/n_slabs of the source rows, which is what lets each 4 MB L2 keep that
 // range's hot rows resident.  Items: all pieces (slab-major, longest first inside a slab), then
 // the unsplit rows by descending degree.
-int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const std::vector<uint32_t> &off,
-               const uint32_t *idx, uint32_t rows, uint32_t edges, uint32_t chunk, uint32_t n_slabs,
-               uint32_t n_index) {
+struct Schedule {
+  std::vector<uint4> items;   // (row, first edge, end edge, partial slot or kNoSlot)
+  std::vector<uint4> splits;  // (row, first slot, slot count, 0)
+  uint32_t n_partials = 0;
+};
+
+// Host-only: needs nothing but the two index arrays.
+void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx, uint32_t rows, uint32_t chunk,
+                   uint32_t n_slabs, uint32_t n_index) {
   std::vector<Piece> pieces;
-  std::vector<uint4> splits;
+  std::vector<uint4> &splits = out.splits;
   uint32_t n_partials = 0;
   std::vector<uint32_t> bucket(static_cast<size_t>(chunk) + 2, 0u);
   const bool slabbed = n_slabs > 1 && idx != nullptr && n_index > 0;
@@ -793,7 +799,7 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
     if (a.slab != b.slab) return a.slab < b.slab;
     return (a.e1 - a.e0) > (b.e1 - b.e0);
   });
-  std::vector<uint4> items;
+  std::vector<uint4> &items = out.items;
   items.reserve(pieces.size() + rows);
   for (const Piece &pc : pieces) items.push_back(make_uint4(pc.row, pc.e0, pc.e1, pc.slot));
   for (size_t i = 1; i < bucket.size(); ++i) bucket[i] += bucket[i - 1];
@@ -804,6 +810,17 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
     if (deg <= chunk && !(wide_ranges && was_cut[r]))
       items[base + bucket[chunk - deg]++] = make_uint4(r, off[r], off[r + 1], nts::kNoSlot);
   }
+  out.n_partials = n_partials;
+}
+
+int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const std::vector<uint32_t> &off,
+               const uint32_t *idx, uint32_t rows, uint32_t edges, uint32_t chunk, uint32_t n_slabs,
+               uint32_t n_index) {
+  Schedule sched;
+  make_schedule(sched, off.data(), idx, rows, chunk, n_slabs, n_index);
+  const std::vector<uint4> &items = sched.items;
+  const std::vector<uint4> &splits = sched.splits;
+  const uint32_t n_partials = sched.n_partials;
 
   nts_spmm_plan *p = new (std::nothrow) nts_spmm_plan();
   if (!p) return nts::fail(NTS_ERR_NOMEM, "nts_spmm_plan_create: host allocation failed");
@@ -877,6 +894,30 @@ int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan_out, const uint32_t *offse
   }
   return build_plan(plan_out, offsets, off, idx.data(), rows, edges, chunk_edges ? chunk_edges : 512u,
                     n_slabs ? n_slabs : 32u, n_index);
+}
+
+int nts_spmm_plan_schedule_host(const uint32_t *offsets_host, const uint32_t *indices_host, uint32_t n_index,
+                                uint32_t rows, uint32_t chunk_edges, uint32_t n_slabs, uint32_t *items_out,
+                                uint64_t items_cap, uint32_t *n_items, uint32_t *n_split_rows, uint32_t *n_partials) {
+  if (rows != 0 && !offsets_host) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_schedule_host: null offsets");
+  for (uint32_t r = 0; r < rows; ++r)
+    if (offsets_host[r + 1] < offsets_host[r])
+      return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_schedule_host: offsets not ascending");
+  if (rows && offsets_host[rows] != 0 && n_slabs > 1 && !indices_host)
+    return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_schedule_host: null indices");
+  Schedule sched;
+  const bool with_ranges = indices_host != nullptr;
+  make_schedule(sched, offsets_host, indices_host, rows, chunk_edges ? chunk_edges : (with_ranges ? 512u : 4096u),
+                with_ranges ? (n_slabs ? n_slabs : 32u) : 1u, n_index);
+  if (n_items) *n_items = static_cast<uint32_t>(sched.items.size());
+  if (n_split_rows) *n_split_rows = static_cast<uint32_t>(sched.splits.size());
+  if (n_partials) *n_partials = sched.n_partials;
+  if (items_out) {
+    if (items_cap < sched.items.size())
+      return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_schedule_host: items_out too small");
+    memcpy(items_out, sched.items.data(), sched.items.size() * sizeof(uint4));
+  }
+  return NTS_OK;
 }
 
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {

@@ -1,0 +1,123 @@
+"""The aggregation schedule as host logic (nts_spmm_plan_schedule_host; no GPU): whatever the degree
+distribution, the work items cover every edge exactly once, the pieces of a split row are
+contiguous, in edge order and own consecutive partial-sum slots, pieces are issued source range by
+source range, and rows below the cutting thresholds stay whole."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from neutronbench_amd import abi
+from neutronbench_amd.abi import call
+
+NO_SLOT = 0xFFFFFFFF
+
+
+def schedule(co, ri, n_index, chunk, slabs):
+    rows = co.size - 1
+    n_items, n_splits, n_partials = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+    ri_ptr = ri.ctypes.data if ri is not None else 0
+    call("nts_spmm_plan_schedule_host", co.ctypes.data, ri_ptr, n_index, rows, chunk, slabs, 0, 0,
+         ctypes.byref(n_items), ctypes.byref(n_splits), ctypes.byref(n_partials))
+    items = np.zeros((n_items.value, 4), dtype=np.uint32)
+    call("nts_spmm_plan_schedule_host", co.ctypes.data, ri_ptr, n_index, rows, chunk, slabs, items.ctypes.data,
+         items.shape[0], None, None, None)
+    return items, n_splits.value, n_partials.value
+
+
+def power_law_block(Vd, Vs, seed, sort_rows=True, hubs=()):
+    rng = np.random.default_rng(seed)
+    deg = np.minimum((rng.pareto(1.1, Vd) * 6).astype(np.int64), 5000)
+    deg[rng.random(Vd) < 0.1] = 0
+    for k, d in enumerate(hubs):
+        deg[(7 * k + 3) % Vd] = d
+    co = np.zeros(Vd + 1, dtype=np.uint32)
+    co[1:] = np.cumsum(deg)
+    ri = rng.integers(0, Vs, int(co[-1])).astype(np.uint32)
+    if sort_rows:
+        for d in range(Vd):
+            ri[co[d]:co[d + 1]].sort()
+    return co, ri, deg
+
+
+def check_invariants(items, n_splits, n_partials, co, ri, deg, chunk, slabs, ranged):
+    rows = co.size - 1
+    covered = np.zeros(int(co[-1]) + 1, dtype=np.int32)
+    whole = items[items[:, 3] == NO_SLOT]
+    pieces = items[items[:, 3] != NO_SLOT]
+    # every edge exactly once, every row exactly once among the whole rows or as pieces
+    for r, e0, e1, _ in items:
+        assert co[r] <= e0 <= e1 <= co[r + 1]
+        covered[e0] += 1
+        covered[e1] -= 1
+    assert np.all(np.cumsum(covered)[:-1] == 1) if co[-1] else True
+    assert np.unique(whole[:, 0]).size == whole.shape[0]
+    assert np.all(whole[:, 1] == co[whole[:, 0]]) and np.all(whole[:, 2] == co[whole[:, 0] + 1])
+    split_rows = np.unique(pieces[:, 0])
+    assert split_rows.size == n_splits and pieces.shape[0] == n_partials
+    assert np.intersect1d(split_rows, whole[:, 0]).size == 0
+    assert split_rows.size + whole.shape[0] == rows  # empty rows are whole rows with no edge
+    # slots: a permutation of 0 .. n_partials-1; inside a row consecutive and in edge order
+    assert np.array_equal(np.sort(pieces[:, 3]), np.arange(n_partials, dtype=np.uint32))
+    order = np.lexsort((pieces[:, 1], pieces[:, 0]))
+    by_row = pieces[order]
+    same = by_row[1:, 0] == by_row[:-1, 0]
+    assert np.all(by_row[1:, 1][same] == by_row[:-1, 2][same])      # contiguous
+    assert np.all(by_row[1:, 3][same] == by_row[:-1, 3][same] + 1)  # consecutive slots in edge order
+    assert np.all(pieces[:, 2] - pieces[:, 1] <= chunk) and np.all(pieces[:, 2] > pieces[:, 1])
+    # thresholds: long rows are always cut; rows of at most chunk/4 edges (chunk without ranges) never
+    second_tier = ranged and slabs >= 8
+    assert set(np.flatnonzero(deg > chunk)) <= set(split_rows.tolist())
+    assert np.all(deg[split_rows] > (chunk // 4 if second_tier else chunk))
+    # whole rows come after all pieces, by descending degree
+    first_whole = np.flatnonzero(items[:, 3] == NO_SLOT)
+    if first_whole.size and pieces.shape[0]:
+        assert first_whole[0] == pieces.shape[0]
+    wd = deg[whole[:, 0]]
+    assert np.all(wd[1:] <= wd[:-1])
+    return pieces
+
+
+@pytest.mark.parametrize("chunk,slabs", [(512, 32), (64, 8), (100, 16), (32, 4), (16, 3), (4096, 1)])
+@pytest.mark.parametrize("seed", [1, 2])
+def test_ranged_schedule_invariants(chunk, slabs, seed):
+    Vd, Vs = 1500, 4000
+    co, ri, deg = power_law_block(Vd, Vs, seed, hubs=(40000, 9000, chunk, chunk + 1, chunk // 4, chunk // 4 + 1))
+    items, n_splits, n_partials = schedule(co, ri, Vs, chunk, slabs)
+    pieces = check_invariants(items, n_splits, n_partials, co, ri, deg, chunk, slabs, ranged=slabs > 1)
+    if slabs > 1:
+        # issue order: the source range of a piece's first edge never decreases along the piece list,
+        # and a piece never crosses a boundary of its row's range width
+        width = -(-Vs // slabs)
+        first_range = ri[pieces[:, 1]] // width
+        last_range = ri[pieces[:, 2] - 1] // width
+        wide = deg[pieces[:, 0]] <= chunk  # second-tier rows use ranges four times as wide
+        issue = np.where(wide, first_range // 4 * 4, first_range)
+        assert np.all(issue[1:] >= issue[:-1])
+        assert np.all(last_range[~wide] == first_range[~wide])
+        assert np.all(last_range[wide] // 4 == first_range[wide] // 4)
+
+
+def test_rows_that_do_not_ascend_fall_back_to_edge_count_pieces():
+    co, ri, deg = power_law_block(800, 3000, 5, sort_rows=False, hubs=(6000, 700))
+    chunk, slabs = 128, 16
+    items, n_splits, n_partials = schedule(co, ri, 3000, chunk, slabs)
+    check_invariants(items, n_splits, n_partials, co, ri, deg, chunk, slabs, ranged=False)
+    assert n_partials == int(np.ceil(deg[deg > chunk] / chunk).sum())
+
+
+def test_schedule_without_indices_and_error_paths():
+    co, ri, deg = power_law_block(500, 900, 9, hubs=(20000,))
+    items, n_splits, n_partials = schedule(co, None, 0, 300, 0)
+    check_invariants(items, n_splits, n_partials, co, ri, deg, 300, 1, ranged=False)
+    empty = np.zeros(1, dtype=np.uint32)
+    items, n_splits, n_partials = schedule(empty, None, 0, 0, 0)
+    assert items.shape[0] == 0 and n_splits == 0 and n_partials == 0
+    bad = np.array([0, 5, 3], dtype=np.uint32)
+    n = ctypes.c_uint32()
+    assert abi.status("nts_spmm_plan_schedule_host", bad.ctypes.data, 0, 0, 2, 0, 0, 0, 0, ctypes.byref(n), None,
+                      None) == abi.NTS_ERR_INVALID
+    assert "ascending" in abi.last_error()
+    small = np.zeros((1, 4), dtype=np.uint32)
+    assert abi.status("nts_spmm_plan_schedule_host", co.ctypes.data, 0, 0, co.size - 1, 300, 0, small.ctypes.data, 1,
+                      None, None, None) == abi.NTS_ERR_INVALID
