@@ -136,8 +136,8 @@ int nts_event_elapsed_ms(float *ms, nts_event_t start, nts_event_t stop);
  * its edges added in order with one fused multiply-add each.  Calls of 65,536 edges or more do not
  * leave long rows to one wavefront: rows of more than P edges are cut into P-edge pieces on the
  * device (no copy to the host), the pieces write partial sums and a second stage adds them in
- * order -- still deterministic, but a long row's sum is then associated piece by piece.  P = 1,024
- * edges, 256 for calls below 2^22 edges (sampled layers).  That path takes stream-ordered scratch
+ * order -- still deterministic, but a long row's sum is then associated piece by piece.  P = 256
+ * edges; from 2^22 edges up the pieces are also issued in source order.  That path takes stream-ordered scratch
  * from the library's pool (see nts_scratch_trim; about (E/P + min(rows, E/P) + 1) * (F * 4 + 48)
  * bytes plus 8 bytes per row, released in stream order before the call returns); a caller that
  * must not allocate, or that runs the same structure many times, uses a plan (below), which also

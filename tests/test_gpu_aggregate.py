@@ -136,10 +136,10 @@ def test_planned_split_rows(device, F, chunk):
 
 @pytest.mark.parametrize("F,hubs,piece", [(16, (60000, 20001), 256), (100, (60000, 20001), 256),
                                           (128, (60000, 20001), 256), (602, (60000, 20001), 256),
-                                          (100, (3000000, 2000000), 1024)])    # rows of millions of edges
+                                          (100, (3000000, 2000000), 256)])     # rows of millions of edges (pieces ordered by source)
 def test_planless_call_balances_hub_rows_on_the_device(device, F, hubs, piece):
-    """nts_spmm_gather without a plan: above 65,536 edges rows longer than 1,024 edges (256 below
-    2^22 edges) are cut into pieces on the device (partial sums + ordered second stage).  Short rows keep the sequential FMA chain bit for
+    """nts_spmm_gather without a plan: above 65,536 edges rows longer than 256 edges are cut into
+    pieces on the device (partial sums + ordered second stage).  Short rows keep the sequential FMA chain bit for
     bit; long rows match within the fp32 tolerance; accumulate still adds; two runs give identical
     bits."""
     print(f"case F={F} hubs={hubs}", flush=True)

@@ -29,11 +29,8 @@ def random_block(Vd, Vs, mean_deg, seed, hub=0, dup=False, empty_frac=0.1):
 def planless_piece_edges(E):
     """Rows of a plan-less aggregation call (nts_spmm_gather, nts_spmm_gather_heads) with at most
     this many edges are summed as one sequential chain, in edge order; longer rows are summed in
-    pieces.  None = no row is cut (calls below 65,536 edges); 256 edges below 2^22 edges (sampled
-    layers: shorter pieces keep the GPU busy), 1,024 from there on."""
-    if E < 1 << 16:
-        return None
-    return 256 if E < 1 << 22 else 1024
+    pieces.  None = no row is cut (calls below 65,536 edges)."""
+    return 256 if E >= 1 << 16 else None
 
 
 def brute_csr(co, ri, Vs):
