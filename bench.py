@@ -60,9 +60,15 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the oracle sample")
     ap.add_argument("--cpu-reference-edges", type=int, default=28_700_000,
                     help="edges of the sample the reference's own CPU operator is timed on (0 = time the oracle instead)")
+    ap.add_argument("--workload", choices=["reddit", "arxiv", "products", "gat"], default="reddit",
+                    help="reddit (default): the aggregation workload above; arxiv / products / gat: per-epoch time of "
+                         "that sampled mini-batch configuration (BASELINE.json configs 2, 4, 5) instead")
+    ap.add_argument("--cpu-batches", type=int, default=3, help="mini-batch workloads: batches the CPU oracle is timed on")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+    if args.workload != "reddit":
+        return run_epoch_workload(args)
 
     import torch
 
@@ -297,6 +303,103 @@ def run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, target_s):
         "kind": "port",
         "sample": f"first {rows} destination rows (forward) and first {rows} source rows (backward) of the same "
                   f"graph, F=602 and F=128, {e_run} edge visits in {t_run:.2f} s",
+    }
+
+
+def run_epoch_workload(args):
+    """Per-epoch time of a sampled mini-batch configuration through the library (every stage through
+    the C ABI, see neutronbench_amd/epoch.py), next to the CPU oracle on a few batches of the same
+    epoch.  One JSON line; `value` is the epoch time with the stages run one after the other, as the
+    reference's default mode does, and config.pipelined_epoch_s the time with the next batch built
+    on a second stream."""
+    import torch
+
+    from neutronbench_amd import epoch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the HIP library has no CPU fallback)")
+    serial = epoch.run(args.workload, pipeline=1, quiet=True)
+    piped = epoch.run(args.workload, pipeline=2, quiet=True)
+    cpu = None
+    if not args.no_cpu_baseline and args.workload != "gat":
+        cpu = epoch_cpu_baseline(torch, args.workload, serial["batches"], args.cpu_batches)
+    cfg = epoch.CONFIGS[args.workload]
+    line = {
+        "metric": "epoch time", "value": serial["epoch_s"], "unit": "s", "n_gpus": 1, "steps": serial["batches"],
+        "warmup": serial["warmup_batches"], "ms_per_step": round(1e3 * serial["epoch_s"] / serial["batches"], 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}-shaped sampled mini-batch epoch, fanout (output side first) "
+                               f"{cfg['fanout']}, batch {cfg['batch']}, {serial['batches']} batches; a step = one batch: "
+                               "sampling, layer construction, feature/label gather, aggregation fwd+bwd of every layer",
+                   "vertices": serial["vertices"], "edges": serial["edges"], "stage_s": serial["stage_s"],
+                   "sampled_edges": serial["sampled_edges"], "gathered_rows": serial["gathered_rows"],
+                   "cache_hit_rate": serial["cache_hit_rate"], "pipelined_epoch_s": piped["epoch_s"]},
+        "roofline": None,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+def epoch_cpu_baseline(torch, name, n_batches, k_batches):
+    """The CPU oracle (restatement of the reference's host steps: sampCSC::postprocessing,
+    generate_csr_from_csc, update_degree + compute_weight_*, get_feature, MiniBatchFuseOp forward and
+    backward) on the first k batches of the epoch, extrapolated to the epoch.  The neighbour pick
+    itself is an input here (the lists the library sampled are used), so the reference's CPU
+    sampling time is not part of the figure."""
+    import numpy as np
+
+    import oracle
+    from neutronbench_amd import epoch, synth
+    from neutronbench_amd.batch import BatchBuilder
+    from neutronbench_amd.layout import as_u32
+
+    cfg = epoch.CONFIGS[name]
+    dev = torch.device("cuda:0")
+    V, E = cfg["V"], cfg["E"]
+    src, dst = synth.rmat_edges(V, E, seed=cfg["seed"], device=dev, sort=True)
+    co, ri = synth.build_csc(src, dst, V)
+    del src, dst
+    gco, gri = as_u32(co), as_u32(ri)
+    feat = synth.normal_features(V, cfg["F"], seed=cfg["seed"] + 40).numpy()
+    train32 = as_u32(synth.permutation(V, cfg["seed"] + 42, dev)[:cfg["train"]])
+    builder = BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"])
+    threads = oracle.max_threads()
+    rng = np.random.default_rng(1)
+    t = {"structure": 0.0, "gather": 0.0, "aggregate": 0.0}
+    k_batches = max(1, min(k_batches, n_batches))
+    u32 = lambda a: a.cpu().numpy().view(np.uint32)  # noqa: E731
+    for b in range(k_batches):
+        layers = builder.sample(train32[b * cfg["batch"]:(b + 1) * cfg["batch"]], 1000 * b)
+        host = [dict(dst=u32(l.dev_destination), co=u32(l.dev_column_offset), src=u32(l.dev_source),
+                     glob=u32(l.dev_source)[u32(l.dev_row_indices)]) for l in layers]
+        outd, ind = np.ones(V, np.uint32), np.ones(V, np.uint32)
+        built = []
+        t0 = time.perf_counter()
+        for h in host[::-1]:  # hop order: the batch's own hop first
+            local, source, n = oracle.postprocess(h["glob"], V)
+            ro, ci = oracle.csr_from_csc(h["co"], local, n)
+            ewf, ewb = oracle.layer_weights(h["co"], local, ro, ci, source, h["dst"], outd, ind)
+            built.append((h["co"], local, ro, ci, ewf, ewb, h["dst"].size, n))
+        t["structure"] += time.perf_counter() - t0
+        built = built[::-1]  # input side first
+        t0 = time.perf_counter()
+        x = oracle.get_feature(feat, host[0]["src"])
+        t["gather"] += time.perf_counter() - t0
+        widths = [cfg["F"]] + [cfg["hidden"]] * (len(built) - 1)
+        for (lco, local, ro, ci, ewf, ewb, Vd, Vs), F in zip(built, widths):
+            xin = x if x.shape == (Vs, F) else rng.standard_normal((Vs, F)).astype(np.float32)
+            g = rng.standard_normal((Vd, F)).astype(np.float32)
+            t0 = time.perf_counter()
+            x = oracle.spmm(xin, ewf, lco, local, Vd, threads=threads)
+            oracle.spmm(g, ewb, ro, ci, Vs, threads=threads)
+            t["aggregate"] += time.perf_counter() - t0
+    builder.close()
+    per_batch = sum(t.values()) / k_batches
+    return {
+        "value": round(per_batch * n_batches, 4), "unit": "s", "cores": threads, "kind": "port",
+        "sample": f"the CPU oracle on the first {k_batches} of {n_batches} batches (the library's sampled neighbour "
+                  f"lists as input; the neighbour pick itself is not timed), extrapolated to the epoch: per batch "
+                  + ", ".join(f"{k} {v / k_batches * 1e3:.2f} ms" for k, v in t.items()),
     }
 
 

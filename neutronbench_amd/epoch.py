@@ -50,7 +50,7 @@ class Timer:
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
-def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1):
+def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False):
     cfg = dict(CONFIGS[name])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
@@ -191,7 +191,10 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         "sampler": sampler, "pipeline": 2 if pipelined else 1, "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
     }
-    print(json.dumps(out))
+    if builder is not None:
+        builder.close()
+    if not quiet:
+        print(json.dumps(out))
     return out
 
 
