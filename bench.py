@@ -13,6 +13,10 @@ the dominant kernel (the F=602 gather) from HIP events recorded around that kern
 baseline timed on the host cores on a bounded sample of the same graph: the reference's own CPU
 operator where the reference-built program oracle/_ref/ref_fullgraph_cpu is present ("reference"),
 else the CPU oracle ("port").
+
+--workload arxiv|products|gat measures the per-epoch time of that sampled mini-batch configuration
+instead (sampling, layer construction, gathers, aggregation fwd+bwd, all through the C ABI) and
+prints it in the same format, with the CPU oracle timed on a few batches of the same epoch.
 """
 import argparse
 import ctypes
