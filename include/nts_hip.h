@@ -159,8 +159,11 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan, const uint32_t *offsets, uint32
  * boundaries of `n_slabs` equal ranges of [index_base, index_base + n_index) and issued slab by slab,
  * so that concurrently running wavefronts gather from the same range of source rows (each XCD's
  * L2 then holds that range's hot rows).  n_slabs = 0 and chunk_edges = 0 select the defaults (32
- * ranges, 512 edges, tuned on a 114.8 M-edge power-law graph at F = 602); rows whose indices do
- * not ascend are split by edge count as above.  With 8 or more ranges, ascending rows of more
+ * ranges, 512 edges, tuned on a 114.8 M-edge power-law graph at F = 602).  A row that is cut but
+ * whose indices do not ascend (an edge file in arbitrary order; the reference's loader leaves CSR
+ * rows in thread-arrival order) is cut in a copy of the index array, owned by the plan, in which
+ * it is sorted (stably); the plan then gathers through that copy (E * 8 more bytes on the device)
+ * and such a row's sum is associated in source order.  With 8 or more ranges, rows of more
  * than chunk_edges / 4 edges are cut as well, at the boundaries of n_slabs / 4 four-times-wider
  * ranges (their pieces run next to the long rows' pieces of the same sources); such a row stays
  * whole when all its edges fall into one wide range.  Results differ from nts_spmm_plan_create only

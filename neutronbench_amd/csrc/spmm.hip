@@ -24,7 +24,9 @@
 #include <rocprim/iterator/counting_iterator.hpp>
 
 #include <algorithm>
+#include <atomic>
 #include <new>
+#include <thread>
 #include <vector>
 
 #include "common.hpp"
@@ -107,7 +109,8 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
                                                         const uint32_t *__restrict__ indices, uint32_t index_base,
                                                         uint32_t n_items, uint32_t F, uint32_t col_base,
                                                         const Item *__restrict__ items, float *__restrict__ partial,
-                                                        int accumulate, HeadArgs heads, uint32_t row_edge_limit) {
+                                                        int accumulate, HeadArgs heads, uint32_t row_edge_limit,
+                                                        const uint32_t *__restrict__ edge_ids) {
   using V = typename Vec<VEC>::type;
   constexpr int U = unroll_for(NACC);
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -155,9 +158,12 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
   uint2 *tile = lds_tile[LDS_TILE ? (threadIdx.x / kWave) : 0];
   // Second component of a pair: the edge weight (as bits), or with per-head weights the id of the
   // edge in alpha's (CSC) order.
+  // edge_ids (a schedule that gathers through its own, re-ordered copy of the indices): position of
+  // edge e in the caller's weight / alpha order.
   auto second_of = [&](uint32_t e) -> uint32_t {
-    if (HEADS) return heads.perm ? heads.perm[e] : e;
-    return w ? __float_as_uint(w[e]) : __float_as_uint(1.f);
+    const uint32_t id = edge_ids ? edge_ids[e] : e;
+    if (HEADS) return heads.perm ? heads.perm[id] : id;
+    return w ? __float_as_uint(w[id]) : __float_as_uint(1.f);
   };
   uint32_t nxt_i = 0;
   uint32_t nxt_s = HEADS ? 0u : __float_as_uint(1.f);
@@ -255,7 +261,8 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
                                                          const uint32_t *__restrict__ indices, uint32_t index_base,
                                                          uint32_t n_items, uint32_t F, const Item *__restrict__ items,
                                                          float *__restrict__ partial, int accumulate, HeadArgs heads,
-                                                         uint32_t row_edge_limit) {
+                                                         uint32_t row_edge_limit,
+                                                         const uint32_t *__restrict__ edge_ids) {
   using V = typename Vec<VEC>::type;
   constexpr int U = 4;
   const uint32_t gl = threadIdx.x & (G - 1);
@@ -288,10 +295,11 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
     uint32_t my_s = HEADS ? 0u : __float_as_uint(1.f);  // weight bits, or the edge's id in alpha's order
     if (gl < n) {
       my_i = indices[eb + gl] - index_base;
+      const uint32_t id = edge_ids ? edge_ids[eb + gl] : eb + gl;
       if (HEADS)
-        my_s = heads.perm ? heads.perm[eb + gl] : eb + gl;
+        my_s = heads.perm ? heads.perm[id] : id;
       else if (w)
-        my_s = __float_as_uint(w[eb + gl]);
+        my_s = __float_as_uint(w[id]);
     }
     uint32_t j = 0;
     for (; j + U <= n; j += U) {
@@ -373,6 +381,7 @@ struct LaunchArgs {
   hipStream_t stream;
   HeadArgs heads = HeadArgs{nullptr, 0u, 0u};  // H == 0: one weight per edge
   uint32_t row_edge_limit = 0xFFFFFFFFu;       // whole-row launches skip rows with more edges than this
+  const uint32_t *edge_ids = nullptr;          // schedules with their own index copy: edge -> caller's edge position
 };
 
 // How the wave kernel hands neighbour pairs to its lanes: through a wave-private LDS tile (default)
@@ -394,7 +403,7 @@ void launch_wave(const LaunchArgs &a, uint32_t col_base) {
 #define NTS_LAUNCH_WAVE(LDS, HD)                                                                                       \
   hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, LDS, HD>), grid, block, 0, a.stream, a.in, a.out, a.w, a.offsets,     \
                      a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate, a.heads,     \
-                     a.row_edge_limit)
+                     a.row_edge_limit, a.edge_ids)
   if (a.heads.H) {
     if (lds_tile_enabled()) NTS_LAUNCH_WAVE(true, true); else NTS_LAUNCH_WAVE(false, true);
   } else {
@@ -410,11 +419,11 @@ void launch_group(const LaunchArgs &a) {
   if (a.heads.H)
     hipLaunchKernelGGL((spmm_group_kernel<G, VEC, true>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
                        a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,
-                       a.row_edge_limit);
+                       a.row_edge_limit, a.edge_ids);
   else
     hipLaunchKernelGGL((spmm_group_kernel<G, VEC, false>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
                        a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,
-                       a.row_edge_limit);
+                       a.row_edge_limit, a.edge_ids);
 }
 
 template <int VEC>
@@ -665,6 +674,24 @@ int check_common(const float *in, float *out, const uint32_t *offsets, const uin
 }  // namespace
 }  // namespace nts
 
+namespace {
+// fn(first, last) over [0, n) on up to 16 host threads, in contiguous blocks.
+template <typename Fn>
+void parallel_blocks(uint32_t n, Fn fn) {
+  unsigned t = std::thread::hardware_concurrency();
+  if (t > 16) t = 16;
+  if (t < 2 || n < 4096) {
+    fn(0u, n);
+    return;
+  }
+  std::vector<std::thread> pool;
+  const uint32_t per = (n + t - 1) / t;
+  for (uint32_t b = 0; b < n; b += per) pool.emplace_back(fn, b, std::min(n, b + per));
+  for (std::thread &th : pool) th.join();
+}
+
+}  // namespace
+
 struct nts_spmm_plan {
   uint32_t rows = 0;
   uint32_t edges = 0;
@@ -677,6 +704,10 @@ struct nts_spmm_plan {
   uint4 *splits = nullptr;            // device
   float *partial = nullptr;           // device, n_partials * partial_F floats
   uint32_t partial_F = 0;
+  // Only when rows had to be re-ordered for the source ranges: the schedule's own copy of the gather
+  // indices (base already subtracted), and for each of its edges the position in the caller's order.
+  uint32_t *sorted_idx = nullptr;     // device, [edges]
+  uint32_t *edge_ids = nullptr;       // device, [edges]
   hipEvent_t ev_start = nullptr;      // optional profiling events around the main kernel
   hipEvent_t ev_stop = nullptr;
 };
@@ -713,11 +744,17 @@ struct Schedule {
   std::vector<uint4> items;   // (row, first edge, end edge, partial slot or kNoSlot)
   std::vector<uint4> splits;  // (row, first slot, slot count, 0)
   uint32_t n_partials = 0;
+  // Empty unless some row that is cut by source range did not have ascending indices: then a copy
+  // of the index array in which those rows are sorted (stable), and the original position of each
+  // of its edges.  Rows that are never cut keep their order.
+  std::vector<uint32_t> sorted_idx;
+  std::vector<uint32_t> edge_ids;
 };
 
 // Host-only: needs nothing but the two index arrays.
-void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx, uint32_t rows, uint32_t chunk,
+void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx_in, uint32_t rows, uint32_t chunk,
                    uint32_t n_slabs, uint32_t n_index) {
+  const uint32_t *idx = idx_in;
   std::vector<Piece> pieces;
   std::vector<uint4> &splits = out.splits;
   uint32_t n_partials = 0;
@@ -736,6 +773,44 @@ void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx, uint
   const uint64_t fine_width = slabbed ? (static_cast<uint64_t>(n_index) + fine - 1) / fine : 0;
   const uint32_t wide_ranges = slabbed && n_slabs >= 8 ? n_slabs / 4 : 0;
   std::vector<uint8_t> was_cut(wide_ranges ? rows : 0, 0);
+  if (slabbed) {
+    // Rows long enough to be cut by source range must ascend.  Edge files are not always sorted
+    // (the reference's loader leaves a CSR row in thread-arrival order), so such rows are sorted in
+    // a copy of the index array that the schedule then gathers through; a stable sort, so equal
+    // indices keep their edge order.  Sums of those rows are associated in source order.
+    const uint32_t cut_above = wide_ranges ? chunk / 4 : chunk;
+    std::vector<uint8_t> unsorted(rows, 0);
+    std::atomic<bool> any(false);
+    parallel_blocks(rows, [&](uint32_t r0, uint32_t r1) {
+      for (uint32_t r = r0; r < r1; ++r) {
+        const uint32_t b = off[r], e = off[r + 1];
+        if (e - b <= cut_above) continue;
+        for (uint32_t k = b + 1; k < e; ++k)
+          if (idx_in[k - 1] > idx_in[k]) {
+            unsorted[r] = 1;
+            any.store(true, std::memory_order_relaxed);
+            break;
+          }
+      }
+    });
+    if (any.load()) {
+      const uint32_t edges = off[rows];
+      out.sorted_idx.assign(idx_in, idx_in + edges);
+      out.edge_ids.resize(edges);
+      parallel_blocks(edges, [&](uint32_t e0, uint32_t e1) {
+        for (uint32_t e = e0; e < e1; ++e) out.edge_ids[e] = e;
+      });
+      parallel_blocks(rows, [&](uint32_t r0, uint32_t r1) {
+        for (uint32_t r = r0; r < r1; ++r) {
+          if (!unsorted[r]) continue;
+          uint32_t *ids = out.edge_ids.data() + off[r], *ids_end = out.edge_ids.data() + off[r + 1];
+          std::stable_sort(ids, ids_end, [&](uint32_t a, uint32_t b) { return idx_in[a] < idx_in[b]; });
+          for (uint32_t k = off[r]; k < off[r + 1]; ++k) out.sorted_idx[k] = idx_in[out.edge_ids[k]];
+        }
+      });
+      idx = out.sorted_idx.data();
+    }
+  }
   std::vector<uint32_t> stops;  // (narrow range id, end edge) of the non-empty ranges of one row
   // Cuts edges [b, e) of a row with ascending indices at `ranges` equal ranges; ranges divides fine.
   auto range_stops = [&](uint32_t b, uint32_t e, uint32_t ranges) {
@@ -756,15 +831,10 @@ void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx, uint
       cut = stop;
     }
   };
-  auto is_ascending = [&](uint32_t b, uint32_t e) {
-    for (uint32_t k = b + 1; k < e; ++k)
-      if (idx[k - 1] > idx[k]) return false;
-    return true;
-  };
   for (uint32_t r = 0; r < rows; ++r) {
     const uint32_t b = off[r], e = off[r + 1], deg = e - b;
     if (deg <= chunk) {
-      if (wide_ranges && deg > chunk / 4 && is_ascending(b, e)) {
+      if (wide_ranges && deg > chunk / 4) {
         range_stops(b, e, wide_ranges);
         if (stops.size() > 2) {
           const uint32_t first = n_partials;
@@ -782,7 +852,7 @@ void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx, uint
       continue;
     }
     const uint32_t first = n_partials;
-    if (slabbed && is_ascending(b, e)) {
+    if (slabbed) {
       range_stops(b, e, n_slabs);
       uint32_t from = b;
       for (size_t q = 0; q < stops.size(); q += 2) {
@@ -842,6 +912,13 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
     err = hipMalloc(reinterpret_cast<void **>(&p->splits), splits.size() * sizeof(uint4));
     if (err == hipSuccess)
       err = hipMemcpy(p->splits, splits.data(), splits.size() * sizeof(uint4), hipMemcpyHostToDevice);
+  }
+  if (err == hipSuccess && !sched.sorted_idx.empty()) {
+    const size_t bytes = sched.sorted_idx.size() * sizeof(uint32_t);
+    err = hipMalloc(reinterpret_cast<void **>(&p->sorted_idx), bytes);
+    if (err == hipSuccess) err = hipMemcpy(p->sorted_idx, sched.sorted_idx.data(), bytes, hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void **>(&p->edge_ids), bytes);
+    if (err == hipSuccess) err = hipMemcpy(p->edge_ids, sched.edge_ids.data(), bytes, hipMemcpyHostToDevice);
   }
   if (err != hipSuccess) {
     nts_spmm_plan_destroy(p);
@@ -927,6 +1004,8 @@ int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {
   hipError_t e1 = plan->items ? hipFree(plan->items) : hipSuccess;
   hipError_t e2 = plan->splits ? hipFree(plan->splits) : hipSuccess;
   hipError_t e3 = plan->partial ? hipFree(plan->partial) : hipSuccess;
+  if (plan->sorted_idx && hipFree(plan->sorted_idx) != hipSuccess) e3 = hipErrorUnknown;
+  if (plan->edge_ids && hipFree(plan->edge_ids) != hipSuccess) e3 = hipErrorUnknown;
   delete plan;
   if (e1 != hipSuccess) return nts::fail_hip(e1, "nts_spmm_plan_destroy");
   if (e2 != hipSuccess) return nts::fail_hip(e2, "nts_spmm_plan_destroy");
@@ -1000,6 +1079,10 @@ int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float 
   nts::LaunchArgs a{in,  out,         alpha,         offsets,    indices, 0u, plan->n_items,
                     F,   plan->items, plan->partial, accumulate, stream};
   a.heads = nts::HeadArgs{perm, H, Fh};
+  if (plan->sorted_idx) {
+    a.indices = plan->sorted_idx;
+    a.edge_ids = plan->edge_ids;
+  }
   nts::launch_spmm(a);
   NTS_LAUNCH_CHECK("nts_spmm_gather_heads_planned");
   if (plan->n_splits) {
@@ -1034,6 +1117,11 @@ int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, 
   if (int rc = nts_spmm_plan_reserve(plan, F)) return rc;
   nts::LaunchArgs a{in,  out,         w,           offsets,       indices,   index_base, plan->n_items,
                     F,   plan->items, plan->partial, accumulate, stream};
+  if (plan->sorted_idx) {  // the schedule's own copy of the indices, base already subtracted
+    a.indices = plan->sorted_idx;
+    a.index_base = 0;
+    a.edge_ids = plan->edge_ids;
+  }
   if (plan->ev_start && plan->ev_stop) NTS_HIP_TRY(hipEventRecord(plan->ev_start, stream));
   nts::launch_spmm(a);
   NTS_LAUNCH_CHECK("nts_spmm_gather_planned");

@@ -228,10 +228,11 @@ def test_empty_and_error_paths(device):
 
 
 @pytest.mark.parametrize("F,chunk,slabs,sorted_rows", [(128, 64, 4, True), (602, 100, 8, True), (41, 32, 16, True),
-                                                       (100, 64, 8, False), (16, 16, 3, True), (64, 48, 32, True)])
+                                                       (100, 64, 8, False), (16, 16, 3, True), (64, 48, 32, True),
+                                                       (602, 64, 4, False), (128, 96, 16, False)])
 def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
-    """Source-range ("slab") schedule: same results as the oracle to tolerance, bit-reproducible, and
-    rows whose indices do not ascend fall back to edge-count chunks."""
+    """Source-range ("slab") schedule: same results as the oracle to tolerance, bit-reproducible, also
+    for rows whose indices do not ascend (cut in the schedule's own sorted copy)."""
     print(f"case F={F} chunk={chunk} slabs={slabs} sorted={sorted_rows}", flush=True)
     Vd, Vs = 400, 900
     co, ri = random_block(Vd, Vs, 25, seed=F + slabs, hub=2500, dup=True)
@@ -245,9 +246,10 @@ def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
     plan = SpmmPlan(dco, Vd, ri.size, chunk, dri, Vs, slabs)
     info = plan.info()
     deg = np.diff(co.astype(np.int64))
-    # With 8 or more source ranges, sorted rows of more than chunk/4 edges are cut as well, at a
-    # quarter as many (wider) ranges, unless all their edges fall into one of those.
-    second_tier = sorted_rows and slabs >= 8
+    # With 8 or more source ranges, rows of more than chunk/4 edges are cut as well, at a quarter as
+    # many (wider) ranges, unless all their edges fall into one of those.  Rows that do not ascend
+    # are cut in the schedule's own sorted copy of the indices, so they behave like sorted ones.
+    second_tier = slabs >= 8
     whole_up_to = chunk // 4 if second_tier else chunk
     long_rows = int((deg > chunk).sum())
     plain = int(np.ceil(deg[deg > chunk] / chunk).sum())
@@ -257,10 +259,7 @@ def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
         assert plain <= info["partials"] <= plain + long_rows * slabs + medium * (slabs // 4)
     else:
         assert info["split_rows"] == long_rows
-        if sorted_rows:
-            assert plain <= info["partials"] <= plain + info["split_rows"] * slabs
-        else:
-            assert info["partials"] == plain
+        assert plain <= info["partials"] <= plain + info["split_rows"] * slabs
     outs = []
     for _ in range(2):
         out = torch.full((Vd, F), float("nan"), device=device)

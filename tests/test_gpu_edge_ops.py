@@ -341,3 +341,53 @@ def test_heads_aggregation_without_a_plan_cuts_hub_rows(device):
         check(out[:, sl], oracle.spmm(xs, w, co, ri, Vd), abs_term_scale(xs, w, co, ri, Vd))
         wb = np.ascontiguousarray(w[perm])
         check(gx[:, sl], oracle.spmm(gs, wb, ro, ci, Vs), abs_term_scale(gs, wb, ro, ci, Vs))
+
+
+@pytest.mark.parametrize("sorted_rows", [True, False])
+def test_heads_aggregation_through_a_schedule(device, sorted_rows):
+    """nts_spmm_gather_heads_planned over the CSC (perm NULL) and over the CSR with alpha kept in CSC
+    order (perm = csr_to_csc), with source-range schedules; with rows that do not ascend the
+    schedule gathers through its own sorted copy and still has to pick each edge's alpha."""
+    from neutronbench_amd.layout import SpmmPlan
+
+    H, Fh = 4, 8
+    F = H * Fh
+    Vd, Vs = 1500, 1200
+    co, ri = random_block(Vd, Vs, 20, seed=93, hub=9000, dup=True)
+    if sorted_rows:
+        for d in range(Vd):
+            ri[co[d]:co[d + 1]] = np.sort(ri[co[d]:co[d + 1]])
+    E = ri.size
+    rng = np.random.default_rng(94)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    g = rng.standard_normal((Vd, F)).astype(np.float32)
+    alpha = rng.random((E, H)).astype(np.float32)
+    ro, ci, perm = brute_csr(co, ri, Vs)
+    if not sorted_rows:  # shuffle inside every CSR row as well (keeping perm consistent)
+        for r in range(Vs):
+            p = rng.permutation(int(ro[r + 1] - ro[r])) + int(ro[r])
+            ci[ro[r]:ro[r + 1]] = ci[p]
+            perm[ro[r]:ro[r + 1]] = perm[p]
+    s = stream()
+    dco, dri, dro, dci, dperm = (dev(a, device) for a in (co, ri, ro, ci, perm))
+    dx, dg, dalpha = dev(x, device), dev(g, device), dev(alpha, device)
+    fwd = SpmmPlan(dco, Vd, E, 64, dri, Vs, 16)
+    bwd = SpmmPlan(dro, Vs, E, 64, dci, Vd, 16)
+    fwd.reserve(F)
+    bwd.reserve(F)
+    out = torch.full((Vd, F), float("nan"), device=device)
+    call("nts_spmm_gather_heads_planned", fwd.handle, ptr(dx), ptr(out), ptr(dalpha), 0, ptr(dco), ptr(dri), H, Fh, 0, s)
+    gx = torch.full((Vs, F), float("nan"), device=device)
+    call("nts_spmm_gather_heads_planned", bwd.handle, ptr(dg), ptr(gx), ptr(dalpha), ptr(dperm), ptr(dro), ptr(dci), H,
+         Fh, 0, s)
+    torch.cuda.synchronize()
+    out, gx = out.cpu().numpy(), gx.cpu().numpy()
+    for h in range(H):
+        sl = slice(h * Fh, (h + 1) * Fh)
+        w = np.ascontiguousarray(alpha[:, h])
+        xs, gs = np.ascontiguousarray(x[:, sl]), np.ascontiguousarray(g[:, sl])
+        check(out[:, sl], oracle.spmm(xs, w, co, ri, Vd), abs_term_scale(xs, w, co, ri, Vd))
+        wb = np.ascontiguousarray(w[perm])
+        check(gx[:, sl], oracle.spmm(gs, wb, ro, ci, Vs), abs_term_scale(gs, wb, ro, ci, Vs))
+    fwd.close()
+    bwd.close()

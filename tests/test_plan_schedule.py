@@ -78,6 +78,19 @@ def check_invariants(items, n_splits, n_partials, co, ri, deg, chunk, slabs, ran
     return pieces
 
 
+def check_ranges(pieces, ri, deg, Vs, chunk, slabs):
+    """Issue order: the source range of a piece's first edge never decreases along the piece list, and
+    a piece never crosses a boundary of its row's range width."""
+    width = -(-Vs // slabs)
+    first_range = ri[pieces[:, 1]] // width
+    last_range = ri[pieces[:, 2] - 1] // width
+    wide = deg[pieces[:, 0]] <= chunk  # second-tier rows use ranges four times as wide
+    issue = np.where(wide, first_range // 4 * 4, first_range)
+    assert np.all(issue[1:] >= issue[:-1])
+    assert np.all(last_range[~wide] == first_range[~wide])
+    assert np.all(last_range[wide] // 4 == first_range[wide] // 4)
+
+
 @pytest.mark.parametrize("chunk,slabs", [(512, 32), (64, 8), (100, 16), (32, 4), (16, 3), (4096, 1)])
 @pytest.mark.parametrize("seed", [1, 2])
 def test_ranged_schedule_invariants(chunk, slabs, seed):
@@ -86,24 +99,23 @@ def test_ranged_schedule_invariants(chunk, slabs, seed):
     items, n_splits, n_partials = schedule(co, ri, Vs, chunk, slabs)
     pieces = check_invariants(items, n_splits, n_partials, co, ri, deg, chunk, slabs, ranged=slabs > 1)
     if slabs > 1:
-        # issue order: the source range of a piece's first edge never decreases along the piece list,
-        # and a piece never crosses a boundary of its row's range width
-        width = -(-Vs // slabs)
-        first_range = ri[pieces[:, 1]] // width
-        last_range = ri[pieces[:, 2] - 1] // width
-        wide = deg[pieces[:, 0]] <= chunk  # second-tier rows use ranges four times as wide
-        issue = np.where(wide, first_range // 4 * 4, first_range)
-        assert np.all(issue[1:] >= issue[:-1])
-        assert np.all(last_range[~wide] == first_range[~wide])
-        assert np.all(last_range[wide] // 4 == first_range[wide] // 4)
+        check_ranges(pieces, ri, deg, Vs, chunk, slabs)
 
 
-def test_rows_that_do_not_ascend_fall_back_to_edge_count_pieces():
-    co, ri, deg = power_law_block(800, 3000, 5, sort_rows=False, hubs=(6000, 700))
-    chunk, slabs = 128, 16
-    items, n_splits, n_partials = schedule(co, ri, 3000, chunk, slabs)
-    check_invariants(items, n_splits, n_partials, co, ri, deg, chunk, slabs, ranged=False)
-    assert n_partials == int(np.ceil(deg[deg > chunk] / chunk).sum())
+@pytest.mark.parametrize("chunk,slabs", [(128, 16), (64, 4)])
+def test_rows_that_do_not_ascend_are_cut_in_a_sorted_copy(chunk, slabs):
+    """Edge files are not always sorted (the reference's loader leaves a CSR row in arrival order):
+    rows long enough to be cut by source range are then cut in a copy of the index array in which
+    they are sorted (stably), so the same invariants hold with respect to that copy."""
+    Vs = 3000
+    co, ri, deg = power_law_block(800, Vs, 5, sort_rows=False, hubs=(6000, 700))
+    items, n_splits, n_partials = schedule(co, ri, Vs, chunk, slabs)
+    pieces = check_invariants(items, n_splits, n_partials, co, ri, deg, chunk, slabs, ranged=True)
+    cut_above = chunk // 4 if slabs >= 8 else chunk
+    ri_cut = ri.copy()
+    for r in np.flatnonzero(deg > cut_above):
+        ri_cut[co[r]:co[r + 1]] = np.sort(ri[co[r]:co[r + 1]], kind="stable")
+    check_ranges(pieces, ri_cut, deg, Vs, chunk, slabs)
 
 
 def test_schedule_without_indices_and_error_paths():
