@@ -172,7 +172,7 @@ def main():
     achieved = algo / (kernel_ms * 1e-3) / 1e9
     roofline = {
         "bound": "hbm",
-        "kernel": "spmm_wave_kernel<1,10,true,false> (F=602 gather, forward and backward launches)",
+        "kernel": "spmm_wave_kernel<1,10,true,false,false> (F=602 gather, forward and backward launches)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",

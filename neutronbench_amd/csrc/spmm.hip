@@ -102,7 +102,7 @@ struct HeadArgs {
   uint32_t Fh;
 };
 
-template <int VEC, int NACC, bool LDS_TILE, bool HEADS>
+template <int VEC, int NACC, bool LDS_TILE, bool HEADS, bool REMAP>
 __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                         const float *__restrict__ w,
                                                         const uint32_t *__restrict__ offsets,
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
   // edge_ids (a schedule that gathers through its own, re-ordered copy of the indices): position of
   // edge e in the caller's weight / alpha order.
   auto second_of = [&](uint32_t e) -> uint32_t {
-    const uint32_t id = edge_ids ? edge_ids[e] : e;
+    const uint32_t id = REMAP ? edge_ids[e] : e;
     if (HEADS) return heads.perm ? heads.perm[id] : id;
     return w ? __float_as_uint(w[id]) : __float_as_uint(1.f);
   };
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
 // Sub-wavefront variant for narrow rows: G lanes per row (G = 4, 8, 16 or 32), 64/G rows per
 // wavefront, one VEC-wide accumulator per lane (F <= G*VEC).  Neighbour pairs are fetched G at a
 // time per group and broadcast inside the group with cross-lane shuffles.
-template <int G, int VEC, bool HEADS>
+template <int G, int VEC, bool HEADS, bool REMAP>
 __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                          const float *__restrict__ w,
                                                          const uint32_t *__restrict__ offsets,
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
     uint32_t my_s = HEADS ? 0u : __float_as_uint(1.f);  // weight bits, or the edge's id in alpha's order
     if (gl < n) {
       my_i = indices[eb + gl] - index_base;
-      const uint32_t id = edge_ids ? edge_ids[eb + gl] : eb + gl;
+      const uint32_t id = REMAP ? edge_ids[eb + gl] : eb + gl;
       if (HEADS)
         my_s = heads.perm ? heads.perm[id] : id;
       else if (w)
@@ -400,14 +400,23 @@ void launch_wave(const LaunchArgs &a, uint32_t col_base) {
   constexpr int kWavesPerBlock = 4;
   const uint32_t blocks = ceil_div(a.n_items, kWavesPerBlock);
   const dim3 grid(blocks), block(kWavesPerBlock * kWave);
-#define NTS_LAUNCH_WAVE(LDS, HD)                                                                                       \
-  hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, LDS, HD>), grid, block, 0, a.stream, a.in, a.out, a.w, a.offsets,     \
+#define NTS_LAUNCH_WAVE(LDS, HD, RM)                                                                                   \
+  hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, LDS, HD, RM>), grid, block, 0, a.stream, a.in, a.out, a.w, a.offsets, \
                      a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate, a.heads,     \
                      a.row_edge_limit, a.edge_ids)
-  if (a.heads.H) {
-    if (lds_tile_enabled()) NTS_LAUNCH_WAVE(true, true); else NTS_LAUNCH_WAVE(false, true);
+  const bool lds = lds_tile_enabled();
+  if (a.edge_ids) {
+    if (a.heads.H) {
+      if (lds) NTS_LAUNCH_WAVE(true, true, true); else NTS_LAUNCH_WAVE(false, true, true);
+    } else {
+      if (lds) NTS_LAUNCH_WAVE(true, false, true); else NTS_LAUNCH_WAVE(false, false, true);
+    }
   } else {
-    if (lds_tile_enabled()) NTS_LAUNCH_WAVE(true, false); else NTS_LAUNCH_WAVE(false, false);
+    if (a.heads.H) {
+      if (lds) NTS_LAUNCH_WAVE(true, true, false); else NTS_LAUNCH_WAVE(false, true, false);
+    } else {
+      if (lds) NTS_LAUNCH_WAVE(true, false, false); else NTS_LAUNCH_WAVE(false, false, false);
+    }
   }
 #undef NTS_LAUNCH_WAVE
 }
@@ -416,14 +425,16 @@ template <int G, int VEC>
 void launch_group(const LaunchArgs &a) {
   const uint32_t per_block = 256 / G;
   const uint32_t blocks = ceil_div(a.n_items, per_block);
-  if (a.heads.H)
-    hipLaunchKernelGGL((spmm_group_kernel<G, VEC, true>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
-                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,
-                       a.row_edge_limit, a.edge_ids);
-  else
-    hipLaunchKernelGGL((spmm_group_kernel<G, VEC, false>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w,
-                       a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,
-                       a.row_edge_limit, a.edge_ids);
+#define NTS_LAUNCH_GROUP(HD, RM)                                                                                  \
+  hipLaunchKernelGGL((spmm_group_kernel<G, VEC, HD, RM>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w, \
+                     a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads, \
+                     a.row_edge_limit, a.edge_ids)
+  if (a.edge_ids) {
+    if (a.heads.H) NTS_LAUNCH_GROUP(true, true); else NTS_LAUNCH_GROUP(false, true);
+  } else {
+    if (a.heads.H) NTS_LAUNCH_GROUP(true, false); else NTS_LAUNCH_GROUP(false, false);
+  }
+#undef NTS_LAUNCH_GROUP
 }
 
 template <int VEC>
