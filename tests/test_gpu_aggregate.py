@@ -309,3 +309,46 @@ def test_scratch_pool_is_kept_between_calls_and_can_be_trimmed(device):
     again = _run_planless(x, None, co, ri, Vd, F, device)
     assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
     call("nts_scratch_trim")
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_shapes_planned_and_planless_agree_with_the_oracle(device, seed):
+    """Random block shapes, widths, piece lengths, range counts (also ones that 4 does not divide),
+    sorted and unsorted rows, weighted or not, accumulating or not: the planned and the plan-less
+    call both match the oracle, and rows that no schedule cuts match it bit for bit."""
+    from neutronbench_amd.layout import SpmmPlan
+
+    rng = np.random.default_rng(1000 + seed)
+    Vd, Vs = int(rng.integers(1, 700)), int(rng.integers(1, 900))
+    F = int(rng.choice([1, 3, 4, 8, 20, 33, 64, 100, 128, 129, 300, 602]))
+    chunk = int(rng.choice([4, 16, 50, 128, 512]))
+    slabs = int(rng.choice([1, 2, 3, 8, 9, 10, 12, 32, 100]))
+    co, ri = random_block(Vd, Vs, float(rng.choice([0.5, 6, 40])), seed=seed, hub=int(rng.choice([0, 300, 5000])), dup=True)
+    if rng.random() < 0.5:
+        for d in range(Vd):
+            ri[co[d]:co[d + 1]] = np.sort(ri[co[d]:co[d + 1]])
+    weighted, accumulate = bool(rng.random() < 0.7), int(rng.random() < 0.5)
+    print(f"case Vd={Vd} Vs={Vs} E={ri.size} F={F} chunk={chunk} slabs={slabs} weighted={weighted} acc={accumulate}", flush=True)
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    w = rng.random(ri.size).astype(np.float32) if weighted else None
+    init = rng.standard_normal((Vd, F)).astype(np.float32)
+    want = oracle.spmm(x, w, co, ri, Vd, fused=True) + (init if accumulate else 0)
+    scale = abs_term_scale(x, w, co, ri, Vd) + (np.abs(init) if accumulate else 0)
+    deg = np.diff(co.astype(np.int64))
+    got = _run_planless(x, w, co, ri, Vd, F, device, accumulate=accumulate, out_init=init if accumulate else None)
+    check(got, want, scale)
+    if not accumulate:
+        whole = deg <= (planless_piece_edges(ri.size) or ri.size + 1)
+        assert np.array_equal(got[whole].view(np.uint32), want[whole].view(np.uint32))
+    dx, dco, dri = _dev(x, device), _dev(co, device), _dev(ri, device)
+    dw = _dev(w, device) if weighted else None
+    plan = SpmmPlan(dco, Vd, ri.size, chunk, dri, Vs, slabs) if slabs > 1 else SpmmPlan(dco, Vd, ri.size, chunk)
+    out = _dev(init, device) if accumulate else torch.full((Vd, F), float("nan"), device=device)
+    call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, F, accumulate, _stream())
+    torch.cuda.synchronize()
+    got_p = out.cpu().numpy()
+    check(got_p, want, scale)
+    if not accumulate:
+        whole = deg <= (chunk // 4 if slabs >= 8 else chunk)
+        assert np.array_equal(got_p[whole].view(np.uint32), want[whole].view(np.uint32))
+    plan.close()
