@@ -353,7 +353,10 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
  *   fanouts[h]   fanout of hop h, hop 0 first (the output-side hop); < 0 = whole neighbourhood, in
  *                which case the batch must not repeat a vertex
  *   arena        nts_batch_builder_arena_bytes(...) bytes of 256-byte-aligned device memory, owned by
- *                the caller, in use until nts_batch_builder_destroy; graph_co / graph_ri likewise
+ *                the caller, in use until nts_batch_builder_destroy; graph_co / graph_ri likewise.
+ *                The size includes the scratch of the library's scan and sort routines for the
+ *                current device, so the call needs a device; 0 = unsupported arguments (no hop,
+ *                more than 8 hops, a fanout of 0, an empty graph or batch).
  *   nts_batch_builder_sample  enqueues everything on `stream` and returns; n <= max_batch
  *   nts_batch_builder_layers  waits for that batch and fills layers[0 .. hops): index 0 is the
  *                input-side layer (its `source` indexes the feature gather), index hops-1 the
