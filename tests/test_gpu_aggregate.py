@@ -95,7 +95,8 @@ def test_accumulate_and_index_base(device):
     assert np.array_equal(got0, oracle.spmm(x, w, co, ri, Vd, fused=True))
 
 
-@pytest.mark.parametrize("F,chunk", [(128, 64), (602, 100), (41, 32), (16, 16), (100, 4096)])
+@pytest.mark.parametrize("F,chunk", [(128, 64), (602, 100), (41, 32), (16, 16), (100, 4096), (300, 48), (1000, 64),
+                                     (1433, 128)])
 def test_planned_split_rows(device, F, chunk):
     """Degree-bucketed schedule with hub rows split into chunks: matches the oracle, reports the
     split, and is bit-reproducible run to run (no atomics)."""
