@@ -659,6 +659,51 @@ __global__ __launch_bounds__(256) void auto_reduce_kernel(float *__restrict__ ou
   *dst = a;
 }
 
+// The same with one block per work item covering all columns (rows of up to 1,024 columns): whole,
+// contiguous partial rows are read, and a third or a quarter as many blocks are launched.
+template <int J>
+__global__ __launch_bounds__(256) void auto_reduce_wide_kernel(float *__restrict__ out,
+                                                               const float *__restrict__ partial,
+                                                               const Item *__restrict__ items,
+                                                               const uint32_t *__restrict__ base, uint32_t F,
+                                                               int accumulate) {
+  const uint32_t i = blockIdx.x;
+  const uint32_t r = items[i].x;
+  if (base[r] != i) return;
+  const uint32_t n = base[r + 1] - i;
+  if (n == 0) return;
+  const float *src = partial + static_cast<size_t>(i) * F;
+  uint32_t c[J];
+  bool live[J];
+  float a[J];
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    c[j] = threadIdx.x + 256u * j;
+    live[j] = c[j] < F;
+    if (!live[j]) c[j] = F - 1;  // re-read the last column, never stored
+    a[j] = src[c[j]];
+  }
+  uint32_t k = 1;
+  for (; k + 8 <= n; k += 8) {
+    float v[8][J];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < J; ++j) v[u][j] = src[static_cast<size_t>(k + u) * F + c[j]];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < J; ++j) a[j] += v[u][j];
+  }
+  for (; k < n; ++k)
+#pragma unroll
+    for (int j = 0; j < J; ++j) a[j] += src[static_cast<size_t>(k) * F + c[j]];
+  float *dst = out + static_cast<size_t>(r) * F;
+#pragma unroll
+  for (int j = 0; j < J; ++j)
+    if (live[j]) dst[c[j]] = accumulate ? a[j] + dst[c[j]] : a[j];
+}
+
 inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 
 // `a` describes the whole-row launch (a.n_items = rows, no items).
@@ -736,8 +781,19 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
   LaunchArgs whole = a;
   whole.row_edge_limit = chunk;
   launch_spmm(whole);
-  hipLaunchKernelGGL(auto_reduce_kernel, dim3(p_max, ceil_div(a.F, 256)), dim3(256), 0, a.stream, a.out, partial, items,
-                     base, a.F, a.accumulate);
+#define NTS_AUTO_REDUCE_WIDE(J)                                                                                     \
+  hipLaunchKernelGGL(auto_reduce_wide_kernel<J>, dim3(p_max), dim3(256), 0, a.stream, a.out, partial, items, base, a.F, \
+                     a.accumulate)
+  if (a.F > 256 && a.F <= 512)
+    NTS_AUTO_REDUCE_WIDE(2);
+  else if (a.F > 512 && a.F <= 768)
+    NTS_AUTO_REDUCE_WIDE(3);
+  else if (a.F > 768 && a.F <= 1024)
+    NTS_AUTO_REDUCE_WIDE(4);
+  else
+    hipLaunchKernelGGL(auto_reduce_kernel, dim3(p_max, ceil_div(a.F, 256)), dim3(256), 0, a.stream, a.out, partial, items,
+                       base, a.F, a.accumulate);
+#undef NTS_AUTO_REDUCE_WIDE
   err = hipGetLastError();
   if (err != hipSuccess) return bail(err, "spmm: balanced launch");
   NTS_HIP_TRY(scratch_free(buf, a.stream));
