@@ -454,6 +454,38 @@ __device__ __forceinline__ void strided_pass(uint64_t first, uint64_t n, uint64_
   for (; i < n; i += stride) use(i, load(i));
 }
 
+// One strided pass that leaves a running (maximum, sum of exp(v - maximum)) pair, so that the maximum
+// and the sum of a segment come out of a single read.  The U values in flight are folded in together:
+// their maximum first, then one rescale of the old sum and U independent exponentials.
+template <int U, typename Load, typename Seen>
+__device__ __forceinline__ void strided_max_sum_pass(uint64_t first, uint64_t n, uint64_t stride, Load load,
+                                                     Seen seen, float &mx, float &sum) {
+  uint64_t i = first;
+  for (; i + (U - 1) * stride < n; i += U * stride) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = load(i + u * stride);
+    float m = mx;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      seen(i + u * stride, v[u]);
+      m = fmaxf(m, v[u]);
+    }
+    float add = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) add += expf(v[u] - m);
+    sum = sum * expf(mx - m) + add;  // mx = -inf at the start: the old sum is 0 and stays 0
+    mx = m;
+  }
+  for (; i < n; i += stride) {
+    const float v = load(i);
+    seen(i, v);
+    const float m = fmaxf(mx, v);
+    sum = sum * expf(mx - m) + expf(v - m);
+    mx = m;
+  }
+}
+
 // Reduction over the lanes of an aligned group of WIDTH lanes that share a head (lane mod H).
 template <int MODE, int WIDTH>  // 0 = max, 1 = sum
 __device__ __forceinline__ float head_reduce_w(float v, uint32_t H) {
@@ -633,22 +665,22 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
         const uint32_t h = lane & (H - 1);
         float erv = 0.f;
         if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
-        float mx = -INFINITY;
-        strided_pass<8>(lane, n, kWave,
-                        [&](uint64_t i) -> float {
-                          if (!FUSED) return xs[i];
-                          const uint32_t src = ri[e0 + i / H];
-                          return leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
-                        },
-                        [&](uint64_t i, float sc) {
-                          if (FUSED) ys[i] = sc;
-                          mx = fmaxf(mx, sc);
-                        });
+        float mx = -INFINITY, sum = 0.f;
+        strided_max_sum_pass<8>(
+            lane, n, kWave,
+            [&](uint64_t i) -> float {
+              if (!FUSED) return xs[i];
+              const uint32_t src = ri[e0 + i / H];
+              return leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
+            },
+            [&](uint64_t i, float sc) {
+              if (FUSED) ys[i] = sc;
+            },
+            mx, sum);
+        // every lane's pair is brought to the head's maximum before the sums are added
+        const float lane_mx = mx;
         mx = head_reduce<0>(mx, H);
-        float sum = 0.f;
-        strided_pass<8>(lane, n, kWave, [&](uint64_t i) -> float { return FUSED ? ys[i] : xs[i]; },
-                        [&](uint64_t, float sc) { sum += expf(sc - mx); });
-        sum = head_reduce<1>(sum, H);
+        sum = head_reduce<1>(sum * expf(lane_mx - mx), H);
         strided_pass<8>(lane, n, kWave, [&](uint64_t i) -> float { return FUSED ? ys[i] : xs[i]; },
                         [&](uint64_t i, float sc) { ys[i] = expf(sc - mx) / sum; });
       } else {
@@ -813,22 +845,21 @@ __global__ __launch_bounds__(kLongBlock) void edge_softmax_fwd_long_kernel(
     const float *xs = FUSED ? nullptr : x + base;
     float erv = 0.f;
     if (FUSED) erv = er[static_cast<size_t>(d) * H + h];
-    float mx = -INFINITY;
-    strided_pass<8>(threadIdx.x, n, kLongBlock,
-                    [&](uint64_t j) -> float {
-                      if (!FUSED) return xs[j];
-                      const uint32_t src = ri[e0 + j / H];
-                      return leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
-                    },
-                    [&](uint64_t j, float sc) {
-                      if (FUSED) ys[j] = sc;
-                      mx = fmaxf(mx, sc);
-                    });
+    float mx = -INFINITY, sum = 0.f;
+    strided_max_sum_pass<8>(
+        threadIdx.x, n, kLongBlock,
+        [&](uint64_t j) -> float {
+          if (!FUSED) return xs[j];
+          const uint32_t src = ri[e0 + j / H];
+          return leaky(el[static_cast<size_t>(src) * H + h] + erv, slope);
+        },
+        [&](uint64_t j, float sc) {
+          if (FUSED) ys[j] = sc;
+        },
+        mx, sum);
+    const float thread_mx = mx;
     mx = block_head_reduce<0>(mx, H, red);
-    float sum = 0.f;
-    strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
-                    [&](uint64_t, float sc) { sum += expf(sc - mx); });
-    sum = block_head_reduce<1>(sum, H, red);
+    sum = block_head_reduce<1>(sum * expf(thread_mx - mx), H, red);
     strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
                     [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) / sum; });
   }
