@@ -314,8 +314,8 @@ def run_epoch_workload(args):
     """Per-epoch time of a sampled mini-batch configuration through the library (every stage through
     the C ABI, see neutronbench_amd/epoch.py), next to the CPU oracle on a few batches of the same
     epoch.  One JSON line; `value` is the epoch time with the stages run one after the other, as the
-    reference's default mode does, and config.pipelined_epoch_s the time with the next batch built
-    on a second stream."""
+    reference's default mode does, and config.pipelined_epoch_s the time with four batches in flight
+    (two being sampled, one gathered, one aggregated, each stage on streams of its own)."""
     import torch
 
     from neutronbench_amd import epoch
@@ -323,7 +323,7 @@ def run_epoch_workload(args):
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (the HIP library has no CPU fallback)")
     serial = epoch.run(args.workload, pipeline=1, quiet=True)
-    piped = epoch.run(args.workload, pipeline=2, quiet=True)
+    piped = epoch.run(args.workload, pipeline=4, quiet=True)
     cpu = None
     if not args.no_cpu_baseline and args.workload != "gat":
         cpu = epoch_cpu_baseline(torch, args.workload, serial["batches"], args.cpu_batches)
@@ -337,7 +337,8 @@ def run_epoch_workload(args):
                                "sampling, layer construction, feature/label gather, aggregation fwd+bwd of every layer",
                    "vertices": serial["vertices"], "edges": serial["edges"], "stage_s": serial["stage_s"],
                    "sampled_edges": serial["sampled_edges"], "gathered_rows": serial["gathered_rows"],
-                   "cache_hit_rate": serial["cache_hit_rate"], "pipelined_epoch_s": piped["epoch_s"]},
+                   "cache_hit_rate": serial["cache_hit_rate"], "pipelined_epoch_s": piped["epoch_s"],
+                   "pipeline_depth": piped["pipeline"]},
         "roofline": None,
         "cpu_baseline": cpu,
     }

@@ -301,7 +301,10 @@ int nts_sddmm_heads(float *galpha, const float *in, const float *gout, const uin
  *                                                                                  remap = cache_node_hashmap
  * For k < n:  i = sel ? sel[k] : k;  g = row_ids[i];  if (remap) g = remap[g];
  *             out[i, :] = table[g, :]          (bit-exact copy)
- * `table`, `sel`, `remap` may be device memory or mapped host memory. */
+ * `table`, `sel`, `remap` may be device memory or mapped host memory.  A gather from a table in host
+ * memory is bound by the link and is launched with a small fixed grid (128 blocks, which keep the
+ * link full), so that work on other streams keeps the rest of the chip; the library learns where
+ * `table` lives from hipPointerGetAttributes. */
 int nts_gather_rows_f32(float *out, const float *table, const uint32_t *row_ids,
                         const uint32_t *sel, const uint32_t *remap, uint32_t n, uint32_t F,
                         nts_stream_t stream);

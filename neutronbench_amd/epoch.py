@@ -15,7 +15,10 @@ stream-ordered sequence with one read-back (nts_batch_builder_*; "sample" then h
 structure together); --sampler library goes hop by hop through the per-step entry points;
 --sampler harness uses the torch sampler of the test harness instead.  Stages are separated by
 stream synchronisation, as every reference operator synchronises its stream.  --pipeline 2 samples
-the next batch on a second stream while the current one is gathered and aggregated.
+the next batch on a second stream while the current one is gathered and aggregated; --pipeline P >= 3
+keeps P batches in flight: P - 2 are sampled ahead, each on a stream of its own, and the next
+batch's features and labels are gathered on another, so that sampling (small dependent kernels), the
+gather (PCIe) and the aggregation (HBM) of consecutive batches overlap.
 """
 import argparse
 import json
@@ -50,7 +53,7 @@ class Timer:
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
-def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False):
+def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False, checksum=False):
     cfg = dict(CONFIGS[name])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
@@ -71,80 +74,43 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     n_batches = (n_train + cfg["batch"] - 1) // cfg["batch"]
     if max_batches:
         n_batches = min(n_batches, max_batches)
-    edges_total, hits_total, rows_total = 0, 0, 0
     builder = BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0) if sampler == "builder" else None
     train32 = as_u32(train_nodes)
-    # The first batches load every kernel's code and grow the allocator's pools; they are run once
-    # untimed, then the epoch starts over from its first batch.
-    n_warm = min(warmup_batches, n_batches)
-    t_epoch = time.perf_counter()
-    sequence = list(range(n_warm)) + list(range(n_batches))
-    # pipeline = 2 (the reference's PIPELINES mode, toolkits/GCN_GPU_NEIGHBOR.hpp:1350-1363, with two
-    # stages in flight): the next batch is sampled on a second stream, by a second builder, while
-    # this one is gathered and aggregated.
+    # pipeline = P > 1 (the reference's PIPELINES mode: P batches in flight, each on a stream of its
+    # own and driven by a thread of its own, one batch at a time in each of the sample, transfer and
+    # train stages; toolkits/GCN_GPU_NEIGHBOR.hpp:1350-1363 and the stage mutexes of its batch loop).
+    # P = 2: the next batch is sampled on a second stream, by a builder of its own, while this one is
+    # gathered and aggregated.  P >= 3: P - 2 batches are sampled ahead, each chain of hops on a stream
+    # of its own (a chain of small dependent launches gains nothing from a busy chip, several chains
+    # side by side do), and the batch after the current one is gathered on a gather stream while the
+    # current one aggregates; an event orders each gather before its aggregation.  One host thread
+    # enqueues all of it: a producer thread of its own was measured and lost to contention for the
+    # interpreter (arxiv 0.039 s against 0.032 s).
     pipelined = builder is not None and pipeline > 1
+    staged_gather = pipelined and pipeline > 2
+    builders = [builder]
     if pipelined:
-        builders = [builder, BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0)]
-        side_stream = torch.cuda.Stream(device=dev)
+        builders += [BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0) for _ in range(pipeline - 1)]
+        sample_streams = [torch.cuda.Stream(device=dev) for _ in range(max(1, pipeline - 2))]
+        gather_stream = torch.cuda.Stream(device=dev) if staged_gather else None
+    totals = {"edges": 0, "hits": 0, "rows": 0, "checksum": 0.0}
 
-        def start_sampling(step):
-            b = sequence[step]
-            builders[step % 2].enqueue(train32[b * cfg["batch"]:(b + 1) * cfg["batch"]], 1000 * b,
-                                       side_stream.cuda_stream)
-        torch.cuda.synchronize()
-        start_sampling(0)
-    for step, b in enumerate(sequence):
-        if step == n_warm:
-            torch.cuda.synchronize()
-            tm.t.clear()
-            edges_total, hits_total, rows_total = 0, 0, 0
-            t_epoch = time.perf_counter()
-        batch = train_nodes[b * cfg["batch"]:(b + 1) * cfg["batch"]]
-        # -- sample (harness) + structure (library) -------------------------------------------
-        layers = []
-        dst_ids = batch
-        if pipelined:
-            t0 = time.perf_counter()
-            layers = builders[step % 2].collect()[::-1]
-            if step + 1 < len(sequence):
-                start_sampling(step + 1)
-            tm.t["sample_wait"] = tm.t.get("sample_wait", 0.0) + time.perf_counter() - t0
-        elif builder is not None:
-            t0 = time.perf_counter()
-            layers = builder.sample(train32[b * cfg["batch"]:(b + 1) * cfg["batch"]], 1000 * b)[::-1]
-            tm.add("sample", t0)
-        for hop, fan in enumerate(cfg["fanout"] if builder is None else []):
-            t0 = time.perf_counter()
-            if sampler == "library":
-                dst32 = dst_ids if dst_ids.dtype == torch.int32 else as_u32(dst_ids)
-                off32, rows32 = sample_hop(gco, gri, dst32, fan, 1000 * b + hop)
-            else:
-                d64 = dst_ids.to(torch.int64) & 0xFFFFFFFF
-                off, rows_global = synth.sample_hop(co, ri, d64, fan, 1000 * b + hop)
-                off32, rows32, dst32 = as_u32(off), as_u32(rows_global), as_u32(d64)
-            tm.add("sample", t0)
-            t0 = time.perf_counter()
-            layer = SampledLayer.from_device_hop(off32, rows32, dst32, V, want_perm=heads > 0)
-            tm.add("structure", t0)
-            layers.append(layer)
-            dst_ids = layer.dev_source
-        layers = layers[::-1]
-        edges_total += sum(l.e_size for l in layers)
-        # -- gather --------------------------------------------------------------------------
-        t0 = time.perf_counter()
+    def batch_ids(b):
+        return train32[b * cfg["batch"]:(b + 1) * cfg["batch"]]
+
+    def gather(stream_obj, layers):
         x = torch.empty(layers[0].src_size, cfg["F"], device=dev)
         if cache is not None:
-            hits = load_feature_gpu_cache(cs, layers[0], x, table.dev_ptr, cache)
+            hits = load_feature_gpu_cache(stream_obj, layers[0], x, table.dev_ptr, cache)
         else:
-            cs.zero_copy_feature_move_gpu(x, table.dev_ptr, layers[0].dev_source, cfg["F"], layers[0].src_size)
+            stream_obj.zero_copy_feature_move_gpu(x, table.dev_ptr, layers[0].dev_source, cfg["F"], layers[0].src_size)
             hits = None
         lab = torch.empty(layers[-1].v_size, dtype=torch.int64, device=dev)
-        load_label_gpu(cs, layers[-1], lab, labels)
-        tm.add("gather", t0)
-        rows_total += layers[0].src_size
-        if hits is not None:
-            hits_total += int(hits.item())
-        # -- aggregation forward, then backward in reverse order --------------------------------
+        load_label_gpu(stream_obj, layers[-1], lab, labels)
+        return x, lab, hits
+
+    def aggregate(layers, x):
+        """Forward through the layers (input side first), then backward in reverse order."""
         ops = []
         for l, layer in enumerate(layers):
             width = cfg["F"] if l == 0 else cfg["hidden"]
@@ -179,8 +145,120 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
             else:
                 g = ops[l].backward(g)
             tm.add("aggregate_bwd", t0)
+        return x, g
+
+    def sample_hop_by_hop(b):
+        layers, dst_ids = [], train_nodes[b * cfg["batch"]:(b + 1) * cfg["batch"]]
+        for hop, fan in enumerate(cfg["fanout"]):
+            t0 = time.perf_counter()
+            if sampler == "library":
+                dst32 = dst_ids if dst_ids.dtype == torch.int32 else as_u32(dst_ids)
+                off32, rows32 = sample_hop(gco, gri, dst32, fan, 1000 * b + hop)
+            else:
+                d64 = dst_ids.to(torch.int64) & 0xFFFFFFFF
+                off, rows_global = synth.sample_hop(co, ri, d64, fan, 1000 * b + hop)
+                off32, rows32, dst32 = as_u32(off), as_u32(rows_global), as_u32(d64)
+            tm.add("sample", t0)
+            t0 = time.perf_counter()
+            layer = SampledLayer.from_device_hop(off32, rows32, dst32, V, want_perm=heads > 0)
+            tm.add("structure", t0)
+            layers.append(layer)
+            dst_ids = layer.dev_source
+        return layers[::-1]  # input-side layer first
+
+    def finish_batch(layers, x, hits):
+        totals["edges"] += sum(l.e_size for l in layers)
+        totals["rows"] += layers[0].src_size
+        if hits is not None:
+            totals["hits"] += int(hits.item())
+        y, g = aggregate(layers, x)
+        if checksum:  # of the last layer's output and the first layer's input gradient: equal in every mode
+            totals["checksum"] += float(y.double().sum()) + float(g.double().sum())
+
+    def run_serial(sequence):
+        for b in sequence:
+            if builder is not None:
+                t0 = time.perf_counter()
+                layers = builder.sample(batch_ids(b), 1000 * b)
+                tm.add("sample", t0)
+            else:
+                layers = sample_hop_by_hop(b)
+            t0 = time.perf_counter()
+            x, _, hits = gather(cs, layers)
+            tm.add("gather", t0)
+            finish_batch(layers, x, hits)
+
+    def run_two_stage(sequence):
+        def start_sampling(step):
+            builders[step % 2].enqueue(batch_ids(sequence[step]), 1000 * sequence[step], sample_streams[0].cuda_stream)
+        start_sampling(0)
+        for step in range(len(sequence)):
+            t0 = time.perf_counter()
+            layers = builders[step % 2].collect()
+            if step + 1 < len(sequence):
+                start_sampling(step + 1)
+            tm.t["sample_wait"] = tm.t.get("sample_wait", 0.0) + time.perf_counter() - t0
+            t0 = time.perf_counter()
+            x, _, hits = gather(cs, layers)
+            tm.add("gather", t0)
+            finish_batch(layers, x, hits)
+
+    def run_staged(sequence):
+        chains = len(sample_streams)
+        started = 0
+
+        def sample_through(last_step):
+            nonlocal started
+            while started <= min(last_step, len(sequence) - 1):
+                builders[started % pipeline].enqueue(batch_ids(sequence[started]), 1000 * sequence[started],
+                                                     sample_streams[started % chains].cuda_stream)
+                started += 1
+
+        def start_gather(step):
+            """Waits for the sampled layers of `step`, then enqueues the gather of its features and labels."""
+            layers = builders[step % pipeline].collect()
+            with torch.cuda.stream(gather_stream):
+                x, lab, hits = gather(CudaStream(gather_stream.cuda_stream, synchronize=False), layers)
+                done = torch.cuda.Event()
+                done.record(gather_stream)
+            return layers, x, lab, hits, done
+
+        main = torch.cuda.current_stream()
+        sample_through(chains - 1)
+        staged = start_gather(0)
+        sample_through(chains)
+        for step in range(len(sequence)):
+            # Batch `step` trains below out of builder step % P; batch step + 1 is gathered out of the
+            # next builder; the P - 2 after it are being sampled.  Builder (step - 1) % P, whose batch
+            # has trained, takes the chain started here.
+            t0 = time.perf_counter()
+            layers, x, lab, hits, gathered = staged
+            if step + 1 < len(sequence):
+                staged = start_gather(step + 1)
+            sample_through(step + pipeline - 1)
+            tm.t["enqueue"] = tm.t.get("enqueue", 0.0) + time.perf_counter() - t0
+            t0 = time.perf_counter()
+            main.wait_event(gathered)
+            for t in (x, lab, hits):
+                if t is not None:
+                    t.record_stream(main)  # allocated on the gather stream, used on this one
+            tm.add("gather_wait", t0)
+            finish_batch(layers, x, hits)
+
+    run_batches = run_staged if staged_gather else run_two_stage if pipelined else run_serial
+    # The first batches load every kernel's code and grow the allocator's pools; they are run once
+    # untimed, as a short epoch of their own (the pipeline drains before the clock starts), then the
+    # epoch starts over from its first batch.
+    n_warm = min(warmup_batches, n_batches)
+    run_batches(list(range(n_warm)))
+    torch.cuda.synchronize()
+    tm.t.clear()
+    totals.update(edges=0, hits=0, rows=0, checksum=0.0)
+    t_epoch = time.perf_counter()
+    run_batches(list(range(n_batches)))
     torch.cuda.synchronize()
     epoch_s = time.perf_counter() - t_epoch
+    edges_total, hits_total, rows_total = totals["edges"], totals["hits"], totals["rows"]
     table.close()
     out = {
         "config": name, "scale": scale, "vertices": V, "edges": E, "batches": n_batches, "batch_size": cfg["batch"],
@@ -188,11 +266,13 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
         "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
-        "sampler": sampler, "pipeline": 2 if pipelined else 1, "sampled_edges": edges_total, "gathered_rows": rows_total,
+        "sampler": sampler, "pipeline": pipeline if pipelined else 1, "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
+        "checksum": totals["checksum"] if checksum else None,
     }
-    if builder is not None:
-        builder.close()
+    for b in builders:
+        if b is not None:
+            b.close()
     if not quiet:
         print(json.dumps(out))
     return out
@@ -205,7 +285,9 @@ if __name__ == "__main__":
     ap.add_argument("--max-batches", type=int, default=0)
     ap.add_argument("--sampler", choices=["builder", "library", "harness"], default="builder")
     ap.add_argument("--warmup-batches", type=int, default=2, help="untimed batches before the epoch starts")
-    ap.add_argument("--pipeline", type=int, default=1, choices=[1, 2],
-                    help="2: the next batch is sampled on a second stream while this one is gathered and aggregated")
+    ap.add_argument("--pipeline", type=int, default=1, choices=[1, 2, 3, 4, 5, 6],
+                    help="batches in flight. 2: the next batch is sampled on a second stream while this one is "
+                         "gathered and aggregated; 3 and more: P - 2 batches are sampled ahead and the next one is "
+                         "gathered on a stream of its own")
     a = ap.parse_args()
     run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline)

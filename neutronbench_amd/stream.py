@@ -14,10 +14,14 @@ from .abi import call, ptr
 
 
 class CudaStream:
-    def __init__(self, stream=None, device=0):
+    def __init__(self, stream=None, device=0, synchronize=True):
+        """synchronize=False: the batch-assembly methods, which in the reference end with a
+        cudaStreamSynchronize, only enqueue their work; for a caller that overlaps the gather of one
+        batch with the training of another and orders them with events."""
         if stream is None:
             stream = torch.cuda.current_stream(device).cuda_stream
         self.stream = int(stream)
+        self.synchronize = bool(synchronize)
 
     # -- stream plumbing ----------------------------------------------------------------------
     def getStream(self):
@@ -28,6 +32,10 @@ class CudaStream:
 
     def CUDA_DEVICE_SYNCHRONIZE(self):
         call("nts_stream_sync", self.stream)
+
+    def _end_of_method(self):
+        if self.synchronize:
+            self.CUDA_DEVICE_SYNCHRONIZE()
 
     # -- aggregation --------------------------------------------------------------------------
     def Gather_By_Dst_From_Src(self, input, output, weight_forward, row_indices, column_offset, src_start, src_end,
@@ -97,29 +105,29 @@ class CudaStream:
     def zero_copy_feature_move_gpu(self, dev_feature, pinned_host_feature, src_vertex, feature_size, vertex_size):
         call("nts_gather_rows_f32", ptr(dev_feature), ptr(pinned_host_feature), ptr(src_vertex), 0, 0, vertex_size,
              feature_size, self.stream)
-        self.CUDA_DEVICE_SYNCHRONIZE()
+        self._end_of_method()
 
     def zero_copy_feature_move_gpu_cache(self, dev_feature, pinned_host_feature, src_vertex, feature_size,
                                          vertex_size, local_idx):
         call("nts_gather_rows_f32", ptr(dev_feature), ptr(pinned_host_feature), ptr(src_vertex), ptr(local_idx), 0,
              vertex_size, feature_size, self.stream)
-        self.CUDA_DEVICE_SYNCHRONIZE()
+        self._end_of_method()
 
     def gather_feature_from_gpu_cache(self, dev_feature, dev_cache_feature, src_vertex, feature_size, vertex_size,
                                       local_idx_cache, cache_node_hashmap):
         call("nts_gather_rows_f32", ptr(dev_feature), ptr(dev_cache_feature), ptr(src_vertex), ptr(local_idx_cache),
              ptr(cache_node_hashmap), vertex_size, feature_size, self.stream)
-        self.CUDA_DEVICE_SYNCHRONIZE()
+        self._end_of_method()
 
     def global_copy_label_move_gpu(self, dev_label, global_dev_label, dst_vertex, vertex_size):
         call("nts_gather_labels_i64", ptr(dev_label), ptr(global_dev_label), ptr(dst_vertex), vertex_size, 1,
              self.stream)
-        self.CUDA_DEVICE_SYNCHRONIZE()
+        self._end_of_method()
 
     def global_copy_mulilabel_move_gpu(self, dev_label, global_dev_label, dst_vertex, vertex_size, label_size):
         call("nts_gather_labels_i64", ptr(dev_label), ptr(global_dev_label), ptr(dst_vertex), vertex_size, label_size,
              self.stream)
-        self.CUDA_DEVICE_SYNCHRONIZE()
+        self._end_of_method()
 
 
 def get_gpu_mem():

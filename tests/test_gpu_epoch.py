@@ -1,0 +1,51 @@
+"""The epoch harness gives the same batches whatever the number of batches in flight: the pipelined
+modes (sampling, gather and aggregation of consecutive batches on streams of their own, ordered by
+events) must reproduce the serial mode's sampled edges, gathered rows, cache hits and a checksum of
+every batch's aggregation output and input gradient, bit for bit."""
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("config,scale", [("arxiv", 0.25), ("products", 0.02), ("gat", 0.02)])
+def test_pipelined_epochs_match_the_serial_one(config, scale):
+    from neutronbench_amd import epoch
+
+    runs = {p: epoch.run(config, scale=scale, max_batches=7, warmup_batches=1, pipeline=p, quiet=True, checksum=True)
+            for p in (1, 2, 3, 5)}
+    serial = runs[1]
+    assert serial["sampled_edges"] > 0 and serial["gathered_rows"] > 0 and serial["checksum"] != 0.0
+    for p, r in runs.items():
+        assert r["pipeline"] == p
+        for key in ("batches", "sampled_edges", "gathered_rows", "cache_hit_rate", "checksum"):
+            assert r[key] == serial[key], (p, key, r[key], serial[key])
+
+
+def test_hop_by_hop_sampler_builds_the_same_batches():
+    from neutronbench_amd import epoch
+
+    a = epoch.run("arxiv", scale=0.25, max_batches=5, warmup_batches=0, sampler="builder", quiet=True, checksum=True)
+    b = epoch.run("arxiv", scale=0.25, max_batches=5, warmup_batches=0, sampler="library", quiet=True, checksum=True)
+    for key in ("sampled_edges", "gathered_rows", "checksum"):
+        assert a[key] == b[key], (key, a[key], b[key])
+
+
+def test_stream_wrapper_can_leave_batch_assembly_unsynchronised():
+    import torch
+
+    from neutronbench_amd.stream import CudaStream
+
+    dev = torch.device("cuda:0")
+    table = torch.arange(64 * 8, dtype=torch.float32, device=dev).view(64, 8)
+    ids = torch.tensor([5, 0, 63, 5], dtype=torch.int32, device=dev)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream())
+    out = torch.zeros(4, 8, device=dev)
+    with torch.cuda.stream(side):
+        cs = CudaStream(side.cuda_stream, synchronize=False)
+        cs.zero_copy_feature_move_gpu(out, table, ids, 8, 4)
+        done = torch.cuda.Event()
+        done.record(side)
+    torch.cuda.current_stream().wait_event(done)
+    assert torch.equal(out, table[ids.long()])
+    assert CudaStream(side.cuda_stream).synchronize is True
