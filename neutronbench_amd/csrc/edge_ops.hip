@@ -152,7 +152,13 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__
 // short row takes the next pending one instead of idling until the longest row of a fixed
 // assignment is done.  Every group adds its row's edge rows in order (eight loads in flight), so
 // the result does not depend on which group happened to take which row.
-template <typename V, int G>
+//
+// Narrow rows (G * sizeof(V) of 16 to 64 bytes) leave a lone lane or two with the whole row: a
+// 1,000-edge row is then 125 dependent rounds of eight loads.  There S slices of G lanes share a
+// row: together they load 8 S consecutive edge rows at once, and every lane of the group then adds
+// those values in edge order, fetching each from the lane that loaded it.  The sum is the same
+// running fp32 sum, bit for bit; only the loads are spread.
+template <typename V, int G, int S>
 __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__restrict__ out,
                                                                           const V *__restrict__ msg,
                                                                           const uint32_t *__restrict__ off,
@@ -161,10 +167,12 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
                                                                           uint32_t long_limit) {
   constexpr int NF = sizeof(V) / 4;
   const uint32_t lane = lane_id();
-  const uint32_t gl = lane & (G - 1), grp = lane / G;
+  constexpr int GG = G * S;  // lanes that share a row
+  const uint32_t gl = lane & (GG - 1), grp = lane / GG;
+  const uint32_t col = gl & (G - 1), slice = gl / G;
   const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
-  const bool col_live = gl < Fv;
+  const bool col_live = col < Fv;
   for (uint64_t base = wave * kWave; base < rows; base += n_waves * kWave) {
     uint32_t my_e0 = 0, my_e1 = 0;
     bool mine = false;
@@ -182,7 +190,7 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
       const uint64_t need_mask = __ballot(!have && gl == 0);
       bool took = false;
       if (!have) {
-        const uint32_t rank = __popcll(need_mask & ((1ull << (grp * G)) - 1ull));
+        const uint32_t rank = __popcll(need_mask & ((1ull << (grp * GG)) - 1ull));
         uint64_t m = pending;
         for (uint32_t t = 0; t < rank && m; ++t) m &= m - 1;
         if (m) {
@@ -202,28 +210,50 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
       for (uint32_t t = __popcll(need_mask); t > 0 && pending; --t) pending &= pending - 1;  // handed out
       if (!__ballot(have)) break;
       if (have) {
-        // up to eight edge rows of this group's row, loaded together, added in order
+        // up to 8 S edge rows of this group's row, loaded together (slice s takes the edges s, s + S,
+        // ...), added in order
         V v[8];
-        const uint32_t n = e1 - k < 8u ? e1 - k : 8u;
+        const uint32_t n = e1 - k < 8u * S ? e1 - k : 8u * S;
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          if (static_cast<uint32_t>(u) < n && col_live) {
-            const uint32_t e = perm ? perm[k + u] : k + u;
-            v[u] = msg[static_cast<size_t>(e) * Fv + gl];
+          v[u] = V{};
+          const uint32_t idx = u * S + slice;
+          if (idx < n && col_live) {
+            const uint32_t e = perm ? perm[k + idx] : k + idx;
+            v[u] = msg[static_cast<size_t>(e) * Fv + col];
           }
         }
+        if (S == 1) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          if (static_cast<uint32_t>(u) < n && col_live) {
+          for (int u = 0; u < 8; ++u) {
+            if (static_cast<uint32_t>(u) < n && col_live) {
+              const float *vf = reinterpret_cast<const float *>(&v[u]);
+#pragma unroll
+              for (int t = 0; t < NF; ++t) a[t] += vf[t];
+            }
+          }
+        } else {
+          const uint32_t first = lane - gl + col;  // the lane of slice 0 that holds this lane's column
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            if (!__ballot(static_cast<uint32_t>(u * S) < n)) break;  // no group of the wavefront has edges left
             const float *vf = reinterpret_cast<const float *>(&v[u]);
 #pragma unroll
-            for (int t = 0; t < NF; ++t) a[t] += vf[t];
+            for (int sl = 0; sl < S; ++sl) {
+              float val[NF];
+#pragma unroll
+              for (int t = 0; t < NF; ++t) val[t] = __shfl(vf[t], first + sl * G, kWave);
+              if (static_cast<uint32_t>(u * S + sl) < n) {
+#pragma unroll
+                for (int t = 0; t < NF; ++t) a[t] += val[t];
+              }
+            }
           }
         }
         k += n;
         if (k >= e1) {
-          if (col_live) {
-            V *p = out + (base + row) * Fv + gl;
+          if (col_live && slice == 0) {
+            V *p = out + (base + row) * Fv + col;
             if (accumulate) {
               const V o = *p;
               const float *of = reinterpret_cast<const float *>(&o);
@@ -1288,17 +1318,17 @@ void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_
     // One group covers a row: wavefronts hand their 64 rows out dynamically (strided launch).
     const uint32_t blocks = ceil_div(rows, 4 * kWave);  // at most 64 rows per wavefront
     const dim3 grid(blocks < 8192u ? blocks : 8192u);
-#define NTS_BALANCED(GG)                                                                                           \
-  hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG>), grid, dim3(256), 0, stream, out, msg, off, perm, \
-                     rows, Fv, accumulate, limit)
-    switch (lanes_for(Fv)) {
-      case 1: NTS_BALANCED(1); break;
-      case 2: NTS_BALANCED(2); break;
-      case 4: NTS_BALANCED(4); break;
-      case 8: NTS_BALANCED(8); break;
-      case 16: NTS_BALANCED(16); break;
-      case 32: NTS_BALANCED(32); break;
-      default: NTS_BALANCED(64); break;
+#define NTS_BALANCED(GG, SS)                                                                                         \
+  hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG, SS>), grid, dim3(256), 0, stream, out, msg, off, \
+                     perm, rows, Fv, accumulate, limit)
+    switch (lanes_for(Fv)) {  // rows narrower than eight lanes are shared by eight lanes all the same
+      case 1: NTS_BALANCED(1, 8); break;
+      case 2: NTS_BALANCED(2, 4); break;
+      case 4: NTS_BALANCED(4, 2); break;
+      case 8: NTS_BALANCED(8, 1); break;
+      case 16: NTS_BALANCED(16, 1); break;
+      case 32: NTS_BALANCED(32, 1); break;
+      default: NTS_BALANCED(64, 1); break;
     }
 #undef NTS_BALANCED
     return;

@@ -308,6 +308,10 @@ def test_long_rows_edge_sums(device, F):
     outs_ = dev(init, device)
     call("nts_gather_edge_to_src", ptr(outs_), ptr(dem), ptr(dro), ptr(dperm), Vs, F, 1, stream())
     check(outs_.cpu().numpy(), want_s + init, scale=sc_s + np.abs(init))
+    outs0 = torch.full((Vs, F), float("nan"), device=device)
+    call("nts_gather_edge_to_src", ptr(outs0), ptr(dem), ptr(dro), ptr(dperm), Vs, F, 0, stream())
+    short_s = np.diff(ro.astype(np.int64)) <= 1024
+    assert np.array_equal(outs0.cpu().numpy()[short_s], want_s[short_s])  # through the permutation as well
 
 
 def test_heads_aggregation_without_a_plan_cuts_hub_rows(device):

@@ -91,7 +91,7 @@ def test_softmax_and_attention_across_size_classes(device, H):
     check(ger_got, seg_sum(gs_want, seg, Vd).astype(np.float32), scale=seg_sum(gs_scale, seg, Vd).astype(np.float32))
 
 
-@pytest.mark.parametrize("F", [1, 4, 32, 100, 260])
+@pytest.mark.parametrize("F", [1, 2, 4, 8, 12, 16, 32, 100, 260])
 def test_edge_sums_across_size_classes(device, F):
     print(f"case F={F}", flush=True)
     rng = np.random.default_rng(2000 + F)
@@ -107,7 +107,10 @@ def test_edge_sums_across_size_classes(device, F):
     scale = seg_sum(np.abs(msg).astype(np.float64), seg, Vd)
     check(got, want.astype(np.float32), scale=scale.astype(np.float32))
     # rows of at most 1,024 edges are sequential chains: exactly the fp32 running sum
-    for r in np.flatnonzero((deg > 0) & (deg <= 1024))[:200]:
+    # (also for rows of 16 to 64 bytes, whose loads are spread over eight lanes): every row above 8
+    # edges, where a spread row takes more than one lane's loads, and 200 of the others
+    chains = (deg > 0) & (deg <= 1024)
+    for r in np.concatenate([np.flatnonzero(chains & (deg > 8)), np.flatnonzero(chains)[:200]]):
         acc = np.zeros(F, dtype=np.float32)
         for e in range(int(co[r]), int(co[r + 1])):
             acc = acc + msg[e]
