@@ -191,13 +191,20 @@ inline unsigned bits_for(uint32_t n) {  // bits needed to represent values in [0
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// The library's radix sort switches to a merge sort below 2^20 items: one block sort and two
+// launches per doubling, about twenty dependent launches for a sampled hop of 400 k edges (230 us of
+// a 570 us batch).  The one-sweep radix path needs a histogram and one launch per eight key bits,
+// and the keys here are local ids of 15 to 22 bits; it takes over from 16 k items.
+using HopSortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                                 rocprim::default_config, 16384>;
+
 // Scratch layout: [sorted keys: E u32][rocprim temporary storage].
 hipError_t sort_temp_bytes(uint32_t E, size_t *bytes) {
   size_t tmp = 0;
   uint32_t *nul = nullptr;
-  hipError_t err = rocprim::radix_sort_pairs(nullptr, tmp, nul, nul,
-                                                              rocprim::counting_iterator<uint32_t>(0u), nul, E ? E : 1u,
-                                                              0u, 32u, static_cast<hipStream_t>(nullptr), false);
+  hipError_t err = rocprim::radix_sort_pairs<HopSortConfig>(nullptr, tmp, nul, nul,
+                                                            rocprim::counting_iterator<uint32_t>(0u), nul, E ? E : 1u,
+                                                            0u, 32u, static_cast<hipStream_t>(nullptr), false);
   *bytes = tmp;
   return err;
 }
@@ -241,9 +248,9 @@ int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co,
   NTS_HIP_TRY(sort_temp_bytes(sort_n, &tmp));
   // Stable LSD radix sort of (local source, CSC edge id): edge ids stay ascending within a source,
   // which is exactly the order the host counting sort produces.
-  NTS_HIP_TRY(rocprim::radix_sort_pairs(w + keys_bytes, tmp, ri, keys_sorted,
-                                                         rocprim::counting_iterator<uint32_t>(0u), perm_out, sort_n,
-                                                         0u, key_bits, stream, false));
+  NTS_HIP_TRY(rocprim::radix_sort_pairs<HopSortConfig>(w + keys_bytes, tmp, ri, keys_sorted,
+                                                       rocprim::counting_iterator<uint32_t>(0u), perm_out, sort_n, 0u,
+                                                       key_bits, stream, false));
   const uint64_t span = static_cast<uint64_t>(Vs.cap) + 1 > E.cap ? static_cast<uint64_t>(Vs.cap) + 1 : E.cap;
   hipLaunchKernelGGL(csr_finish_kernel, dim3(ceil_div(span, 256)), dim3(256), 0, stream, ro, ci, keys_sorted, perm_out,
                      co, Vd, Vs, E);
