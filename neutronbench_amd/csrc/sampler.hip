@@ -41,6 +41,13 @@ struct HopCount {
   }
 };
 using HopCountIterator = rocprim::transform_iterator<rocprim::counting_iterator<uint32_t>, HopCount, uint32_t>;
+// Every input of this scan costs three dependent loads (live count, destination, its offsets), and a
+// thread works through its items one after the other: with the library's default of 8 to 16 items
+// per thread the scan of 4,097 slots took 26 us.  Two items per thread make it a matter of more
+// blocks instead.
+using HopScanConfig = rocprim::scan_config<256, 2, rocprim::block_load_method::block_load_transpose,
+                                           rocprim::block_store_method::block_store_transpose,
+                                           rocprim::block_scan_algorithm::using_warp_scan>;
 
 // True if `pred` holds on any lane of the caller's aligned group of G lanes (all of them active).
 template <int G>
@@ -123,8 +130,9 @@ hipError_t scan_bytes(uint32_t n, size_t *bytes) {
   size_t tmp = 0;
   uint32_t *nul = nullptr;
   HopCountIterator in(rocprim::counting_iterator<uint32_t>(0u), HopCount{nullptr, nullptr, host_count(0), 0});
-  hipError_t err = rocprim::exclusive_scan(nullptr, tmp, in, nul, 0u, n ? n : 1u, rocprim::plus<uint32_t>(),
-                                           static_cast<hipStream_t>(nullptr), false);
+  hipError_t err = rocprim::exclusive_scan<HopScanConfig>(nullptr, tmp, in, nul, 0u, n ? n : 1u,
+                                                          rocprim::plus<uint32_t>(), static_cast<hipStream_t>(nullptr),
+                                                          false);
   *bytes = tmp;
   return err;
 }
@@ -142,8 +150,8 @@ int hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, Dev
                 size_t scan_tmp_bytes, hipStream_t stream) {
   // One scan whose input is computed on the fly; slot n.cap (count 0) receives the edge total.
   HopCountIterator in(rocprim::counting_iterator<uint32_t>(0u), HopCount{graph_co, dst, n, fanout});
-  NTS_HIP_TRY(rocprim::exclusive_scan(scan_tmp, scan_tmp_bytes, in, co, 0u, n.cap + 1, rocprim::plus<uint32_t>(), stream,
-                                      false));
+  NTS_HIP_TRY(rocprim::exclusive_scan<HopScanConfig>(scan_tmp, scan_tmp_bytes, in, co, 0u, n.cap + 1,
+                                                     rocprim::plus<uint32_t>(), stream, false));
   return NTS_OK;
 }
 
