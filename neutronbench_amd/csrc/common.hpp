@@ -138,6 +138,38 @@ __device__ __forceinline__ uint32_t owner_of(const uint32_t *__restrict__ off, u
   return lo;
 }
 
+// Owners of the 64 consecutive edge positions base .. base + 63, one per lane, for a wavefront that
+// walks a contiguous span of edges: a binary search per lane is ~log2(n) dependent loads per step,
+// while consecutive edges belong to a handful of consecutive rows.  `d0` (wave-uniform) enters as
+// any row with off[d0] <= base, e.g. the owner found for an earlier step, and leaves as the owner
+// of `base`.  The wavefront reads the 64 offsets after d0 in one load; a lane's owner is d0 plus the
+// number of those offsets that are <= its position (found with six shuffles).  Only a step that
+// spans more than 64 rows (runs of empty rows) falls back to the search.  Lanes at or beyond
+// off[n] return n.  All 64 lanes must call it.
+__device__ __forceinline__ uint32_t owners_of_step(const uint32_t *__restrict__ off, uint32_t n, uint32_t base,
+                                                   uint32_t &d0) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t total = off[n];
+  uint32_t win;
+  while (true) {
+    const uint32_t idx = d0 + 1 + lane;
+    win = off[idx < n ? idx : n];
+    const uint32_t behind = __popcll(__ballot(win <= base));  // offsets of the window not beyond `base`
+    if (behind == 0 || base >= total) break;
+    d0 = behind < static_cast<uint32_t>(kWave) ? d0 + behind : owner_of(off, n, base);
+  }
+  const uint32_t e = base + lane;
+  uint32_t pos = 0;
+#pragma unroll
+  for (uint32_t step = kWave / 2; step >= 1; step >>= 1) {
+    const uint32_t v = __shfl(win, pos + step - 1, kWave);
+    if (v <= e) pos += step;
+  }
+  const uint32_t last = __shfl(win, kWave - 1, kWave);
+  if (e >= total) return n;
+  return last <= e ? owner_of(off, n, e) : d0 + pos;
+}
+
 // Butterfly reductions over the `width` lanes of an aligned lane group (width = power of two <= 64).
 template <int WIDTH>
 __device__ __forceinline__ float group_max(float v) {

@@ -25,8 +25,9 @@ inline dim3 wave_block() { return dim3(kWavesPerBlock * kWave); }
 //
 // Edge-parallel: the edge count is read on the device (co[Vd]); a wavefront takes 64 consecutive
 // edges per step, every lane looks up the feature row its edge copies from (the source id, or the
-// destination that owns the edge by binary search in co), and sub-wavefront groups of G lanes then
-// move 64/G rows at a time.  Work per wave does not depend on any vertex's degree.
+// destination that owns the edge, followed along the wavefront's contiguous span of edges), and
+// sub-wavefront groups of G lanes then move 64/G rows at a time.  Work per wave does not depend on
+// any vertex's degree.
 
 enum CopyMode { kFromSrc = 0, kFromDst = 1, kAddFromDst = 2 };
 
@@ -42,16 +43,25 @@ __global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, con
   constexpr uint32_t kEdgesPerStep = kWave / G;
   const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
-  for (uint64_t base = wave * kWave; base < E; base += n_waves * kWave) {
+  // A wavefront walks a contiguous span of wave steps: the destination that owns each step's edges
+  // follows from the previous step's (owners_of_step) instead of a search per lane.
+  const uint64_t total_steps = (static_cast<uint64_t>(E) + kWave - 1) / kWave;
+  const uint64_t per_wave = (total_steps + n_waves - 1) / n_waves;
+  const uint64_t first_step = wave * per_wave;
+  const uint64_t end_step = first_step + per_wave < total_steps ? first_step + per_wave : total_steps;
+  if (first_step >= end_step) return;
+  uint32_t d0 = mode == kFromSrc ? 0u : owner_of(co, Vd, static_cast<uint32_t>(first_step * kWave));
+  for (uint64_t step = first_step; step < end_step; ++step) {
+    const uint64_t base = step * kWave;
     const uint64_t e = base + lane;
     uint32_t row = 0;
-    if (e < E) {
-      if (mode == kFromSrc) {
+    if (mode == kFromSrc) {
+      if (e < E) {
         row = ri[e];
         if (mirror) row = mirror[row];
-      } else {
-        row = owner_of(co, Vd, static_cast<uint32_t>(e));
       }
+    } else {
+      row = owners_of_step(co, Vd, static_cast<uint32_t>(base), d0);
     }
     for (uint32_t j = 0; j < G; ++j) {
       const uint32_t holder = j * kEdgesPerStep + grp;  // lane that looked up this group's edge
@@ -1129,13 +1139,19 @@ __global__ __launch_bounds__(256) void sddmm_edge_kernel(float *__restrict__ gal
   uint32_t d_held = 0xFFFFFFFFu;
   float4 y4 = make_float4(0.f, 0.f, 0.f, 0.f);
   float y1 = 0.f;
-  for (uint64_t base = wave * kWave; base < E; base += n_waves * kWave) {
+  // A wavefront walks a contiguous span of wave steps, so that the owner of each step's edges is
+  // found from the previous step's instead of by a search per lane.
+  const uint64_t total_steps = (static_cast<uint64_t>(E) + kWave - 1) / kWave;
+  const uint64_t per_wave = (total_steps + n_waves - 1) / n_waves;
+  const uint64_t first_step = wave * per_wave;
+  const uint64_t end_step = first_step + per_wave < total_steps ? first_step + per_wave : total_steps;
+  if (first_step >= end_step) return;
+  uint32_t d0 = owner_of(co, Vd, static_cast<uint32_t>(first_step * kWave));
+  for (uint64_t step = first_step; step < end_step; ++step) {
+    const uint64_t base = step * kWave;
     const uint64_t e = base + lane;
-    uint32_t src = 0, own = 0;
-    if (e < E) {
-      src = ri[e];
-      own = owner_of(co, Vd, static_cast<uint32_t>(e));
-    }
+    const uint32_t own = owners_of_step(co, Vd, static_cast<uint32_t>(base), d0);
+    const uint32_t src = e < E ? ri[e] : 0u;
     // Four edges at a time: their gathered rows are requested before the first is used.
     constexpr uint32_t U = 4;
     for (uint32_t j0 = 0; j0 < G; j0 += U) {
