@@ -18,7 +18,9 @@ stream synchronisation, as every reference operator synchronises its stream.  --
 the next batch on a second stream while the current one is gathered and aggregated; --pipeline P >= 3
 keeps P batches in flight: P - 2 are sampled ahead, each on a stream of its own, and the next
 batch's features and labels are gathered on another, so that sampling (small dependent kernels), the
-gather (PCIe) and the aggregation (HBM) of consecutive batches overlap.
+gather (PCIe) and the aggregation (HBM) of consecutive batches overlap; from that depth on the host
+does not wait for any aggregation either (--stage-sync 0): batches are ordered by events, and the stage
+times printed are host enqueue times.
 """
 import argparse
 import json
@@ -43,17 +45,20 @@ CONFIGS = {
 
 
 class Timer:
-    def __init__(self):
+    def __init__(self, sync=True):
         self.t = {}
+        self.sync = sync  # False: stages are not waited for, the times are host enqueue times
 
     def add(self, key, t0):
         # Only the stream the stages run on: a device-wide wait would also wait for the next batch
         # being sampled on the second stream of the pipelined mode.
-        torch.cuda.current_stream().synchronize()
+        if self.sync:
+            torch.cuda.current_stream().synchronize()
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
-def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False, checksum=False):
+def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False, checksum=False,
+        stage_sync=None):
     cfg = dict(CONFIGS[name])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
@@ -69,7 +74,13 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     cache = FeatureCache(feat_cpu, out_deg.cpu(), int(V * cfg["cache"]), dev) if cfg["cache"] > 0 else None
     train_nodes = synth.permutation(V, cfg["seed"] + 42, dev)[:n_train]
     cs = CudaStream()
-    tm = Timer()
+    # Stages separated by a stream synchronisation, as every reference operator ends with one -- except
+    # from three batches in flight on, where the one host thread of this harness would stall all the
+    # streams it feeds: there the batches are ordered by events only and the host never waits for an
+    # aggregation (the reference gets the same effect from one host thread per pipeline).
+    if stage_sync is None:
+        stage_sync = not (sampler == "builder" and pipeline > 2)
+    tm = Timer(sync=stage_sync)
     heads = cfg.get("heads", 0)
     n_batches = (n_train + cfg["batch"] - 1) // cfg["batch"]
     if max_batches:
@@ -94,6 +105,7 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         sample_streams = [torch.cuda.Stream(device=dev) for _ in range(max(1, pipeline - 2))]
         gather_stream = torch.cuda.Stream(device=dev) if staged_gather else None
     totals = {"edges": 0, "hits": 0, "rows": 0, "checksum": 0.0}
+    hits_on_device = torch.zeros(1, dtype=torch.int64, device=dev)  # summed there when no stage is waited for
 
     def batch_ids(b):
         return train32[b * cfg["batch"]:(b + 1) * cfg["batch"]]
@@ -128,7 +140,7 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
                 y = agg.forward(x, att.forward(el, er))
                 ops.append((att, agg))
             else:
-                op = SingleGPUSampleGraphOp(layers, l, cs)
+                op = SingleGPUSampleGraphOp(layers, l, cs, sync=stage_sync)
                 y = op.forward(x)
                 ops.append(op)
             tm.add("aggregate_fwd", t0)
@@ -170,7 +182,10 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         totals["edges"] += sum(l.e_size for l in layers)
         totals["rows"] += layers[0].src_size
         if hits is not None:
-            totals["hits"] += int(hits.item())
+            if stage_sync:
+                totals["hits"] += int(hits.item())
+            else:
+                hits_on_device.add_(hits)
         y, g = aggregate(layers, x)
         if checksum:  # of the last layer's output and the first layer's input gradient: equal in every mode
             totals["checksum"] += float(y.double().sum()) + float(g.double().sum())
@@ -207,11 +222,16 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         chains = len(sample_streams)
         started = 0
 
+        trained = [None] * pipeline  # per builder: recorded when the batch built in it has been aggregated
+
         def sample_through(last_step):
             nonlocal started
             while started <= min(last_step, len(sequence) - 1):
+                stream = sample_streams[started % chains]
+                if trained[started % pipeline] is not None:
+                    stream.wait_event(trained[started % pipeline])  # the arena's last batch is still being read
                 builders[started % pipeline].enqueue(batch_ids(sequence[started]), 1000 * sequence[started],
-                                                     sample_streams[started % chains].cuda_stream)
+                                                     stream.cuda_stream)
                 started += 1
 
         def start_gather(step):
@@ -244,6 +264,8 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
                     t.record_stream(main)  # allocated on the gather stream, used on this one
             tm.add("gather_wait", t0)
             finish_batch(layers, x, hits)
+            trained[step % pipeline] = torch.cuda.Event()
+            trained[step % pipeline].record(main)
 
     run_batches = run_staged if staged_gather else run_two_stage if pipelined else run_serial
     # The first batches load every kernel's code and grow the allocator's pools; they are run once
@@ -254,11 +276,12 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     torch.cuda.synchronize()
     tm.t.clear()
     totals.update(edges=0, hits=0, rows=0, checksum=0.0)
+    hits_on_device.zero_()
     t_epoch = time.perf_counter()
     run_batches(list(range(n_batches)))
     torch.cuda.synchronize()
     epoch_s = time.perf_counter() - t_epoch
-    edges_total, hits_total, rows_total = totals["edges"], totals["hits"], totals["rows"]
+    edges_total, hits_total, rows_total = totals["edges"], totals["hits"] + int(hits_on_device.item()), totals["rows"]
     table.close()
     out = {
         "config": name, "scale": scale, "vertices": V, "edges": E, "batches": n_batches, "batch_size": cfg["batch"],
@@ -266,7 +289,7 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
         "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
-        "sampler": sampler, "pipeline": pipeline if pipelined else 1, "sampled_edges": edges_total, "gathered_rows": rows_total,
+        "sampler": sampler, "pipeline": pipeline if pipelined else 1, "stage_sync": stage_sync, "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
         "checksum": totals["checksum"] if checksum else None,
     }
@@ -289,5 +312,10 @@ if __name__ == "__main__":
                     help="batches in flight. 2: the next batch is sampled on a second stream while this one is "
                          "gathered and aggregated; 3 and more: P - 2 batches are sampled ahead and the next one is "
                          "gathered on a stream of its own")
+    ap.add_argument("--stage-sync", type=int, default=None, choices=[0, 1],
+                    help="1: wait for the stream after every stage (stage times are device times; default up to "
+                         "--pipeline 2); 0: never wait for an aggregation, batches are ordered by events (stage times "
+                         "are host enqueue times; default from --pipeline 3)")
     a = ap.parse_args()
-    run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline)
+    run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline,
+        stage_sync=None if a.stage_sync is None else bool(a.stage_sync))
