@@ -104,8 +104,9 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         builders += [BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0) for _ in range(pipeline - 1)]
         sample_streams = [torch.cuda.Stream(device=dev) for _ in range(max(1, pipeline - 2))]
         gather_stream = torch.cuda.Stream(device=dev) if staged_gather else None
-    totals = {"edges": 0, "hits": 0, "rows": 0, "checksum": 0.0}
+    totals = {"edges": 0, "hits": 0, "rows": 0}
     hits_on_device = torch.zeros(1, dtype=torch.int64, device=dev)  # summed there when no stage is waited for
+    checksum_on_device = torch.zeros((), dtype=torch.float64, device=dev)
 
     def batch_ids(b):
         return train32[b * cfg["batch"]:(b + 1) * cfg["batch"]]
@@ -188,7 +189,7 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
                 hits_on_device.add_(hits)
         y, g = aggregate(layers, x)
         if checksum:  # of the last layer's output and the first layer's input gradient: equal in every mode
-            totals["checksum"] += float(y.double().sum()) + float(g.double().sum())
+            checksum_on_device.add_(y.double().sum() + g.double().sum())  # no read-back: nothing waits here
 
     def run_serial(sequence):
         for b in sequence:
@@ -275,8 +276,9 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     run_batches(list(range(n_warm)))
     torch.cuda.synchronize()
     tm.t.clear()
-    totals.update(edges=0, hits=0, rows=0, checksum=0.0)
+    totals.update(edges=0, hits=0, rows=0)
     hits_on_device.zero_()
+    checksum_on_device.zero_()
     t_epoch = time.perf_counter()
     run_batches(list(range(n_batches)))
     torch.cuda.synchronize()
@@ -291,7 +293,7 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
         "sampler": sampler, "pipeline": pipeline if pipelined else 1, "stage_sync": stage_sync, "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
-        "checksum": totals["checksum"] if checksum else None,
+        "checksum": float(checksum_on_device.item()) if checksum else None,
     }
     for b in builders:
         if b is not None:
