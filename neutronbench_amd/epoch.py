@@ -205,6 +205,9 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
             finish_batch(layers, x, hits)
 
     def run_two_stage(sequence):
+        if not sequence:
+            return
+
         def start_sampling(step):
             builders[step % 2].enqueue(batch_ids(sequence[step]), 1000 * sequence[step], sample_streams[0].cuda_stream)
         start_sampling(0)
@@ -220,9 +223,10 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
             finish_batch(layers, x, hits)
 
     def run_staged(sequence):
+        if not sequence:
+            return
         chains = len(sample_streams)
         started = 0
-
         trained = [None] * pipeline  # per builder: recorded when the batch built in it has been aggregated
 
         def sample_through(last_step):
@@ -291,7 +295,8 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
         "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
-        "sampler": sampler, "pipeline": pipeline if pipelined else 1, "stage_sync": stage_sync, "sampled_edges": edges_total, "gathered_rows": rows_total,
+        "sampler": sampler, "pipeline": pipeline if pipelined else 1, "stage_sync": stage_sync,
+        "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
         "checksum": float(checksum_on_device.item()) if checksum else None,
     }

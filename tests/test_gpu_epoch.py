@@ -21,6 +21,15 @@ def test_pipelined_epochs_match_the_serial_one(config, scale):
             assert r[key] == serial[key], (p, key, r[key], serial[key])
 
 
+def test_pipelined_epoch_without_warm_up_batches():
+    from neutronbench_amd import epoch
+
+    a = epoch.run("arxiv", scale=0.25, max_batches=3, warmup_batches=0, pipeline=1, quiet=True, checksum=True)
+    for p in (2, 4):
+        b = epoch.run("arxiv", scale=0.25, max_batches=3, warmup_batches=0, pipeline=p, quiet=True, checksum=True)
+        assert (b["sampled_edges"], b["checksum"]) == (a["sampled_edges"], a["checksum"])
+
+
 def test_hop_by_hop_sampler_builds_the_same_batches():
     from neutronbench_amd import epoch
 
