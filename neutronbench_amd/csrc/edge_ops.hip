@@ -570,10 +570,11 @@ __device__ __forceinline__ void softmax_fwd_regs(float *__restrict__ ys, const f
     sum += v[k];
   }
   sum = head_reduce_w<1, WIDTH>(sum, H);
+  const float inv = 1.f / sum;  // one division per lane instead of one per value
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     const uint32_t i = gl + WIDTH * k;
-    if (i < n) ys[i] = v[k] / sum;
+    if (i < n) ys[i] = v[k] * inv;
   }
 }
 
@@ -621,6 +622,28 @@ __device__ __forceinline__ void softmax_bwd_regs(float *__restrict__ gxs, float 
   }
 }
 
+// These kernels are bound by their vector instructions, not by memory (253 per 256-value segment
+// were counted, a wave64 instruction holding its SIMD for four cycles: 80 % of the launch time), and
+// most of them served register slots beyond the segment's end.  The register paths are therefore
+// instantiated for 1, 2, 4 and 8 slots per lane and called with the smallest count that covers
+// every segment the wavefront is working on (`n`, the caller's segment size, must be in scope).
+#define NTS_BY_SLOTS(WIDTH, FN, ...)                                        \
+  do {                                                                      \
+    if (!any_lane(n > 4u * (WIDTH))) {                                      \
+      if (!any_lane(n > 2u * (WIDTH))) {                                    \
+        if (!any_lane(n > 1u * (WIDTH))) FN<FUSED, WIDTH, 1>(__VA_ARGS__);  \
+        else FN<FUSED, WIDTH, 2>(__VA_ARGS__);                              \
+      } else {                                                              \
+        FN<FUSED, WIDTH, 4>(__VA_ARGS__);                                   \
+      }                                                                     \
+    } else {                                                                \
+      FN<FUSED, WIDTH, 8>(__VA_ARGS__);                                     \
+    }                                                                       \
+  } while (0)
+
+// True if `pred` holds on any active lane of the wavefront.
+__device__ __forceinline__ bool any_lane(bool pred) { return __ballot(pred) != 0; }
+
 // Short segments (n <= kShortValues; power-of-two H <= kShortG): a group of kShortG lanes per
 // destination, striding over the destinations.  BWD selects the backward formula.
 template <bool FUSED, bool BWD>
@@ -642,12 +665,12 @@ __global__ __launch_bounds__(256) void edge_softmax_short_kernel(float *__restri
     const uint32_t n = static_cast<uint32_t>(n64);
     const size_t base = static_cast<size_t>(e0) * H;
     if (BWD) {
-      softmax_bwd_regs<FUSED, kShortG, kShortK>(out + base, ger, x_or_gy + base, y + base, el, er, ri, d, e0, n, H,
-                                                slope, gl);
+      NTS_BY_SLOTS(kShortG, softmax_bwd_regs, out + base, ger, x_or_gy + base, y + base, el, er, ri, d, e0, n, H, slope,
+                   gl);
     } else {
       if (n == 0) continue;
-      softmax_fwd_regs<FUSED, kShortG, kShortK>(out + base, FUSED ? nullptr : x_or_gy + base, el, er, ri, d, e0, n, H,
-                                                slope, gl);
+      NTS_BY_SLOTS(kShortG, softmax_fwd_regs, out + base, FUSED ? nullptr : x_or_gy + base, el, er, ri, d, e0, n, H,
+                   slope, gl);
     }
   }
 }
@@ -699,7 +722,7 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
 
       if (POW2) {
         if (n <= kWaveRegValues) {
-          softmax_fwd_regs<FUSED, kWave, kWaveK>(ys, xs, el, er, ri, d, e0, n, H, slope, lane);
+          NTS_BY_SLOTS(kWave, softmax_fwd_regs, ys, xs, el, er, ri, d, e0, n, H, slope, lane);
           continue;
         }
         const uint32_t h = lane & (H - 1);
@@ -721,8 +744,9 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
         const float lane_mx = mx;
         mx = head_reduce<0>(mx, H);
         sum = head_reduce<1>(sum * expf(lane_mx - mx), H);
+        const float inv = 1.f / sum;
         strided_pass<8>(lane, n, kWave, [&](uint64_t i) -> float { return FUSED ? ys[i] : xs[i]; },
-                        [&](uint64_t i, float sc) { ys[i] = expf(sc - mx) / sum; });
+                        [&](uint64_t i, float sc) { ys[i] = expf(sc - mx) * inv; });
       } else {
         const uint32_t deg = e1 - e0;
         for (uint32_t h = 0; h < H; ++h) {
@@ -747,9 +771,10 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
             sum += expf(sc - mx);
           }
           sum = group_sum<kWave>(sum);
+          const float inv = 1.f / sum;
           for (uint32_t k = lane; k < deg; k += kWave) {
             const float sc = FUSED ? ys[static_cast<size_t>(k) * H + h] : xs[static_cast<size_t>(k) * H + h];
-            ys[static_cast<size_t>(k) * H + h] = expf(sc - mx) / sum;
+            ys[static_cast<size_t>(k) * H + h] = expf(sc - mx) * inv;
           }
         }
       }
@@ -791,7 +816,7 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
 
       if (POW2) {
         if (n <= kWaveRegValues) {
-          softmax_bwd_regs<FUSED, kWave, kWaveK>(gxs, ger, gys, ys, el, er, ri, d, e0, n, H, slope, lane);
+          NTS_BY_SLOTS(kWave, softmax_bwd_regs, gxs, ger, gys, ys, el, er, ri, d, e0, n, H, slope, lane);
           continue;
         }
         const uint32_t h = lane & (H - 1);
@@ -900,8 +925,9 @@ __global__ __launch_bounds__(kLongBlock) void edge_softmax_fwd_long_kernel(
     const float thread_mx = mx;
     mx = block_head_reduce<0>(mx, H, red);
     sum = block_head_reduce<1>(sum * expf(thread_mx - mx), H, red);
+    const float inv = 1.f / sum;
     strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
-                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) / sum; });
+                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) * inv; });
   }
 }
 
@@ -1046,8 +1072,9 @@ __global__ __launch_bounds__(kLongBlock) void giant_softmax_apply_kernel(float *
     const float sum = rowstat[static_cast<size_t>(pc.x) * 2 * H + H + h];
     float *ys = y + base;
     const float *xs = FUSED ? ys : x + base;  // the fused forward left the raw score in y
+    const float inv = 1.f / sum;
     strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return xs[j]; },
-                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) / sum; });
+                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) * inv; });
   }
 }
 
