@@ -665,8 +665,13 @@ __global__ __launch_bounds__(256) void edge_softmax_short_kernel(float *__restri
     const uint32_t n = static_cast<uint32_t>(n64);
     const size_t base = static_cast<size_t>(e0) * H;
     if (BWD) {
-      NTS_BY_SLOTS(kShortG, softmax_bwd_regs, out + base, ger, x_or_gy + base, y + base, el, er, ri, d, e0, n, H, slope,
-                   gl);
+      if (FUSED) {  // the four instances together would cost this kernel a wavefront per SIMD
+        softmax_bwd_regs<FUSED, kShortG, kShortK>(out + base, ger, x_or_gy + base, y + base, el, er, ri, d, e0, n, H,
+                                                  slope, gl);
+      } else {
+        NTS_BY_SLOTS(kShortG, softmax_bwd_regs, out + base, ger, x_or_gy + base, y + base, el, er, ri, d, e0, n, H,
+                     slope, gl);
+      }
     } else {
       if (n == 0) continue;
       NTS_BY_SLOTS(kShortG, softmax_fwd_regs, out + base, FUSED ? nullptr : x_or_gy + base, el, er, ri, d, e0, n, H,
