@@ -175,6 +175,9 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
                                                                           const uint32_t *__restrict__ perm,
                                                                           uint32_t rows, uint32_t Fv, int accumulate,
                                                                           uint32_t long_limit) {
+  // Rows a wavefront takes at a time: eight per lane group, so that a wavefront with two groups
+  // (128-byte-wide vectors) is not left with 32 rows per group while others have finished.
+  constexpr uint32_t kSet = (kWave / (G * S)) * 8 < kWave ? (kWave / (G * S)) * 8 : kWave;
   constexpr int NF = sizeof(V) / 4;
   const uint32_t lane = lane_id();
   constexpr int GG = G * S;  // lanes that share a row
@@ -183,10 +186,10 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
   const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
   const bool col_live = col < Fv;
-  for (uint64_t base = wave * kWave; base < rows; base += n_waves * kWave) {
+  for (uint64_t base = wave * kSet; base < rows; base += n_waves * kSet) {
     uint32_t my_e0 = 0, my_e1 = 0;
     bool mine = false;
-    if (base + lane < rows) {
+    if (lane < kSet && base + lane < rows) {
       my_e0 = off[base + lane];
       my_e1 = off[base + lane + 1];
       mine = my_e1 - my_e0 <= long_limit;  // longer rows belong to the block kernels
@@ -354,73 +357,103 @@ __global__ __launch_bounds__(256) void giant_plan_kernel(uint32_t *__restrict__ 
   }
 }
 
-// Sum of the edge rows [e0, e1) by one 1024-thread block, added into dst[0 .. F).  Columns are taken
-// in tiles of `tile` (a power of two <= 1024); thread t owns column t % tile of slice t / tile, a
-// slice adds every (1024/tile)-th edge of the range in ascending order (eight loads in flight), and
-// slice 0 then adds the slices' sums in slice order.
-__device__ __forceinline__ void block_sum_edge_rows(float *__restrict__ dst, const float *__restrict__ msg,
+__device__ __forceinline__ void vadd(float &a, const float &b) { a += b; }
+__device__ __forceinline__ void vadd(float4 &a, const float4 &b) {
+  a.x += b.x;
+  a.y += b.y;
+  a.z += b.z;
+  a.w += b.w;
+}
+template <typename V>
+__device__ __forceinline__ V vnull();
+template <>
+__device__ __forceinline__ float vnull<float>() {
+  return 0.f;
+}
+template <>
+__device__ __forceinline__ float4 vnull<float4>() {
+  return make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// Sum of the edge rows [e0, e1) by one 1024-thread block, added into dst[0 .. Fv) (V = float, or
+// float4 when rows are 16-byte aligned: a quarter of the load instructions and of the rounds a row
+// takes).  Columns are taken in tiles of `tile` vectors (a power of two <= 1024); thread t owns
+// column t % tile of slice t / tile, a slice adds every (1024/tile)-th edge of the range in ascending
+// order (eight loads in flight), and the slices' sums are then added pairwise in a fixed tree.
+template <typename V>
+__device__ __forceinline__ void block_sum_edge_rows(V *__restrict__ dst, const V *__restrict__ msg,
                                                     const uint32_t *__restrict__ perm, uint32_t e0, uint32_t e1,
-                                                    uint32_t F, uint32_t tile, int accumulate, float *part) {
+                                                    uint32_t Fv, uint32_t tile, int accumulate, V *part) {
   const uint32_t c = threadIdx.x & (tile - 1);
   const uint32_t slice = threadIdx.x / tile;
   const uint32_t n_slices = kLongBlock / tile;
-  for (uint32_t cb = 0; cb < F; cb += tile) {
+  for (uint32_t cb = 0; cb < Fv; cb += tile) {
     const uint32_t col = cb + c;
-    float a = 0.f;
-    if (col < F) {
+    V a = vnull<V>();
+    if (col < Fv) {
       uint32_t k = e0 + slice;
       for (; static_cast<uint64_t>(k) + 7ull * n_slices < e1; k += 8 * n_slices) {
-        float v[8];
+        V v[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const uint32_t kk = k + u * n_slices;
           const uint32_t e = perm ? perm[kk] : kk;
-          v[u] = msg[static_cast<size_t>(e) * F + col];
+          v[u] = msg[static_cast<size_t>(e) * Fv + col];
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) a += v[u];
+        for (int u = 0; u < 8; ++u) vadd(a, v[u]);
       }
       for (; k < e1; k += n_slices) {
         const uint32_t e = perm ? perm[k] : k;
-        a += msg[static_cast<size_t>(e) * F + col];
+        vadd(a, msg[static_cast<size_t>(e) * Fv + col]);
       }
     }
     part[threadIdx.x] = a;
     __syncthreads();
-    if (slice == 0 && col < F) {
-      float total = part[c];
-      for (uint32_t sidx = 1; sidx < n_slices; ++sidx) total += part[sidx * tile + c];
-      dst[col] = accumulate ? dst[col] + total : total;
+    for (uint32_t stride = n_slices / 2; stride >= 1; stride >>= 1) {
+      if (slice < stride) {
+        V lo = part[threadIdx.x];
+        vadd(lo, part[threadIdx.x + stride * tile]);
+        part[threadIdx.x] = lo;
+      }
+      __syncthreads();
+    }
+    if (slice == 0 && col < Fv) {
+      V total = part[c];
+      if (accumulate) vadd(total, dst[col]);
+      dst[col] = total;
     }
     __syncthreads();
   }
 }
 
 // One 1024-thread block per listed long row.
+template <typename V>
 __global__ __launch_bounds__(kLongBlock) void gather_edge_to_row_long_kernel(
-    float *__restrict__ out, const float *__restrict__ msg, const uint32_t *__restrict__ off,
+    V *__restrict__ out, const V *__restrict__ msg, const uint32_t *__restrict__ off,
     const uint32_t *__restrict__ perm, const uint32_t *__restrict__ list, const uint32_t *__restrict__ count,
-    uint32_t F, uint32_t tile, int accumulate) {
-  __shared__ float part[kLongBlock];
+    uint32_t Fv, uint32_t tile, int accumulate) {
+  __shared__ V part[kLongBlock];
   const uint32_t n_rows = *count;
   for (uint32_t i = blockIdx.x; i < n_rows; i += gridDim.x) {
     const uint32_t r = list[i];
-    block_sum_edge_rows(out + static_cast<size_t>(r) * F, msg, perm, off[r], off[r + 1], F, tile, accumulate, part);
+    block_sum_edge_rows(out + static_cast<size_t>(r) * Fv, msg, perm, off[r], off[r + 1], Fv, tile, accumulate, part);
   }
 }
 
 // One block per piece of a giant row: partial[piece, :] = sum of the piece's edge rows.
-__global__ __launch_bounds__(kLongBlock) void giant_sum_pieces_kernel(float *__restrict__ partial,
-                                                                      const float *__restrict__ msg,
+template <typename V>
+__global__ __launch_bounds__(kLongBlock) void giant_sum_pieces_kernel(V *__restrict__ partial,
+                                                                      const V *__restrict__ msg,
                                                                       const uint32_t *__restrict__ perm,
                                                                       const uint32_t *__restrict__ hdr,
-                                                                      const uint4 *__restrict__ pieces, uint32_t F,
+                                                                      const uint4 *__restrict__ pieces, uint32_t Fv,
                                                                       uint32_t tile) {
-  __shared__ float part[kLongBlock];
+  __shared__ V part[kLongBlock];
   const uint32_t n_pieces = hdr[1];
   for (uint32_t p = blockIdx.x; p < n_pieces; p += gridDim.x) {
     const uint4 pc = pieces[p];
-    block_sum_edge_rows(partial + static_cast<size_t>(p) * F, msg, perm, pc.z, pc.w, F, tile, 0, part);
+    block_sum_edge_rows(partial + static_cast<size_t>(p) * Fv, msg, perm, pc.z, pc.w, Fv, tile, 0, part);
   }
 }
 
@@ -1364,11 +1397,13 @@ void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_
                         int accumulate, uint32_t limit, hipStream_t stream) {
   if (Fv <= 64 && rows >= 4096) {
     // One group covers a row: wavefronts hand their 64 rows out dynamically (strided launch).
-    const uint32_t blocks = ceil_div(rows, 4 * kWave);  // at most 64 rows per wavefront
-    const dim3 grid(blocks < 8192u ? blocks : 8192u);
-#define NTS_BALANCED(GG, SS)                                                                                         \
-  hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG, SS>), grid, dim3(256), 0, stream, out, msg, off, \
-                     perm, rows, Fv, accumulate, limit)
+#define NTS_BALANCED(GG, SS)                                                                                    \
+  do {                                                                                                          \
+    const uint32_t set = (kWave / ((GG) * (SS))) * 8 < kWave ? (kWave / ((GG) * (SS))) * 8 : kWave;            \
+    const uint32_t blocks = ceil_div(rows, 4 * set); /* at most `set` rows per wavefront at a time */          \
+    hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG, SS>), dim3(blocks < 16384u ? blocks : 16384u), \
+                       dim3(256), 0, stream, out, msg, off, perm, rows, Fv, accumulate, limit);                 \
+  } while (0)
     switch (lanes_for(Fv)) {  // rows narrower than eight lanes are shared by eight lanes all the same
       case 1: NTS_BALANCED(1, 8); break;
       case 2: NTS_BALANCED(2, 4); break;
@@ -1411,17 +1446,30 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
     launch_gather_rows(out, msg, off, perm, rows, F, accumulate, limit, stream);
   NTS_LAUNCH_CHECK(who);
   if (lr.list) {
+    // The block kernels take 16-byte vectors under the same condition as the row kernels above.
+    const bool v4 = F % 4 == 0 && aligned_to(out, 16) && aligned_to(msg, 16);
+    const uint32_t Fv = v4 ? F / 4 : F;
     uint32_t tile = 1;
-    while (tile < F && tile < static_cast<uint32_t>(kLongBlock)) tile <<= 1;
-    hipLaunchKernelGGL(gather_edge_to_row_long_kernel, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, msg, off,
-                       perm, lr.list, lr.count, F, tile, accumulate);
+    while (tile < Fv && tile < static_cast<uint32_t>(kLongBlock)) tile <<= 1;
+    if (v4)
+      hipLaunchKernelGGL(gather_edge_to_row_long_kernel<float4>, dim3(kLongGrid), dim3(kLongBlock), 0, stream,
+                         reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, lr.list,
+                         lr.count, Fv, tile, accumulate);
+    else
+      hipLaunchKernelGGL(gather_edge_to_row_long_kernel<float>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, msg,
+                         off, perm, lr.list, lr.count, Fv, tile, accumulate);
     NTS_LAUNCH_CHECK(who);
     // Giant rows: pieces by separate blocks into stream-ordered scratch, then the ordered combine.
     float *partial = nullptr;
     NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&partial), static_cast<size_t>(kPieceCap) * F * sizeof(float),
                                stream));
-    hipLaunchKernelGGL(giant_sum_pieces_kernel, dim3(kLongGrid), dim3(kLongBlock), 0, stream, partial, msg, perm, lr.hdr,
-                       lr.pieces, F, tile);
+    if (v4)
+      hipLaunchKernelGGL(giant_sum_pieces_kernel<float4>, dim3(kLongGrid), dim3(kLongBlock), 0, stream,
+                         reinterpret_cast<float4 *>(partial), reinterpret_cast<const float4 *>(msg), perm, lr.hdr,
+                         lr.pieces, Fv, tile);
+    else
+      hipLaunchKernelGGL(giant_sum_pieces_kernel<float>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, partial, msg,
+                         perm, lr.hdr, lr.pieces, Fv, tile);
     hipLaunchKernelGGL(giant_sum_combine_kernel, dim3(kGiantCap / 4), dim3(256), 0, stream, out, partial, lr.hdr,
                        lr.giant_rows, lr.first, F, accumulate);
     const hipError_t launch_err = hipGetLastError();
