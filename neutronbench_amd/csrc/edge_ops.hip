@@ -912,7 +912,8 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
 //                ger[d,h] = sum_seg gx[e,h].
 // Visits the destinations with min_values <= n <= max_values (empty segments included when
 // min_values is 0, so that ger is written for every destination).
-template <bool FUSED, bool POW2>
+// PART as in the forward kernel: the fused form is launched in two parts.
+template <bool FUSED, bool POW2, int PART>
 __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict__ gx, float *__restrict__ ger,
                                                                const float *__restrict__ gy,
                                                                const float *__restrict__ y,
@@ -921,7 +922,7 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
                                                                const uint32_t *__restrict__ co,
                                                                const uint32_t *__restrict__ ri, uint32_t Vd,
                                                                uint32_t H, float slope, uint32_t min_values,
-                                                               uint32_t max_values) {
+                                                               uint32_t max_values, uint32_t vec4) {
   const uint32_t lane = lane_id();
   const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
@@ -940,8 +941,55 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
       float *gxs = gx + base;
 
       if (POW2) {
-        if (n <= kWaveRegValues) {
+        if (PART <= 1 && n <= kWaveRegValues) {
           NTS_BY_SLOTS(kWave, softmax_bwd_regs, gxs, ger, gys, ys, el, er, ri, d, e0, n, H, slope, lane);
+          continue;
+        }
+        if (PART == 1) continue;
+        if (PART == 2 && FUSED && vec4 && n >= 2048u) {
+          // 16-byte lanes: four consecutive values = heads (4 lane mod H) .. +3 of one edge
+          const uint32_t h0 = (lane * 4u) & (H - 1);
+          const uint32_t hq = H / 4;
+          const float4 *gys4 = reinterpret_cast<const float4 *>(gys);
+          const float4 *ys4 = reinterpret_cast<const float4 *>(ys);
+          float4 *gxs4 = reinterpret_cast<float4 *>(gxs);
+          float dot4[4] = {0.f, 0.f, 0.f, 0.f};
+          strided_pass<4>(lane, n / 4, kWave, [&](uint64_t i) -> float4 { return gys4[i]; },
+                          [&](uint64_t i, float4 g) {
+                            const float4 a = ys4[i];
+                            dot4[0] += g.x * a.x;
+                            dot4[1] += g.y * a.y;
+                            dot4[2] += g.z * a.z;
+                            dot4[3] += g.w * a.w;
+                          });
+#pragma unroll
+          for (int c = 0; c < 4; ++c) dot4[c] = head_reduce<1>(dot4[c], hq);
+          const float4 erv = *reinterpret_cast<const float4 *>(er + static_cast<size_t>(d) * H + h0);
+          float gsum4[4] = {0.f, 0.f, 0.f, 0.f};
+          strided_pass<4>(lane, n / 4, kWave,
+                          [&](uint64_t i) -> float4 {
+                            const uint32_t src = ri[e0 + static_cast<uint32_t>(i * 4 / H)];
+                            return *reinterpret_cast<const float4 *>(el + static_cast<size_t>(src) * H + h0);
+                          },
+                          [&](uint64_t i, float4 e) {
+                            const float4 g = gys4[i], a = ys4[i];
+                            float4 r;
+                            r.x = a.x * (g.x - dot4[0]) * (e.x + erv.x > 0.f ? 1.f : slope);
+                            r.y = a.y * (g.y - dot4[1]) * (e.y + erv.y > 0.f ? 1.f : slope);
+                            r.z = a.z * (g.z - dot4[2]) * (e.z + erv.z > 0.f ? 1.f : slope);
+                            r.w = a.w * (g.w - dot4[3]) * (e.w + erv.w > 0.f ? 1.f : slope);
+                            gsum4[0] += r.x;
+                            gsum4[1] += r.y;
+                            gsum4[2] += r.z;
+                            gsum4[3] += r.w;
+                            gxs4[i] = r;
+                          });
+#pragma unroll
+          for (int c = 0; c < 4; ++c) gsum4[c] = head_reduce<1>(gsum4[c], hq);
+          if (lane < hq) {
+            *reinterpret_cast<float4 *>(ger + static_cast<size_t>(d) * H + h0) =
+                make_float4(gsum4[0], gsum4[1], gsum4[2], gsum4[3]);
+          }
           continue;
         }
         const uint32_t h = lane & (H - 1);
@@ -1579,7 +1627,7 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   // 16-byte lanes for the segments that do not fit the register paths: whole heads per lane and
   // every array 16-byte aligned (a segment starts at e0 * H floats).
   const uint32_t vec4 = pow2 && H % 4 == 0 && aligned_to(out, 16) && aligned_to(x_or_gy, 16) && aligned_to(y, 16) &&
-                        aligned_to(el, 16) && aligned_to(er, 16);
+                        aligned_to(el, 16) && aligned_to(er, 16) && aligned_to(ger, 16);
   const bool use_short = pow2 && H <= static_cast<uint32_t>(kShortG);
   const uint32_t min_values = use_short ? kShortValues + 1 : 0u;
   // Both strided kernels: enough wavefronts to fill the chip several times, never more than the work.
@@ -1623,11 +1671,18 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
       NTS_LAUNCH_CHECK(who);
     }
   } else {
-#define NTS_BWD(FU, P2)                                                                                           \
-  hipLaunchKernelGGL((edge_softmax_bwd_kernel<FU, P2>), grid, block, 0, stream, out, ger, x_or_gy, y, el, er, co, ri, \
-                     Vd, H, slope, min_values, max_values)
-    if (fused) { if (pow2) NTS_BWD(true, true); else NTS_BWD(true, false); }
-    else       { if (pow2) NTS_BWD(false, true); else NTS_BWD(false, false); }
+#define NTS_BWD(FU, P2, PART, LO, HI)                                                                            \
+  hipLaunchKernelGGL((edge_softmax_bwd_kernel<FU, P2, PART>), grid, block, 0, stream, out, ger, x_or_gy, y, el, er, co, \
+                     ri, Vd, H, slope, LO, HI, vec4)
+    if (pow2 && fused) {
+      const uint32_t regs_hi = max_values < kWaveRegValues ? max_values : kWaveRegValues;
+      NTS_BWD(true, true, 1, min_values, regs_hi);
+      if (max_values > kWaveRegValues) NTS_BWD(true, true, 2, kWaveRegValues + 1, max_values);
+    } else if (pow2) {
+      NTS_BWD(false, true, 0, min_values, max_values);
+    } else {
+      if (fused) NTS_BWD(true, false, 0, min_values, max_values); else NTS_BWD(false, false, 0, min_values, max_values);
+    }
 #undef NTS_BWD
     NTS_LAUNCH_CHECK(who);
     if (lr.list) {

@@ -90,6 +90,27 @@ def test_softmax_and_attention_across_size_classes(device, H):
     assert not np.isnan(ger_got).any()  # empty destinations get zeros
     check(ger_got, seg_sum(gs_want, seg, Vd).astype(np.float32), scale=seg_sum(gs_scale, seg, Vd).astype(np.float32))
 
+    # The same call with every float array one float off a 16-byte boundary: the library may only use
+    # 16-byte lanes when all of them allow it, and must give the same results when they do not.
+    def off1(t):
+        buf = torch.empty(t.numel() + 1, dtype=t.dtype, device=t.device)
+        view = buf[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 == 4
+        return view
+
+    u_el, u_er, u_gy, u_alpha_in = off1(d_el), off1(d_er), off1(dgy), off1(d_alpha)
+    u_alpha = off1(torch.full((E, H), float("nan"), device=device))
+    call("nts_gat_attention_fwd", ptr(u_alpha), ptr(u_el), ptr(u_er), ptr(dco), ptr(dri), Vd, H, 0.2, stream())
+    check(u_alpha.cpu().numpy(), alpha_ref.astype(np.float32), scale=1.0, floor=1e-7)
+    u_gs = off1(torch.full((E, H), float("nan"), device=device))
+    u_ger = off1(torch.full((Vd, H), float("nan"), device=device))
+    call("nts_gat_attention_bwd", ptr(u_gs), ptr(u_ger), ptr(u_gy), ptr(u_alpha_in), ptr(u_el), ptr(u_er), ptr(dco),
+         ptr(dri), Vd, H, 0.2, stream())
+    check(u_gs.cpu().numpy(), gs_want.astype(np.float32), scale=gs_scale.astype(np.float32))
+    check(u_ger.cpu().numpy(), seg_sum(gs_want, seg, Vd).astype(np.float32),
+          scale=seg_sum(gs_scale, seg, Vd).astype(np.float32))
+
 
 @pytest.mark.parametrize("F", [1, 2, 4, 8, 12, 16, 32, 100, 260])
 def test_edge_sums_across_size_classes(device, F):
