@@ -216,8 +216,11 @@ int nts_scatter_dst_to_edge(float *msg, const float *feat, const uint32_t *co, u
 int nts_scatter_grad_to_edge(float *msg_grad, const float *gout, const uint32_t *co, uint32_t Vd,
                              uint32_t F, nts_stream_t stream);
 /* Cuda_Stream::Gather_Msg_to_Dst (cuda/ntsCUDA.hpp:157-159; kernel
- * cuda/ntsCUDADistKernel.cuh:81-95): out[d,:] (+)= sum_{e in CSC(d)} msg[e,:], summed in edge
- * order.  accumulate as in nts_spmm_gather. */
+ * cuda/ntsCUDADistKernel.cuh:81-95): out[d,:] (+)= sum_{e in CSC(d)} msg[e,:].  Rows of at most
+ * 1,024 edges are summed in edge order (the running fp32 sum); longer rows are spread over the
+ * slices of a block (and, above 16,384 edges, over several blocks) whose partial sums are added in
+ * a fixed order: the same bits on every call, within rounding of the edge-order sum.  accumulate as
+ * in nts_spmm_gather. */
 int nts_gather_edge_to_dst(float *out, const float *msg, const uint32_t *co, uint32_t Vd,
                            uint32_t F, int accumulate, nts_stream_t stream);
 /* Cuda_Stream::Gather_Msg_To_Src_Mirror (cuda/ntsCUDA.hpp:149-151; kernel :46-63), made
