@@ -395,3 +395,38 @@ def test_heads_aggregation_through_a_schedule(device, sorted_rows):
         check(gx[:, sl], oracle.spmm(gs, wb, ro, ci, Vs), abs_term_scale(gs, wb, ro, ci, Vs))
     fwd.close()
     bwd.close()
+
+
+def test_edge_parallel_kernels_over_runs_of_empty_rows(device):
+    """The edge-parallel kernels follow the owning destination along a wavefront's span of edges and
+    read the 64 offsets after the current row; where 64 consecutive edges spread over more rows than
+    that (sparse rows between runs of empty ones), or a span starts after hundreds of empty rows, they
+    must still find every edge's owner."""
+    rng = np.random.default_rng(77)
+    Vd, Vs, H, Fh = 30000, 4000, 4, 8
+    deg = np.zeros(Vd, dtype=np.int64)
+    deg[::7] = 1                          # one edge every seventh row: 64 edges span 448 rows
+    deg[3000:3400] = 0                    # a run of empty rows
+    deg[3400] = 300                       # then a row longer than a wavefront's step
+    deg[9000:9100] = rng.integers(0, 3, 100)
+    deg[15000:29000] = 0                  # a long empty run before the last rows
+    deg[29990:] = 5
+    co = np.concatenate([[0], np.cumsum(deg)]).astype(np.uint32)
+    E = int(co[-1])
+    ri = rng.integers(0, Vs, E).astype(np.uint32)
+    seg = np.repeat(np.arange(Vd), deg)
+    F = H * Fh
+    xd = rng.standard_normal((Vd, F)).astype(np.float32)
+    hs = rng.standard_normal((Vs, F)).astype(np.float32)
+    dco, dri, dxd, dhs = dev(co, device), dev(ri, device), dev(xd, device), dev(hs, device)
+    msg = torch.full((E, F), float("nan"), device=device)
+    call("nts_scatter_dst_to_edge", ptr(msg), ptr(dxd), ptr(dco), Vd, F, stream())
+    assert np.array_equal(msg.cpu().numpy(), xd[seg])
+    acc = torch.ones((E, F), device=device)
+    call("nts_scatter_grad_to_edge", ptr(acc), ptr(dxd), ptr(dco), Vd, F, stream())
+    assert np.array_equal(acc.cpu().numpy(), np.float32(1) + xd[seg])
+    galpha = torch.full((E, H), float("nan"), device=device)
+    call("nts_sddmm_heads", ptr(galpha), ptr(dhs), ptr(dxd), ptr(dco), ptr(dri), Vd, H, Fh, stream())
+    want = (hs[ri].reshape(E, H, Fh).astype(np.float64) * xd[seg].reshape(E, H, Fh)).sum(2)
+    scale = np.abs(hs[ri].reshape(E, H, Fh).astype(np.float64) * xd[seg].reshape(E, H, Fh)).sum(2)
+    check(galpha.cpu().numpy(), want.astype(np.float32), scale=scale.astype(np.float32))
