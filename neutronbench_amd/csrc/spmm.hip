@@ -88,7 +88,13 @@ __device__ __forceinline__ void vadd(float4 &a, float4 x) {
 }
 
 // Edges processed per inner step: keeps 8..16 independent row loads in flight per lane.
-__host__ __device__ constexpr int unroll_for(int nacc) { return nacc >= 6 ? 1 : nacc >= 4 ? 2 : nacc >= 2 ? 4 : 8; }
+// With 4-byte lanes and six to ten accumulators (F = 602: ten) four edges per step were measured
+// against one, two and three: 11.04 ms against 11.54 / 11.13 / 11.13 for the Reddit-shaped F=602 pass --
+// a step's loads are all requested before the first is used, so a wavefront then has 40 row loads in
+// flight instead of 10.  With 16-byte lanes the same count would cost 160 registers.
+__host__ __device__ constexpr int unroll_for(int nacc, int vec) {
+  return nacc >= 6 ? (vec == 1 ? 4 : 1) : nacc >= 4 ? 2 : nacc >= 2 ? 4 : 8;
+}
 
 // Work item of a planned launch: row, first edge, one-past-last edge, partial slot (kNoSlot = the
 // item is a whole row and writes `out` directly).
@@ -112,7 +118,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
                                                         int accumulate, HeadArgs heads, uint32_t row_edge_limit,
                                                         const uint32_t *__restrict__ edge_ids) {
   using V = typename Vec<VEC>::type;
-  constexpr int U = unroll_for(NACC);
+  constexpr int U = unroll_for(NACC, VEC);
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t item = blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
   if (item >= n_items) return;
