@@ -38,7 +38,7 @@ HBM_PEAK_GBS = 8000.0
 # Bytes per launch of the F=602 gather kernel that cross the L2 <-> fabric boundary, from rocprofv3
 # FETCH_SIZE (x1.986 calibration) + WRITE_SIZE at the default schedule
 # (profiles/spmm_wave_f602_reddit_shaped_pmc.txt).  Reported only for the configuration it was measured on.
-TRAFFIC_BYTES_F602 = 43_126_634_100
+TRAFFIC_BYTES_F602 = 44_601_740_400
 TRAFFIC_MEASURED_AT = dict(vertices=V_REDDIT, edges=E_REDDIT, chunk=512, slabs=32)
 
 
