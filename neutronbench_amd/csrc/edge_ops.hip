@@ -495,6 +495,13 @@ __device__ __forceinline__ float head_reduce(float v, uint32_t H) {
 
 __device__ __forceinline__ float leaky(float s, float slope) { return s > 0.f ? s : s * slope; }
 
+// exp for the softmax kernels: the hardware's 2^x of x * log2(e), two instructions instead of the
+// fourteen of the correctly rounded library routine -- these kernels are bound by their vector
+// instructions for short segments.  Arguments are <= 0 (a value minus its segment's maximum); the
+// product's rounding puts the relative error at |x| * 6e-8 (1e-6 at x = -20, where the result is
+// 2e-9 of the segment's largest term), well inside the 1e-4 these operators are held to.
+__device__ __forceinline__ float softmax_exp(float x) { return __expf(x); }
+
 // Multi-pass softmax forward of one segment with 16-byte lanes (H a multiple of 4, 16-byte aligned
 // arrays): lane l of a group of WIDTH threads takes the vectors l, l + WIDTH, ... of the segment, i.e.
 // four consecutive values = heads (4 l mod H) .. +3 of one edge, so a pass needs a quarter of the load
@@ -513,14 +520,14 @@ __device__ __forceinline__ void strided_max_sum_pass4(uint64_t first, uint64_t n
     }
     float add[4] = {0.f, 0.f, 0.f, 0.f};
     for (int u = 0; u < count; ++u) {
-      add[0] += expf(v[u].x - m[0]);
-      add[1] += expf(v[u].y - m[1]);
-      add[2] += expf(v[u].z - m[2]);
-      add[3] += expf(v[u].w - m[3]);
+      add[0] += softmax_exp(v[u].x - m[0]);
+      add[1] += softmax_exp(v[u].y - m[1]);
+      add[2] += softmax_exp(v[u].z - m[2]);
+      add[3] += softmax_exp(v[u].w - m[3]);
     }
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      sum[c] = sum[c] * expf(mx[c] - m[c]) + add[c];  // mx = -inf at the start: the old sum is 0 and stays 0
+      sum[c] = sum[c] * softmax_exp(mx[c] - m[c]) + add[c];  // mx = -inf at the start: the old sum is 0 and stays 0
       mx[c] = m[c];
     }
   };
@@ -591,15 +598,15 @@ __device__ __forceinline__ void strided_max_sum_pass(uint64_t first, uint64_t n,
     }
     float add = 0.f;
 #pragma unroll
-    for (int u = 0; u < U; ++u) add += expf(v[u] - m);
-    sum = sum * expf(mx - m) + add;  // mx = -inf at the start: the old sum is 0 and stays 0
+    for (int u = 0; u < U; ++u) add += softmax_exp(v[u] - m);
+    sum = sum * softmax_exp(mx - m) + add;  // mx = -inf at the start: the old sum is 0 and stays 0
     mx = m;
   }
   for (; i < n; i += stride) {
     const float v = load(i);
     seen(i, v);
     const float m = fmaxf(mx, v);
-    sum = sum * expf(mx - m) + expf(v - m);
+    sum = sum * softmax_exp(mx - m) + softmax_exp(v - m);
     mx = m;
   }
 }
@@ -644,7 +651,7 @@ __device__ __forceinline__ void softmax_fwd_regs(float *__restrict__ ys, const f
   float sum = 0.f;
 #pragma unroll
   for (int k = 0; k < K; ++k) {
-    v[k] = (gl + WIDTH * k < n) ? expf(v[k] - mx) : 0.f;
+    v[k] = (gl + WIDTH * k < n) ? softmax_exp(v[k] - mx) : 0.f;
     sum += v[k];
   }
   sum = head_reduce_w<1, WIDTH>(sum, H);
@@ -840,13 +847,13 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
           for (int c = 0; c < 4; ++c) {
             const float lane_mx = mx4[c];
             mx4[c] = head_reduce<0>(mx4[c], hq);
-            sum4[c] = head_reduce<1>(sum4[c] * expf(lane_mx - mx4[c]), hq);
+            sum4[c] = head_reduce<1>(sum4[c] * softmax_exp(lane_mx - mx4[c]), hq);
             inv4[c] = 1.f / sum4[c];
           }
           strided_pass<4>(lane, n / 4, kWave, [&](uint64_t i) -> float4 { return FUSED ? ys4[i] : xs4[i]; },
                           [&](uint64_t i, float4 sc) {
-                            ys4[i] = make_float4(expf(sc.x - mx4[0]) * inv4[0], expf(sc.y - mx4[1]) * inv4[1],
-                                                 expf(sc.z - mx4[2]) * inv4[2], expf(sc.w - mx4[3]) * inv4[3]);
+                            ys4[i] = make_float4(softmax_exp(sc.x - mx4[0]) * inv4[0], softmax_exp(sc.y - mx4[1]) * inv4[1],
+                                                 softmax_exp(sc.z - mx4[2]) * inv4[2], softmax_exp(sc.w - mx4[3]) * inv4[3]);
                           });
           continue;
         }
@@ -868,10 +875,10 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
         // every lane's pair is brought to the head's maximum before the sums are added
         const float lane_mx = mx;
         mx = head_reduce<0>(mx, H);
-        sum = head_reduce<1>(sum * expf(lane_mx - mx), H);
+        sum = head_reduce<1>(sum * softmax_exp(lane_mx - mx), H);
         const float inv = 1.f / sum;
         strided_pass<8>(lane, n, kWave, [&](uint64_t i) -> float { return FUSED ? ys[i] : xs[i]; },
-                        [&](uint64_t i, float sc) { ys[i] = expf(sc - mx) * inv; });
+                        [&](uint64_t i, float sc) { ys[i] = softmax_exp(sc - mx) * inv; });
       } else {
         const uint32_t deg = e1 - e0;
         for (uint32_t h = 0; h < H; ++h) {
@@ -893,13 +900,13 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
           float sum = 0.f;
           for (uint32_t k = lane; k < deg; k += kWave) {
             const float sc = FUSED ? ys[static_cast<size_t>(k) * H + h] : xs[static_cast<size_t>(k) * H + h];
-            sum += expf(sc - mx);
+            sum += softmax_exp(sc - mx);
           }
           sum = group_sum<kWave>(sum);
           const float inv = 1.f / sum;
           for (uint32_t k = lane; k < deg; k += kWave) {
             const float sc = FUSED ? ys[static_cast<size_t>(k) * H + h] : xs[static_cast<size_t>(k) * H + h];
-            ys[static_cast<size_t>(k) * H + h] = expf(sc - mx) * inv;
+            ys[static_cast<size_t>(k) * H + h] = softmax_exp(sc - mx) * inv;
           }
         }
       }
@@ -1097,10 +1104,10 @@ __global__ __launch_bounds__(kLongBlock) void edge_softmax_fwd_long_kernel(
         mx, sum);
     const float thread_mx = mx;
     mx = block_head_reduce<0>(mx, H, red);
-    sum = block_head_reduce<1>(sum * expf(thread_mx - mx), H, red);
+    sum = block_head_reduce<1>(sum * softmax_exp(thread_mx - mx), H, red);
     const float inv = 1.f / sum;
     strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
-                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) * inv; });
+                    [&](uint64_t j, float sc) { ys[j] = softmax_exp(sc - mx) * inv; });
   }
 }
 
@@ -1186,7 +1193,7 @@ __global__ __launch_bounds__(kLongBlock) void giant_softmax_stats_kernel(
     mx = block_head_reduce<0>(mx, H, red);
     float sum = 0.f;
     strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return FUSED ? ys[j] : xs[j]; },
-                    [&](uint64_t, float sc) { sum += expf(sc - mx); });
+                    [&](uint64_t, float sc) { sum += softmax_exp(sc - mx); });
     sum = block_head_reduce<1>(sum, H, red);
     if (threadIdx.x < H) {
       stats[static_cast<size_t>(p) * 2 * H + threadIdx.x] = mx;
@@ -1216,7 +1223,7 @@ __global__ __launch_bounds__(64) void giant_softmax_combine_kernel(float *__rest
       for (uint32_t p = p0; p < p1; ++p) m = fmaxf(m, stats[static_cast<size_t>(p) * width + h]);
       float sum = 0.f;
       for (uint32_t p = p0; p < p1; ++p)
-        sum += stats[static_cast<size_t>(p) * width + H + h] * expf(stats[static_cast<size_t>(p) * width + h] - m);
+        sum += stats[static_cast<size_t>(p) * width + H + h] * softmax_exp(stats[static_cast<size_t>(p) * width + h] - m);
       rowstat[static_cast<size_t>(i) * 2 * H + h] = m;
       rowstat[static_cast<size_t>(i) * 2 * H + H + h] = sum;
     } else {
@@ -1247,7 +1254,7 @@ __global__ __launch_bounds__(kLongBlock) void giant_softmax_apply_kernel(float *
     const float *xs = FUSED ? ys : x + base;  // the fused forward left the raw score in y
     const float inv = 1.f / sum;
     strided_pass<8>(threadIdx.x, n, kLongBlock, [&](uint64_t j) -> float { return xs[j]; },
-                    [&](uint64_t j, float sc) { ys[j] = expf(sc - mx) * inv; });
+                    [&](uint64_t j, float sc) { ys[j] = softmax_exp(sc - mx) * inv; });
   }
 }
 
