@@ -295,18 +295,26 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
   const uint32_t head = HEADS ? lcol / heads.Fh : 0u;
   V acc = vzero<VEC>();
 
+  // The (index, weight) pairs of the next G edges are requested while the current ones are used, so
+  // that a group does not wait for them at the start of every tile.
+  auto fetch_pair = [&](uint32_t e, uint32_t &pi, uint32_t &ps) {
+    pi = 0;
+    ps = HEADS ? 0u : __float_as_uint(1.f);  // weight bits, or the edge's id in alpha's order
+    if (e < e1) {
+      pi = indices[e] - index_base;
+      const uint32_t id = REMAP ? edge_ids[e] : e;
+      if (HEADS)
+        ps = heads.perm ? heads.perm[id] : id;
+      else if (w)
+        ps = __float_as_uint(w[id]);
+    }
+  };
+  uint32_t nxt_i, nxt_s;
+  fetch_pair(e0 + gl, nxt_i, nxt_s);
   for (uint32_t eb = e0; eb < e1; eb += G) {
     const uint32_t n = min(static_cast<uint32_t>(G), e1 - eb);
-    uint32_t my_i = 0;
-    uint32_t my_s = HEADS ? 0u : __float_as_uint(1.f);  // weight bits, or the edge's id in alpha's order
-    if (gl < n) {
-      my_i = indices[eb + gl] - index_base;
-      const uint32_t id = REMAP ? edge_ids[eb + gl] : eb + gl;
-      if (HEADS)
-        my_s = heads.perm ? heads.perm[id] : id;
-      else if (w)
-        my_s = __float_as_uint(w[id]);
-    }
+    const uint32_t my_i = nxt_i, my_s = nxt_s;
+    fetch_pair(eb + G + gl, nxt_i, nxt_s);
     uint32_t j = 0;
     for (; j + U <= n; j += U) {
       uint32_t si[U];
