@@ -146,6 +146,23 @@ int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t 
                     const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
                     uint32_t F, int accumulate, nts_stream_t stream);
 
+/* nts_spmm_gather for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments, same kernels and bit-identical results; the scratch of calls that cut long rows
+ * lives in a fixed array inside the library's code object (NTS_SPMM_STATIC_SCRATCH_BYTES, held by
+ * every device that loads the library until the process ends) instead of the stream-ordered pool.
+ * The call itself allocates and frees nothing (the first call on a device looks the array's address
+ * up once; do that call before a capture).  A call whose scratch, by the formula given with
+ * nts_spmm_gather plus the scan / sort work area, exceeds the array returns NTS_ERR_INVALID with
+ * both sizes in nts_last_error() and launches nothing; calls below 65,536 edges need no scratch.
+ * Every call on a device uses the same array: calls that overlap on one device (two streams, two
+ * host threads) race, so a caller serialises them.  Nothing in the array has to be zero on entry:
+ * each call writes every word before it reads it. */
+#define NTS_SPMM_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int nts_spmm_gather_static_scratch(const float *in, float *out, const float *w, const uint32_t *offsets,
+                                   const uint32_t *indices, uint32_t index_base, uint32_t rows,
+                                   uint32_t edges, uint32_t F, int accumulate, nts_stream_t stream);
+
 /* Degree-bucketed schedule for a fixed offsets array (full-graph chunks: CSC_segment_pinned,
  * core/GraphSegment.h:54-133).  Rows are ordered by descending degree class; rows longer than
  * `chunk_edges` are split into chunks whose partial sums are combined by a second kernel in a

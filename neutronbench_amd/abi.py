@@ -53,6 +53,7 @@ SIGNATURES = {
     "nts_event_elapsed_ms": [ctypes.POINTER(_f32), _vp, _vp],
     "nts_spmm_plan_set_events": [_vp, _vp, _vp],
     "nts_spmm_gather": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
+    "nts_spmm_gather_static_scratch": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
     "nts_spmm_plan_create": [ctypes.POINTER(_vp), _vp, _u32, _u32, _u32, _vp],
     "nts_spmm_plan_create_slabs": [ctypes.POINTER(_vp), _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _vp],
     "nts_spmm_plan_schedule_host": [_vp, _vp, _u32, _u32, _u32, _u32, _vp, _u64, ctypes.POINTER(_u32),

@@ -25,14 +25,42 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <new>
 #include <thread>
 #include <vector>
 
 #include "common.hpp"
 
+// Fixed scratch of nts_spmm_gather_static_scratch, the entry point for callers that must not allocate:
+// each device that loads this library holds one copy of the array until the process ends.  Host code
+// never passes the array's name to a kernel (on the host the name is only a stand-in for the symbol):
+// its device address is looked up once per device and kept in g_static_scratch_ptr.
+constexpr size_t kStaticScratchBytes = NTS_SPMM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace nts {
 namespace {
+
+constexpr int kMaxScratchDevices = 64;
+std::mutex g_static_scratch_mutex;
+unsigned char *g_static_scratch_ptr[kMaxScratchDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch_address(unsigned char **out) {
+  int dev = -1;
+  NTS_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxScratchDevices) return fail(NTS_ERR_INVALID, "static scratch: device ordinal out of range");
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (!g_static_scratch_ptr[dev]) {
+    unsigned char *p = nullptr;
+    NTS_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+    if (!p) return fail(NTS_ERR_HIP, "static scratch: hipGetSymbolAddress returned a null address");
+    g_static_scratch_ptr[dev] = p;
+  }
+  *out = g_static_scratch_ptr[dev];
+  return NTS_OK;
+}
 
 template <int VEC>
 struct Vec;
@@ -720,8 +748,10 @@ __global__ __launch_bounds__(256) void auto_reduce_wide_kernel(float *__restrict
 
 inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 
-// `a` describes the whole-row launch (a.n_items = rows, no items).
-int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
+// `a` describes the whole-row launch (a.n_items = rows, no items).  Scratch comes from the library's
+// stream-ordered pool, or, when `fixed` is set, from that caller-held region of `fixed_cap` bytes
+// (nothing is allocated or freed then; a call that needs more is refused).
+int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nullptr, size_t fixed_cap = 0) {
   const uint32_t rows = a.n_items;
   if (edges < kAutoMinEdges) {
     launch_spmm(a);
@@ -744,9 +774,18 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
   const size_t n_items_b = up256(static_cast<size_t>(p_max) * sizeof(Item));
   const size_t n_keys_b = up256(static_cast<size_t>(p_max) * sizeof(uint32_t));
   const size_t n_partial = up256(static_cast<size_t>(p_max) * a.F * sizeof(float));
-  unsigned char *buf = nullptr;
-  NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&buf),
-                             2 * n_off + 2 * n_items_b + 3 * n_keys_b + tmp_bytes + n_partial, a.stream));
+  const size_t need = 2 * n_off + 2 * n_items_b + 3 * n_keys_b + tmp_bytes + n_partial;
+  unsigned char *buf = fixed;
+  if (fixed) {
+    if (need > fixed_cap) {
+      char msg[200];
+      snprintf(msg, sizeof msg, "spmm: the call needs %zu bytes of scratch, the fixed scratch holds %zu", need,
+               fixed_cap);
+      return fail(NTS_ERR_INVALID, msg);
+    }
+  } else {
+    NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&buf), need, a.stream));
+  }
   unsigned char *cursor = buf;
   auto take = [&cursor](size_t bytes) {
     unsigned char *p = cursor;
@@ -763,7 +802,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
   void *tmp = take(tmp_bytes);
   float *partial = reinterpret_cast<float *>(take(n_partial));
   auto bail = [&](hipError_t err, const char *what) {
-    (void)scratch_free(buf, a.stream);
+    if (!fixed) (void)scratch_free(buf, a.stream);
     return fail_hip(err, what);
   };
   hipLaunchKernelGGL(auto_count_kernel, dim3(ceil_div(static_cast<uint64_t>(rows) + 1, 256)), dim3(256), 0, a.stream,
@@ -810,7 +849,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges) {
 #undef NTS_AUTO_REDUCE_WIDE
   err = hipGetLastError();
   if (err != hipSuccess) return bail(err, "spmm: balanced launch");
-  NTS_HIP_TRY(scratch_free(buf, a.stream));
+  if (!fixed) NTS_HIP_TRY(scratch_free(buf, a.stream));
   return NTS_OK;
 }
 
@@ -875,6 +914,22 @@ int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t 
   nts::LaunchArgs a{in, out, w, offsets, indices, index_base, rows, F, nullptr, nullptr, accumulate, stream};
   if (int rc = nts::launch_spmm_balanced(a, edges)) return rc;
   NTS_LAUNCH_CHECK("nts_spmm_gather");
+  return NTS_OK;
+}
+
+int nts_spmm_gather_static_scratch(const float *in, float *out, const float *w, const uint32_t *offsets,
+                                   const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
+                                   uint32_t F, int accumulate, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_gather_static_scratch");
+  if (int rc = nts::check_common(in, out, offsets, indices, rows, edges, F,
+                                 "nts_spmm_gather_static_scratch: null pointer"))
+    return rc;
+  if (rows == 0) return NTS_OK;
+  unsigned char *fixed = nullptr;
+  if (int rc = nts::static_scratch_address(&fixed)) return rc;
+  nts::LaunchArgs a{in, out, w, offsets, indices, index_base, rows, F, nullptr, nullptr, accumulate, stream};
+  if (int rc = nts::launch_spmm_balanced(a, edges, fixed, kStaticScratchBytes)) return rc;
+  NTS_LAUNCH_CHECK("nts_spmm_gather_static_scratch");
   return NTS_OK;
 }
 
