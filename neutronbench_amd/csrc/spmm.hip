@@ -677,11 +677,13 @@ __global__ __launch_bounds__(256) void auto_order_items_kernel(Item *__restrict_
 __global__ __launch_bounds__(256) void auto_reduce_kernel(float *__restrict__ out, const float *__restrict__ partial,
                                                           const Item *__restrict__ items,
                                                           const uint32_t *__restrict__ base, uint32_t F,
-                                                          int accumulate) {
+                                                          int accumulate, uint32_t p_max) {
   const uint32_t i = blockIdx.x;
   const uint32_t r = items[i].x;
   if (base[r] != i) return;
-  const uint32_t n = base[r + 1] - i;
+  // Slots at or beyond p_max were never written (only possible when the caller's edge count is
+  // smaller than offsets[rows]): they are not read.
+  const uint32_t n = min(base[r + 1], p_max) - i;
   if (n == 0) return;
   const uint32_t c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= F) return;
@@ -708,11 +710,11 @@ __global__ __launch_bounds__(256) void auto_reduce_wide_kernel(float *__restrict
                                                                const float *__restrict__ partial,
                                                                const Item *__restrict__ items,
                                                                const uint32_t *__restrict__ base, uint32_t F,
-                                                               int accumulate) {
+                                                               int accumulate, uint32_t p_max) {
   const uint32_t i = blockIdx.x;
   const uint32_t r = items[i].x;
   if (base[r] != i) return;
-  const uint32_t n = base[r + 1] - i;
+  const uint32_t n = min(base[r + 1], p_max) - i;  // as in auto_reduce_kernel
   if (n == 0) return;
   const float *src = partial + static_cast<size_t>(i) * F;
   uint32_t c[J];
@@ -836,7 +838,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
   launch_spmm(whole);
 #define NTS_AUTO_REDUCE_WIDE(J)                                                                                     \
   hipLaunchKernelGGL(auto_reduce_wide_kernel<J>, dim3(p_max), dim3(256), 0, a.stream, a.out, partial, items, base, a.F, \
-                     a.accumulate)
+                     a.accumulate, p_max)
   if (a.F > 256 && a.F <= 512)
     NTS_AUTO_REDUCE_WIDE(2);
   else if (a.F > 512 && a.F <= 768)
@@ -845,7 +847,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
     NTS_AUTO_REDUCE_WIDE(4);
   else
     hipLaunchKernelGGL(auto_reduce_kernel, dim3(p_max, ceil_div(a.F, 256)), dim3(256), 0, a.stream, a.out, partial, items,
-                       base, a.F, a.accumulate);
+                       base, a.F, a.accumulate, p_max);
 #undef NTS_AUTO_REDUCE_WIDE
   err = hipGetLastError();
   if (err != hipSuccess) return bail(err, "spmm: balanced launch");
