@@ -4,7 +4,10 @@ aggregate backward.  Dense layers are not part of this library and are left out.
 
     python -m neutronbench_amd.epoch --config arxiv|products|gat [--scale S]
 
-Configurations (BASELINE.json configs 2, 4, 5):
+Configurations (BASELINE.json configs 2, 4, 5).  Fanouts are listed in hop order, the batch's own hop
+first: the reference reverses its FANOUT string ("10,25" for the first one) and gives entry i to hop i
+(toolkits/GCN_GPU_NEIGHBOR.hpp:126-130, core/ntsSampler.hpp:857-921), so the batch's hop takes the
+largest fanout:
   arxiv     169,343 nodes, 2.48M R-MAT edges, 128 features, fanout [25,10], batch 1,024, 90,941 train nodes
   products  2,449,029 nodes, 126.2M R-MAT edges, 100 features in mapped pinned host memory, HBM cache of the
             top 20 % out-degree nodes, fanout [15,10,5], batch 6,000, 196,615 train nodes
@@ -35,9 +38,9 @@ from .ops import GATAggregateOp, GATAttentionOp, SingleGPUSampleGraphOp
 from .stream import CudaStream
 
 CONFIGS = {
-    "arxiv": dict(V=169_343, E=2_480_000, F=128, hidden=128, classes=40, fanout=[10, 25], batch=1024, train=90_941,
+    "arxiv": dict(V=169_343, E=2_480_000, F=128, hidden=128, classes=40, fanout=[25, 10], batch=1024, train=90_941,
                   seed=2, cache=0.0),
-    "products": dict(V=2_449_029, E=126_200_000, F=100, hidden=128, classes=47, fanout=[5, 10, 15], batch=6000,
+    "products": dict(V=2_449_029, E=126_200_000, F=100, hidden=128, classes=47, fanout=[15, 10, 5], batch=6000,
                      train=196_615, seed=4, cache=0.2),
     "gat": dict(V=2_449_029, E=126_200_000, F=100, hidden=128, classes=47, fanout=[10, 10], batch=4096, train=196_615,
                 seed=4, cache=0.2, heads=4),

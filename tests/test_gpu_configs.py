@@ -76,14 +76,15 @@ def test_config1_cora_shaped_full_graph(device):
 
 
 def test_config2_arxiv_shaped_minibatch(device):
-    """169,343-node, 2.48M-edge R-MAT graph, 128 features, fanout [25,10] (output-side hop 10),
+    """169,343-node, 2.48M-edge R-MAT graph, 128 features, fanout [25,10] (the batch's own hop 25, as the
+    reference's reversed FANOUT string "10,25" gives it),
     batch 1,024: sampled-layer construction bit-exact, feature/label gather bit-exact, aggregation
     forward and backward of both layers against MiniBatchFuseOp's arithmetic."""
     V, E, F = 169_343, 2_480_000, 128
     src, dst = synth.rmat_edges(V, E, seed=2)
     co, ri = synth.build_csc(src, dst, V)
     batch = synth.permutation(V, 22)[:1024]
-    hops = _sample_batch(co, ri, V, batch, [10, 25], seed=22)
+    hops = _sample_batch(co, ri, V, batch, [25, 10], seed=22)
     feat = synth.normal_features(V, F, seed=23).numpy()
     labels = synth.uniform_labels(V, 40, seed=24).numpy()
     layers = [SampledLayer.from_host_csc(*(torch.from_numpy(h[k].astype(np.int64)) for k in
@@ -203,7 +204,7 @@ def test_config4_products_shaped_cached_gather(device):
     co, ri = co.cpu(), ri.cpu()
     del src, dst
     batch = synth.permutation(V, 44)[:6000]
-    hops = _sample_batch(co, ri, V, batch, [5, 10, 15], seed=44)
+    hops = _sample_batch(co, ri, V, batch, [15, 10, 5], seed=44)
     feat_t = synth.normal_features(V, F, seed=45)
     feat = feat_t.numpy()
     n_cache = V // 5
