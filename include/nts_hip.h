@@ -201,12 +201,25 @@ int nts_spmm_plan_destroy(nts_spmm_plan_t *plan);
 /* Number of work items, split rows and partial-sum slots of a plan (for tests and reports). */
 int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows,
                        uint32_t *partials);
-/* Grow the plan's partial-sum scratch so that widths up to F need no allocation later. */
+/* Grow the plan's scratch (partial sums of split rows; for a schedule with runs of equal indices
+ * also a copy of the input with padded rows, see below) so that a later call of width F allocates
+ * nothing. */
 int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F);
 /* NtsScheduler::GatherByDstFromSrc / GatherBySrcFromDst on a full-graph chunk
  * (core/NtsScheduler.hpp:146-178, 239-271; core/graph.hpp:3432-3478).  `offsets` must be the
- * array the plan was built from.  A plan must not be used by two streams at the same time (its
- * scratch is shared). */
+ * array the plan was built from.
+ * Parallel edges.  When at least 1 edge in 20 repeats the gather index of the edge before it (a
+ * multigraph with sorted rows; nts_spmm_plan_create_slabs counts them), the call loads a source row
+ * once per run of equal indices and still adds it once per edge, with that edge's weight and in edge
+ * order, so every sum keeps its bits.  Such a schedule also gathers rows that are wider than 128
+ * floats and not a multiple of four floats wide from a copy of `in` whose rows are padded to whole
+ * 128-byte lines (made by the call, in the plan's scratch, n_index * 4 * ceil(F / 32) * 32 bytes), so
+ * that the row loads are 16 bytes per lane.
+ * Concurrency.  A plan's scratch is shared by all calls on it.  The host side of a call is
+ * serialised per plan, and a call on another stream than the previous one first waits, on the
+ * device, for that call's last kernel; calls on one plan therefore never overlap on the device,
+ * from however many streams or host threads they come (use one plan per stream for overlap).  The
+ * caller must not destroy a plan while a call on it is being made. */
 int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *w,
                             const uint32_t *offsets, const uint32_t *indices, uint32_t index_base,
                             uint32_t F, int accumulate, nts_stream_t stream);

@@ -136,7 +136,7 @@ struct HeadArgs {
   uint32_t Fh;
 };
 
-template <int VEC, int NACC, bool LDS_TILE, bool HEADS, bool REMAP>
+template <int VEC, int NACC, bool LDS_TILE, bool HEADS, bool REMAP, bool RUNS>
 __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                         const float *__restrict__ w,
                                                         const uint32_t *__restrict__ offsets,
@@ -144,7 +144,8 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
                                                         uint32_t n_items, uint32_t F, uint32_t col_base,
                                                         const Item *__restrict__ items, float *__restrict__ partial,
                                                         int accumulate, HeadArgs heads, uint32_t row_edge_limit,
-                                                        const uint32_t *__restrict__ edge_ids) {
+                                                        const uint32_t *__restrict__ edge_ids, uint32_t in_ld,
+                                                        uint32_t partial_ld, int out_scalar) {
   using V = typename Vec<VEC>::type;
   constexpr int U = unroll_for(NACC, VEC);
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -177,7 +178,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
   for (int k = 0; k < NACC; ++k) {
     col[k] = col_base + (lane + kWave * k) * VEC;
     live[k] = col[k] < F;
-    lcol[k] = live[k] ? col[k] : F - VEC;
+    lcol[k] = live[k] ? col[k] : in_ld - VEC;
     head[k] = HEADS ? lcol[k] / heads.Fh : 0u;
     acc[k] = vzero<VEC>();
   }
@@ -231,6 +232,48 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
         second = wave_read(my_s, j);
       }
     };
+    if (RUNS && LDS_TILE && !HEADS) {
+      // Runs of consecutive edges with the same neighbour (a multigraph's parallel edges, adjacent in
+      // sorted rows): the row is loaded once and added once per edge of the run, in edge order with
+      // each edge's own weight, so the result is the same bit for bit.  Up to U runs per step.
+      const uint32_t prev = tile[lane ? lane - 1 : 0].x;
+      uint64_t starts = __ballot(lane < n && (lane == 0 || my_i != prev));
+      while (starts) {
+        uint32_t rs[U + 1];
+        int nr = 0;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          rs[u] = n;
+          if (starts) {
+            rs[u] = static_cast<uint32_t>(__builtin_ctzll(starts));
+            starts &= starts - 1;
+            nr = u + 1;
+          }
+        }
+        rs[U] = starts ? static_cast<uint32_t>(__builtin_ctzll(starts)) : n;
+        V v[U][NACC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (u < nr) {
+            const float *src = in + static_cast<size_t>(wave_first(tile[rs[u]].x)) * in_ld;
+#pragma unroll
+            for (int k = 0; k < NACC; ++k) v[u][k] = *reinterpret_cast<const V *>(src + lcol[k]);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (u < nr) {
+            const uint32_t end = (u + 1 < U) ? rs[u + 1] : rs[U];
+            for (uint32_t q = rs[u]; q < end; ++q) {
+              const float wgt = __uint_as_float(wave_first(tile[q].y));
+#pragma unroll
+              for (int k = 0; k < NACC; ++k) vfma(acc[k], v[u][k], wgt);
+            }
+          }
+        }
+      }
+      continue;
+    }
     uint32_t j = 0;
     for (; j + U <= n; j += U) {
       const float *src[U];
@@ -239,7 +282,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
       for (int u = 0; u < U; ++u) {
         uint32_t si;
         pair_at(j + u, si, ss[u]);
-        src[u] = in + static_cast<size_t>(si) * F;
+        src[u] = in + static_cast<size_t>(si) * in_ld;
       }
       V v[U][NACC];
       float wv[U][HEADS ? NACC : 1];
@@ -263,7 +306,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
     for (; j < n; ++j) {
       uint32_t si, ss;
       pair_at(j, si, ss);
-      const float *src = in + static_cast<size_t>(si) * F;
+      const float *src = in + static_cast<size_t>(si) * in_ld;
 #pragma unroll
       for (int k = 0; k < NACC; ++k) {
         const float wgt = HEADS ? w[static_cast<size_t>(ss) * heads.H + head[k]] : __uint_as_float(ss);
@@ -272,7 +315,23 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
     }
   }
 
-  float *dst = (slot == kNoSlot) ? out + static_cast<size_t>(row) * F : partial + static_cast<size_t>(slot) * F;
+  if (VEC > 1 && out_scalar && slot == kNoSlot) {
+    // Output rows that do not start on a 16-byte boundary (F not a multiple of four while the gather
+    // runs over a padded copy of the input): the row is stored one float at a time.
+    float *dst = out + static_cast<size_t>(row) * F;
+#pragma unroll
+    for (int k = 0; k < NACC; ++k) {
+      const float *r = reinterpret_cast<const float *>(&acc[k]);
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) {
+        const uint32_t cc = col[k] + c;
+        if (cc < F) dst[cc] = accumulate ? r[c] + dst[cc] : r[c];
+      }
+    }
+    return;
+  }
+  float *dst =
+      (slot == kNoSlot) ? out + static_cast<size_t>(row) * F : partial + static_cast<size_t>(slot) * partial_ld;
   const bool add = accumulate && slot == kNoSlot;
 #pragma unroll
   for (int k = 0; k < NACC; ++k) {
@@ -388,21 +447,21 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
 __global__ __launch_bounds__(256) void spmm_reduce_partials_kernel(float *__restrict__ out,
                                                                    const float *__restrict__ partial,
                                                                    const uint4 *__restrict__ splits, uint32_t F,
-                                                                   int accumulate) {
+                                                                   int accumulate, uint32_t ld) {
   const uint4 s = splits[blockIdx.x];
   const uint32_t c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= F) return;
-  const float *src = partial + static_cast<size_t>(s.y) * F + c;
+  const float *src = partial + static_cast<size_t>(s.y) * ld + c;
   float a = src[0];
   uint32_t k = 1;
   for (; k + 8 <= s.z; k += 8) {
     float v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = src[static_cast<size_t>(k + u) * F];
+    for (int u = 0; u < 8; ++u) v[u] = src[static_cast<size_t>(k + u) * ld];
 #pragma unroll
     for (int u = 0; u < 8; ++u) a += v[u];
   }
-  for (; k < s.z; ++k) a += src[static_cast<size_t>(k) * F];
+  for (; k < s.z; ++k) a += src[static_cast<size_t>(k) * ld];
   float *dst = out + static_cast<size_t>(s.x) * F + c;
   if (accumulate) a += *dst;
   *dst = a;
@@ -414,9 +473,9 @@ template <int J>
 __global__ __launch_bounds__(256) void spmm_reduce_partials_wide_kernel(float *__restrict__ out,
                                                                         const float *__restrict__ partial,
                                                                         const uint4 *__restrict__ splits, uint32_t F,
-                                                                        int accumulate) {
+                                                                        int accumulate, uint32_t ld) {
   const uint4 s = splits[blockIdx.x];
-  const float *src = partial + static_cast<size_t>(s.y) * F;
+  const float *src = partial + static_cast<size_t>(s.y) * ld;
   uint32_t c[J];
   bool live[J];
   float a[J];
@@ -433,7 +492,7 @@ __global__ __launch_bounds__(256) void spmm_reduce_partials_wide_kernel(float *_
 #pragma unroll
     for (int u = 0; u < 8; ++u)
 #pragma unroll
-      for (int j = 0; j < J; ++j) v[u][j] = src[static_cast<size_t>(k + u) * F + c[j]];
+      for (int j = 0; j < J; ++j) v[u][j] = src[static_cast<size_t>(k + u) * ld + c[j]];
 #pragma unroll
     for (int u = 0; u < 8; ++u)
 #pragma unroll
@@ -444,7 +503,7 @@ __global__ __launch_bounds__(256) void spmm_reduce_partials_wide_kernel(float *_
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int j = 0; j < J; ++j) v[u][j] = src[static_cast<size_t>(k + u) * F + c[j]];
+      for (int j = 0; j < J; ++j) v[u][j] = src[static_cast<size_t>(k + u) * ld + c[j]];
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -452,7 +511,7 @@ __global__ __launch_bounds__(256) void spmm_reduce_partials_wide_kernel(float *_
   }
   for (; k < s.z; ++k)
 #pragma unroll
-    for (int j = 0; j < J; ++j) a[j] += src[static_cast<size_t>(k) * F + c[j]];
+    for (int j = 0; j < J; ++j) a[j] += src[static_cast<size_t>(k) * ld + c[j]];
   float *dst = out + static_cast<size_t>(s.x) * F;
 #pragma unroll
   for (int j = 0; j < J; ++j)
@@ -461,12 +520,13 @@ __global__ __launch_bounds__(256) void spmm_reduce_partials_wide_kernel(float *_
 
 // Launches the second stage for a plan's split rows.
 inline void launch_reduce_partials(float *out, const float *partial, const uint4 *splits, uint32_t n_splits, uint32_t F,
-                                   int accumulate, hipStream_t stream) {
+                                   int accumulate, hipStream_t stream, uint32_t ld = 0) {
+  if (!ld) ld = F;  // row stride of the partial sums
   // Up to 1,024 columns one block adds whole rows (contiguous reads: 29.6 -> 29.2 ms per step on the
   // Reddit-shaped F=602 workload); wider rows are tiled 256 columns per block.
 #define NTS_REDUCE_WIDE(J)                                                                                          \
   hipLaunchKernelGGL(spmm_reduce_partials_wide_kernel<J>, dim3(n_splits), dim3(256), 0, stream, out, partial, splits, \
-                     F, accumulate)
+                     F, accumulate, ld)
   if (F > 256 && F <= 512)
     NTS_REDUCE_WIDE(2);
   else if (F > 512 && F <= 768)
@@ -475,8 +535,29 @@ inline void launch_reduce_partials(float *out, const float *partial, const uint4
     NTS_REDUCE_WIDE(4);
   else
     hipLaunchKernelGGL(spmm_reduce_partials_kernel, dim3(n_splits, ceil_div(F, 256)), dim3(256), 0, stream, out, partial,
-                       splits, F, accumulate);
+                       splits, F, accumulate, ld);
 #undef NTS_REDUCE_WIDE
+}
+
+// Copy of a [rows, F] matrix with the row stride padded to `ld` floats (a multiple of four; the pad
+// columns are zero), so that every row starts on a 16-byte boundary and the gather can use 16-byte
+// lanes.  One thread per 16 bytes written.
+__global__ __launch_bounds__(256) void pad_rows_kernel(float4 *__restrict__ dst, const float *__restrict__ src,
+                                                       uint32_t rows, uint32_t F, uint32_t ld) {
+  const uint32_t per_row = ld / 4;
+  const uint64_t total = static_cast<uint64_t>(rows) * per_row;
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+       i += static_cast<uint64_t>(gridDim.x) * blockDim.x) {
+    const uint32_t r = static_cast<uint32_t>(i / per_row);
+    const uint32_t c = static_cast<uint32_t>(i % per_row) * 4;
+    const float *p = src + static_cast<size_t>(r) * F + c;
+    float4 v;
+    v.x = c + 0 < F ? p[0] : 0.f;
+    v.y = c + 1 < F ? p[1] : 0.f;
+    v.z = c + 2 < F ? p[2] : 0.f;
+    v.w = c + 3 < F ? p[3] : 0.f;
+    dst[i] = v;
+  }
 }
 
 struct LaunchArgs {
@@ -495,41 +576,32 @@ struct LaunchArgs {
   HeadArgs heads = HeadArgs{nullptr, 0u, 0u};  // H == 0: one weight per edge
   uint32_t row_edge_limit = 0xFFFFFFFFu;       // whole-row launches skip rows with more edges than this
   const uint32_t *edge_ids = nullptr;          // schedules with their own index copy: edge -> caller's edge position
+  uint32_t in_ld = 0;                          // row stride of `in` in floats (0 = F)
+  uint32_t partial_ld = 0;                     // row stride of `partial` in floats (0 = F)
+  bool dup_runs = false;                       // rows hold runs of equal indices worth loading once per run
 };
-
-// How the wave kernel hands neighbour pairs to its lanes: through a wave-private LDS tile (default)
-// or by register broadcast (NTS_SPMM_LDS_TILE=0).  The two measure the same on MI355X (12.44 ms vs
-// 12.40 ms for the 114.8 M-edge F=602 gather); the variable is read once per process.
-bool lds_tile_enabled() {
-  static const bool enabled = [] {
-    const char *e = getenv("NTS_SPMM_LDS_TILE");
-    return e ? e[0] != '0' : true;
-  }();
-  return enabled;
-}
 
 template <int VEC, int NACC>
 void launch_wave(const LaunchArgs &a, uint32_t col_base) {
   constexpr int kWavesPerBlock = 4;
   const uint32_t blocks = ceil_div(a.n_items, kWavesPerBlock);
   const dim3 grid(blocks), block(kWavesPerBlock * kWave);
-#define NTS_LAUNCH_WAVE(LDS, HD, RM)                                                                                   \
-  hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, LDS, HD, RM>), grid, block, 0, a.stream, a.in, a.out, a.w, a.offsets, \
-                     a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate, a.heads,     \
-                     a.row_edge_limit, a.edge_ids)
-  const bool lds = lds_tile_enabled();
+  // Neighbour pairs always go through the wave-private LDS tile (a register-broadcast variant measured
+  // the same: 12.44 ms against 12.40 ms for the 114.8 M-edge F=602 gather).
+#define NTS_LAUNCH_WAVE(HD, RM, RUNS)                                                                                  \
+  hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, true, HD, RM, RUNS>), grid, block, 0, a.stream, a.in, a.out, a.w,    \
+                     a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate,  \
+                     a.heads, a.row_edge_limit, a.edge_ids, a.in_ld ? a.in_ld : a.F,                                  \
+                     a.partial_ld ? a.partial_ld : a.F,                                                                \
+                     (VEC > 1 && (a.F % VEC != 0 || !aligned_to(a.out, 4 * VEC))) ? 1 : 0)
   if (a.edge_ids) {
-    if (a.heads.H) {
-      if (lds) NTS_LAUNCH_WAVE(true, true, true); else NTS_LAUNCH_WAVE(false, true, true);
-    } else {
-      if (lds) NTS_LAUNCH_WAVE(true, false, true); else NTS_LAUNCH_WAVE(false, false, true);
-    }
+    if (a.heads.H) NTS_LAUNCH_WAVE(true, true, false);
+    else if (a.dup_runs) NTS_LAUNCH_WAVE(false, true, true);
+    else NTS_LAUNCH_WAVE(false, true, false);
   } else {
-    if (a.heads.H) {
-      if (lds) NTS_LAUNCH_WAVE(true, true, false); else NTS_LAUNCH_WAVE(false, true, false);
-    } else {
-      if (lds) NTS_LAUNCH_WAVE(true, false, false); else NTS_LAUNCH_WAVE(false, false, false);
-    }
+    if (a.heads.H) NTS_LAUNCH_WAVE(true, false, false);
+    else if (a.dup_runs) NTS_LAUNCH_WAVE(false, false, true);
+    else NTS_LAUNCH_WAVE(false, false, false);
   }
 #undef NTS_LAUNCH_WAVE
 }
@@ -585,8 +657,17 @@ void launch_wave_vec(const LaunchArgs &a) {
 // used: measured on MI355X, dwordx2 gathers run ~20 % slower than either dword or dwordx4 gathers of
 // the same bytes (F=512: 15.4 ms vs 12.8 / 11.7 ms; F=602: 18.8 ms vs 15.3 ms with dword lanes).
 int pick_vec(const LaunchArgs &a) {
-  const bool a16 = aligned_to(a.in, 16) && aligned_to(a.out, 16) && (!a.partial || aligned_to(a.partial, 16));
   const bool heads_ok = a.heads.H == 0 || a.heads.Fh % 4 == 0;  // a 16-byte lane must stay inside one head
+  if (a.in_ld) {
+    // Gather over a padded copy of the input (row stride a multiple of four floats): 16-byte lanes
+    // whatever F is; output rows off a 16-byte boundary are stored float by float.
+    const uint32_t pld = a.partial_ld ? a.partial_ld : a.F;
+    if (a.in_ld % 4 == 0 && aligned_to(a.in, 16) && (!a.partial || (pld % 4 == 0 && aligned_to(a.partial, 16))) &&
+        a.heads.H == 0)
+      return 4;
+    return 1;
+  }
+  const bool a16 = aligned_to(a.in, 16) && aligned_to(a.out, 16) && (!a.partial || aligned_to(a.partial, 16));
   if (a.F % 4 == 0 && a16 && heads_ok) return 4;
   return 1;
 }
@@ -895,8 +976,23 @@ struct nts_spmm_plan {
   const uint32_t *offsets = nullptr;  // identity check only
   uint4 *items = nullptr;             // device
   uint4 *splits = nullptr;            // device
-  float *partial = nullptr;           // device, n_partials * partial_F floats
-  uint32_t partial_F = 0;
+  // Scratch shared by every call on this plan: the partial sums of split rows and, for widths whose
+  // rows do not start on 16-byte boundaries, a padded copy of the input.  `mu` serialises the host
+  // side of the calls (growing the scratch, enqueueing); `done` is recorded after the last kernel of
+  // each call, and a call on another stream waits for it before it touches the scratch.
+  float *partial = nullptr;           // device
+  size_t partial_floats = 0;          // its capacity
+  float *in_padded = nullptr;         // device
+  size_t in_padded_floats = 0;
+  uint32_t n_index = 0;               // rows of the gathered matrix (0 = not known: no padded copy)
+  // At least 1 in 20 edges repeats the gather index of the edge before it: the wave kernel then loads
+  // a row once per run of equal indices (and widths off 16-byte boundaries get the padded copy).
+  bool dup_runs = false;
+  uint64_t repeated_edges = 0;
+  std::mutex mu;
+  hipEvent_t done = nullptr;
+  hipStream_t last_stream = nullptr;
+  bool in_flight = false;
   // Only when rows had to be re-ordered for the source ranges: the schedule's own copy of the gather
   // indices (base already subtracted), and for each of its edges the position in the caller's order.
   uint32_t *sorted_idx = nullptr;     // device, [edges]
@@ -958,6 +1054,9 @@ struct Schedule {
   // of its edges.  Rows that are never cut keep their order.
   std::vector<uint32_t> sorted_idx;
   std::vector<uint32_t> edge_ids;
+  // Edges whose gather index equals that of the edge before them in the same row (parallel edges of
+  // a multigraph, adjacent when rows are sorted); counted in the index array the schedule gathers through.
+  uint64_t repeated_edges = 0;
 };
 
 // Host-only: needs nothing but the two index arrays.
@@ -1074,6 +1173,16 @@ void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx_in, u
     }
     splits.push_back(make_uint4(r, first, n_partials - first, 0u));
   }
+  if (idx) {
+    std::atomic<uint64_t> repeated(0);
+    parallel_blocks(rows, [&](uint32_t r0, uint32_t r1) {
+      uint64_t n = 0;
+      for (uint32_t r = r0; r < r1; ++r)
+        for (uint32_t k = off[r] + 1; k < off[r + 1]; ++k) n += idx[k] == idx[k - 1];
+      repeated.fetch_add(n, std::memory_order_relaxed);
+    });
+    out.repeated_edges = repeated.load();
+  }
   std::stable_sort(splits.begin(), splits.end(), [](const uint4 &a, const uint4 &b) { return a.z > b.z; });
   std::stable_sort(pieces.begin(), pieces.end(), [](const Piece &a, const Piece &b) {
     if (a.slab != b.slab) return a.slab < b.slab;
@@ -1111,8 +1220,11 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
   p->n_items = static_cast<uint32_t>(items.size());
   p->n_splits = static_cast<uint32_t>(splits.size());
   p->n_partials = n_partials;
-  hipError_t err = hipSuccess;
-  if (!items.empty()) {
+  p->n_index = n_index;
+  p->repeated_edges = sched.repeated_edges;
+  p->dup_runs = edges > 0 && sched.repeated_edges * 20 >= edges;
+  hipError_t err = hipEventCreateWithFlags(&p->done, hipEventDisableTiming);
+  if (err == hipSuccess && !items.empty()) {
     err = hipMalloc(reinterpret_cast<void **>(&p->items), items.size() * sizeof(uint4));
     if (err == hipSuccess)
       err = hipMemcpy(p->items, items.data(), items.size() * sizeof(uint4), hipMemcpyHostToDevice);
@@ -1210,9 +1322,12 @@ int nts_spmm_plan_schedule_host(const uint32_t *offsets_host, const uint32_t *in
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {
   NTS_TRACE_RANGE("nts_spmm_plan_destroy");
   if (!plan) return NTS_OK;
+  { std::lock_guard<std::mutex> lock(plan->mu); }  // a call that is still enqueueing finishes first
   hipError_t e1 = plan->items ? hipFree(plan->items) : hipSuccess;
   hipError_t e2 = plan->splits ? hipFree(plan->splits) : hipSuccess;
   hipError_t e3 = plan->partial ? hipFree(plan->partial) : hipSuccess;
+  if (plan->in_padded && hipFree(plan->in_padded) != hipSuccess) e3 = hipErrorUnknown;
+  if (plan->done && hipEventDestroy(plan->done) != hipSuccess) e3 = hipErrorUnknown;
   if (plan->sorted_idx && hipFree(plan->sorted_idx) != hipSuccess) e3 = hipErrorUnknown;
   if (plan->edge_ids && hipFree(plan->edge_ids) != hipSuccess) e3 = hipErrorUnknown;
   delete plan;
@@ -1231,20 +1346,84 @@ int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *s
   return NTS_OK;
 }
 
+namespace {
+
+// Row stride, in floats, of the padded input copy and of the partial sums for width F: rows of more
+// than 128 floats that do not start on 16-byte boundaries can be gathered from a copy whose rows are
+// padded to a multiple of 32 floats (whole 128-byte lines), so that the gather runs with 16-byte
+// lanes -- three loads per neighbour row at F = 602 instead of ten.  0 = no copy (F itself is the
+// stride).  Measured on the 114.8 M-edge R-MAT graph at F = 602: with one load per run of equal
+// indices the copy pays (9.75 -> 9.21 ms per pass, the 0.25 ms copy not included; 25.7 -> 25.0 ms per
+// four-pass step with it); without runs it does not (11.05 -> 11.7 ms, and 8.79 -> 8.93 ms on the same
+// graph with its parallel edges removed), so only schedules with runs use it.  NTS_SPMM_PAD=0 / 1 in
+// the environment forces it off / on.
+uint32_t padded_stride(const nts_spmm_plan *plan, uint32_t F, bool heads) {
+  static const int forced = [] {
+    const char *e = getenv("NTS_SPMM_PAD");
+    return e ? (e[0] != '0' ? 1 : 0) : -1;
+  }();
+  if (heads || plan->n_index == 0 || F <= 128 || F % 4 == 0) return 0;
+  if (forced == 0 || (forced < 0 && !plan->dup_runs)) return 0;
+  return (F + 31) / 32 * 32;
+}
+
+// NTS_SPMM_RUNS=0 / 1 forces the one-load-per-run kernel off / on whatever the schedule found.
+bool use_runs(const nts_spmm_plan *plan) {
+  static const int forced = [] {
+    const char *e = getenv("NTS_SPMM_RUNS");
+    return e ? (e[0] != '0' ? 1 : 0) : -1;
+  }();
+  return forced < 0 ? plan->dup_runs : forced == 1;
+}
+
+// Grows the plan's scratch for width F.  Caller holds plan->mu.
+int reserve_locked(nts_spmm_plan *plan, uint32_t F, bool heads) {
+  const uint32_t ld = padded_stride(plan, F, heads);
+  const size_t want_partial = static_cast<size_t>(plan->n_partials) * (ld ? ld : F);
+  const size_t want_padded = ld ? static_cast<size_t>(plan->n_index) * ld : 0;
+  if (want_partial > plan->partial_floats) {
+    // The old buffer may still be read by work queued earlier: hipFree waits for the device.
+    if (plan->partial) {
+      NTS_HIP_TRY(hipFree(plan->partial));
+      plan->partial = nullptr;
+      plan->partial_floats = 0;
+    }
+    NTS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&plan->partial), want_partial * sizeof(float)));
+    plan->partial_floats = want_partial;
+  }
+  if (want_padded > plan->in_padded_floats) {
+    if (plan->in_padded) {
+      NTS_HIP_TRY(hipFree(plan->in_padded));
+      plan->in_padded = nullptr;
+      plan->in_padded_floats = 0;
+    }
+    NTS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&plan->in_padded), want_padded * sizeof(float)));
+    plan->in_padded_floats = want_padded;
+  }
+  return NTS_OK;
+}
+
+// A call on `stream` is about to use the plan's scratch: if the previous call ran on another stream,
+// `stream` first waits for it (in stream order, the host does not block).  Caller holds plan->mu.
+int enter_stream(nts_spmm_plan *plan, hipStream_t stream) {
+  if (plan->in_flight && plan->last_stream != stream) NTS_HIP_TRY(hipStreamWaitEvent(stream, plan->done, 0));
+  return NTS_OK;
+}
+int leave_stream(nts_spmm_plan *plan, hipStream_t stream) {
+  NTS_HIP_TRY(hipEventRecord(plan->done, stream));
+  plan->last_stream = stream;
+  plan->in_flight = true;
+  return NTS_OK;
+}
+
+}  // namespace
+
 int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F) {
   NTS_TRACE_RANGE("nts_spmm_plan_reserve");
   if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_reserve: null plan");
-  if (plan->n_partials == 0 || F <= plan->partial_F) return NTS_OK;
-  // The old buffer may still be read by work queued earlier: hipFree waits for the device.
-  if (plan->partial) {
-    NTS_HIP_TRY(hipFree(plan->partial));
-    plan->partial = nullptr;
-    plan->partial_F = 0;
-  }
-  NTS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&plan->partial),
-                        static_cast<size_t>(plan->n_partials) * F * sizeof(float)));
-  plan->partial_F = F;
-  return NTS_OK;
+  if (F == 0) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_reserve: F is 0");
+  std::lock_guard<std::mutex> lock(plan->mu);
+  return reserve_locked(plan, F, false);
 }
 
 namespace {
@@ -1284,7 +1463,9 @@ int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float 
                                  "nts_spmm_gather_heads_planned: null pointer"))
     return rc;
   if (plan->rows == 0) return NTS_OK;
-  if (int rc = nts_spmm_plan_reserve(plan, F)) return rc;
+  std::lock_guard<std::mutex> lock(plan->mu);
+  if (int rc = reserve_locked(plan, F, true)) return rc;
+  if (int rc = enter_stream(plan, stream)) return rc;
   nts::LaunchArgs a{in,  out,         alpha,         offsets,    indices, 0u, plan->n_items,
                     F,   plan->items, plan->partial, accumulate, stream};
   a.heads = nts::HeadArgs{perm, H, Fh};
@@ -1298,7 +1479,7 @@ int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float 
     nts::launch_reduce_partials(out, plan->partial, plan->splits, plan->n_splits, F, accumulate, stream);
     NTS_LAUNCH_CHECK("spmm_reduce_partials_kernel");
   }
-  return NTS_OK;
+  return leave_stream(plan, stream);
 }
 
 int nts_spmm_plan_set_events(nts_spmm_plan_t *plan, nts_event_t start, nts_event_t stop) {
@@ -1322,7 +1503,9 @@ int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, 
                                  "nts_spmm_gather_planned: null pointer"))
     return rc;
   if (plan->rows == 0) return NTS_OK;
-  if (int rc = nts_spmm_plan_reserve(plan, F)) return rc;
+  std::lock_guard<std::mutex> lock(plan->mu);
+  if (int rc = reserve_locked(plan, F, false)) return rc;
+  if (int rc = enter_stream(plan, stream)) return rc;
   nts::LaunchArgs a{in,  out,         w,           offsets,       indices,   index_base, plan->n_items,
                     F,   plan->items, plan->partial, accumulate, stream};
   if (plan->sorted_idx) {  // the schedule's own copy of the indices, base already subtracted
@@ -1330,15 +1513,27 @@ int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, 
     a.index_base = 0;
     a.edge_ids = plan->edge_ids;
   }
+  a.dup_runs = use_runs(plan);
+  if (const uint32_t ld = padded_stride(plan, F, false)) {
+    // Rows off 16-byte boundaries: gather from a padded copy with 16-byte lanes.
+    const uint64_t vecs = static_cast<uint64_t>(plan->n_index) * (ld / 4);
+    const uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>((vecs + 255) / 256, 1u << 16));
+    hipLaunchKernelGGL(nts::pad_rows_kernel, dim3(blocks), dim3(256), 0, stream,
+                       reinterpret_cast<float4 *>(plan->in_padded), in, plan->n_index, F, ld);
+    NTS_LAUNCH_CHECK("pad_rows_kernel");
+    a.in = plan->in_padded;
+    a.in_ld = ld;
+    a.partial_ld = ld;
+  }
   if (plan->ev_start && plan->ev_stop) NTS_HIP_TRY(hipEventRecord(plan->ev_start, stream));
   nts::launch_spmm(a);
   NTS_LAUNCH_CHECK("nts_spmm_gather_planned");
   if (plan->ev_start && plan->ev_stop) NTS_HIP_TRY(hipEventRecord(plan->ev_stop, stream));
   if (plan->n_splits) {
-    nts::launch_reduce_partials(out, plan->partial, plan->splits, plan->n_splits, F, accumulate, stream);
+    nts::launch_reduce_partials(out, plan->partial, plan->splits, plan->n_splits, F, accumulate, stream, a.partial_ld);
     NTS_LAUNCH_CHECK("spmm_reduce_partials_kernel");
   }
-  return NTS_OK;
+  return leave_stream(plan, stream);
 }
 
 }  // extern "C"

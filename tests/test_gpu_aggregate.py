@@ -274,20 +274,102 @@ def test_cache_aware_plan(device, F, chunk, slabs, sorted_rows):
     plan.close()
 
 
-def test_register_broadcast_variant_in_a_fresh_process(device):
-    """The library hands neighbour pairs to the lanes through an LDS tile by default and by register
-    broadcast when NTS_SPMM_LDS_TILE=0 (read once per process): the other variant passes the same
-    parity cases."""
+@pytest.mark.parametrize("runs,pad", [("1", "1"), ("0", "0")])
+def test_forced_kernel_variants_in_a_fresh_process(device, runs, pad):
+    """A schedule picks by itself whether rows are loaded once per run of equal indices and whether
+    widths off 16-byte boundaries are gathered from a padded copy (both when at least 1 edge in 20
+    repeats its predecessor's index).  NTS_SPMM_RUNS / NTS_SPMM_PAD (read once per process) force the
+    choice: both settings pass the same parity cases, bit-exact rows included."""
     import os
     import subprocess
     import sys
 
-    env = dict(os.environ, NTS_SPMM_LDS_TILE="0")
+    env = dict(os.environ, NTS_SPMM_RUNS=runs, NTS_SPMM_PAD=pad)
     here = os.path.dirname(os.path.abspath(__file__))
     r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(here, "test_gpu_aggregate.py"), "-q", "-x", "-m", "gpu",
-                        "-k", "forward_matches_oracle or planned_split_rows or cache_aware", "--timeout", "120",
+                        "-k", "planned_split_rows or cache_aware or random_shapes or runs_of_equal", "--timeout", "120",
                         "--timeout-method", "thread"], env=env, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-1500:]
+
+
+@pytest.mark.parametrize("F", [130, 200, 301, 602, 256, 1433])
+def test_runs_of_equal_indices_are_loaded_once_and_added_edge_by_edge(device, F):
+    """A multigraph block with sorted rows: two thirds of the edges repeat their predecessor's index,
+    so the schedule turns on the one-load-per-run kernel (and, for widths that are not multiples of
+    four, the padded copy of the input).  Every edge is still added with its own weight in edge order:
+    rows that are not cut equal the oracle's fused chain bit for bit."""
+    print(f"case F={F}", flush=True)
+    rng = np.random.default_rng(F)
+    Vd, Vs, chunk, slabs = 600, 400, 64, 8
+    deg = rng.integers(0, 60, Vd)
+    deg[[3, 299]] = [5000, 700]
+    co = np.zeros(Vd + 1, dtype=np.uint32)
+    co[1:] = np.cumsum(deg)
+    ri = np.concatenate([np.sort(np.repeat(rng.integers(0, Vs, (d + 2) // 3), 3)[:d]) for d in deg]).astype(np.uint32)
+    assert (ri[1:] == ri[:-1]).mean() > 0.5
+    x = rng.standard_normal((Vs, F)).astype(np.float32)
+    w = rng.random(ri.size).astype(np.float32)
+    dx, dw, dco, dri = _dev(x, device), _dev(w, device), _dev(co, device), _dev(ri, device)
+    plan = SpmmPlan(dco, Vd, ri.size, chunk, dri, Vs, slabs)
+    ref_fma = oracle.spmm(x, w, co, ri, Vd, fused=True)
+    scale = abs_term_scale(x, w, co, ri, Vd)
+    for accumulate in (0, 1):
+        init = rng.standard_normal((Vd, F)).astype(np.float32)
+        out = _dev(init, device) if accumulate else torch.full((Vd, F), float("nan"), device=device)
+        call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, F, accumulate,
+             _stream())
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        if accumulate:
+            check(got, oracle.spmm(x, w, co, ri, Vd) + init, scale + np.abs(init))
+        else:
+            check(got, oracle.spmm(x, w, co, ri, Vd), scale)
+            keep = deg <= chunk // 4
+            assert keep.sum() > 100
+            assert np.array_equal(got[keep].view(np.uint32), ref_fma[keep].view(np.uint32))
+    # unweighted through the same schedule
+    out = torch.full((Vd, F), float("nan"), device=device)
+    call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), 0, ptr(dco), ptr(dri), 0, F, 0, _stream())
+    torch.cuda.synchronize()
+    check(out.cpu().numpy(), oracle.spmm(x, None, co, ri, Vd), abs_term_scale(x, None, co, ri, Vd))
+    plan.close()
+
+
+def test_one_plan_called_from_two_streams(device):
+    """A plan's scratch (partial sums, padded input copy) is shared by all calls on it.  Calls from
+    different streams are ordered by the library (the later stream waits, on the device, for the
+    earlier call's last kernel), so two streams that use one plan without any host-side wait still
+    get the results of calls made one at a time."""
+    rng = np.random.default_rng(77)
+    Vd, Vs, F, chunk, slabs = 30000, 20000, 602, 64, 8
+    deg = rng.integers(0, 120, Vd)
+    deg[[5, 77, 1500]] = [200000, 50000, 9000]
+    co = np.zeros(Vd + 1, dtype=np.uint32)
+    co[1:] = np.cumsum(deg)
+    ri = np.concatenate([np.sort(rng.integers(0, Vs, d)) for d in deg]).astype(np.uint32)
+    w = rng.random(ri.size).astype(np.float32)
+    xs = [rng.standard_normal((Vs, F)).astype(np.float32) for _ in range(2)]
+    dw, dco, dri = _dev(w, device), _dev(co, device), _dev(ri, device)
+    dxs = [_dev(x, device) for x in xs]
+    plan = SpmmPlan(dco, Vd, ri.size, chunk, dri, Vs, slabs)
+    assert plan.info()["partials"] > 20000
+    want = []
+    for dx in dxs:  # one at a time
+        out = torch.empty(Vd, F, device=device)
+        call("nts_spmm_gather_planned", plan.handle, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, F, 0, _stream())
+        torch.cuda.synchronize()
+        want.append(out.cpu().numpy())
+    streams = [torch.cuda.Stream(device=device) for _ in range(2)]
+    outs = [torch.empty(Vd, F, device=device) for _ in range(2)]
+    torch.cuda.synchronize()
+    for _ in range(6):  # alternate streams back to back, no host wait in between
+        for k in range(2):
+            call("nts_spmm_gather_planned", plan.handle, ptr(dxs[k]), ptr(outs[k]), ptr(dw), ptr(dco), ptr(dri), 0, F, 0,
+                 streams[k].cuda_stream)
+    torch.cuda.synchronize()
+    for k in range(2):
+        assert np.array_equal(outs[k].cpu().numpy().view(np.uint32), want[k].view(np.uint32)), f"stream {k}"
+    plan.close()
 
 
 def test_scratch_pool_is_kept_between_calls_and_can_be_trimmed(device):
