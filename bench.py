@@ -8,11 +8,13 @@ aggregate-then-transform order: layer-0 forward (F=602), layer-1 forward (F=128)
 (F=128), layer-0 backward (F=602).  Forward gathers by destination over the CSC, backward gathers
 by source over the CSR.  Inputs are resident in HBM before the timed region.
 
-Prints one JSON line: edges aggregated per second (4 * E edges per step), the roofline figure of
-the dominant kernel (the F=602 gather) from HIP events recorded around that kernel, and a CPU
-baseline timed on the host cores on a bounded sample of the same graph: the reference's own CPU
-operator where the reference-built program oracle/_ref/ref_fullgraph_cpu is present ("reference"),
-else the CPU oracle ("port").
+Prints one JSON line: edges aggregated per second (4 * E edges per step); the roofline figure of the
+dominant kernel (the F=602 gather): its HBM-side bytes per launch from the committed rocprofv3
+counter summary over the kernel time this run measures with HIP events recorded around that kernel;
+a check of the last timed step's outputs against the CPU oracle; and the CPU baselines timed on the
+host cores on the same graph: the reference's own CPU operator where the reference-built program
+oracle/_ref/ref_fullgraph_cpu is present ("reference"), and the CPU oracle ("port") at both thread
+settings.  The run exits with status 1 when the check fails.
 
 --workload arxiv|products|gat measures the per-epoch time of that sampled mini-batch configuration
 instead (sampling, layer construction, gathers, aggregation fwd+bwd, all through the C ABI) and
@@ -32,20 +34,59 @@ if ROOT not in sys.path:
 V_REDDIT = 232_965
 E_REDDIT = 114_800_000
 F_IN, F_HID = 602, 128
-# The reference's own CPU operator, built from the reference tree where that is present (test infrastructure).
+# The reference's own operators, built from the reference tree where that is present (test infrastructure):
+# its CPU operator, and its GPU operator class compiled against this library's host veneer.
 REFERENCE_PROGRAM = os.path.join(ROOT, "oracle", "_ref", "ref_fullgraph_cpu")
+REFERENCE_GPU_PROGRAM = os.path.join(ROOT, "oracle", "_ref", "ref_fullgraph_gpu")
 HBM_PEAK_GBS = 8000.0
-# Bytes per launch of the F=602 gather kernel that cross the L2 <-> fabric boundary, from rocprofv3
-# FETCH_SIZE (x1.986 calibration) + WRITE_SIZE at the default schedule
-# (profiles/spmm_wave_f602_reddit_shaped_pmc.txt).  Reported only for the configuration it was measured on.
-TRAFFIC_BYTES_F602 = 44_601_740_400
-TRAFFIC_MEASURED_AT = dict(vertices=V_REDDIT, edges=E_REDDIT, chunk=512, slabs=32)
+# rocprofv3 counter summary of the dominant kernel on this workload; it names the kernel sources it was
+# measured with, and its traffic figure is only quoted while those sources are unchanged.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "spmm_wave_f602_reddit_shaped_pmc.txt")
+KERNEL_SOURCES = [os.path.join(ROOT, "neutronbench_amd", "csrc", n) for n in ("spmm.hip", "common.hpp")]
 
 
 def algorithmic_bytes(E, V_out, F, weighted=True):
     """Edge-gather model of one aggregation pass: one source row, one index and one weight per
     edge; one output row and one offset per output row."""
     return E * (4 * F + 4 + (4 if weighted else 0)) + V_out * 4 * F + (V_out + 1) * 4
+
+
+def compulsory_bytes(E, V_in, V_out, F):
+    """Every input and output row once, every index and weight once, every offset once."""
+    return (V_in + V_out) * 4 * F + E * 8 + (V_out + 1) * 4
+
+
+def kernel_sources_digest():
+    import hashlib
+
+    h = hashlib.sha256()
+    for path in KERNEL_SOURCES:
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """HBM-side bytes per launch of the dominant kernel from the committed rocprofv3 summary
+    (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain copy), or None
+    when the summary is missing, was taken on another workload / schedule, or with other kernel
+    sources than the ones this run uses."""
+    try:
+        fields = {}
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if ":" in line and not line.startswith(" "):
+                    k, v = line.split(":", 1)
+                    fields[k.strip()] = v.strip()
+        if fields.get("kernel_sources_sha256_16") != kernel_sources_digest():
+            return None
+        if fields.get("workload") != workload:
+            return None
+        return {"traffic": int(fields["traffic_bytes_per_launch"]), "fetch": int(fields["fetch_bytes_per_launch"]),
+                "write": int(fields["write_bytes_per_launch"]), "kernel": fields.get("kernel"),
+                "l2_hit_rate": float(fields["l2_hit_rate"]) if "l2_hit_rate" in fields else None}
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def main():
@@ -58,12 +99,15 @@ def main():
     ap.add_argument("--chunk", type=int, default=512, help="largest number of edges in one piece of a split hub row")
     ap.add_argument("--slabs", type=int, default=32,
                     help="source ranges of the cache-aware schedule (1 = split hub rows by edge count only)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true",
+                    help="skip everything that runs on the host after the timed region: the check of the timed "
+                         "outputs against the CPU oracle, the CPU baselines and the reference operator's time")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB row copy (identity gather) so that HBM byte counters can be scaled")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the oracle sample")
-    ap.add_argument("--cpu-reference-edges", type=int, default=28_700_000,
-                    help="edges of the sample the reference's own CPU operator is timed on (0 = time the oracle instead)")
+    ap.add_argument("--cpu-reps", type=int, default=5, help="timed repetitions of each CPU baseline (median reported)")
+    ap.add_argument("--cpu-reference-edges", type=int, default=0,
+                    help="edges of the graph the reference's own operators are timed on (0 = the whole graph; a "
+                         "smaller number takes the edges of the lowest-numbered source vertices)")
     ap.add_argument("--workload", choices=["reddit", "arxiv", "products", "gat"], default="reddit",
                     help="reddit (default): the aggregation workload above; arxiv / products / gat: per-epoch time of "
                          "that sampled mini-batch configuration (BASELINE.json configs 2, 4, 5) instead")
@@ -99,6 +143,7 @@ def main():
     op = ForwardSingleGPUfuseOp(chunk, with_weight=True)
     chunk.plan_forward.reserve(F_IN)
     chunk.plan_backward.reserve(F_IN)
+    scratch = [p.scratch_info(F_IN) for p in (chunk.plan_forward, chunk.plan_backward)]
 
     def step():
         y0 = op.forward(x0)    # layer 0: aggregate the 602-wide input features
@@ -125,7 +170,6 @@ def main():
     # One HIP event pair per aggregation launch of the timed region (4 per step).  The library records
     # them on the launch stream immediately before and after its main gather kernel; nothing waits on
     # them until the timed region is over.
-    stream = torch.cuda.current_stream().cuda_stream
     n_ev = 4 * args.steps
     events = []
     for _ in range(n_ev):
@@ -134,16 +178,17 @@ def main():
         call("nts_event_create", ctypes.byref(b))
         events.append((a, b))
     fwd, bwd = chunk.plan_forward.handle, chunk.plan_backward.handle
+    outs = [None] * 4
 
     def timed_step(i):
         call("nts_spmm_plan_set_events", fwd, *events[4 * i + 0])
-        op.forward(x0)
+        outs[0] = op.forward(x0)
         call("nts_spmm_plan_set_events", fwd, *events[4 * i + 1])
-        op.forward(h1)
+        outs[1] = op.forward(h1)
         call("nts_spmm_plan_set_events", bwd, *events[4 * i + 2])
-        op.backward(g1)
+        outs[2] = op.backward(g1)
         call("nts_spmm_plan_set_events", bwd, *events[4 * i + 3])
-        op.backward(g0)
+        outs[3] = op.backward(g0)
 
     # Timed region: exactly `steps` steps between two synchronisations.
     torch.cuda.synchronize()
@@ -165,32 +210,59 @@ def main():
         call("nts_event_destroy", a)
         call("nts_event_destroy", b)
     per_pass = [sum(durs[k::4]) / args.steps for k in range(4)]  # fwd602, fwd128, bwd128, bwd602
-    # Dominant kernel: the F=602 gather (spmm_wave_kernel<1,10>), launched twice per step: forward
-    # over the CSC and backward over the CSR.  Same algorithmic bytes per launch for both.
+    # Dominant kernel: the F=602 gather (spmm_wave_kernel), launched twice per step: forward over the
+    # CSC and backward over the CSR.  Same algorithmic bytes per launch for both.
     kernel_ms = (per_pass[0] + per_pass[3]) / 2
     algo = algorithmic_bytes(E, V, F_IN)
-    achieved = algo / (kernel_ms * 1e-3) / 1e9
+    model_gbs = algo / (kernel_ms * 1e-3) / 1e9
+    workload_key = f"V={V} E={E} chunk={args.chunk} slabs={args.slabs} F={F_IN}"
+    measured = measured_traffic(workload_key)
+    padded = scratch[0]["padded_input_bytes"] > 0
     roofline = {
+        # `achieved` and `frac` are the bytes rocprofv3 counts between the L2 and the fabric (Infinity
+        # Cache / HBM) per launch over this run's kernel time: the figure the 60 %-of-peak target is
+        # judged on.  null when no counter summary matches the kernel sources of this run.
         "bound": "hbm",
-        "kernel": "spmm_wave_kernel<1,10,true,false,false> (F=602 gather, forward and backward launches)",
-        "achieved": round(achieved, 1),
+        "kernel": (measured or {}).get("kernel") or
+        ("spmm_wave_kernel<4,3,...> over a padded input copy" if padded else "spmm_wave_kernel<1,10,...>")
+        + " (F=602 gather, forward and backward launches)",
+        "achieved": round(measured["traffic"] / (kernel_ms * 1e-3) / 1e9, 1) if measured else None,
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": TRAFFIC_BYTES_F602 if dict(vertices=V, edges=E, chunk=args.chunk, slabs=args.slabs) ==
-        TRAFFIC_MEASURED_AT else None,
+        "frac": round(measured["traffic"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if measured else None,
+        "traffic": measured["traffic"] if measured else None,
+        "target_frac": 0.6,
+        "target_met": bool(measured and measured["traffic"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS >= 0.6),
+        "limited_by": "L2 misses through the fabric: this library's plain streaming kernels move 4.9-6.1 TB/s by the "
+                      "same counters, and the gather fetches many times its compulsory bytes because one source "
+                      f"range does not fit a 4 MB L2 (L2 hit rate {(measured or {}).get('l2_hit_rate')})",
+        # the edge-gather model (one source row per edge) counts every re-read served by L2 as a byte
+        # moved; it exceeds the HBM peak and is reported for comparison only
+        "model_gbs": round(model_gbs, 1),
+        "model_frac": round(model_gbs / HBM_PEAK_GBS, 4),
         "algorithmic_bytes": algo,
+        "compulsory_bytes": compulsory_bytes(E, V, V, F_IN),
         "kernel_ms": round(kernel_ms, 3),
         "per_pass_ms": {"fwd_F602": round(per_pass[0], 3), "fwd_F128": round(per_pass[1], 3),
                         "bwd_F128": round(per_pass[2], 3), "bwd_F602": round(per_pass[3], 3)},
     }
 
-    cpu_baseline = None
+    check = cpu_baseline = None
+    reference_operator = None
     if not args.no_cpu_baseline:
-        if args.cpu_reference_edges > 0 and os.path.exists(REFERENCE_PROGRAM):
-            cpu_baseline = run_reference_cpu_baseline(torch, chunk, x0, h1, V, min(E, args.cpu_reference_edges))
+        inputs = dict(fwd_F602=x0, fwd_F128=h1, bwd_F128=g1, bwd_F602=g0)
+        check = check_against_oracle(torch, chunk, inputs, dict(zip(inputs, outs)), V)
+        if not check["ok"]:
+            print(json.dumps({"error": "timed outputs differ from the CPU oracle", "check": check}))
+            sys.exit(1)
+        ref_edges = min(E, args.cpu_reference_edges) if args.cpu_reference_edges > 0 else E
+        cpu_baseline, reference_operator = run_reference_programs(torch, chunk, x0, h1, V, ref_edges, args.cpu_reps)
+        port = run_cpu_port_baseline(torch, chunk, x0, h1, g1, g0, V, args.cpu_reps)
         if cpu_baseline is None:
-            cpu_baseline = run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, args.cpu_seconds)
+            cpu_baseline = port.pop("all_threads")
+            cpu_baseline["other_thread_setting"] = port.pop("reference_default_threads")
+        else:
+            cpu_baseline["port"] = port
 
     out = {
         "metric": "edges aggregated/s (fwd+bwd)",
@@ -210,27 +282,119 @@ def main():
             "vertices": V,
             "edges": E,
             "graph": "R-MAT a=.57 b=.19 c=.19, seed 3, ids permuted, edge list in (src, dst) order, duplicates kept",
+            "parallel_edges": {"forward": scratch[0]["repeated_edges"], "backward": scratch[1]["repeated_edges"],
+                               "note": "edges that repeat the source (forward) / destination (backward) of the edge "
+                                       "before them in their row; the kernel loads such a row once per run and adds "
+                                       "it once per edge (NTS_SPMM_RUNS=0 NTS_SPMM_PAD=0 times the kernel without that)",
+                               "loads_once_per_run": scratch[0]["loads_once_per_run"]},
             "passes_per_step": 4,
             "plan": dict(chunk.plan_forward.info(), chunk_edges=args.chunk, slabs=args.slabs),
+            "plan_build_s": round(chunk.plan_build_s, 3),
+            "plan_scratch_bytes": {"forward": scratch[0]["partial_bytes"] + scratch[0]["padded_input_bytes"],
+                                   "backward": scratch[1]["partial_bytes"] + scratch[1]["padded_input_bytes"],
+                                   "of_which_padded_input_copy": scratch[0]["padded_input_bytes"]},
             "setup_s": round(setup_s, 2),
+            "timed_path": "Python operator mirror: torch.empty_like output, accumulate=0, nts_spmm_gather_planned",
+            "reference_operator": reference_operator,
         },
         "roofline": roofline,
+        "check": check,
         "cpu_baseline": cpu_baseline,
     }
     print(json.dumps(out))
 
 
-def run_reference_cpu_baseline(torch, chunk, x0, h1, V, sample_edges):
-    """The reference's own CPU operator (ForwardCPUfuseOp behind oracle/_ref/ref_fullgraph_cpu, built
-    from the reference tree by oracle/build_ref.sh) on the edges of the lowest-numbered source
-    vertices of the same graph: its loader, partitioner and operator run unchanged on this host's
-    cores.  Returns None when the program fails, so that the caller can fall back to the oracle."""
+def check_against_oracle(torch, chunk, inputs, outputs, V, n_rows=400, n_hubs=4):
+    """The outputs of the last timed step against the CPU oracle: n_rows seeded rows per pass (rows that
+    the schedule never cuts must equal the oracle's fused chain bit for bit, the others within 1e-4 of
+    max(|a|, |b|, 1e-2 * sum|terms|)), and the n_hubs longest rows against a float64 sum -- the oracle's
+    strictly sequential fp32 chain over 10^5..10^6 edges is itself several 1e-4 off there, so for those
+    rows the kernel has to meet the tolerance against float64 and must not be less accurate than the
+    oracle."""
+    import numpy as np
+
+    import oracle
+    from neutronbench_amd import synth
+    from neutronbench_amd.layout import u32_to_i64
+
+    rows = synth.permutation(V, 7, chunk.column_offset_gpu.device)[:n_rows]
+    worst, worst_hub, exact_rows, checked = 0.0, 0.0, 0, 0
+    detail = {}
+    for name, x in inputs.items():
+        out = outputs[name]
+        fwd = name.startswith("fwd")
+        off = chunk.column_offset_gpu if fwd else chunk.row_offset_gpu
+        idx = chunk.row_indices_gpu if fwd else chunk.column_indices_gpu
+        w = chunk.edge_weight_forward_gpu if fwd else chunk.edge_weight_backward_gpu
+        off64 = u32_to_i64(off)
+        deg = off64[1:] - off64[:-1]
+        hubs = torch.topk(deg, n_hubs).indices
+        xh = x.cpu().numpy()
+
+        def sub(sel):
+            starts = off64[sel]
+            lens = off64[sel + 1] - starts
+            so = torch.zeros(sel.numel() + 1, dtype=torch.int64, device=off.device)
+            so[1:] = torch.cumsum(lens, 0)
+            eid = torch.repeat_interleave(starts - so[:-1], lens) + torch.arange(int(so[-1]), device=off.device)
+            return so.cpu().numpy().astype(np.uint32), eid
+
+        def err(a, b, scale):
+            den = np.maximum(np.maximum(np.abs(a), np.abs(b)), 1e-2 * scale + 1e-30)
+            return float((np.abs(a.astype(np.float64) - b) / den).max())
+
+        so, eid = sub(rows)
+        si, sw = idx[eid].cpu().numpy().view(np.uint32), w[eid].cpu().numpy()
+        got = out[rows].cpu().numpy()
+        ref = oracle.spmm(xh, sw, so, si, rows.numel())
+        scale = oracle.spmm(np.abs(xh), sw, so, si, rows.numel())
+        uncut = np.diff(so.astype(np.int64)) <= 128  # rows of at most chunk/4 edges are never cut
+        fused = oracle.spmm(xh, sw, so, si, rows.numel(), fused=True)
+        bits_ok = bool(np.array_equal(got[uncut].view(np.uint32), fused[uncut].view(np.uint32)))
+        e_rows = err(got, ref, scale)
+        ho, heid = sub(hubs)
+        hi64, hw = u32_to_i64(idx[heid]), w[heid]
+        exact = np.zeros((n_hubs, x.shape[1]))
+        for k in range(n_hubs):
+            acc = torch.zeros(x.shape[1], dtype=torch.float64, device=x.device)
+            for s in range(int(ho[k]), int(ho[k + 1]), 1 << 15):
+                e = min(s + (1 << 15), int(ho[k + 1]))
+                acc += (x[hi64[s:e]].double() * hw[s:e, None].double()).sum(0)
+            exact[k] = acc.cpu().numpy()
+        hscale = oracle.spmm(np.abs(xh), hw.cpu().numpy(), ho, idx[heid].cpu().numpy().view(np.uint32), n_hubs)
+        href = oracle.spmm(xh, hw.cpu().numpy(), ho, idx[heid].cpu().numpy().view(np.uint32), n_hubs)
+        e_hub, e_hub_oracle = err(out[hubs].cpu().numpy(), exact, hscale), err(href, exact, hscale)
+        detail[name] = {"rows_max_rel_err": e_rows, "uncut_rows_bit_exact": bits_ok, "uncut_rows": int(uncut.sum()),
+                        "hub_max_rel_err_vs_f64": e_hub, "oracle_hub_max_rel_err_vs_f64": e_hub_oracle}
+        worst, worst_hub = max(worst, e_rows), max(worst_hub, e_hub)
+        exact_rows += int(uncut.sum()) if bits_ok else 0
+        checked += rows.numel() + n_hubs
+        if not bits_ok or e_rows > 1e-4 or e_hub > 1e-4 or e_hub > max(e_hub_oracle, 1e-5):
+            return {"ok": False, "failed_pass": name, "detail": detail}
+    return {"ok": True, "checked_rows": checked, "max_rel_err": worst, "bit_exact_rows": exact_rows,
+            "hub_rows_max_rel_err_vs_f64": worst_hub, "tolerance": 1e-4,
+            "note": "sampled rows of all four timed passes against the CPU oracle; the longest rows of each pass are "
+                    "held to float64 (the oracle's sequential fp32 chain is less accurate there than the kernel)",
+            "detail": detail}
+
+
+def run_reference_programs(torch, chunk, x0, h1, V, sample_edges, reps):
+    """The reference's own operators on the same graph, from the programs oracle/build_ref.sh builds out
+    of the reference tree: ForwardCPUfuseOp on this host's cores (its loader, partitioner and operator
+    unchanged) -> the CPU baseline; and ForwardSingleGPUfuseOp, the reference's GPU operator class
+    compiled unchanged against this library's host veneer (torch::zeros output, accumulate = 1, the
+    operator's own stream synchronisation) -> what an unchanged caller gets, outside the timed region.
+    Returns (cpu_baseline or None, reference_operator or None)."""
     import re
     import shutil
     import subprocess
     import tempfile
 
+    if not os.path.exists(REFERENCE_PROGRAM):
+        return None, None
+    E = chunk.E
     tmp = tempfile.mkdtemp(prefix="nts_ref_")
+    cpu = gpu = None
     try:
         ro = chunk.row_offset_gpu.to(torch.int64)
         pos = torch.arange(sample_edges, device=ro.device)
@@ -240,74 +404,84 @@ def run_reference_cpu_baseline(torch, chunk, x0, h1, V, sample_edges):
         del ro, pos, src, dst
         x0.cpu().numpy().tofile(os.path.join(tmp, f"p.x{F_IN}"))
         h1.cpu().numpy().tofile(os.path.join(tmp, f"p.x{F_HID}"))
-        r = subprocess.run([REFERENCE_PROGRAM, os.path.join(tmp, "g.edge"), str(V), f"{F_IN},{F_HID}", "1",
-                            os.path.join(tmp, "p"), "agg-cpu"], capture_output=True, text=True, timeout=240)
-        rows = re.findall(r"timing: V=\d+ E=(\d+) F=(\d+) forward_s=([0-9.]+) backward_s=([0-9.]+) threads=(\d+)", r.stdout)
-        if r.returncode != 0 or len(rows) != 2:
-            return None
-        total_s = sum(float(f) + float(b) for _, _, f, b, _ in rows)
-        edges = int(rows[0][0])
-        return {
-            "value": round(4 * edges / total_s, 1),
-            "unit": "edges/s",
-            "cores": int(rows[0][4]),
-            "kind": "reference",
-            "sample": f"the reference's ForwardCPUfuseOp (its own loader, partitioner and operator, built from the "
-                      f"reference sources) on the {edges} edges of the lowest-numbered source vertices of the same "
-                      f"graph, forward and backward at F={F_IN} and F={F_HID}, best of 3: "
-                      + ", ".join(f"F={w} fwd {float(f):.3f} s bwd {float(b):.3f} s" for _, w, f, b, _ in rows),
-        }
+        env = dict(os.environ, NTS_REF_WARMUP="1", NTS_REF_REPS=str(reps))
+        pat = (r"timing: V=\d+ E=(\d+) F=(\d+) forward_s=([0-9.]+) backward_s=([0-9.]+)(?: threads=(\d+))? "
+               r"best_forward_s=([0-9.]+) best_backward_s=([0-9.]+)")
+        argv = [os.path.join(tmp, "g.edge"), str(V), f"{F_IN},{F_HID}", "1", os.path.join(tmp, "p")]
+        r = subprocess.run([REFERENCE_PROGRAM] + argv + ["agg-cpu"], capture_output=True, text=True, timeout=400, env=env)
+        rows = re.findall(pat, r.stdout)
+        if r.returncode == 0 and len(rows) == 2:
+            total_s = sum(float(f) + float(b) for _, _, f, b, _, _, _ in rows)
+            edges = int(rows[0][0])
+            cpu = {
+                "value": round(4 * edges / total_s, 1),
+                "unit": "edges/s",
+                "cores": int(rows[0][4]),
+                "kind": "reference",
+                "sample": f"the reference's ForwardCPUfuseOp (its own loader, partitioner and operator, built from the "
+                          f"reference sources) on {'the whole graph' if edges == E else 'the lowest-numbered source vertices'}"
+                          f" ({edges} edges), forward and backward at F={F_IN} and F={F_HID}, median of {reps} after 1 "
+                          f"warm-up, {rows[0][4]} threads (the operator's only setting: every configured CPU): "
+                          + ", ".join(f"F={w} fwd {float(f):.3f} s bwd {float(b):.3f} s" for _, w, f, b, _, _, _ in rows),
+            }
+        if os.path.exists(REFERENCE_GPU_PROGRAM):
+            r = subprocess.run([REFERENCE_GPU_PROGRAM] + argv + ["agg-gpu"], capture_output=True, text=True, timeout=400,
+                               env=env)
+            rows = re.findall(pat, r.stdout)
+            if r.returncode == 0 and len(rows) == 2:
+                gpu = {"what": "the reference's ForwardSingleGPUfuseOp class, unchanged, over the host veneer "
+                               "(torch::zeros output, accumulate=1, stream synchronisation per call); wall time per "
+                               f"call, median of {reps} after 1 warm-up; the veneer builds its schedule on the third "
+                               "identical call, so the best time is the steady state",
+                       "edges": int(rows[0][0])}
+                for _, w, f, b, _, bf, bb in rows:
+                    gpu[f"F{w}_forward_ms"] = round(float(f) * 1e3, 3)
+                    gpu[f"F{w}_backward_ms"] = round(float(b) * 1e3, 3)
+                    gpu[f"F{w}_best_forward_ms"] = round(float(bf) * 1e3, 3)
+                    gpu[f"F{w}_best_backward_ms"] = round(float(bb) * 1e3, 3)
     except (OSError, subprocess.SubprocessError):
-        return None
+        pass
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
+    return cpu, gpu
 
 
-def run_cpu_baseline(torch, chunk, x0, h1, g1, g0, V, target_s):
-    """The CPU oracle (restatement of the reference's CPU operators, OpenMP over rows) on the first
-    R output rows of each of the four passes of the same graph, all host cores."""
+def run_cpu_port_baseline(torch, chunk, x0, h1, g1, g0, V, reps):
+    """The CPU oracle (restatement of the reference's CPU operators, OpenMP over rows) on the whole graph,
+    the four passes of a step, at the two thread settings the reference uses: every hardware thread
+    (its full-graph operators) and max(1, ncpu / 2 - 1) (its sampler's default, core/coocsc.hpp:50).
+    Median of `reps` after one warm-up each."""
     import numpy as np
 
     import oracle
     from neutronbench_amd.layout import u32_to_i64
 
-    threads = oracle.max_threads()
-    co = u32_to_i64(chunk.column_offset_gpu).cpu().numpy()
-    ro = u32_to_i64(chunk.row_offset_gpu).cpu().numpy()
+    all_threads = oracle.max_threads()
+    co = u32_to_i64(chunk.column_offset_gpu).cpu().numpy().astype(np.uint32)
+    ro = u32_to_i64(chunk.row_offset_gpu).cpu().numpy().astype(np.uint32)
+    fi = chunk.row_indices_gpu.cpu().numpy().view(np.uint32)
+    bi = chunk.column_indices_gpu.cpu().numpy().view(np.uint32)
+    fw, bw = chunk.edge_weight_forward_gpu.cpu().numpy(), chunk.edge_weight_backward_gpu.cpu().numpy()
     xs = [t.cpu().numpy() for t in (x0, h1, g1, g0)]
+    E = chunk.E
 
-    def slice_rows(offsets, indices_dev, weights_dev, rows):
-        e = int(offsets[rows])
-        idx = indices_dev[:e].cpu().numpy().view(np.uint32)
-        w = weights_dev[:e].cpu().numpy()
-        return offsets[: rows + 1].astype(np.uint32), idx, w, e
-
-    def run(rows):
-        fo, fi, fw, fe = slice_rows(co, chunk.row_indices_gpu, chunk.edge_weight_forward_gpu, rows)
-        bo, bi, bw, be = slice_rows(ro, chunk.column_indices_gpu, chunk.edge_weight_backward_gpu, rows)
+    def one(threads):
         t = time.perf_counter()
-        oracle.spmm(xs[0], fw, fo, fi, rows, threads=threads)
-        oracle.spmm(xs[1], fw, fo, fi, rows, threads=threads)
-        oracle.spmm(xs[2], bw, bo, bi, rows, threads=threads)
-        oracle.spmm(xs[3], bw, bo, bi, rows, threads=threads)
-        return time.perf_counter() - t, 2 * (fe + be)
+        oracle.spmm(xs[0], fw, co, fi, V, threads=threads)
+        oracle.spmm(xs[1], fw, co, fi, V, threads=threads)
+        oracle.spmm(xs[2], bw, ro, bi, V, threads=threads)
+        oracle.spmm(xs[3], bw, ro, bi, V, threads=threads)
+        return time.perf_counter() - t
 
-    probe_rows = min(V, 512)
-    t_probe, e_probe = run(probe_rows)
-    rate = e_probe / max(t_probe, 1e-6)
-    # rows whose four passes need about target_s at the probed rate
-    want_edges = rate * target_s
-    per_row = (co[V] + ro[V]) * 2 / V
-    rows = int(max(probe_rows, min(V, want_edges / max(per_row, 1))))
-    t_run, e_run = run(rows)
-    return {
-        "value": round(e_run / t_run, 1),
-        "unit": "edges/s",
-        "cores": threads,
-        "kind": "port",
-        "sample": f"first {rows} destination rows (forward) and first {rows} source rows (backward) of the same "
-                  f"graph, F=602 and F=128, {e_run} edge visits in {t_run:.2f} s",
-    }
+    out = {}
+    for key, threads in (("all_threads", all_threads), ("reference_default_threads", max(1, all_threads // 2 - 1))):
+        one(threads)
+        times = sorted(one(threads) for _ in range(reps))
+        med = times[len(times) // 2] if len(times) % 2 else 0.5 * (times[len(times) // 2 - 1] + times[len(times) // 2])
+        out[key] = {"value": round(4 * E / med, 1), "unit": "edges/s", "cores": threads, "kind": "port",
+                    "sample": f"the CPU oracle on the whole graph ({E} edges), four passes (F=602 and F=128, forward "
+                              f"and backward), median of {reps} after 1 warm-up: {med:.3f} s per step"}
+    return out
 
 
 def run_epoch_workload(args):

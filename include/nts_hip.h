@@ -180,7 +180,8 @@ int nts_spmm_plan_create(nts_spmm_plan_t **plan, const uint32_t *offsets, uint32
  * whose indices do not ascend (an edge file in arbitrary order; the reference's loader leaves CSR
  * rows in thread-arrival order) is cut in a copy of the index array, owned by the plan, in which
  * it is sorted (stably); the plan then gathers through that copy (E * 8 more bytes on the device)
- * and such a row's sum is associated in source order.  With 8 or more ranges, rows of more
+ * and such a row's sum is associated in source order.  With 8 or more ranges, rows of at most
+ * 4 * chunk_edges edges are cut at n_slabs / 2 ranges of twice the width, and rows of more
  * than chunk_edges / 4 edges are cut as well, at the boundaries of n_slabs / 4 four-times-wider
  * ranges (their pieces run next to the long rows' pieces of the same sources); such a row stays
  * whole when all its edges fall into one wide range.  Results differ from nts_spmm_plan_create only
@@ -201,6 +202,12 @@ int nts_spmm_plan_destroy(nts_spmm_plan_t *plan);
 /* Number of work items, split rows and partial-sum slots of a plan (for tests and reports). */
 int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows,
                        uint32_t *partials);
+/* What a call of width F through this plan keeps in the plan's scratch, and what the schedule found:
+ * bytes of partial sums, bytes of the padded input copy (0 when the call gathers from `in` itself),
+ * the number of edges that repeat the gather index of the edge before them in their row, and whether
+ * calls load a source row once per run of such edges.  Any out-pointer may be NULL. */
+int nts_spmm_plan_scratch_info(nts_spmm_plan_t *plan, uint32_t F, size_t *partial_bytes, size_t *padded_input_bytes,
+                               uint64_t *repeated_edges, int *loads_once_per_run);
 /* Grow the plan's scratch (partial sums of split rows; for a schedule with runs of equal indices
  * also a copy of the input with padded rows, see below) so that a later call of width F allocates
  * nothing. */

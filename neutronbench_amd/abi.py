@@ -60,6 +60,8 @@ SIGNATURES = {
                                     ctypes.POINTER(_u32), ctypes.POINTER(_u32)],
     "nts_spmm_plan_destroy": [_vp],
     "nts_spmm_plan_info": [_vp, ctypes.POINTER(_u32), ctypes.POINTER(_u32), ctypes.POINTER(_u32)],
+    "nts_spmm_plan_scratch_info": [_vp, _u32, ctypes.POINTER(_sz), ctypes.POINTER(_sz), ctypes.POINTER(_u64),
+                                   ctypes.POINTER(_int)],
     "nts_spmm_plan_reserve": [_vp, _u32],
     "nts_spmm_gather_planned": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _int, _vp],
     "nts_scatter_src_to_edge": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],

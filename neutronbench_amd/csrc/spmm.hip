@@ -347,7 +347,7 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
 // Sub-wavefront variant for narrow rows: G lanes per row (G = 4, 8, 16 or 32), 64/G rows per
 // wavefront, one VEC-wide accumulator per lane (F <= G*VEC).  Neighbour pairs are fetched G at a
 // time per group and broadcast inside the group with cross-lane shuffles.
-template <int G, int VEC, bool HEADS, bool REMAP>
+template <int G, int VEC, bool HEADS, bool REMAP, bool RUNS>
 __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict__ in, float *__restrict__ out,
                                                          const float *__restrict__ w,
                                                          const uint32_t *__restrict__ offsets,
@@ -398,6 +398,8 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
   };
   uint32_t nxt_i, nxt_s;
   fetch_pair(e0 + gl, nxt_i, nxt_s);
+  V held = vzero<VEC>();            // RUNS: the row loaded last and its index
+  uint32_t held_i = 0xFFFFFFFFu;
   for (uint32_t eb = e0; eb < e1; eb += G) {
     const uint32_t n = min(static_cast<uint32_t>(G), e1 - eb);
     const uint32_t my_i = nxt_i, my_s = nxt_s;
@@ -413,6 +415,25 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
       }
       V v[U];
       float wv[U];
+      if (RUNS) {
+        // An edge that repeats its predecessor's index (a parallel edge) does not load the row again:
+        // the group keeps the last row it loaded in `held` and adds it with the edge's own weight.
+        bool fresh[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          fresh[u] = si[u] != (u ? si[u - 1] : held_i);
+          v[u] = vzero<VEC>();
+          if (fresh[u]) v[u] = *reinterpret_cast<const V *>(in + static_cast<size_t>(si[u]) * F + lcol);
+          wv[u] = HEADS ? w[static_cast<size_t>(ss[u]) * heads.H + head] : __uint_as_float(ss[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (fresh[u]) held = v[u];
+          vfma(acc, held, wv[u]);
+        }
+        held_i = si[U - 1];
+        continue;
+      }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         v[u] = *reinterpret_cast<const V *>(in + static_cast<size_t>(si[u]) * F + lcol);
@@ -427,6 +448,12 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
       const uint32_t si = __shfl(my_i, j, G);
       const uint32_t ss = __shfl(my_s, j, G);
       const float wgt = HEADS ? w[static_cast<size_t>(ss) * heads.H + head] : __uint_as_float(ss);
+      if (RUNS) {
+        if (si != held_i) held = *reinterpret_cast<const V *>(in + static_cast<size_t>(si) * F + lcol);
+        held_i = si;
+        vfma(acc, held, wgt);
+        continue;
+      }
       vfma(acc, *reinterpret_cast<const V *>(in + static_cast<size_t>(si) * F + lcol), wgt);
     }
   }
@@ -610,14 +637,18 @@ template <int G, int VEC>
 void launch_group(const LaunchArgs &a) {
   const uint32_t per_block = 256 / G;
   const uint32_t blocks = ceil_div(a.n_items, per_block);
-#define NTS_LAUNCH_GROUP(HD, RM)                                                                                  \
-  hipLaunchKernelGGL((spmm_group_kernel<G, VEC, HD, RM>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w, \
-                     a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads, \
+#define NTS_LAUNCH_GROUP(HD, RM, RUNS)                                                                                  \
+  hipLaunchKernelGGL((spmm_group_kernel<G, VEC, HD, RM, RUNS>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w, \
+                     a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,     \
                      a.row_edge_limit, a.edge_ids)
   if (a.edge_ids) {
-    if (a.heads.H) NTS_LAUNCH_GROUP(true, true); else NTS_LAUNCH_GROUP(false, true);
+    if (a.heads.H) NTS_LAUNCH_GROUP(true, true, false);
+    else if (a.dup_runs) NTS_LAUNCH_GROUP(false, true, true);
+    else NTS_LAUNCH_GROUP(false, true, false);
   } else {
-    if (a.heads.H) NTS_LAUNCH_GROUP(true, false); else NTS_LAUNCH_GROUP(false, false);
+    if (a.heads.H) NTS_LAUNCH_GROUP(true, false, false);
+    else if (a.dup_runs) NTS_LAUNCH_GROUP(false, false, true);
+    else NTS_LAUNCH_GROUP(false, false, false);
   }
 #undef NTS_LAUNCH_GROUP
 }
@@ -1068,10 +1099,12 @@ void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx_in, u
   uint32_t n_partials = 0;
   std::vector<uint32_t> bucket(static_cast<size_t>(chunk) + 2, 0u);
   const bool slabbed = n_slabs > 1 && idx != nullptr && n_index > 0;
-  // Source ranges come in two widths and a row is cut at the width that suits its length: every
+  // Source ranges come in three widths and a row is cut at the width that suits its length: every
   // piece costs one partial row (written, then read by the second stage), so shorter rows get
   // fewer, wider ranges.
-  //   more than chunk edges        n_slabs ranges
+  //   more than 4 * chunk edges    n_slabs ranges
+  //   more than chunk edges        n_slabs / 2 ranges (2,048-edge rows at 32 ranges would be cut into 19-edge
+  //                                pieces on average; 24.7 -> 24.2 ms per four-pass step on the 114.8 M-edge graph)
   //   more than chunk / 4 edges    n_slabs / 4 ranges; a row whose edges all fall into one of them stays whole
   // A piece is issued with the first narrow range it covers, so that wavefronts resident at the
   // same time gather from the same part of the source rows whatever the width of their ranges.
@@ -1161,7 +1194,7 @@ void make_schedule(Schedule &out, const uint32_t *off, const uint32_t *idx_in, u
     }
     const uint32_t first = n_partials;
     if (slabbed) {
-      range_stops(b, e, n_slabs);
+      range_stops(b, e, (wide_ranges && deg <= 4 * static_cast<uint64_t>(chunk)) ? n_slabs / 2 : n_slabs);
       uint32_t from = b;
       for (size_t q = 0; q < stops.size(); q += 2) {
         for (uint32_t k = from; k < stops[q + 1]; k += chunk)
@@ -1417,6 +1450,19 @@ int leave_stream(nts_spmm_plan *plan, hipStream_t stream) {
 }
 
 }  // namespace
+
+int nts_spmm_plan_scratch_info(nts_spmm_plan_t *plan, uint32_t F, size_t *partial_bytes, size_t *padded_input_bytes,
+                               uint64_t *repeated_edges, int *loads_once_per_run) {
+  NTS_TRACE_RANGE("nts_spmm_plan_scratch_info");
+  if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_scratch_info: null plan");
+  if (F == 0) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_scratch_info: F is 0");
+  const uint32_t ld = padded_stride(plan, F, false);
+  if (partial_bytes) *partial_bytes = static_cast<size_t>(plan->n_partials) * (ld ? ld : F) * sizeof(float);
+  if (padded_input_bytes) *padded_input_bytes = ld ? static_cast<size_t>(plan->n_index) * ld * sizeof(float) : 0;
+  if (repeated_edges) *repeated_edges = plan->repeated_edges;
+  if (loads_once_per_run) *loads_once_per_run = use_runs(plan) ? 1 : 0;
+  return NTS_OK;
+}
 
 int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F) {
   NTS_TRACE_RANGE("nts_spmm_plan_reserve");

@@ -8,6 +8,7 @@ torch has no uint32 arithmetic, so tensors are stored as int32 with the same bit
 kernels read them as uint32.
 """
 import ctypes
+import time
 
 import torch
 
@@ -51,6 +52,14 @@ class SpmmPlan:
     def reserve(self, F):
         call("nts_spmm_plan_reserve", self.handle, F)
 
+    def scratch_info(self, F):
+        """Scratch a call of width F keeps in the plan and what the schedule found about parallel edges."""
+        pb, ib, rep, runs = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_uint64(), ctypes.c_int()
+        call("nts_spmm_plan_scratch_info", self.handle, F, ctypes.byref(pb), ctypes.byref(ib), ctypes.byref(rep),
+             ctypes.byref(runs))
+        return dict(partial_bytes=pb.value, padded_input_bytes=ib.value, repeated_edges=rep.value,
+                    loads_once_per_run=bool(runs.value))
+
     def close(self):
         if self.handle:
             call("nts_spmm_plan_destroy", self.handle)
@@ -77,12 +86,15 @@ class FullGraphChunk:
         self.edge_weight_backward_gpu = ewb
         self.src_range = (0, V)
         self.dst_range = (0, V)
+        torch.cuda.current_stream(column_offset.device).synchronize()
+        t0 = time.perf_counter()
         if n_slabs == 1:
             self.plan_forward = SpmmPlan(column_offset, V, self.E, chunk_edges)
             self.plan_backward = SpmmPlan(row_offset, V, self.E, chunk_edges)
         else:
             self.plan_forward = SpmmPlan(column_offset, V, self.E, chunk_edges, row_indices, V, n_slabs)
             self.plan_backward = SpmmPlan(row_offset, V, self.E, chunk_edges, column_indices, V, n_slabs)
+        self.plan_build_s = time.perf_counter() - t0  # both schedules (host side, read-backs and uploads included)
 
     @classmethod
     def from_edges(cls, src, dst, V, chunk_edges=0, n_slabs=1):

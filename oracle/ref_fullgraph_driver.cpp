@@ -16,11 +16,12 @@
 //
 //   usage: ref_fullgraph <edge_file> <vertices> <F> <H> <prefix> <cpu|gpu|both|agg-cpu>
 //   agg-cpu runs ForwardCPUfuseOp only; <F> may be a comma-separated list, and for every width the
-//   input is <prefix>.x<F>.  Three timed repetitions per width, best forward and backward time
-//   printed: the CPU baseline of the aggregation benchmark.
+//   input is <prefix>.x<F>.  NTS_REF_WARMUP (default 2) untimed and NTS_REF_REPS (default 5) timed
+//   repetitions per width; the median and the best forward and backward times are printed: the CPU
+//   baseline of the aggregation benchmark.
 //   agg-gpu (GPU build only): ForwardSingleGPUfuseOp only, on the reference's GPU chunk
-//   (GenerateAll(GPU_T) + CopyGraphToDevice), same width list and inputs as agg-cpu; prints the best
-//   wall time of forward and backward (each call ends with the operator's own stream synchronisation).
+//   (GenerateAll(GPU_T) + CopyGraphToDevice), same width list, inputs and repetitions as agg-cpu; prints
+//   the median and best wall time of forward and backward (each call ends with the operator's own stream synchronisation).
 //   samp (GPU build only, but makes no device call): <H> is a number of sampled layers; for layer k
 //   the files <prefix>.l<k>.dst [Vd], .co [Vd+1], .ri [E] (uint32; ri = GLOBAL source ids of the
 //   sampled edges) are run through the reference's sampCSC (core/coocsc.hpp): postprocessing,
@@ -61,6 +62,13 @@
 #include <vector>
 
 static std::string g_prefix;
+static int g_warmup = 2, g_reps = 5;  // NTS_REF_WARMUP / NTS_REF_REPS (timing modes)
+
+static double median(std::vector<double> v) {
+  std::sort(v.begin(), v.end());
+  const size_t n = v.size();
+  return n == 0 ? 0.0 : (n % 2 ? v[n / 2] : 0.5 * (v[n / 2 - 1] + v[n / 2]));
+}
 
 static NtsVar read_matrix(const std::string &name, long rows, long cols) {
   const std::string path = g_prefix + "." + name;
@@ -179,6 +187,8 @@ int main(int argc, char **argv) {
   const int F = widths.at(0);
   const int H = std::stoi(argv[4]);
   g_prefix = argv[5];
+  if (const char *e = getenv("NTS_REF_WARMUP")) g_warmup = std::max(0, atoi(e));
+  if (const char *e = getenv("NTS_REF_REPS")) g_reps = std::max(1, atoi(e));
   const std::string mode = argv[6];
   const bool agg_only = mode == "agg-cpu";
   const bool run_cpu = mode == "cpu" || mode == "both";
@@ -211,18 +221,22 @@ int main(int argc, char **argv) {
     nts::op::ForwardSingleGPUfuseOp op(pgg, all);
     for (int width : widths) {
       NtsVar X = read_matrix("x" + std::to_string(width), vertices, width).cuda();
-      double best_f = 1e30, best_b = 1e30;
-      for (int rep = 0; rep < 5; ++rep) {
+      std::vector<double> tf, tb;
+      for (int rep = 0; rep < g_warmup + g_reps; ++rep) {
         double t0 = now();
         NtsVar Y = op.forward(X);
         double t1 = now();
         NtsVar G = op.backward(X);
         double t2 = now();
-        best_f = std::min(best_f, t1 - t0);
-        best_b = std::min(best_b, t2 - t1);
+        if (rep >= g_warmup) {
+          tf.push_back(t1 - t0);
+          tb.push_back(t2 - t1);
+        }
       }
-      printf("reference ForwardSingleGPUfuseOp over libntship timing: V=%u E=%u F=%d forward_s=%.6f backward_s=%.6f\n",
-             vertices, pgg->owned_edges, width, best_f, best_b);
+      printf("reference ForwardSingleGPUfuseOp over libntship timing: V=%u E=%u F=%d forward_s=%.6f backward_s=%.6f "
+             "best_forward_s=%.6f best_backward_s=%.6f reps=%d warmup=%d\n",
+             vertices, pgg->owned_edges, width, median(tf), median(tb), *std::min_element(tf.begin(), tf.end()),
+             *std::min_element(tb.begin(), tb.end()), g_reps, g_warmup);
     }
     return 0;
   }
@@ -272,18 +286,22 @@ int main(int argc, char **argv) {
     nts::op::ForwardCPUfuseOp op(pg, active);
     for (int width : widths) {
       NtsVar X = read_matrix("x" + std::to_string(width), V, width);
-      double best_f = 1e30, best_b = 1e30;
-      for (int rep = 0; rep < 3; ++rep) {
+      std::vector<double> tf, tb;
+      for (int rep = 0; rep < g_warmup + g_reps; ++rep) {
         double t0 = now();
         NtsVar Y = op.forward(X);
         double t1 = now();
         NtsVar G = op.backward(X);
         double t2 = now();
-        best_f = std::min(best_f, t1 - t0);
-        best_b = std::min(best_b, t2 - t1);
+        if (rep >= g_warmup) {
+          tf.push_back(t1 - t0);
+          tb.push_back(t2 - t1);
+        }
       }
-      printf("reference ForwardCPUfuseOp timing: V=%ld E=%ld F=%d forward_s=%.6f backward_s=%.6f threads=%d\n", V, E,
-             width, best_f, best_b, graph->threads);
+      printf("reference ForwardCPUfuseOp timing: V=%ld E=%ld F=%d forward_s=%.6f backward_s=%.6f threads=%d "
+             "best_forward_s=%.6f best_backward_s=%.6f reps=%d warmup=%d\n",
+             V, E, width, median(tf), median(tb), graph->threads, *std::min_element(tf.begin(), tf.end()),
+             *std::min_element(tb.begin(), tb.end()), g_reps, g_warmup);
     }
     return 0;
   }

@@ -292,7 +292,7 @@ def test_forced_kernel_variants_in_a_fresh_process(device, runs, pad):
     assert r.returncode == 0, r.stdout[-1500:]
 
 
-@pytest.mark.parametrize("F", [130, 200, 301, 602, 256, 1433])
+@pytest.mark.parametrize("F", [16, 100, 128, 130, 200, 301, 602, 256, 1433])
 def test_runs_of_equal_indices_are_loaded_once_and_added_edge_by_edge(device, F):
     """A multigraph block with sorted rows: two thirds of the edges repeat their predecessor's index,
     so the schedule turns on the one-load-per-run kernel (and, for widths that are not multiples of

@@ -84,11 +84,13 @@ def check_ranges(pieces, ri, deg, Vs, chunk, slabs):
     width = -(-Vs // slabs)
     first_range = ri[pieces[:, 1]] // width
     last_range = ri[pieces[:, 2] - 1] // width
-    wide = deg[pieces[:, 0]] <= chunk  # second-tier rows use ranges four times as wide
-    issue = np.where(wide, first_range // 4 * 4, first_range)
+    # with 8 or more ranges: rows of at most `chunk` edges use ranges four times as wide, rows of at
+    # most 4 * chunk edges ranges twice as wide
+    d = deg[pieces[:, 0]]
+    m = np.where(d <= chunk, 4, np.where(d <= 4 * chunk, 2, 1)) if slabs >= 8 else np.ones_like(d)
+    issue = first_range // m * m
     assert np.all(issue[1:] >= issue[:-1])
-    assert np.all(last_range[~wide] == first_range[~wide])
-    assert np.all(last_range[wide] // 4 == first_range[wide] // 4)
+    assert np.all(last_range // m == first_range // m)
 
 
 @pytest.mark.parametrize("chunk,slabs", [(512, 32), (64, 8), (100, 16), (32, 4), (16, 3), (4096, 1)])
