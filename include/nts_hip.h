@@ -363,6 +363,25 @@ int nts_gather_rows_cached_f32(float *out, const float *table, const float *cach
 int nts_gather_labels_i64(int64_t *out, const int64_t *table, const uint32_t *ids, uint32_t n,
                           uint32_t classes, nts_stream_t stream);
 
+/* Vertex rows that arrive as message records.  The reference's full-graph GPU operators
+ * (ForwardGPUfuseOp, core/ntsDistGPUFusedGraphOp.hpp:49-91; scheduler calls core/NtsScheduler.hpp:300-314)
+ * exchange rows between partitions as records {uint32 vertex id, F floats} in a pinned host buffer --
+ * also when the one partition of a single-GPU run sends to itself.  `records` (device memory or mapped
+ * host memory) holds n_records records of 4 * (F + 1) bytes; records whose id lies outside
+ * [id_begin, id_end) are skipped.
+ *   nts_message_rows_unpack  Cuda_Stream::deSerializeToGPU (cuda/ntsCUDA.hpp:118-121; kernel
+ *                            cuda/ntsCUDATransferKernel.cuh:66-93): rows[id - id_begin, :] = record values
+ *   nts_message_rows_add     Cuda_Stream::aggregate_comm_result_debug (cuda/ntsCUDA.hpp:113-117; kernel
+ *                            :43-64): rows[id - id_begin, :] += record values, without the reference's
+ *                            float atomics: records that name distinct rows are added in parallel,
+ *                            and a buffer that names a row twice is added in record order, so the
+ *                            result is reproducible either way.  Takes 4 * (id_end - id_begin + 1) bytes
+ *                            of stream-ordered scratch (see nts_scratch_trim). */
+int nts_message_rows_unpack(float *rows, const float *records, uint32_t n_records, uint32_t F, uint32_t id_begin,
+                            uint32_t id_end, nts_stream_t stream);
+int nts_message_rows_add(float *rows, const float *records, uint32_t n_records, uint32_t F, uint32_t id_begin,
+                         uint32_t id_end, nts_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Sampled-layer index construction on the device (sampCSC, core/coocsc.hpp)
  * ------------------------------------------------------------------------------------------- */
@@ -507,6 +526,12 @@ int nts_read_feature_label_mask(const char *path_f, const char *path_l, const ch
                                 uint32_t F, uint32_t classes, float *local_feature, int64_t *local_label,
                                 int32_t *local_mask, int64_t *global_label, int32_t *global_mask,
                                 int threads);
+/* Writes the feature file nts_read_feature_label_mask reads, in the form the reference's data
+ * preparation produces (data/generate_nts_dataset.py:308, 356-359: "%.4f" after the id): record r is
+ * "id f0 .. fF-1" with id = ids[r] (ids NULL: r) and every value printed with `decimals` (0..9) digits
+ * after the point.  Formatting runs on `threads` host threads (<= 0: all). */
+int nts_feature_text_write(const char *path, const float *table, const uint32_t *ids, uint32_t V, uint32_t F,
+                           int decimals, int threads);
 /* Comma-separated feature file of readFeature_Label_Mask_OGB (core/ntsDataloador.hpp:397-437): line k
  * holds the F values of vertex k; each field is converted with atof and narrowed to float. */
 int nts_feature_csv_read(const char *path, float *table, uint32_t V, uint32_t F, int threads);

@@ -80,6 +80,8 @@ SIGNATURES = {
     "nts_gather_rows_f32": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],
     "nts_gather_rows_cached_f32": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp],
     "nts_gather_labels_i64": [_vp, _vp, _vp, _u32, _u32, _vp],
+    "nts_message_rows_unpack": [_vp, _vp, _u32, _u32, _u32, _u32, _vp],
+    "nts_message_rows_add": [_vp, _vp, _u32, _u32, _u32, _u32, _vp],
     "nts_sample_hop_work_bytes": [_u32],
     "nts_sample_hop_offsets": [_vp, _vp, _vp, _u32, ctypes.c_int32, _vp, _vp],
     "nts_sample_hop_neighbors": [_vp, _vp, _vp, _vp, _vp, _u32, ctypes.c_int32, ctypes.c_uint64, _vp],
@@ -99,6 +101,7 @@ SIGNATURES = {
     "nts_edge_file_count": [_str, ctypes.POINTER(_u64)],
     "nts_edge_file_read": [_str, _vp, _u64, _u64, ctypes.POINTER(_u32)],
     "nts_read_feature_label_mask": [_str, _str, _str, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _int],
+    "nts_feature_text_write": [_str, _vp, _vp, _u32, _u32, _int, _int],
     "nts_feature_csv_read": [_str, _vp, _u32, _u32, _int],
     "nts_int_list_text_read": [_str, _vp, _u64, ctypes.POINTER(_u64)],
     "nts_table_bin_write": [_str, _vp, _u64, _u64, _u32],

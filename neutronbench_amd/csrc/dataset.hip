@@ -524,6 +524,37 @@ int nts_table_bin_write(const char *path, const void *data, uint64_t rows, uint6
   return ok ? NTS_OK : fail(NTS_ERR_INVALID, "nts_table_bin_write: write failed");
 }
 
+int nts_feature_text_write(const char *path, const float *table, const uint32_t *ids, uint32_t V, uint32_t F,
+                           int decimals, int threads) {
+  NTS_TRACE_RANGE("nts_feature_text_write");
+  if (!path || (!table && static_cast<uint64_t>(V) * F)) return fail(NTS_ERR_INVALID, "nts_feature_text_write: null argument");
+  if (decimals < 0 || decimals > 9) return fail(NTS_ERR_INVALID, "nts_feature_text_write: decimals outside 0..9");
+  const int T = clamp_threads(threads, static_cast<size_t>(V) * F * 4);
+  // Each thread formats a contiguous block of records into its own buffer; the buffers are then
+  // written in order.
+  std::vector<std::string> parts(T);
+  const uint32_t per = (V + T - 1) / T;
+  run_threads(T, [&](int t) {
+    const uint32_t r0 = std::min<uint64_t>(V, static_cast<uint64_t>(t) * per), r1 = std::min<uint64_t>(V, r0 + per);
+    std::string &out = parts[t];
+    out.reserve(static_cast<size_t>(r1 - r0) * (12 + static_cast<size_t>(F) * (decimals + 6)));
+    char buf[64];
+    for (uint32_t r = r0; r < r1; ++r) {
+      out.append(buf, static_cast<size_t>(snprintf(buf, sizeof buf, "%u", ids ? ids[r] : r)));
+      const float *row = table + static_cast<size_t>(r) * F;
+      for (uint32_t c = 0; c < F; ++c)
+        out.append(buf, static_cast<size_t>(snprintf(buf, sizeof buf, " %.*f", decimals, static_cast<double>(row[c]))));
+      out.push_back('\n');
+    }
+  });
+  FILE *f = fopen(path, "wb");
+  if (!f) return fail(NTS_ERR_INVALID, (std::string("nts_feature_text_write: cannot create ") + path).c_str());
+  bool ok = true;
+  for (const std::string &part : parts) ok = ok && fwrite(part.data(), 1, part.size(), f) == part.size();
+  ok = fclose(f) == 0 && ok;
+  return ok ? NTS_OK : fail(NTS_ERR_INVALID, "nts_feature_text_write: write failed");
+}
+
 int nts_table_bin_info(const char *path, uint64_t *rows, uint64_t *cols, uint32_t *elem_bytes) {
   NTS_TRACE_RANGE("nts_table_bin_info");
   if (!path) return fail(NTS_ERR_INVALID, "nts_table_bin_info: null path");

@@ -5,6 +5,8 @@
 // A group of G lanes (G chosen so that G*VEC*4 bytes covers a row with little idle width) moves
 // one row with 4/8/16-byte accesses; 64/G rows per wavefront.  Wide accesses matter most on the
 // zero-copy path, where every wave load becomes PCIe read requests.
+#include <algorithm>
+
 #include "common.hpp"
 
 namespace nts {
@@ -167,12 +169,115 @@ void launch_rows_any(const RowsArgs &a) {
   return launch_rows_v<float>(a, a.F);
 }
 
+// ---- rows that arrive as message records -----------------------------------------------------------
+// The reference's full-graph GPU operators (ForwardGPUfuseOp, core/ntsDistGPUFusedGraphOp.hpp:49-91) move
+// vertex rows between partitions as records {uint32 vertex id, F floats} in a pinned host buffer, also
+// when the one partition sends to itself.  A wavefront takes one record at a time; its lanes cover
+// the columns (records are 4 * (F + 1) bytes long, so rows are only 4-byte aligned).
+
+__global__ __launch_bounds__(256) void message_rows_unpack_kernel(float *__restrict__ rows,
+                                                                  const float *__restrict__ records, uint32_t n,
+                                                                  uint32_t F, uint32_t id_begin, uint32_t id_end) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint64_t waves = static_cast<uint64_t>(gridDim.x) * (blockDim.x / kWave);
+  for (uint64_t k = static_cast<uint64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave; k < n; k += waves) {
+    const float *rec = records + k * (static_cast<uint64_t>(F) + 1);
+    const uint32_t id = __float_as_uint(rec[0]);
+    if (id < id_begin || id >= id_end) continue;
+    float *dst = rows + static_cast<size_t>(id - id_begin) * F;
+    for (uint32_t c = lane; c < F; c += kWave) dst[c] = rec[1 + c];
+  }
+}
+
+// Counts how many records name each row; *repeated becomes non-zero when some row is named twice.
+__global__ __launch_bounds__(256) void message_rows_claim_kernel(uint32_t *__restrict__ claims,
+                                                                 uint32_t *__restrict__ repeated,
+                                                                 const float *__restrict__ records, uint32_t n,
+                                                                 uint32_t F, uint32_t id_begin, uint32_t id_end) {
+  const uint64_t k = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (k >= n) return;
+  const uint32_t id = __float_as_uint(records[k * (static_cast<uint64_t>(F) + 1)]);
+  if (id < id_begin || id >= id_end) return;
+  if (atomicAdd(&claims[id - id_begin], 1u) != 0u) atomicOr(repeated, 1u);
+}
+
+// rows[id - id_begin, :] += record values.  Records that name distinct rows (what the reference's
+// operators send: one record per vertex and buffer) are added in parallel, each row by one
+// wavefront, without atomics.  If two records of the buffer name the same row, the additions run in
+// record order instead (one thread per column walks the buffer), so the result does not depend on
+// scheduling either way.
+__global__ __launch_bounds__(256) void message_rows_add_kernel(float *__restrict__ rows,
+                                                               const float *__restrict__ records, uint32_t n,
+                                                               uint32_t F, uint32_t id_begin, uint32_t id_end,
+                                                               const uint32_t *__restrict__ repeated) {
+  const uint64_t stride = static_cast<uint64_t>(F) + 1;
+  if (*repeated) {
+    const uint64_t c = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= F) return;
+    for (uint64_t k = 0; k < n; ++k) {
+      const uint32_t id = __float_as_uint(records[k * stride]);
+      if (id < id_begin || id >= id_end) continue;
+      rows[static_cast<size_t>(id - id_begin) * F + c] += records[k * stride + 1 + c];
+    }
+    return;
+  }
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint64_t waves = static_cast<uint64_t>(gridDim.x) * (blockDim.x / kWave);
+  for (uint64_t k = static_cast<uint64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave; k < n; k += waves) {
+    const float *rec = records + k * stride;
+    const uint32_t id = __float_as_uint(rec[0]);
+    if (id < id_begin || id >= id_end) continue;
+    float *dst = rows + static_cast<size_t>(id - id_begin) * F;
+    for (uint32_t c = lane; c < F; c += kWave) dst[c] += rec[1 + c];
+  }
+}
+
 }  // namespace
 }  // namespace nts
 
 using namespace nts;
 
 extern "C" {
+
+int nts_message_rows_unpack(float *rows, const float *records, uint32_t n_records, uint32_t F, uint32_t id_begin,
+                            uint32_t id_end, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_message_rows_unpack");
+  if (F == 0) return fail(NTS_ERR_INVALID, "nts_message_rows_unpack: F is 0");
+  if (n_records == 0 || id_end <= id_begin) return NTS_OK;
+  if (!rows || !records) return fail(NTS_ERR_INVALID, "nts_message_rows_unpack: null pointer");
+  const uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>((static_cast<uint64_t>(n_records) + 3) / 4, 16384));
+  hipLaunchKernelGGL(message_rows_unpack_kernel, dim3(blocks), dim3(256), 0, stream, rows, records, n_records, F,
+                     id_begin, id_end);
+  NTS_LAUNCH_CHECK("nts_message_rows_unpack");
+  return NTS_OK;
+}
+
+int nts_message_rows_add(float *rows, const float *records, uint32_t n_records, uint32_t F, uint32_t id_begin,
+                         uint32_t id_end, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_message_rows_add");
+  if (F == 0) return fail(NTS_ERR_INVALID, "nts_message_rows_add: F is 0");
+  if (n_records == 0 || id_end <= id_begin) return NTS_OK;
+  if (!rows || !records) return fail(NTS_ERR_INVALID, "nts_message_rows_add: null pointer");
+  const size_t words = static_cast<size_t>(id_end - id_begin) + 1;  // claims per row, then the flag
+  uint32_t *claims = nullptr;
+  NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&claims), words * sizeof(uint32_t), stream));
+  int rc = nts_memset_zero(claims, words * sizeof(uint32_t), stream);
+  if (rc == NTS_OK) {
+    uint32_t *repeated = claims + (words - 1);
+    hipLaunchKernelGGL(message_rows_claim_kernel, dim3((n_records + 255) / 256), dim3(256), 0, stream, claims, repeated,
+                       records, n_records, F, id_begin, id_end);
+    // enough blocks for one wavefront per record and for one thread per column
+    const uint64_t want = std::max<uint64_t>((static_cast<uint64_t>(n_records) + 3) / 4, (static_cast<uint64_t>(F) + 255) / 256);
+    const uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>(want, 16384));
+    hipLaunchKernelGGL(message_rows_add_kernel, dim3(std::max(blocks, (F + 255) / 256)), dim3(256), 0, stream, rows,
+                       records, n_records, F, id_begin, id_end, repeated);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) rc = fail_hip(err, "nts_message_rows_add");
+  }
+  const hipError_t ferr = scratch_free(claims, stream);
+  if (rc == NTS_OK && ferr != hipSuccess) rc = fail_hip(ferr, "nts_message_rows_add: scratch_free");
+  return rc;
+}
 
 int nts_gather_rows_f32(float *out, const float *table, const uint32_t *row_ids, const uint32_t *sel,
                         const uint32_t *remap, uint32_t n, uint32_t F, nts_stream_t stream) {

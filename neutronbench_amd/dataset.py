@@ -74,6 +74,36 @@ def write_edge_file(path, pairs):
     np.ascontiguousarray(pairs, dtype=np.uint32).tofile(path)
 
 
+def write_feature_file(path, features, ids=None, decimals=4, threads=0):
+    """Text feature file as data/generate_nts_dataset.py writes it: one record per line,
+    "id f0 f1 ... fF-1", values printed with `decimals` digits after the point (so the file holds the
+    rounded values, which is what a reader then sees)."""
+    features = np.ascontiguousarray(features, dtype=np.float32)
+    V, F = features.shape
+    ids32 = None if ids is None else np.ascontiguousarray(ids, dtype=np.uint32)
+    call("nts_feature_text_write", _path(path), _np_ptr(features), _np_ptr(ids32) if ids32 is not None else 0, V, F,
+         decimals, threads)
+
+
+def write_label_file(path, labels, ids=None):
+    """"id label" per line (single-label form)."""
+    labels = np.asarray(labels).astype(np.int64)
+    ids = np.arange(labels.size) if ids is None else np.asarray(ids)
+    np.savetxt(path, np.stack([ids, labels], 1), fmt="%d")
+
+
+MASK_WORDS = ("train", "val", "test")
+
+
+def write_mask_file(path, mask, ids=None):
+    """"id word" per line; mask values 0 / 1 / 2 are written as train / val / test, anything else
+    as "unknown" (which the readers store as 3)."""
+    mask = np.asarray(mask)
+    ids = np.arange(mask.size) if ids is None else np.asarray(ids)
+    with open(path, "w") as f:
+        f.write("".join(f"{i} {MASK_WORDS[m] if 0 <= m < 3 else 'unknown'}\n" for i, m in zip(ids.tolist(), mask.tolist())))
+
+
 class GNNDatum:
     """local_feature [V, F] float32, local_label / global_label int64, local_mask / global_mask int32
     of one partition that owns every vertex (core/ntsDataloador.hpp:36-88)."""

@@ -490,16 +490,28 @@ class Cuda_Stream {
                                   VertexId_CUDA feature_size, bool with_weight = false, bool tensor_weight = false);
   void zero_copy_embedding_move_gpu(float *dev_feature, float *pinned_host_feature, VertexId_CUDA feature_size,
                                     VertexId_CUDA vertex_size);
-  // Unpacking of multi-rank MPI message buffers (cuda/ntsCUDATransferKernel.cuh:30-93): part of the
-  // distributed path, which this single-GPU library does not implement.  They fail loudly.
+  // Rows that arrive as message records {vertex id, F floats} (cuda/ntsCUDATransferKernel.cuh:43-93): the
+  // full-graph operators ForwardGPUfuseOp / DistGPUGetDepNbrOp exchange rows this way, also when the
+  // one partition of a single-GPU run sends to itself (core/NtsScheduler.hpp:300-314).
+  void aggregate_comm_result_debug(float *aggregate_buffer, float *input_buffer, VertexId_CUDA data_size,
+                                   VertexId_CUDA feature_size, VertexId_CUDA partition_start,
+                                   VertexId_CUDA partition_end, bool sync) {
+    (void)sync;
+    nts_veneer::note_write(aggregate_buffer);
+    NTS_VENEER_CHECK(nts_message_rows_add(aggregate_buffer, input_buffer, data_size, feature_size, partition_start,
+                                          partition_end, stream));
+  }
+  void deSerializeToGPU(float *input_gpu_buffer, float *input_buffer, VertexId_CUDA data_size,
+                        VertexId_CUDA feature_size, VertexId_CUDA partition_start, VertexId_CUDA partition_end,
+                        bool sync) {
+    (void)sync;
+    nts_veneer::note_write(input_gpu_buffer);
+    NTS_VENEER_CHECK(nts_message_rows_unpack(input_gpu_buffer, input_buffer, data_size, feature_size, partition_start,
+                                             partition_end, stream));
+  }
+  // The reference's kernel behind this one adds the message buffer to itself and prints
+  // (cuda/ntsCUDATransferKernel.cuh:30-41); nothing in core/ calls it.  It fails loudly.
   void aggregate_comm_result(float *, float *, VertexId_CUDA, int, int, bool = true) { dist_unsupported(); }
-  void aggregate_comm_result_debug(float *, float *, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA,
-                                   bool) {
-    dist_unsupported();
-  }
-  void deSerializeToGPU(float *, float *, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA, VertexId_CUDA, bool) {
-    dist_unsupported();
-  }
 
   // Mini-batch assembly; like the reference these return with the result complete.
   void zero_copy_feature_move_gpu(float *dev_feature, float *pinned_host_feature, VertexId_CUDA *src_vertex,
@@ -542,7 +554,7 @@ class Cuda_Stream {
 
  private:
   static void dist_unsupported() {
-    printf("the distributed (MPI message buffer) GPU path is not part of the single-GPU HIP library\n");
+    printf("Cuda_Stream::aggregate_comm_result has no defined result in the reference and is not implemented\n");
     exit(1);
   }
   static void reject_tensor_weight(bool tensor) {
