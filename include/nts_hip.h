@@ -3,9 +3,13 @@
  * single-GPU graph-operator kernels of NeutronBench.
  *
  * Every entry point is `extern "C"`, takes plain pointers and sizes, receives the HIP stream
- * explicitly, returns an int status (0 = NTS_OK) and never prints or exits.  There is no global
- * mutable state: calls on different streams are independent and the library is re-entrant, which
- * is what the reference's pipelined mini-batch loop needs (one Cuda_Stream per host thread,
+ * explicitly, returns an int status (0 = NTS_OK) and never prints or exits.  State that outlives a
+ * call is either in a handle the caller owns (a schedule, a batch builder: calls on one handle are
+ * serialised by the library, see each) or one of three process-wide items that are safe to share: a
+ * per-device pool that keeps freed scratch (thread-safe, stream-ordered), the per-thread last-error
+ * text, and the fixed scratch array of nts_spmm_gather_static_scratch (whose calls a caller must
+ * serialise).  Calls on different streams and host threads are otherwise independent, which is what
+ * the reference's pipelined mini-batch loop needs (one Cuda_Stream per host thread,
  * toolkits/GCN_GPU_NEIGHBOR.hpp:1350-1363).
  *
  * Conventions: indices are uint32 (VertexId_CUDA, cuda/cuda_type.h:21), values are fp32, labels
@@ -104,6 +108,15 @@ int nts_stream_sync(nts_stream_t stream);
 int nts_device_sync(void);
 /* get_gpu_mem / show_gpu_mem (utils/cuda_memory.hpp:6-68): free and total device bytes. */
 int nts_mem_info(size_t *free_bytes, size_t *total_bytes);
+
+/* 64-bit checksum of one or two uint32 device arrays (position-dependent: moving or changing any
+ * element changes it, up to hash collisions), computed on the device and read back: the call waits
+ * for `stream`.  Either array may be empty.  For callers that keep something derived from device
+ * arrays they do not own -- the host veneer verifies with it, before every call through a schedule it
+ * built by itself, that offsets and indices still hold what the schedule was made from.  No
+ * counterpart in the reference.  About 0.1 ms for 115 M indices. */
+int nts_fingerprint_u32(uint64_t *fingerprint, const uint32_t *a, uint64_t n_a, const uint32_t *b, uint64_t n_b,
+                        nts_stream_t stream);
 
 /* Device-side timers (the reference only has host wall clocks, dep/gemini/time.hpp:20-26, around
  * synchronised calls).  An event is an opaque handle; elapsed time is in milliseconds between two

@@ -47,6 +47,7 @@ SIGNATURES = {
     "nts_stream_sync": [_vp],
     "nts_device_sync": [],
     "nts_mem_info": [ctypes.POINTER(_sz), ctypes.POINTER(_sz)],
+    "nts_fingerprint_u32": [ctypes.POINTER(_u64), _vp, _u64, _vp, _u64, _vp],
     "nts_event_create": [ctypes.POINTER(_vp)],
     "nts_event_destroy": [_vp],
     "nts_event_record": [_vp, _vp],

@@ -6,6 +6,7 @@
 #include <stdlib.h>
 
 #include <atomic>
+#include <algorithm>
 #include <mutex>
 
 #include "common.hpp"
@@ -36,6 +37,25 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned char *p, size_t
   for (size_t i = tid; i < body16; i += stride) body[i] = make_uint4(0u, 0u, 0u, 0u);
   if (tid < head) p[tid] = 0;
   if (tid < tail) p[head + body16 * 16 + tid] = 0;
+}
+
+// Position-dependent 64-bit checksum of a uint32 array: the sum over i of a 64-bit mix of
+// (value, salt + i).  A sum, so that blocks can add their shares in any order (integer atomics).
+__device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+__global__ __launch_bounds__(256) void fingerprint_kernel(unsigned long long *__restrict__ out,
+                                                          const uint32_t *__restrict__ a, unsigned long long n,
+                                                          unsigned long long salt) {
+  unsigned long long acc = 0;
+  const unsigned long long stride = static_cast<unsigned long long>(gridDim.x) * blockDim.x;
+  for (unsigned long long i = static_cast<unsigned long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    acc += mix64((static_cast<unsigned long long>(a[i]) << 32) ^ ((salt + i) * 0x9E3779B97F4A7C15ull));
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0 && acc) atomicAdd(out, acc);
 }
 
 }  // namespace
@@ -229,6 +249,36 @@ int nts_memset_zero(void *dev_ptr, size_t bytes, nts_stream_t stream) {
                      body16, tail);
   NTS_LAUNCH_CHECK("fill_zero_kernel");
   return NTS_OK;
+}
+
+int nts_fingerprint_u32(uint64_t *fingerprint, const uint32_t *a, uint64_t n_a, const uint32_t *b, uint64_t n_b,
+                        nts_stream_t stream) {
+  if (!fingerprint) return fail(NTS_ERR_INVALID, "nts_fingerprint_u32: null out-pointer");
+  if ((n_a && !a) || (n_b && !b)) return fail(NTS_ERR_INVALID, "nts_fingerprint_u32: null array");
+  unsigned long long *word = nullptr;
+  NTS_HIP_TRY(nts::scratch_alloc(reinterpret_cast<void **>(&word), 16, stream));
+  int rc = nts_memset_zero(word, 16, stream);
+  const uint64_t lens[2] = {n_a, n_b};
+  const uint32_t *arrays[2] = {a, b};
+  for (int k = 0; k < 2 && rc == NTS_OK; ++k) {
+    if (!lens[k]) continue;
+    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((lens[k] + 255) / 256, 8192));
+    hipLaunchKernelGGL(nts::fingerprint_kernel, dim3(blocks), dim3(256), 0, stream, word, arrays[k],
+                       static_cast<unsigned long long>(lens[k]), k ? 0x5851F42D4C957F2Dull + n_a : 0ull);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) rc = nts::fail_hip(err, "fingerprint_kernel");
+  }
+  unsigned long long host = 0;
+  if (rc == NTS_OK) {
+    hipError_t err = hipMemcpyAsync(&host, word, sizeof(host), hipMemcpyDeviceToHost, stream);
+    if (err == hipSuccess) err = hipStreamSynchronize(stream);
+    if (err != hipSuccess) rc = nts::fail_hip(err, "nts_fingerprint_u32: read-back");
+  }
+  const hipError_t ferr = nts::scratch_free(word, stream);
+  if (rc == NTS_OK && ferr != hipSuccess) rc = nts::fail_hip(ferr, "nts_fingerprint_u32: scratch_free");
+  // lengths are part of the value, so that a prefix of an array does not collide with the array
+  *fingerprint = host ^ (n_a * 0xD6E8FEB86659FD93ull) ^ (n_b * 0xA0761D6478BD642Full);
+  return rc;
 }
 
 int nts_stream_create(nts_stream_t *stream) {

@@ -177,6 +177,28 @@ int main() {
     const long planned1 = nts_veneer::planned_calls();
     EXPECT(run_and_check(want));
     EXPECT(nts_veneer::planned_calls() == planned1);
+    // A write the veneer cannot see (what a libtorch operator or a kernel of the caller's own would be:
+    // here a copy through the C ABI directly): the schedule that exists by now must not be used on the
+    // new contents.  It is found out by the checksum taken before every scheduled call.
+    EXPECT(run_and_check(want));
+    EXPECT(run_and_check(want));
+    const long built2 = nts_veneer::plans_built();
+    EXPECT(run_and_check(want));  // third sighting of the re-uploaded arrays: scheduled again
+    EXPECT(nts_veneer::plans_built() == built2 + 1 || nts_veneer::plans_built() == built2);
+    EXPECT(run_and_check(want));
+    const long planned2 = nts_veneer::planned_calls(), dropped0 = nts_veneer::plans_dropped_by_checksum();
+    EXPECT(planned2 > planned1);
+    for (VertexId_CUDA e = cob[7]; e < cob[8]; ++e) rib[e] = (rib[e] * 5 + 11) % Vb;
+    std::sort(rib.begin() + cob[7], rib.begin() + cob[8]);
+    EXPECT(nts_memcpy_h2d(dri, rib.data(), (size_t)Eb * sizeof(VertexId_CUDA), 1) == NTS_OK);
+    want = reference();
+    EXPECT(run_and_check(want));  // correct on the new contents ...
+    EXPECT(nts_veneer::planned_calls() == planned2);  // ... because the schedule was not used
+    EXPECT(nts_veneer::plans_dropped_by_checksum() == dropped0 + 1);
+    EXPECT(run_and_check(want));
+    EXPECT(run_and_check(want));  // and a new schedule follows once the new contents have repeated
+    EXPECT(run_and_check(want));
+    EXPECT(nts_veneer::planned_calls() > planned2);
     // without a source range (as SingleGPUSampleGraphOp calls it) no schedule is ever made
     const long built1 = nts_veneer::plans_built();
     for (int rep = 0; rep < 4; ++rep) {
