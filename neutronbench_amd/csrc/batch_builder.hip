@@ -42,7 +42,7 @@ bool plan_layout(Layout *L, uint32_t V, uint32_t graph_edges, const int32_t *fan
   };
   L->sizes = take((hops + 1) * kSizeWords * sizeof(uint32_t));
   L->dst0 = take(static_cast<size_t>(max_batch) * sizeof(uint32_t));
-  uint32_t vd = max_batch < V ? max_batch : V;
+  uint32_t vd = max_batch;  // the caller's batch may repeat vertices, so it may be longer than V
   uint32_t e_max = 0;
   for (uint32_t h = 0; h < hops; ++h) {
     HopLayout &H = L->hop[h];
@@ -140,8 +140,11 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
   if (hops == 0 || hops > kMaxHops) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: 1 to 8 hops");
   if (max_batch == 0 || V == 0 || graph_edges == 0)
     return fail(NTS_ERR_INVALID, "nts_batch_builder_create: empty graph or batch");
-  for (uint32_t h = 0; h < hops; ++h)
+  for (uint32_t h = 0; h < hops; ++h) {
     if (fanouts[h] == 0) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: fanout 0");
+    if (fanouts[h] > kWidestFanout)
+      return fail(NTS_ERR_UNSUPPORTED, "nts_batch_builder_create: fanouts above 1,024 are not supported");
+  }
   if (!aligned_to(arena, 256)) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: arena must be 256-byte aligned");
   nts_batch_builder *b = new (std::nothrow) nts_batch_builder();
   if (!b) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: out of host memory");

@@ -65,6 +65,28 @@ hipError_t scratch_alloc(void **ptr, size_t bytes, hipStream_t stream);
 hipError_t scratch_free(void *ptr, hipStream_t stream);
 hipError_t scratch_trim();  // gives the current device's unused scratch back to the driver
 
+// A scratch block that is returned to the pool when its scope ends, whichever way the function is
+// left (the error paths included); release() frees it early and reports the result.
+struct ScratchBlock {
+  void *ptr = nullptr;
+  hipStream_t stream = nullptr;
+  ScratchBlock() = default;
+  ScratchBlock(const ScratchBlock &) = delete;
+  ScratchBlock &operator=(const ScratchBlock &) = delete;
+  hipError_t alloc(size_t bytes, hipStream_t s) {
+    stream = s;
+    return scratch_alloc(&ptr, bytes, s);
+  }
+  hipError_t release() {
+    const hipError_t e = ptr ? scratch_free(ptr, stream) : hipSuccess;
+    ptr = nullptr;
+    return e;
+  }
+  ~ScratchBlock() {
+    if (ptr) (void)scratch_free(ptr, stream);
+  }
+};
+
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 inline uint32_t ceil_div(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
@@ -92,6 +114,10 @@ inline DevCount device_count(const uint32_t *n, uint32_t cap) { return DevCount{
 inline DevCount device_edge_count(const uint32_t *off, const uint32_t *n, uint32_t n_cap, uint32_t cap) {
   return DevCount{cap, n, off, n_cap};
 }
+
+// Largest finite fanout of the neighbour pick (distinct uniform positions: up to 64 inside lane
+// groups with Floyd's algorithm, up to this many by a keyed permutation of the positions).
+constexpr int32_t kWidestFanout = 1024;
 
 // Steps of a sampled layer's construction with sizes that may live on the device (sampler.hip,
 // layout.hip); the C entry points pass host counts, the batch builder device counts.

@@ -1491,6 +1491,7 @@ int edge_copy_impl(float *msg, const float *feat, const uint32_t *ri, const uint
 // Scratch of the long-row path in one stream-ordered allocation: list[rows], its counter, and the
 // tables of the giant rows (header, row list, first-piece prefix, piece table).
 struct LongRows {
+  ScratchBlock block;  // owns the allocation: returned to the pool on every way out of the caller
   uint32_t *list = nullptr;
   uint32_t *count = nullptr;
   uint32_t *hdr = nullptr;
@@ -1507,9 +1508,8 @@ int collect_long_rows(LongRows &lr, const uint32_t *off, uint32_t rows, uint32_t
   if (rows < kLongMinVertices) return NTS_OK;
   const size_t list_bytes = (static_cast<size_t>(rows) + 1 + 7) / 8 * 8 * sizeof(uint32_t);  // list + counter, 32-byte multiple
   const size_t small_bytes = (8 + kGiantCap + kGiantCap + 8) * sizeof(uint32_t);             // hdr, rows, first
-  unsigned char *buf = nullptr;
-  NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&buf), list_bytes + small_bytes + kPieceCap * sizeof(uint4),
-                             stream));
+  NTS_HIP_TRY(lr.block.alloc(list_bytes + small_bytes + kPieceCap * sizeof(uint4), stream));
+  unsigned char *buf = static_cast<unsigned char *>(lr.block.ptr);
   lr.list = reinterpret_cast<uint32_t *>(buf);
   lr.count = lr.list + rows;
   lr.hdr = reinterpret_cast<uint32_t *>(buf + list_bytes);
@@ -1526,9 +1526,9 @@ int collect_long_rows(LongRows &lr, const uint32_t *off, uint32_t rows, uint32_t
   return NTS_OK;
 }
 
-int release_long_rows(LongRows &lr, hipStream_t stream) {
-  if (lr.list) NTS_HIP_TRY(scratch_free(lr.list, stream));
-  lr = LongRows();
+int release_long_rows(LongRows &lr) {
+  lr.list = nullptr;
+  NTS_HIP_TRY(lr.block.release());
   return NTS_OK;
 }
 
@@ -1602,9 +1602,9 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
                          off, perm, lr.list, lr.count, Fv, tile, accumulate);
     NTS_LAUNCH_CHECK(who);
     // Giant rows: pieces by separate blocks into stream-ordered scratch, then the ordered combine.
-    float *partial = nullptr;
-    NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&partial), static_cast<size_t>(kPieceCap) * F * sizeof(float),
-                               stream));
+    ScratchBlock partial_block;
+    NTS_HIP_TRY(partial_block.alloc(static_cast<size_t>(kPieceCap) * F * sizeof(float), stream));
+    float *partial = static_cast<float *>(partial_block.ptr);
     if (v4)
       hipLaunchKernelGGL(giant_sum_pieces_kernel<float4>, dim3(kLongGrid), dim3(kLongBlock), 0, stream,
                          reinterpret_cast<float4 *>(partial), reinterpret_cast<const float4 *>(msg), perm, lr.hdr,
@@ -1615,10 +1615,10 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
     hipLaunchKernelGGL(giant_sum_combine_kernel, dim3(kGiantCap / 4), dim3(256), 0, stream, out, partial, lr.hdr,
                        lr.giant_rows, lr.first, F, accumulate);
     const hipError_t launch_err = hipGetLastError();
-    NTS_HIP_TRY(scratch_free(partial, stream));
+    NTS_HIP_TRY(partial_block.release());
     if (launch_err != hipSuccess) return fail_hip(launch_err, who);
   }
-  return release_long_rows(lr, stream);
+  return release_long_rows(lr);
 }
 
 // Edge softmax / fused attention, forward (gy == nullptr) or backward; x / el / er / ri / ger are
@@ -1704,9 +1704,10 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   }
   if (lr.list) {
     // Giant segments: per-piece statistics, ordered combine, apply (see the kernels above).
-    float *stats = nullptr;
     const size_t stats_floats = static_cast<size_t>(kPieceCap) * 2 * H, row_floats = static_cast<size_t>(kGiantCap) * 2 * H;
-    NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&stats), (stats_floats + row_floats) * sizeof(float), stream));
+    ScratchBlock stats_block;
+    NTS_HIP_TRY(stats_block.alloc((stats_floats + row_floats) * sizeof(float), stream));
+    float *stats = static_cast<float *>(stats_block.ptr);
     float *rowstat = stats + stats_floats;
     const dim3 pgrid(kLongGrid), pblock(kLongBlock), cgrid(kGiantCap / 4), cblock(64);
     if (!backward) {
@@ -1739,10 +1740,10 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
       }
     }
     const hipError_t launch_err = hipGetLastError();
-    NTS_HIP_TRY(scratch_free(stats, stream));
+    NTS_HIP_TRY(stats_block.release());
     if (launch_err != hipSuccess) return fail_hip(launch_err, who);
   }
-  return release_long_rows(lr, stream);
+  return release_long_rows(lr);
 }
 }  // namespace
 

@@ -5,8 +5,8 @@
 //                positions of the destination's CSC segment, uniformly at random
 // The reference draws positions with a per-thread mt19937 and iterates an unordered_set, so which
 // neighbours it picks (and in which order) is implementation-defined; here positions come from a
-// counter-based hash of (seed, destination slot) through Floyd's sampling and are emitted in
-// ascending position order, which keeps source ids ascending inside a destination for graphs with
+// counter-based hash of (seed, destination slot) through Floyd's sampling (fanouts up to 64) or a
+// keyed permutation of the positions (up to 1,024) and are emitted in ascending position order, which keeps source ids ascending inside a destination for graphs with
 // sorted adjacency.  Results depend only on the arguments: the same seed gives the same sample.
 #include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
@@ -98,15 +98,7 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
     return;
   }
   const uint64_t state0 = mix64(seed ^ (static_cast<uint64_t>(i) << 32) ^ d);
-  if (take > kMaxFanout || take > G) {
-    // Very large fanouts: a window of consecutive positions from a random start (distinct by
-    // construction), emitted in ascending position order: [0, wrap) then [start, start + take - wrap).
-    const uint32_t start = static_cast<uint32_t>(state0 % deg);
-    const uint32_t wrap = start + take > deg ? start + take - deg : 0;
-    for (uint32_t k = gl; k < take; k += G)
-      emit(ri_out, mark, out + k, graph_ri[base + (k < wrap ? k : start + (k - wrap))]);
-    return;
-  }
+  if (take > kMaxFanout || take > G) return;  // fanouts above one wavefront: hop_pick_wide_kernel
   // Lane gl < take: step j = deg - take + gl, hash chain advanced gl + 1 times.
   uint64_t state = state0;
   for (uint32_t q = 0; q <= gl && q < take; ++q) state = mix64(state);
@@ -122,6 +114,63 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
   if (gl < take) {
     uint32_t rank = 0;
     for (uint32_t q = 0; q < take; ++q) rank += __shfl(v, q, G) < v ? 1u : 0u;
+    emit(ri_out, mark, out + rank, graph_ri[base + v]);
+  }
+}
+
+// Fanouts of 65 .. 1,024: one wavefront per destination.  The positions are the first `take` values of
+// a keyed pseudo-random permutation of [0, deg): three rounds of (multiply by an odd constant, add a
+// key, fold the high bits down) are a bijection on [0, 2^b) for the smallest 2^b >= deg, and values
+// that land at or beyond deg are sent through the rounds again until they fall inside (cycle walking:
+// still a bijection, on [0, deg)), so the picks are distinct by construction and spread over the whole
+// neighbourhood.  They are staged in LDS, ranked, and emitted in ascending position order like the
+// narrower fanouts.  Destinations with at most `fanout` neighbours were copied whole by hop_pick_kernel.
+__global__ __launch_bounds__(256) void hop_pick_wide_kernel(uint32_t *__restrict__ ri_out,
+                                                            const uint32_t *__restrict__ co,
+                                                            const uint32_t *__restrict__ graph_co,
+                                                            const uint32_t *__restrict__ graph_ri,
+                                                            const uint32_t *__restrict__ dst, DevCount n,
+                                                            uint32_t edge_cap, uint64_t seed,
+                                                            uint32_t *__restrict__ mark) {
+  __shared__ uint32_t picked[4][kWidestFanout];
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint32_t *mine = picked[threadIdx.x / kWave];
+  const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  if (i >= n.get()) return;  // whole wavefronts leave together
+  const uint32_t d = dst[i];
+  const uint32_t base = graph_co[d];
+  const uint32_t deg = graph_co[d + 1] - base;
+  const uint32_t out = co[i];
+  const uint32_t take = co[i + 1] - out;
+  if (co[i + 1] > edge_cap || take == deg || take <= static_cast<uint32_t>(kMaxFanout)) return;
+  const uint64_t key = mix64(seed ^ (static_cast<uint64_t>(i) << 32) ^ d);
+  uint32_t bits = 1;
+  while ((1ull << bits) < deg) ++bits;
+  const uint32_t mask = bits >= 32 ? 0xFFFFFFFFu : (1u << bits) - 1u;
+  const uint32_t k0 = static_cast<uint32_t>(key), k1 = static_cast<uint32_t>(key >> 32),
+                 k2 = static_cast<uint32_t>(mix64(key));
+  const uint32_t fold = bits > 1 ? bits / 2 : 1;
+  auto rounds = [&](uint32_t x) {
+    x = (x * 0x9E3779B1u + k0) & mask;
+    x ^= x >> fold;
+    x = (x * 0x85EBCA6Bu + k1) & mask;
+    x ^= x >> fold;
+    x = (x * 0xC2B2AE35u + k2) & mask;
+    x ^= x >> fold;
+    return x;
+  };
+  for (uint32_t k = lane; k < take; k += kWave) {
+    uint32_t x = rounds(k);
+    while (x >= deg) x = rounds(x);
+    mine[k] = x;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  for (uint32_t k = lane; k < take; k += kWave) {
+    const uint32_t v = mine[k];
+    uint32_t rank = 0;
+    for (uint32_t q = 0; q < take; ++q) rank += mine[q] < v ? 1u : 0u;
     emit(ri_out, mark, out + rank, graph_ri[base + v]);
   }
 }
@@ -177,6 +226,13 @@ int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph
   }
 #undef NTS_LAUNCH_PICK
   NTS_LAUNCH_CHECK("hop_pick_kernel");
+  if (fanout > kMaxFanout) {
+    if (fanout > kWidestFanout)
+      return fail(NTS_ERR_UNSUPPORTED, "neighbour pick: fanouts above 1,024 are not supported");
+    hipLaunchKernelGGL(hop_pick_wide_kernel, dim3(ceil_div(static_cast<uint64_t>(n.cap) * kWave, 256)), dim3(256), 0,
+                       stream, ri_global, co, graph_co, graph_ri, dst, n, edge_cap, seed, mark_bits);
+    NTS_LAUNCH_CHECK("hop_pick_wide_kernel");
+  }
   return NTS_OK;
 }
 

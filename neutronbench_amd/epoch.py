@@ -211,7 +211,13 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         if not sequence:
             return
 
+        trained = [None, None]  # per builder: recorded when the batch built in it has been aggregated
+
         def start_sampling(step):
+            # the arena of this builder may still be read by the aggregation of the batch before last
+            # (only when the stages are not separated by waits): the sampling stream waits for it
+            if trained[step % 2] is not None:
+                sample_streams[0].wait_event(trained[step % 2])
             builders[step % 2].enqueue(batch_ids(sequence[step]), 1000 * sequence[step], sample_streams[0].cuda_stream)
         start_sampling(0)
         for step in range(len(sequence)):
@@ -224,6 +230,8 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
             x, _, hits = gather(cs, layers)
             tm.add("gather", t0)
             finish_batch(layers, x, hits)
+            trained[step % 2] = torch.cuda.Event()
+            trained[step % 2].record(torch.cuda.current_stream())
 
     def run_staged(sequence):
         if not sequence:

@@ -228,7 +228,7 @@ def test_fully_device_side_layer_construction(device):
     assert layer.dev_ewf().cpu().numpy().tobytes() == ewf.tobytes() and layer.dev_ewb().cpu().numpy().tobytes() == ewb.tobytes()
 
 
-@pytest.mark.parametrize("fanout", [-1, 1, 5, 25, 64, 100])
+@pytest.mark.parametrize("fanout", [-1, 1, 5, 25, 64, 65, 100, 700])
 def test_device_sampler_properties(device, fanout):
     """The hop sampler's contract: offsets equal init_co (bit-exact); with nothing dropped a
     destination's neighbours come out in CSC order; otherwise `fanout` DISTINCT positions of its
@@ -287,3 +287,29 @@ def test_device_sampler_is_uniform(device):
     expect = n * fanout / deg
     assert counts.sum() == n * fanout
     assert np.all(np.abs(counts - expect) < 6 * np.sqrt(expect)), counts
+
+
+def test_wide_fanouts_pick_spread_positions_uniformly(device):
+    """Fanouts above one wavefront (65 .. 1,024) take their positions from a keyed permutation of the
+    neighbourhood: every position about equally often, and the picks of one destination are spread
+    over the whole list instead of forming a run of neighbouring positions."""
+    deg, n, fanout = 1000, 4000, 100
+    gco = torch.tensor([0, deg], dtype=torch.int32, device=device)
+    gri = torch.arange(deg, dtype=torch.int32, device=device)
+    dst = torch.zeros(n, dtype=torch.int32, device=device)
+    co, ri = sample_hop(gco, gri, dst, fanout, 9)
+    picks = ri.cpu().numpy().reshape(n, fanout)
+    assert all(np.unique(row).size == fanout for row in picks[:200])
+    assert np.all(np.diff(picks, axis=1) > 0)  # ascending inside a destination
+    counts = np.bincount(picks.ravel(), minlength=deg)
+    expect = n * fanout / deg
+    assert np.all(np.abs(counts - expect) < 6 * np.sqrt(expect)), (counts.min(), counts.max(), expect)
+    # a window of consecutive positions would give a span of about `fanout`; spread picks span nearly the list
+    spans = picks[:, -1] - picks[:, 0]
+    assert np.median(spans) > 0.9 * deg
+    # pairs of positions are not tied together: positions 0 and 1 are picked together about (fanout/deg)^2 of the time
+    both = np.mean((picks == 0).any(1) & (picks == 1).any(1))
+    assert both < 3 * (fanout / deg) ** 2 + 0.01
+    # fanouts beyond the supported width are refused
+    assert abi.status("nts_sample_hop_neighbors", ptr(ri), ptr(co), ptr(gco), ptr(gri), ptr(dst), n, 2000, 1,
+                      torch.cuda.current_stream().cuda_stream) == abi.NTS_ERR_UNSUPPORTED

@@ -50,7 +50,7 @@ def assert_same_layers(got, want):
     (30000, 600000, 1024, [25, 10], 1),          # the Arxiv-shaped configuration's hops
     (50000, 2000000, 3000, [15, 10, 5], 2),      # Products-shaped hops
     (4000, 30000, 500, [3, 2, 2, 2], 3),         # more hops than layers of the configurations, sparse graph
-    (2000, 400000, 64, [64, 100], 4),            # fanout of a whole wavefront and the window pick above it
+    (2000, 400000, 64, [64, 100], 4),            # fanout of a whole wavefront and the permutation pick above it
     (3000, 40000, 700, [-1, 4], 5),              # whole neighbourhoods first
 ])
 def test_builder_equals_the_per_hop_entry_points(device, V, E, batch, fanouts, seed):

@@ -30,6 +30,19 @@ def test_pipelined_epoch_without_warm_up_batches():
         assert (b["sampled_edges"], b["checksum"]) == (a["sampled_edges"], a["checksum"])
 
 
+def test_two_batches_in_flight_without_stage_waits():
+    """With two batches in flight and no host-side wait between the stages, the sampling of batch k+2
+    re-uses the arena batch k was built in while batch k may still be aggregated: the sampling stream
+    waits for an event recorded after that aggregation.  Same results as the serial epoch."""
+    from neutronbench_amd import epoch
+
+    a = epoch.run("products", scale=0.05, max_batches=8, warmup_batches=0, pipeline=1, quiet=True, checksum=True)
+    b = epoch.run("products", scale=0.05, max_batches=8, warmup_batches=0, pipeline=2, stage_sync=False, quiet=True,
+                  checksum=True)
+    for key in ("sampled_edges", "gathered_rows", "cache_hit_rate", "checksum"):
+        assert a[key] == b[key], (key, a[key], b[key])
+
+
 def test_hop_by_hop_sampler_builds_the_same_batches():
     from neutronbench_amd import epoch
 
