@@ -4,6 +4,7 @@
 // algorithms; everything is order-independent, so the outputs are deterministic.
 #include <string.h>
 
+#include <rocprim/block/block_radix_sort.hpp>
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
@@ -191,24 +192,173 @@ inline unsigned bits_for(uint32_t n) {  // bits needed to represent values in [0
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// The library's radix sort switches to a merge sort below 2^20 items: one block sort and two
-// launches per doubling, about twenty dependent launches for a sampled hop of 400 k edges (230 us of
-// a 570 us batch).  The one-sweep radix path needs a histogram and one launch per eight key bits,
-// and the keys here are local ids of 15 to 22 bits; it takes over from 16 k items.
-// (Other digit widths and items per thread for the one-sweep passes were measured: five-bit digits
-// make a 256 k-edge hop 8 % faster and a 4.5 M-edge hop 15 % slower; the library's own choice stays.)
-using HopSortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
-                                                 rocprim::default_config, 16384>;
+// ---- stable sort of a sampled hop's edges by local source ------------------------------------------
+//
+// generate_csr_from_csc is a stable counting sort of (local source, CSC edge id).  A sampled hop has
+// 10^4 .. 10^6 edges and keys of 15 to 22 bits.  The library's device-wide radix sort spends ~24 us per
+// eight-bit pass whatever the size and clears its histograms with memset nodes, which keeps a batch's
+// construction out of a HIP graph.  This one is sized for hops: a least-significant-digit radix sort
+// in ceil(key_bits / 9) passes of equal width, three launches per pass and no memset:
+//   hop_sort_count    block b counts the digits of edges [2048 b, 2048 (b + 1)) in an LDS histogram and
+//                     writes its column of the digit-major table counts[digit][block]
+//   hop_sort_rows     one block per digit: exclusive scan of that digit's row over the blocks, and
+//                     the digit's total
+//   hop_sort_scatter  block b turns the totals into the digits' first positions, adds its entries of
+//                     the table, sorts its 2,048 (digit, position) pairs with the block-wide stable
+//                     sort, so that equal digits lie next to each other in their original order, and
+//                     writes every edge to start[digit] + its rank inside the chunk's run of that digit
+// Equal keys keep their order in every pass: the result is the stable order, bit for bit.  Only
+// blocks below ceil(E / 2048) of the launched ceil(capacity / 2048) do anything.
+constexpr int kHopSortThreads = 256;
+constexpr int kHopSortItems = 8;
+constexpr uint32_t kHopSortChunk = kHopSortThreads * kHopSortItems;  // 2,048 edges
+constexpr unsigned kHopSortMaxDigitBits = 9;
+constexpr uint32_t kHopSortMaxBins = 1u << kHopSortMaxDigitBits;
 
-// Scratch layout: [sorted keys: E u32][rocprim temporary storage].
-hipError_t sort_temp_bytes(uint32_t E, size_t *bytes) {
-  size_t tmp = 0;
-  uint32_t *nul = nullptr;
-  hipError_t err = rocprim::radix_sort_pairs<HopSortConfig>(nullptr, tmp, nul, nul,
-                                                            rocprim::counting_iterator<uint32_t>(0u), nul, E ? E : 1u,
-                                                            0u, 32u, static_cast<hipStream_t>(nullptr), false);
-  *bytes = tmp;
-  return err;
+struct HopSortShape {
+  uint32_t blocks;
+  unsigned passes;
+  unsigned digit_bits;
+};
+inline HopSortShape hop_sort_shape(uint32_t capacity, unsigned key_bits) {
+  HopSortShape sh;
+  sh.blocks = capacity ? static_cast<uint32_t>((static_cast<uint64_t>(capacity) + kHopSortChunk - 1) / kHopSortChunk) : 1u;
+  if (key_bits == 0) key_bits = 1;
+  sh.passes = (key_bits + kHopSortMaxDigitBits - 1) / kHopSortMaxDigitBits;
+  sh.digit_bits = (key_bits + sh.passes - 1) / sh.passes;
+  return sh;
+}
+
+// Exclusive prefix of `mine` over the 256 threads of a block, in thread order; *total = the sum.
+__device__ __forceinline__ uint32_t block_prefix_256(uint32_t mine, uint32_t *wave_sums, uint32_t *total) {
+  const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  uint32_t incl = mine;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t up = __shfl_up(incl, d, kWave);
+    if (lane >= static_cast<uint32_t>(d)) incl += up;
+  }
+  __syncthreads();  // wave_sums may still be read from an earlier call
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  uint32_t before = 0, all = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < kHopSortThreads / kWave; ++w) {
+    const uint32_t v = wave_sums[w];
+    if (w < wave) before += v;
+    all += v;
+  }
+  *total = all;
+  return before + incl - mine;
+}
+
+__global__ __launch_bounds__(kHopSortThreads) void hop_sort_count_kernel(uint32_t *__restrict__ table,
+                                                                         const uint32_t *__restrict__ keys,
+                                                                         DevCount edges, unsigned shift,
+                                                                         unsigned digit_bits) {
+  __shared__ uint32_t hist[kHopSortMaxBins];
+  const uint32_t E = edges.get();
+  const uint64_t first = static_cast<uint64_t>(blockIdx.x) * kHopSortChunk;
+  if (first >= E) return;
+  const uint32_t bins = 1u << digit_bits, mask = bins - 1u;
+  for (uint32_t d = threadIdx.x; d < bins; d += kHopSortThreads) hist[d] = 0;
+  __syncthreads();
+  const uint64_t last = first + kHopSortChunk < E ? first + kHopSortChunk : E;
+  for (uint64_t e = first + threadIdx.x; e < last; e += kHopSortThreads) atomicAdd(&hist[(keys[e] >> shift) & mask], 1u);
+  __syncthreads();
+  for (uint32_t d = threadIdx.x; d < bins; d += kHopSortThreads) table[static_cast<size_t>(d) * gridDim.x + blockIdx.x] = hist[d];
+}
+
+// One block per digit; table rows are `blocks` long, totals follow the table.
+__global__ __launch_bounds__(kHopSortThreads) void hop_sort_rows_kernel(uint32_t *__restrict__ table,
+                                                                        uint32_t *__restrict__ totals, uint32_t blocks,
+                                                                        DevCount edges) {
+  __shared__ uint32_t wave_sums[kHopSortThreads / kWave];
+  const uint32_t E = edges.get();
+  const uint32_t live = static_cast<uint32_t>((static_cast<uint64_t>(E) + kHopSortChunk - 1) / kHopSortChunk);
+  uint32_t *row = table + static_cast<size_t>(blockIdx.x) * blocks;
+  const uint32_t per = (live + kHopSortThreads - 1) / kHopSortThreads;
+  const uint32_t b = threadIdx.x * per, e = b + per < live ? b + per : live;
+  uint32_t sum = 0;
+  for (uint32_t i = b; i < e; ++i) sum += row[i];
+  uint32_t total;
+  uint32_t run = block_prefix_256(sum, wave_sums, &total);
+  for (uint32_t i = b; i < e; ++i) {
+    const uint32_t v = row[i];
+    row[i] = run;
+    run += v;
+  }
+  if (threadIdx.x == 0) totals[blockIdx.x] = total;
+}
+
+// vals_in == nullptr: the value of edge e is e.
+__global__ __launch_bounds__(kHopSortThreads) void hop_sort_scatter_kernel(uint32_t *__restrict__ keys_out,
+                                                                           uint32_t *__restrict__ vals_out,
+                                                                           const uint32_t *__restrict__ keys_in,
+                                                                           const uint32_t *__restrict__ vals_in,
+                                                                           const uint32_t *__restrict__ table,
+                                                                           const uint32_t *__restrict__ totals,
+                                                                           DevCount edges, unsigned shift,
+                                                                           unsigned digit_bits) {
+  using Sort = rocprim::block_radix_sort<uint32_t, kHopSortThreads, kHopSortItems, uint32_t>;
+  __shared__ typename Sort::storage_type sort_storage;
+  __shared__ uint32_t start[kHopSortMaxBins];     // output position of the first edge of each digit from this block
+  __shared__ uint32_t first_at[kHopSortMaxBins];  // where the chunk's run of each digit begins
+  __shared__ uint32_t chunk_keys[kHopSortChunk], chunk_vals[kHopSortChunk];
+  __shared__ uint16_t sorted_digit[kHopSortChunk];
+  __shared__ uint32_t wave_sums[kHopSortThreads / kWave];
+  const uint32_t E = edges.get();
+  const uint64_t c0 = static_cast<uint64_t>(blockIdx.x) * kHopSortChunk;
+  if (c0 >= E) return;
+  const uint32_t n = static_cast<uint32_t>(E - c0 < kHopSortChunk ? E - c0 : kHopSortChunk);
+  const uint32_t bins = 1u << digit_bits, mask = bins - 1u;
+  {  // first position of every digit: exclusive scan of the totals, plus this block's entry of the table
+    const uint32_t per = (bins + kHopSortThreads - 1) / kHopSortThreads;  // 1 or 2
+    const uint32_t b = threadIdx.x * per, e = b + per < bins ? b + per : bins;
+    uint32_t sum = 0;
+    for (uint32_t d = b; d < e; ++d) sum += totals[d];
+    uint32_t total;
+    uint32_t run = block_prefix_256(sum, wave_sums, &total);
+    for (uint32_t d = b; d < e; ++d) {
+      start[d] = run + table[static_cast<size_t>(d) * gridDim.x + blockIdx.x];
+      run += totals[d];
+    }
+  }
+  uint32_t digit[kHopSortItems], idx[kHopSortItems];
+#pragma unroll
+  for (int j = 0; j < kHopSortItems; ++j) {  // coalesced load into LDS
+    const uint32_t p = j * kHopSortThreads + threadIdx.x;
+    if (p < n) {
+      chunk_keys[p] = keys_in[c0 + p];
+      chunk_vals[p] = vals_in ? vals_in[c0 + p] : static_cast<uint32_t>(c0 + p);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kHopSortItems; ++j) {
+    const uint32_t p = threadIdx.x * kHopSortItems + j;  // blocked arrangement keeps the input order
+    idx[j] = p;
+    digit[j] = p < n ? ((chunk_keys[p] >> shift) & mask) : bins;  // the chunk's unused tail sorts last
+  }
+  Sort().sort(digit, idx, sort_storage, 0, digit_bits + 1);
+#pragma unroll
+  for (int j = 0; j < kHopSortItems; ++j) sorted_digit[threadIdx.x * kHopSortItems + j] = static_cast<uint16_t>(digit[j]);
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kHopSortItems; ++j) {  // the first element of every run records where the run begins
+    const uint32_t p = threadIdx.x * kHopSortItems + j;
+    if (p < n && (p == 0 || sorted_digit[p - 1] != sorted_digit[p])) first_at[digit[j]] = p;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kHopSortItems; ++j) {
+    const uint32_t p = threadIdx.x * kHopSortItems + j;
+    if (p < n) {
+      const uint32_t pos = start[digit[j]] + (p - first_at[digit[j]]);
+      keys_out[pos] = chunk_keys[idx[j]];
+      vals_out[pos] = chunk_vals[idx[j]];
+    }
+  }
 }
 
 // Splits the (src, dst) pairs of an edge list into two key arrays.
@@ -232,27 +382,47 @@ hipError_t sort_pairs_temp_bytes(uint32_t E, size_t *bytes) {
 
 }  // namespace
 
+// Scratch layout: [sorted keys: n][keys between passes: n][values between passes: n]
+//                 [digit table: 512 x ceil(n / 2048)][digit totals: 512], all u32.
 size_t csr_from_csc_bytes(uint32_t sort_n) {
-  size_t tmp = 0;
-  if (sort_temp_bytes(sort_n, &tmp) != hipSuccess) return 0;
-  return align_up(static_cast<size_t>(sort_n) * sizeof(uint32_t), 256) + align_up(tmp, 256) + 256;
+  const size_t arr = align_up(static_cast<size_t>(sort_n ? sort_n : 1) * sizeof(uint32_t), 256);
+  const HopSortShape sh = hop_sort_shape(sort_n, 32);
+  const size_t table = align_up((static_cast<size_t>(sh.blocks) + 1) * kHopSortMaxBins * sizeof(uint32_t), 256);
+  return 3 * arr + table + 256;
 }
 
 int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, DevCount Vd,
                  DevCount Vs, DevCount E, uint32_t sort_n, unsigned key_bits, void *work, hipStream_t stream) {
   unsigned char *w = static_cast<unsigned char *>(work);
+  const size_t arr = align_up(static_cast<size_t>(sort_n ? sort_n : 1) * sizeof(uint32_t), 256);
   uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(w);
-  size_t keys_bytes = align_up(static_cast<size_t>(sort_n) * sizeof(uint32_t), 256);
+  uint32_t *keys_mid[2] = {reinterpret_cast<uint32_t *>(w + arr), keys_sorted};
+  uint32_t *vals_mid = reinterpret_cast<uint32_t *>(w + 2 * arr);
+  uint32_t *table = reinterpret_cast<uint32_t *>(w + 3 * arr);
   // Without a caller buffer for perm, ci doubles as the sorted edge-id array and is rewritten in
   // place by a second pass (each thread reads its own element before writing it).
   uint32_t *perm_out = perm ? perm : ci;
-  size_t tmp = 0;
-  NTS_HIP_TRY(sort_temp_bytes(sort_n, &tmp));
-  // Stable LSD radix sort of (local source, CSC edge id): edge ids stay ascending within a source,
-  // which is exactly the order the host counting sort produces.
-  NTS_HIP_TRY(rocprim::radix_sort_pairs<HopSortConfig>(w + keys_bytes, tmp, ri, keys_sorted,
-                                                       rocprim::counting_iterator<uint32_t>(0u), perm_out, sort_n, 0u,
-                                                       key_bits, stream, false));
+  // Stable sort of (local source, CSC edge id): edge ids stay ascending within a source, which is
+  // exactly the order the host counting sort produces.  Keys and values alternate between two
+  // buffers so that the last pass lands in keys_sorted / perm_out.
+  const HopSortShape sh = hop_sort_shape(sort_n, key_bits);
+  uint32_t *totals = table + static_cast<size_t>(sh.blocks) * kHopSortMaxBins;
+  uint32_t *vals_buf[2] = {vals_mid, perm_out};
+  const uint32_t *kin = ri, *vin = nullptr;
+  for (unsigned pass = 0; pass < sh.passes; ++pass) {
+    const unsigned to = (sh.passes - 1 - pass) & 1u ? 0u : 1u;  // the last pass writes buffer 1
+    uint32_t *kout = keys_mid[to], *vout = vals_buf[to];
+    const unsigned shift = pass * sh.digit_bits;
+    hipLaunchKernelGGL(hop_sort_count_kernel, dim3(sh.blocks), dim3(kHopSortThreads), 0, stream, table, kin, E, shift,
+                       sh.digit_bits);
+    hipLaunchKernelGGL(hop_sort_rows_kernel, dim3(1u << sh.digit_bits), dim3(kHopSortThreads), 0, stream, table, totals,
+                       sh.blocks, E);
+    hipLaunchKernelGGL(hop_sort_scatter_kernel, dim3(sh.blocks), dim3(kHopSortThreads), 0, stream, kout, vout, kin, vin,
+                       table, totals, E, shift, sh.digit_bits);
+    NTS_LAUNCH_CHECK("hop_sort kernels");
+    kin = kout;
+    vin = vout;
+  }
   const uint64_t span = static_cast<uint64_t>(Vs.cap) + 1 > E.cap ? static_cast<uint64_t>(Vs.cap) + 1 : E.cap;
   hipLaunchKernelGGL(csr_finish_kernel, dim3(ceil_div(span, 256)), dim3(256), 0, stream, ro, ci, keys_sorted, perm_out,
                      co, Vd, Vs, E);
@@ -401,7 +571,9 @@ int nts_gather_edge_to_src_unsorted(float *out, const float *msg, const uint32_t
   NTS_HIP_TRY(hipStreamSynchronize(stream));
   if (E == 0) return NTS_OK;
   size_t tmp = 0;
-  NTS_HIP_TRY(sort_temp_bytes(E, &tmp));
+  NTS_HIP_TRY(rocprim::radix_sort_pairs(nullptr, tmp, static_cast<uint32_t *>(nullptr), static_cast<uint32_t *>(nullptr),
+                                        rocprim::counting_iterator<uint32_t>(0u), static_cast<uint32_t *>(nullptr), E, 0u,
+                                        32u, stream, false));
   const size_t arr = align_up(static_cast<size_t>(E) * sizeof(uint32_t), 256);
   unsigned char *work = nullptr;
   NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&work), 3 * arr + align_up(tmp, 256), stream));
