@@ -441,9 +441,16 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
  *                Pointers address the arena and stay valid until the next nts_batch_builder_sample
  *                on the same builder; a pipeline that samples batch k+1 while batch k trains uses
  *                one builder per stage in flight, as the reference uses one SampledSubgraph each.
+ *   nts_batch_builder_use_graph  enable != 0: nts_batch_builder_sample records the launches of the
+ *                hops (and the copy of the layer shapes to the host) once, at the builder's next
+ *                batch, as a HIP graph, and replays that graph for every later batch; only one small
+ *                launch that stores the batch's ids, their count and the seed stays outside.  The
+ *                arrays are the same bit for bit (every launch reads counts and the seed from the
+ *                arena, none is a memset node); what changes is the host time per batch.  The
+ *                recording is thread-local and runs on a stream the library creates for it; the
+ *                graph is then launched on the caller's stream.  Off by default.
  * Calls on one builder must not overlap: consecutive nts_batch_builder_sample calls go to the same
- * stream, or the earlier batch is waited for first (nts_batch_builder_layers does).  The sequence
- * contains a device-to-host copy and an event record and is not meant for HIP-graph capture. */
+ * stream, or the earlier batch is waited for first (nts_batch_builder_layers does). */
 typedef struct nts_batch_builder nts_batch_builder_t;
 typedef struct nts_sampled_layer {
   uint32_t v_size, e_size, src_size, reserved; /* destinations, edges, distinct sources */
@@ -464,6 +471,7 @@ int nts_batch_builder_create(nts_batch_builder_t **builder, const uint32_t *grap
                              uint32_t max_batch, int want_perm, void *arena, size_t arena_bytes);
 int nts_batch_builder_sample(nts_batch_builder_t *builder, const uint32_t *batch_ids, uint32_t n, uint64_t seed,
                              nts_stream_t stream);
+int nts_batch_builder_use_graph(nts_batch_builder_t *builder, int enable);
 int nts_batch_builder_layers(nts_batch_builder_t *builder, nts_sampled_layer_t *layers);
 int nts_batch_builder_destroy(nts_batch_builder_t *builder);
 

@@ -143,9 +143,11 @@ class BatchBuilder:
 
     graph_co / graph_ri: int32 device tensors (uint32 bit patterns) of the whole graph's CSC;
     fanouts: hop 0 (the batch's own hop) first.  The layers returned by `sample` are views into
-    this object's arena: they are overwritten by the next `sample`."""
+    this object's arena: they are overwritten by the next `sample`.  graph=True: the launches of the
+    hops are recorded once as a HIP graph and replayed for every later batch (same arrays, less host
+    time per batch)."""
 
-    def __init__(self, graph_co, graph_ri, fanouts, max_batch, want_perm=False):
+    def __init__(self, graph_co, graph_ri, fanouts, max_batch, want_perm=False, graph=False):
         self.device = graph_co.device
         self.graph_co, self.graph_ri = graph_co, graph_ri
         self.hops = len(fanouts)
@@ -160,6 +162,8 @@ class BatchBuilder:
         call("nts_batch_builder_create", ctypes.byref(handle), ptr(graph_co), ptr(graph_ri), V, E, fan, self.hops,
              max_batch, int(want_perm), self.arena.data_ptr() + self._skew, nbytes)
         self.handle = handle.value
+        if graph:
+            call("nts_batch_builder_use_graph", self.handle, 1)
         self._desc = (SampledLayerDesc * self.hops)()
 
     def _array(self, address, count, dtype):

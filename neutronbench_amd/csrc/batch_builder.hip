@@ -28,7 +28,7 @@ struct HopLayout {
 
 struct Layout {
   HopLayout hop[kMaxHops];
-  size_t dst0, sizes, ri_global, relabel_work, csr_work, scan_work, total;
+  size_t dst0, sizes, seed, ri_global, relabel_work, csr_work, scan_work, total;
   size_t relabel_bytes, csr_bytes, scan_bytes;
 };
 
@@ -41,6 +41,7 @@ bool plan_layout(Layout *L, uint32_t V, uint32_t graph_edges, const int32_t *fan
     return here;
   };
   L->sizes = take((hops + 1) * kSizeWords * sizeof(uint32_t));
+  L->seed = take(sizeof(uint64_t));
   L->dst0 = take(static_cast<size_t>(max_batch) * sizeof(uint32_t));
   uint32_t vd = max_batch;  // the caller's batch may repeat vertices, so it may be longer than V
   uint32_t e_max = 0;
@@ -95,10 +96,14 @@ inline unsigned bits_for(uint32_t n) {  // bits needed to represent values in [0
 }
 
 // The batch's vertex ids become hop 0's destinations; the live destination count of hop 0 is n.
+// Everything that changes from batch to batch enters here -- the ids, their count and the seed go
+// to fixed places in the arena -- so that the launches after this one are the same for every batch.
 __global__ __launch_bounds__(256) void start_batch_kernel(uint32_t *__restrict__ dst0, const uint32_t *__restrict__ ids,
-                                                          uint32_t n, uint32_t *__restrict__ sizes) {
+                                                          uint32_t n, uint32_t *__restrict__ sizes, uint32_t size_words,
+                                                          uint64_t *__restrict__ seed_word, uint64_t seed) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i == 0) sizes[0] = n;
+  if (i < size_words) sizes[i] = i == 0 ? n : 0u;
+  if (i == 0) *seed_word = seed;
   if (i < n) dst0[i] = ids[i];
 }
 
@@ -118,7 +123,91 @@ struct nts_batch_builder {
   hipEvent_t done;
   bool pending;
   bool bitmap_clean;  // the bitmap of sampled sources is all zero (each hop's last kernel leaves it so)
+  bool use_graph;     // replay the hops' launches as one HIP graph, captured at the first batch
+  hipGraph_t graph;
+  hipGraphExec_t graph_exec;
 };
+
+namespace {
+
+// Every launch of a batch after start_batch_kernel: the hops, then the copy of the size table to the
+// host.  All arguments are addresses inside the arena, capacities and device-resident counts, so the
+// sequence is the same for every batch of a builder.
+int enqueue_hops(nts_batch_builder *b, hipStream_t stream) {
+  unsigned char *A = b->arena;
+  uint32_t *sizes = reinterpret_cast<uint32_t *>(A + b->L.sizes);
+  const uint64_t *seed_word = reinterpret_cast<const uint64_t *>(A + b->L.seed);
+  uint32_t *dst = reinterpret_cast<uint32_t *>(A + b->L.dst0);
+  uint32_t *ri_global = reinterpret_cast<uint32_t *>(A + b->L.ri_global);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(A + b->L.relabel_work);
+  const uint32_t words = (b->V + 31) / 32;
+  for (uint32_t h = 0; h < b->hops; ++h) {
+    const HopLayout &H = b->L.hop[h];
+    uint32_t *hop_sizes = sizes + h * kSizeWords;
+    uint32_t *co = reinterpret_cast<uint32_t *>(A + H.co);
+    uint32_t *ri = reinterpret_cast<uint32_t *>(A + H.ri_local);
+    uint32_t *source = reinterpret_cast<uint32_t *>(A + H.source);
+    uint32_t *ro = reinterpret_cast<uint32_t *>(A + H.ro);
+    uint32_t *ci = reinterpret_cast<uint32_t *>(A + H.ci);
+    uint32_t *perm = b->want_perm ? reinterpret_cast<uint32_t *>(A + H.perm) : nullptr;
+    float *ewf = reinterpret_cast<float *>(A + H.ewf);
+    float *ewb = reinterpret_cast<float *>(A + H.ewb);
+    const DevCount Vd = device_count(hop_sizes + 0, H.vd_cap);
+    const DevCount Vs = device_count(hop_sizes + 2, H.vs_cap);
+    const DevCount E = device_edge_count(co, hop_sizes + 0, H.vd_cap, H.e_cap);
+    if (int rc = hop_offsets(co, b->graph_co, dst, Vd, b->fanout[h], A + b->L.scan_work, b->L.scan_bytes, stream))
+      return rc;
+    if (int rc = hop_neighbors(ri_global, co, b->graph_co, b->graph_ri, dst, Vd, H.e_cap, b->fanout[h],
+                               device_seed(seed_word, h), bits, stream))
+      return rc;
+    // Local ids; the unused tail of the edge array is padded with a key that sorts after every
+    // source.
+    if (int rc = relabel_sources(source, hop_sizes + 2, hop_sizes + kSizeWords, ri, ri_global, E, H.e_cap, H.vs_cap,
+                                 hop_sizes + 1, b->V, A + b->L.relabel_work, true, stream))
+      return rc;
+    if (int rc = csr_from_csc(ro, ci, perm, co, ri, Vd, Vs, E, H.e_cap, bits_for(H.vs_cap + 1), A + b->L.csr_work,
+                              stream))
+      return rc;
+    if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, bits, words, stream)) return rc;
+    dst = source;  // the next hop's destinations are this hop's sources (init_dst)
+  }
+  const size_t size_bytes = (b->hops + 1) * kSizeWords * sizeof(uint32_t);
+  NTS_HIP_TRY(hipMemcpyAsync(b->host_sizes, sizes, size_bytes, hipMemcpyDeviceToHost, stream));
+  return NTS_OK;
+}
+
+// Records enqueue_hops into a graph and instantiates it.  The recording runs on a stream created for
+// it (the caller's may be the null stream, which cannot record; nothing executes while recording)
+// in thread-local mode: other host threads keep using the device meanwhile.
+int capture_hops(nts_batch_builder *b) {
+  hipStream_t stream = nullptr;
+  NTS_HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+  hipError_t begin = hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal);
+  if (begin != hipSuccess) {
+    (void)hipStreamDestroy(stream);
+    return fail_hip(begin, "nts_batch_builder_sample: hipStreamBeginCapture");
+  }
+  const int rc = enqueue_hops(b, stream);
+  hipGraph_t graph = nullptr;
+  const hipError_t end = hipStreamEndCapture(stream, &graph);  // always ends the recording, also after an error
+  (void)hipStreamDestroy(stream);
+  if (rc != NTS_OK) {
+    if (graph) (void)hipGraphDestroy(graph);
+    return rc;
+  }
+  if (end != hipSuccess) return fail_hip(end, "nts_batch_builder_sample: hipStreamEndCapture");
+  hipGraphExec_t exec = nullptr;
+  const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (inst != hipSuccess) {
+    (void)hipGraphDestroy(graph);
+    return fail_hip(inst, "nts_batch_builder_sample: hipGraphInstantiate");
+  }
+  b->graph = graph;
+  b->graph_exec = exec;
+  return NTS_OK;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -163,6 +252,9 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
   b->host_sizes = nullptr;
   b->pending = false;
   b->bitmap_clean = false;
+  b->use_graph = false;
+  b->graph = nullptr;
+  b->graph_exec = nullptr;
   hipError_t err = hipHostMalloc(reinterpret_cast<void **>(&b->host_sizes), (hops + 1) * kSizeWords * sizeof(uint32_t),
                                  hipHostMallocDefault);
   if (err == hipSuccess) {
@@ -180,6 +272,8 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
 int nts_batch_builder_destroy(nts_batch_builder_t *b) {
   NTS_TRACE_RANGE("nts_batch_builder_destroy");
   if (!b) return NTS_OK;
+  if (b->graph_exec) (void)hipGraphExecDestroy(b->graph_exec);
+  if (b->graph) (void)hipGraphDestroy(b->graph);
   hipError_t e1 = hipEventDestroy(b->done);
   hipError_t e2 = hipHostFree(b->host_sizes);
   delete b;
@@ -197,8 +291,8 @@ int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, 
   unsigned char *A = b->arena;
   uint32_t *sizes = reinterpret_cast<uint32_t *>(A + b->L.sizes);
   uint32_t *dst = reinterpret_cast<uint32_t *>(A + b->L.dst0);
-  uint32_t *ri_global = reinterpret_cast<uint32_t *>(A + b->L.ri_global);
-  const size_t size_bytes = (b->hops + 1) * kSizeWords * sizeof(uint32_t);
+  uint64_t *seed_word = reinterpret_cast<uint64_t *>(A + b->L.seed);
+  const uint32_t size_words = (b->hops + 1) * kSizeWords;
   // The neighbour pick sets the bits of the sources it emits, the relabelling reads them, and the
   // hop's last kernel clears them again; only a first or an interrupted batch clears them up front.
   uint32_t *bits = reinterpret_cast<uint32_t *>(A + b->L.relabel_work);
@@ -206,43 +300,26 @@ int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, 
   if (!b->bitmap_clean)
     if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
   b->bitmap_clean = false;
-  if (int rc = nts_memset_zero(sizes, size_bytes, stream)) return rc;
-  hipLaunchKernelGGL(start_batch_kernel, dim3(ceil_div(n ? n : 1, 256)), dim3(256), 0, stream, dst, batch_ids, n, sizes);
+  const uint32_t start_threads = n > size_words ? n : size_words;
+  hipLaunchKernelGGL(start_batch_kernel, dim3(ceil_div(start_threads, 256)), dim3(256), 0, stream, dst, batch_ids, n,
+                     sizes, size_words, seed_word, seed);
   NTS_LAUNCH_CHECK("start_batch_kernel");
-  for (uint32_t h = 0; h < b->hops; ++h) {
-    const HopLayout &H = b->L.hop[h];
-    uint32_t *hop_sizes = sizes + h * kSizeWords;
-    uint32_t *co = reinterpret_cast<uint32_t *>(A + H.co);
-    uint32_t *ri = reinterpret_cast<uint32_t *>(A + H.ri_local);
-    uint32_t *source = reinterpret_cast<uint32_t *>(A + H.source);
-    uint32_t *ro = reinterpret_cast<uint32_t *>(A + H.ro);
-    uint32_t *ci = reinterpret_cast<uint32_t *>(A + H.ci);
-    uint32_t *perm = b->want_perm ? reinterpret_cast<uint32_t *>(A + H.perm) : nullptr;
-    float *ewf = reinterpret_cast<float *>(A + H.ewf);
-    float *ewb = reinterpret_cast<float *>(A + H.ewb);
-    const DevCount Vd = device_count(hop_sizes + 0, H.vd_cap);
-    const DevCount Vs = device_count(hop_sizes + 2, H.vs_cap);
-    const DevCount E = device_edge_count(co, hop_sizes + 0, H.vd_cap, H.e_cap);
-    if (int rc = hop_offsets(co, b->graph_co, dst, Vd, b->fanout[h], A + b->L.scan_work, b->L.scan_bytes, stream))
-      return rc;
-    if (int rc = hop_neighbors(ri_global, co, b->graph_co, b->graph_ri, dst, Vd, H.e_cap, b->fanout[h], seed + h, bits,
-                               stream))
-      return rc;
-    // Local ids; the unused tail of the edge array is padded with a key that sorts after every
-    // source, so that the sort below can run over the fixed capacity.
-    if (int rc = relabel_sources(source, hop_sizes + 2, hop_sizes + kSizeWords, ri, ri_global, E, H.e_cap, H.vs_cap,
-                                 hop_sizes + 1, b->V, A + b->L.relabel_work, true, stream))
-      return rc;
-    if (int rc = csr_from_csc(ro, ci, perm, co, ri, Vd, Vs, E, H.e_cap, bits_for(H.vs_cap + 1), A + b->L.csr_work,
-                              stream))
-      return rc;
-    if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, bits, words, stream)) return rc;
-    dst = source;  // the next hop's destinations are this hop's sources (init_dst)
+  if (b->use_graph) {
+    if (!b->graph_exec)
+      if (int rc = capture_hops(b)) return rc;
+    NTS_HIP_TRY(hipGraphLaunch(b->graph_exec, stream));
+  } else {
+    if (int rc = enqueue_hops(b, stream)) return rc;
   }
-  NTS_HIP_TRY(hipMemcpyAsync(b->host_sizes, sizes, size_bytes, hipMemcpyDeviceToHost, stream));
   NTS_HIP_TRY(hipEventRecord(b->done, stream));
   b->pending = true;
   b->bitmap_clean = true;
+  return NTS_OK;
+}
+
+int nts_batch_builder_use_graph(nts_batch_builder_t *b, int enable) {
+  if (!b) return fail(NTS_ERR_INVALID, "nts_batch_builder_use_graph: null builder");
+  b->use_graph = enable != 0;
   return NTS_OK;
 }
 

@@ -115,6 +115,18 @@ inline DevCount device_edge_count(const uint32_t *off, const uint32_t *n, uint32
   return DevCount{cap, n, off, n_cap};
 }
 
+// A seed that is either a host value or a device word plus an offset (the batch builder keeps the
+// batch's seed on the device, so that the same launches serve every batch).
+struct DevSeed {
+  const uint64_t *base;
+  uint64_t add;
+#if defined(__HIPCC__)
+  __device__ __forceinline__ uint64_t get() const { return (base ? *base : 0ull) + add; }
+#endif
+};
+inline DevSeed host_seed(uint64_t v) { return DevSeed{nullptr, v}; }
+inline DevSeed device_seed(const uint64_t *base, uint64_t add) { return DevSeed{base, add}; }
+
 // Largest finite fanout of the neighbour pick (distinct uniform positions: up to 64 inside lane
 // groups with Floyd's algorithm, up to this many by a keyed permutation of the positions).
 constexpr int32_t kWidestFanout = 1024;
@@ -124,7 +136,7 @@ constexpr int32_t kWidestFanout = 1024;
 int hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, DevCount n, int32_t fanout, void *scan_tmp,
                 size_t scan_tmp_bytes, hipStream_t stream);
 int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co, const uint32_t *graph_ri,
-                  const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, uint64_t seed, uint32_t *mark_bits,
+                  const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, DevSeed seed, uint32_t *mark_bits,
                   hipStream_t stream);
 size_t hop_scan_bytes(uint32_t n);
 // fill_to > E: local[E .. fill_to) = fill_value (padding for a sort over a fixed capacity);

@@ -198,7 +198,7 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // 10^4 .. 10^6 edges and keys of 15 to 22 bits.  The library's device-wide radix sort spends ~24 us per
 // eight-bit pass whatever the size and clears its histograms with memset nodes, which keeps a batch's
 // construction out of a HIP graph.  This one is sized for hops: a least-significant-digit radix sort
-// in ceil(key_bits / 9) passes of equal width, three launches per pass and no memset:
+// in ceil(key_bits / 10) passes of equal width, three launches per pass and no memset:
 //   hop_sort_count    block b counts the digits of edges [2048 b, 2048 (b + 1)) in an LDS histogram and
 //                     writes its column of the digit-major table counts[digit][block]
 //   hop_sort_rows     one block per digit: exclusive scan of that digit's row over the blocks, and
@@ -212,7 +212,7 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 constexpr int kHopSortThreads = 256;
 constexpr int kHopSortItems = 8;
 constexpr uint32_t kHopSortChunk = kHopSortThreads * kHopSortItems;  // 2,048 edges
-constexpr unsigned kHopSortMaxDigitBits = 9;
+constexpr unsigned kHopSortMaxDigitBits = 10;
 constexpr uint32_t kHopSortMaxBins = 1u << kHopSortMaxDigitBits;
 
 struct HopSortShape {
@@ -229,8 +229,9 @@ inline HopSortShape hop_sort_shape(uint32_t capacity, unsigned key_bits) {
   return sh;
 }
 
-// Exclusive prefix of `mine` over the 256 threads of a block, in thread order; *total = the sum.
-__device__ __forceinline__ uint32_t block_prefix_256(uint32_t mine, uint32_t *wave_sums, uint32_t *total) {
+// Exclusive prefix of `mine` over the THREADS threads of a block, in thread order; *total = the sum.
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_prefix(uint32_t mine, uint32_t *wave_sums, uint32_t *total) {
   const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   uint32_t incl = mine;
 #pragma unroll
@@ -243,7 +244,7 @@ __device__ __forceinline__ uint32_t block_prefix_256(uint32_t mine, uint32_t *wa
   __syncthreads();
   uint32_t before = 0, all = 0;
 #pragma unroll
-  for (uint32_t w = 0; w < kHopSortThreads / kWave; ++w) {
+  for (uint32_t w = 0; w < THREADS / kWave; ++w) {
     const uint32_t v = wave_sums[w];
     if (w < wave) before += v;
     all += v;
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(kHopSortThreads) void hop_sort_rows_kernel(uint32_t
   uint32_t sum = 0;
   for (uint32_t i = b; i < e; ++i) sum += row[i];
   uint32_t total;
-  uint32_t run = block_prefix_256(sum, wave_sums, &total);
+  uint32_t run = block_prefix<kHopSortThreads>(sum, wave_sums, &total);
   for (uint32_t i = b; i < e; ++i) {
     const uint32_t v = row[i];
     row[i] = run;
@@ -291,8 +292,10 @@ __global__ __launch_bounds__(kHopSortThreads) void hop_sort_rows_kernel(uint32_t
   if (threadIdx.x == 0) totals[blockIdx.x] = total;
 }
 
-// vals_in == nullptr: the value of edge e is e.
-__global__ __launch_bounds__(kHopSortThreads) void hop_sort_scatter_kernel(uint32_t *__restrict__ keys_out,
+// vals_in == nullptr: the value of edge e is e.  THREADS x ITEMS = 2,048: the block-wide sort ranks a
+// thread's items one after the other, so more threads with fewer items each shorten the chain.
+template <int THREADS, int ITEMS>
+__global__ __launch_bounds__(THREADS) void hop_sort_scatter_kernel(uint32_t *__restrict__ keys_out,
                                                                            uint32_t *__restrict__ vals_out,
                                                                            const uint32_t *__restrict__ keys_in,
                                                                            const uint32_t *__restrict__ vals_in,
@@ -300,34 +303,36 @@ __global__ __launch_bounds__(kHopSortThreads) void hop_sort_scatter_kernel(uint3
                                                                            const uint32_t *__restrict__ totals,
                                                                            DevCount edges, unsigned shift,
                                                                            unsigned digit_bits) {
-  using Sort = rocprim::block_radix_sort<uint32_t, kHopSortThreads, kHopSortItems, uint32_t>;
+  // one ranking round over the whole digit (the library's default is eight bits per round)
+  using Sort = rocprim::block_radix_sort<uint32_t, THREADS, ITEMS, uint32_t, 1, 1, kHopSortMaxDigitBits>;
   __shared__ typename Sort::storage_type sort_storage;
   __shared__ uint32_t start[kHopSortMaxBins];     // output position of the first edge of each digit from this block
   __shared__ uint32_t first_at[kHopSortMaxBins];  // where the chunk's run of each digit begins
   __shared__ uint32_t chunk_keys[kHopSortChunk], chunk_vals[kHopSortChunk];
   __shared__ uint16_t sorted_digit[kHopSortChunk];
-  __shared__ uint32_t wave_sums[kHopSortThreads / kWave];
+  __shared__ uint32_t wave_sums[THREADS / kWave];
+  static_assert(THREADS * ITEMS == static_cast<int>(kHopSortChunk), "one chunk per block");
   const uint32_t E = edges.get();
   const uint64_t c0 = static_cast<uint64_t>(blockIdx.x) * kHopSortChunk;
   if (c0 >= E) return;
   const uint32_t n = static_cast<uint32_t>(E - c0 < kHopSortChunk ? E - c0 : kHopSortChunk);
   const uint32_t bins = 1u << digit_bits, mask = bins - 1u;
   {  // first position of every digit: exclusive scan of the totals, plus this block's entry of the table
-    const uint32_t per = (bins + kHopSortThreads - 1) / kHopSortThreads;  // 1 or 2
+    const uint32_t per = (bins + THREADS - 1) / THREADS;
     const uint32_t b = threadIdx.x * per, e = b + per < bins ? b + per : bins;
     uint32_t sum = 0;
     for (uint32_t d = b; d < e; ++d) sum += totals[d];
     uint32_t total;
-    uint32_t run = block_prefix_256(sum, wave_sums, &total);
+    uint32_t run = block_prefix<THREADS>(sum, wave_sums, &total);
     for (uint32_t d = b; d < e; ++d) {
       start[d] = run + table[static_cast<size_t>(d) * gridDim.x + blockIdx.x];
       run += totals[d];
     }
   }
-  uint32_t digit[kHopSortItems], idx[kHopSortItems];
+  uint32_t digit[ITEMS], idx[ITEMS];
 #pragma unroll
-  for (int j = 0; j < kHopSortItems; ++j) {  // coalesced load into LDS
-    const uint32_t p = j * kHopSortThreads + threadIdx.x;
+  for (int j = 0; j < ITEMS; ++j) {  // coalesced load into LDS
+    const uint32_t p = j * THREADS + threadIdx.x;
     if (p < n) {
       chunk_keys[p] = keys_in[c0 + p];
       chunk_vals[p] = vals_in ? vals_in[c0 + p] : static_cast<uint32_t>(c0 + p);
@@ -335,24 +340,26 @@ __global__ __launch_bounds__(kHopSortThreads) void hop_sort_scatter_kernel(uint3
   }
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < kHopSortItems; ++j) {
-    const uint32_t p = threadIdx.x * kHopSortItems + j;  // blocked arrangement keeps the input order
+  for (int j = 0; j < ITEMS; ++j) {
+    const uint32_t p = threadIdx.x * ITEMS + j;  // blocked arrangement keeps the input order
     idx[j] = p;
-    digit[j] = p < n ? ((chunk_keys[p] >> shift) & mask) : bins;  // the chunk's unused tail sorts last
+    // The chunk's unused tail takes the largest digit: it comes last in the input, so the stable
+    // sort leaves it behind every edge, at positions n and above.
+    digit[j] = p < n ? ((chunk_keys[p] >> shift) & mask) : mask;
   }
-  Sort().sort(digit, idx, sort_storage, 0, digit_bits + 1);
+  Sort().sort(digit, idx, sort_storage, 0, digit_bits);
 #pragma unroll
-  for (int j = 0; j < kHopSortItems; ++j) sorted_digit[threadIdx.x * kHopSortItems + j] = static_cast<uint16_t>(digit[j]);
+  for (int j = 0; j < ITEMS; ++j) sorted_digit[threadIdx.x * ITEMS + j] = static_cast<uint16_t>(digit[j]);
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < kHopSortItems; ++j) {  // the first element of every run records where the run begins
-    const uint32_t p = threadIdx.x * kHopSortItems + j;
+  for (int j = 0; j < ITEMS; ++j) {  // the first element of every run records where the run begins
+    const uint32_t p = threadIdx.x * ITEMS + j;
     if (p < n && (p == 0 || sorted_digit[p - 1] != sorted_digit[p])) first_at[digit[j]] = p;
   }
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < kHopSortItems; ++j) {
-    const uint32_t p = threadIdx.x * kHopSortItems + j;
+  for (int j = 0; j < ITEMS; ++j) {
+    const uint32_t p = threadIdx.x * ITEMS + j;
     if (p < n) {
       const uint32_t pos = start[digit[j]] + (p - first_at[digit[j]]);
       keys_out[pos] = chunk_keys[idx[j]];
@@ -383,7 +390,7 @@ hipError_t sort_pairs_temp_bytes(uint32_t E, size_t *bytes) {
 }  // namespace
 
 // Scratch layout: [sorted keys: n][keys between passes: n][values between passes: n]
-//                 [digit table: 512 x ceil(n / 2048)][digit totals: 512], all u32.
+//                 [digit table: 1,024 x ceil(n / 2048)][digit totals: 1,024], all u32.
 size_t csr_from_csc_bytes(uint32_t sort_n) {
   const size_t arr = align_up(static_cast<size_t>(sort_n ? sort_n : 1) * sizeof(uint32_t), 256);
   const HopSortShape sh = hop_sort_shape(sort_n, 32);
@@ -417,8 +424,9 @@ int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co,
                        sh.digit_bits);
     hipLaunchKernelGGL(hop_sort_rows_kernel, dim3(1u << sh.digit_bits), dim3(kHopSortThreads), 0, stream, table, totals,
                        sh.blocks, E);
-    hipLaunchKernelGGL(hop_sort_scatter_kernel, dim3(sh.blocks), dim3(kHopSortThreads), 0, stream, kout, vout, kin, vin,
-                       table, totals, E, shift, sh.digit_bits);
+    // (512 x 4 and 1,024 x 2 were measured as well: the same within 3 %)
+    hipLaunchKernelGGL((hop_sort_scatter_kernel<kHopSortThreads, kHopSortItems>), dim3(sh.blocks), dim3(kHopSortThreads), 0,
+                       stream, kout, vout, kin, vin, table, totals, E, shift, sh.digit_bits);
     NTS_LAUNCH_CHECK("hop_sort kernels");
     kin = kout;
     vin = vout;

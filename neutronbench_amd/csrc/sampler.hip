@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
                                                        const uint32_t *__restrict__ graph_co,
                                                        const uint32_t *__restrict__ graph_ri,
                                                        const uint32_t *__restrict__ dst, DevCount n,
-                                                       uint32_t edge_cap, int32_t fanout, uint64_t seed,
+                                                       uint32_t edge_cap, int32_t fanout, DevSeed seed,
                                                        uint32_t *__restrict__ mark) {
   const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) / G;
   if (i >= n.get()) return;  // whole groups leave together
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
     for (uint32_t k = gl; k < deg; k += G) emit(ri_out, mark, out + k, graph_ri[base + k]);
     return;
   }
-  const uint64_t state0 = mix64(seed ^ (static_cast<uint64_t>(i) << 32) ^ d);
+  const uint64_t state0 = mix64(seed.get() ^ (static_cast<uint64_t>(i) << 32) ^ d);
   if (take > kMaxFanout || take > G) return;  // fanouts above one wavefront: hop_pick_wide_kernel
   // Lane gl < take: step j = deg - take + gl, hash chain advanced gl + 1 times.
   uint64_t state = state0;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void hop_pick_wide_kernel(uint32_t *__restrict
                                                             const uint32_t *__restrict__ graph_co,
                                                             const uint32_t *__restrict__ graph_ri,
                                                             const uint32_t *__restrict__ dst, DevCount n,
-                                                            uint32_t edge_cap, uint64_t seed,
+                                                            uint32_t edge_cap, DevSeed seed,
                                                             uint32_t *__restrict__ mark) {
   __shared__ uint32_t picked[4][kWidestFanout];
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void hop_pick_wide_kernel(uint32_t *__restrict
   const uint32_t out = co[i];
   const uint32_t take = co[i + 1] - out;
   if (co[i + 1] > edge_cap || take == deg || take <= static_cast<uint32_t>(kMaxFanout)) return;
-  const uint64_t key = mix64(seed ^ (static_cast<uint64_t>(i) << 32) ^ d);
+  const uint64_t key = mix64(seed.get() ^ (static_cast<uint64_t>(i) << 32) ^ d);
   uint32_t bits = 1;
   while ((1ull << bits) < deg) ++bits;
   const uint32_t mask = bits >= 32 ? 0xFFFFFFFFu : (1u << bits) - 1u;
@@ -205,7 +205,7 @@ int hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, Dev
 }
 
 int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co, const uint32_t *graph_ri,
-                  const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, uint64_t seed, uint32_t *mark_bits,
+                  const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, DevSeed seed, uint32_t *mark_bits,
                   hipStream_t stream) {
   // Lanes per destination: the fanout rounded up to a power of two (full neighbourhoods and
   // fanouts above one wavefront are strided copies, for which a quarter wavefront serves well).
@@ -267,7 +267,7 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
   if (n == 0) return NTS_OK;
   if (!ri_global || !co || !graph_co || !graph_ri || !dst)
     return fail(NTS_ERR_INVALID, "nts_sample_hop_neighbors: null pointer");
-  return hop_neighbors(ri_global, co, graph_co, graph_ri, dst, host_count(n), 0xFFFFFFFFu, fanout, seed, nullptr,
+  return hop_neighbors(ri_global, co, graph_co, graph_ri, dst, host_count(n), 0xFFFFFFFFu, fanout, host_seed(seed), nullptr,
                        stream);
 }
 

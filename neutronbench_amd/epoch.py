@@ -61,7 +61,7 @@ class Timer:
 
 
 def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False, checksum=False,
-        stage_sync=None):
+        stage_sync=None, graph=True):
     cfg = dict(CONFIGS[name])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
@@ -88,7 +88,9 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     n_batches = (n_train + cfg["batch"] - 1) // cfg["batch"]
     if max_batches:
         n_batches = min(n_batches, max_batches)
-    builder = BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0) if sampler == "builder" else None
+    # graph: a builder records the launches of its hops once and replays them as a HIP graph
+    builder = (BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0, graph=graph)
+               if sampler == "builder" else None)
     train32 = as_u32(train_nodes)
     # pipeline = P > 1 (the reference's PIPELINES mode: P batches in flight, each on a stream of its
     # own and driven by a thread of its own, one batch at a time in each of the sample, transfer and
@@ -104,7 +106,8 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     staged_gather = pipelined and pipeline > 2
     builders = [builder]
     if pipelined:
-        builders += [BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0) for _ in range(pipeline - 1)]
+        builders += [BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0, graph=graph)
+                     for _ in range(pipeline - 1)]
         sample_streams = [torch.cuda.Stream(device=dev) for _ in range(max(1, pipeline - 2))]
         gather_stream = torch.cuda.Stream(device=dev) if staged_gather else None
     totals = {"edges": 0, "hits": 0, "rows": 0}
@@ -306,7 +309,8 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         "fanout_output_side_first": cfg["fanout"], "epoch_s": round(epoch_s, 4),
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
         "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
-        "sampler": sampler, "pipeline": pipeline if pipelined else 1, "stage_sync": stage_sync,
+        "sampler": sampler, "hop_launches_as_graph": bool(graph and sampler == "builder"),
+        "pipeline": pipeline if pipelined else 1, "stage_sync": stage_sync,
         "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
         "checksum": float(checksum_on_device.item()) if checksum else None,
@@ -334,6 +338,9 @@ if __name__ == "__main__":
                     help="1: wait for the stream after every stage (stage times are device times; default up to "
                          "--pipeline 2); 0: never wait for an aggregation, batches are ordered by events (stage times "
                          "are host enqueue times; default from --pipeline 3)")
+    ap.add_argument("--graph", type=int, default=1, choices=[0, 1],
+                    help="1 (default): each builder replays the launches of its hops as a HIP graph recorded at its "
+                         "first batch; 0: the launches are enqueued one by one for every batch")
     a = ap.parse_args()
     run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline,
-        stage_sync=None if a.stage_sync is None else bool(a.stage_sync))
+        stage_sync=None if a.stage_sync is None else bool(a.stage_sync), graph=bool(a.graph))

@@ -178,3 +178,56 @@ def test_two_builders_on_two_streams_overlap_without_interference(device):
                 assert getattr(l, name).cpu().numpy().tobytes() == expect[name].tobytes(), f"batch {k} {name}"
     for b in builders:
         b.close()
+
+
+@pytest.mark.parametrize("fanouts,want_perm", [([25, 10], True), ([15, 10, 5], True), ([64, 100], True)])
+def test_builder_replaying_a_graph_equals_the_launch_by_launch_builder(device, fanouts, want_perm):
+    """nts_batch_builder_use_graph: the hops' launches are recorded at the first batch and replayed
+    for every later one.  Replays are interleaved with eager work and synchronisations of the
+    program's own (the per-hop path run for comparison, read-backs), batch sizes and seeds change
+    from replay to replay, and every replay must give the arrays of the eager builder bit for bit."""
+    V, E, cap = 30000, 700000, 1500
+    gco, gri = graph(V, E, 61, device)
+    perm = synth.permutation(V, 62, device)
+    eager = BatchBuilder(gco, gri, fanouts, cap, want_perm=want_perm)
+    replay = BatchBuilder(gco, gri, fanouts, cap, want_perm=want_perm, graph=True)
+    sizes = [1500, 1500, 640, 1, 0, 1499, 77, 1500]
+    at = 0
+    for k, n in enumerate(sizes):
+        ids = as_u32(perm[at:at + n])
+        at += n
+        got = replay.sample(ids, 7000 + 13 * k)
+        want = eager.sample(ids, 7000 + 13 * k)
+        assert_same_layers(got, want)
+        if n and k % 3 == 0:  # and both equal the per-hop entry points
+            assert_same_layers(got, per_hop_layers(gco, gri, ids, fanouts, 7000 + 13 * k, V))
+        torch.cuda.synchronize()
+    eager.close()
+    replay.close()
+
+
+def test_graph_builders_on_two_streams(device):
+    """Two builders in graph mode, each captured on and replayed to a stream of its own while the
+    other one's batch is still in flight."""
+    V, E, fanouts, batch = 40000, 900000, [10, 15], 2000
+    gco, gri = graph(V, E, 71, device)
+    perm = as_u32(synth.permutation(V, 72, device))
+    lone = BatchBuilder(gco, gri, fanouts, batch, want_perm=True)
+    want = []
+    for k in range(6):
+        layers = lone.sample(perm[k * batch:(k + 1) * batch], 190 + k)
+        want.append([{name: getattr(l, name).cpu().numpy().copy() for name in ARRAYS} for l in layers])
+    lone.close()
+    builders = [BatchBuilder(gco, gri, fanouts, batch, want_perm=True, graph=True) for _ in range(2)]
+    streams = [torch.cuda.Stream(device=device) for _ in range(2)]
+    torch.cuda.synchronize()
+    builders[0].enqueue(perm[0:batch], 190, streams[0].cuda_stream)
+    for k in range(6):
+        if k + 1 < 6:
+            builders[(k + 1) % 2].enqueue(perm[(k + 1) * batch:(k + 2) * batch], 191 + k, streams[(k + 1) % 2].cuda_stream)
+        layers = builders[k % 2].collect()
+        for l, expect in zip(layers, want[k]):
+            for name in ARRAYS:
+                assert getattr(l, name).cpu().numpy().tobytes() == expect[name].tobytes(), f"batch {k} {name}"
+    for b in builders:
+        b.close()
