@@ -22,6 +22,7 @@
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
+#include <rocprim/iterator/transform_iterator.hpp>
 
 #include <algorithm>
 #include <atomic>
@@ -141,8 +142,9 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
                                                         const float *__restrict__ w,
                                                         const uint32_t *__restrict__ offsets,
                                                         const uint32_t *__restrict__ indices, uint32_t index_base,
-                                                        uint32_t n_items, uint32_t F, uint32_t col_base,
-                                                        const Item *__restrict__ items, float *__restrict__ partial,
+                                                        uint32_t n_items, uint32_t n_list, uint32_t F,
+                                                        uint32_t col_base, const Item *__restrict__ items,
+                                                        float *__restrict__ partial,
                                                         int accumulate, HeadArgs heads, uint32_t row_edge_limit,
                                                         const uint32_t *__restrict__ edge_ids, uint32_t in_ld,
                                                         uint32_t partial_ld, int out_scalar) {
@@ -152,17 +154,19 @@ __global__ __launch_bounds__(256) void spmm_wave_kernel(const float *__restrict_
   const uint32_t item = blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
   if (item >= n_items) return;
 
+  // Work items [0, n_list) come from the list, the ones after it are the rows 0, 1, ... themselves
+  // (a launch may hold both: the pieces of long rows first, then every row that fits one wavefront).
   uint32_t row, e0, e1, slot;
-  if (items) {
+  if (item < n_list) {
     const Item it = items[item];
     row = wave_first(it.x);
     e0 = wave_first(it.y);
     e1 = wave_first(it.z);
     slot = wave_first(it.w);
   } else {
-    row = item;
-    e0 = wave_first(offsets[item]);
-    e1 = wave_first(offsets[item + 1]);
+    row = item - n_list;
+    e0 = wave_first(offsets[row]);
+    e1 = wave_first(offsets[row + 1]);
     slot = kNoSlot;
     if (e1 - e0 > row_edge_limit) return;  // a long row: its pieces are separate work items
   }
@@ -352,8 +356,9 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
                                                          const float *__restrict__ w,
                                                          const uint32_t *__restrict__ offsets,
                                                          const uint32_t *__restrict__ indices, uint32_t index_base,
-                                                         uint32_t n_items, uint32_t F, const Item *__restrict__ items,
-                                                         float *__restrict__ partial, int accumulate, HeadArgs heads,
+                                                         uint32_t n_items, uint32_t n_list, uint32_t F,
+                                                         const Item *__restrict__ items, float *__restrict__ partial,
+                                                         int accumulate, HeadArgs heads,
                                                          uint32_t row_edge_limit,
                                                          const uint32_t *__restrict__ edge_ids) {
   using V = typename Vec<VEC>::type;
@@ -363,16 +368,16 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
   if (item >= n_items) return;  // whole groups leave together; shuffles stay inside a group
 
   uint32_t row, e0, e1, slot;
-  if (items) {
+  if (item < n_list) {  // listed work items first, then the rows themselves
     const Item it = items[item];
     row = it.x;
     e0 = it.y;
     e1 = it.z;
     slot = it.w;
   } else {
-    row = item;
-    e0 = offsets[item];
-    e1 = offsets[item + 1];
+    row = item - n_list;
+    e0 = offsets[row];
+    e1 = offsets[row + 1];
     slot = kNoSlot;
     if (e1 - e0 > row_edge_limit) return;  // a long row: its pieces are separate work items
   }
@@ -606,18 +611,21 @@ struct LaunchArgs {
   uint32_t in_ld = 0;                          // row stride of `in` in floats (0 = F)
   uint32_t partial_ld = 0;                     // row stride of `partial` in floats (0 = F)
   bool dup_runs = false;                       // rows hold runs of equal indices worth loading once per run
+  uint32_t rows_after_items = 0;               // with items: this many whole rows follow the listed items in the launch
 };
 
 template <int VEC, int NACC>
 void launch_wave(const LaunchArgs &a, uint32_t col_base) {
   constexpr int kWavesPerBlock = 4;
-  const uint32_t blocks = ceil_div(a.n_items, kWavesPerBlock);
+  const uint32_t n_list = a.items ? a.n_items : 0u, n_total = a.n_items + (a.items ? a.rows_after_items : 0u);
+  const uint32_t blocks = ceil_div(n_total, kWavesPerBlock);
   const dim3 grid(blocks), block(kWavesPerBlock * kWave);
   // Neighbour pairs always go through the wave-private LDS tile (a register-broadcast variant measured
   // the same: 12.44 ms against 12.40 ms for the 114.8 M-edge F=602 gather).
 #define NTS_LAUNCH_WAVE(HD, RM, RUNS)                                                                                  \
   hipLaunchKernelGGL((spmm_wave_kernel<VEC, NACC, true, HD, RM, RUNS>), grid, block, 0, a.stream, a.in, a.out, a.w,    \
-                     a.offsets, a.indices, a.index_base, a.n_items, a.F, col_base, a.items, a.partial, a.accumulate,  \
+                     a.offsets, a.indices, a.index_base, n_total, n_list, a.F, col_base, a.items, a.partial,         \
+                     a.accumulate,                                                                                     \
                      a.heads, a.row_edge_limit, a.edge_ids, a.in_ld ? a.in_ld : a.F,                                  \
                      a.partial_ld ? a.partial_ld : a.F,                                                                \
                      (VEC > 1 && (a.F % VEC != 0 || !aligned_to(a.out, 4 * VEC))) ? 1 : 0)
@@ -636,10 +644,12 @@ void launch_wave(const LaunchArgs &a, uint32_t col_base) {
 template <int G, int VEC>
 void launch_group(const LaunchArgs &a) {
   const uint32_t per_block = 256 / G;
-  const uint32_t blocks = ceil_div(a.n_items, per_block);
+  const uint32_t n_list = a.items ? a.n_items : 0u, n_total = a.n_items + (a.items ? a.rows_after_items : 0u);
+  const uint32_t blocks = ceil_div(n_total, per_block);
 #define NTS_LAUNCH_GROUP(HD, RM, RUNS)                                                                                  \
   hipLaunchKernelGGL((spmm_group_kernel<G, VEC, HD, RM, RUNS>), dim3(blocks), dim3(256), 0, a.stream, a.in, a.out, a.w, \
-                     a.offsets, a.indices, a.index_base, a.n_items, a.F, a.items, a.partial, a.accumulate, a.heads,     \
+                     a.offsets, a.indices, a.index_base, n_total, n_list, a.F, a.items, a.partial, a.accumulate,        \
+                     a.heads,                                                                                          \
                      a.row_edge_limit, a.edge_ids)
   if (a.edge_ids) {
     if (a.heads.H) NTS_LAUNCH_GROUP(true, true, false);
@@ -743,18 +753,19 @@ constexpr uint32_t kAutoChunk = 256;
 // source rows fit the caches anyway and every launch saved counts at this size.
 constexpr uint32_t kAutoLargeEdges = 1u << 22;
 
-__global__ __launch_bounds__(256) void auto_count_kernel(uint32_t *__restrict__ pieces,
-                                                         const uint32_t *__restrict__ off, uint32_t rows,
-                                                         uint32_t chunk) {
-  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
-  if (r > rows) return;
-  uint32_t n = 0;
-  if (r < rows) {
+// Pieces of row r: 0 for a row that fits one wavefront, else ceil(degree / chunk); 0 for r == rows,
+// so that the exclusive scan's last entry is the total.  Evaluated inside the scan (no launch and no
+// array of its own).
+struct PieceCount {
+  const uint32_t *off;
+  uint32_t rows, chunk;
+  __host__ __device__ uint32_t operator()(uint32_t r) const {
+    if (r >= rows) return 0u;
     const uint32_t deg = off[r + 1] - off[r];
-    if (deg > chunk) n = (deg + chunk - 1) / chunk;
+    return deg > chunk ? (deg + chunk - 1) / chunk : 0u;
   }
-  pieces[r] = n;  // pieces[rows] = 0, so that the scan's last entry is the total
-}
+};
+using PieceCountIterator = rocprim::transform_iterator<rocprim::counting_iterator<uint32_t>, PieceCount, uint32_t>;
 
 // Also writes keys[i] = the gather index of the piece's first edge (0xFFFFFFFF for an empty item):
 // the pieces are then issued in ascending key order, so that wavefronts resident at the same time
@@ -878,7 +889,8 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
   size_t scan_bytes = 0, sort_bytes = 0;
   {
     uint32_t *nul = nullptr;
-    NTS_HIP_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, nul, nul, 0u, static_cast<size_t>(rows) + 1,
+    PieceCountIterator none(rocprim::counting_iterator<uint32_t>(0u), PieceCount{nullptr, 0u, chunk});
+    NTS_HIP_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, none, nul, 0u, static_cast<size_t>(rows) + 1,
                                         rocprim::plus<uint32_t>(), a.stream, false));
     NTS_HIP_TRY(rocprim::radix_sort_pairs(nullptr, sort_bytes, nul, nul, rocprim::counting_iterator<uint32_t>(0u), nul,
                                           p_max, 0u, 32u, a.stream, false));
@@ -888,7 +900,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
   const size_t n_items_b = up256(static_cast<size_t>(p_max) * sizeof(Item));
   const size_t n_keys_b = up256(static_cast<size_t>(p_max) * sizeof(uint32_t));
   const size_t n_partial = up256(static_cast<size_t>(p_max) * a.F * sizeof(float));
-  const size_t need = 2 * n_off + 2 * n_items_b + 3 * n_keys_b + tmp_bytes + n_partial;
+  const size_t need = n_off + 2 * n_items_b + 3 * n_keys_b + tmp_bytes + n_partial;
   unsigned char *buf = fixed;
   if (fixed) {
     if (need > fixed_cap) {
@@ -906,7 +918,6 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
     cursor += bytes;
     return p;
   };
-  uint32_t *pieces = reinterpret_cast<uint32_t *>(take(n_off));
   uint32_t *base = reinterpret_cast<uint32_t *>(take(n_off));
   Item *items = reinterpret_cast<Item *>(take(n_items_b));
   Item *ordered = reinterpret_cast<Item *>(take(n_items_b));
@@ -919,12 +930,9 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
     if (!fixed) (void)scratch_free(buf, a.stream);
     return fail_hip(err, what);
   };
-  hipLaunchKernelGGL(auto_count_kernel, dim3(ceil_div(static_cast<uint64_t>(rows) + 1, 256)), dim3(256), 0, a.stream,
-                     pieces, a.offsets, rows, chunk);
-  hipError_t err = hipGetLastError();
-  if (err != hipSuccess) return bail(err, "auto_count_kernel");
-  err = rocprim::exclusive_scan(tmp, scan_bytes, pieces, base, 0u, static_cast<size_t>(rows) + 1,
-                                rocprim::plus<uint32_t>(), a.stream, false);
+  PieceCountIterator counts(rocprim::counting_iterator<uint32_t>(0u), PieceCount{a.offsets, rows, chunk});
+  hipError_t err = rocprim::exclusive_scan(tmp, scan_bytes, counts, base, 0u, static_cast<size_t>(rows) + 1,
+                                           rocprim::plus<uint32_t>(), a.stream, false);
   if (err != hipSuccess) return bail(err, "spmm: scan of piece counts");
   hipLaunchKernelGGL(auto_items_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, items, keys, base, a.offsets,
                      a.indices, a.index_base, rows, chunk, p_max);
@@ -939,15 +947,15 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
     err = hipGetLastError();
     if (err != hipSuccess) return bail(err, "auto_order_items_kernel");
   }
-  // Pieces first (the heavy, uniform work), then the rows that fit one wavefront.
+  // One launch: the pieces first (the heavy, uniform work), then the rows that fit one wavefront,
+  // so that the rows fill the chip while the last pieces, each a serial chain, finish.
   LaunchArgs pc = a;
   pc.n_items = p_max;
   pc.items = large ? ordered : items;
   pc.partial = partial;
+  pc.rows_after_items = rows;
+  pc.row_edge_limit = chunk;
   launch_spmm(pc);
-  LaunchArgs whole = a;
-  whole.row_edge_limit = chunk;
-  launch_spmm(whole);
 #define NTS_AUTO_REDUCE_WIDE(J)                                                                                     \
   hipLaunchKernelGGL(auto_reduce_wide_kernel<J>, dim3(p_max), dim3(256), 0, a.stream, a.out, partial, items, base, a.F, \
                      a.accumulate, p_max)
