@@ -152,7 +152,7 @@ int nts_event_elapsed_ms(float *ms, nts_event_t start, nts_event_t stop);
  * order -- still deterministic, but a long row's sum is then associated piece by piece.  P = 256
  * edges; from 2^22 edges up the pieces are also issued in source order.  That path takes stream-ordered scratch
  * from the library's pool (see nts_scratch_trim; about (E/P + min(rows, E/P) + 1) * (F * 4 + 48)
- * bytes plus 8 bytes per row, released in stream order before the call returns); a caller that
+ * bytes plus 4 bytes per row, released in stream order before the call returns); a caller that
  * must not allocate, or that runs the same structure many times, uses a plan (below), which also
  * orders the pieces for the L2. */
 int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t *offsets,
