@@ -313,3 +313,48 @@ def test_wide_fanouts_pick_spread_positions_uniformly(device):
     # fanouts beyond the supported width are refused
     assert abi.status("nts_sample_hop_neighbors", ptr(ri), ptr(co), ptr(gco), ptr(gri), ptr(dst), n, 2000, 1,
                       torch.cuda.current_stream().cuda_stream) == abi.NTS_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("Vs,E,skew", [
+    (1, 5000, 0.0),            # one source: every key equal, one digit, one pass
+    (700, 2047, 0.0),          # one edge short of a chunk
+    (1024, 2048, 0.5),         # exactly one chunk, ten key bits: one pass
+    (1025, 2049, 0.5),         # eleven key bits: two passes; one edge into the second chunk
+    (40000, 100_000, 0.9),     # sixteen bits, a hub source holding most edges
+    (1_100_000, 300_000, 0.3), # twenty-one bits: three passes, most sources without an edge
+    (3_000_000, 70_000, 0.0),  # twenty-two bits
+])
+def test_hop_sort_over_digit_widths_and_chunk_boundaries(device, Vs, E, skew):
+    """nts_csr_from_csc sorts (local source, CSC edge id) with the library's own radix sort: passes of
+    equal width over ceil(bits / 10) digits, 2,048 edges per block.  Against numpy's stable sort, for
+    key widths that take one to three passes, edge counts on both sides of a chunk boundary, equal
+    keys in bulk (stability) and sparse keys."""
+    rng = np.random.default_rng(Vs + E)
+    Vd = max(1, E // 7)
+    cuts = np.sort(rng.integers(0, E + 1, Vd - 1))
+    co = np.concatenate([[0], cuts, [E]]).astype(np.uint32)
+    ri = rng.integers(0, Vs, E).astype(np.uint32)
+    if skew:
+        hub = rng.integers(0, Vs)
+        ri[rng.random(E) < skew] = hub
+    order = np.argsort(ri, kind="stable").astype(np.uint32)
+    ro_want = np.searchsorted(ri[order], np.arange(Vs + 1)).astype(np.uint32)
+    owner = (np.searchsorted(co, np.arange(E), side="right") - 1).astype(np.uint32)
+    ci_want = owner[order]
+    d_co, d_ri = torch.from_numpy(co.view(np.int32)).to(device), torch.from_numpy(ri.view(np.int32)).to(device)
+    ro = torch.empty(Vs + 1, dtype=torch.int32, device=device)
+    ci = torch.empty(E, dtype=torch.int32, device=device)
+    perm = torch.empty(E, dtype=torch.int32, device=device)
+    nbytes = call("nts_csr_from_csc_work_bytes", Vd, Vs, E)
+    work = torch.empty(nbytes + 256, dtype=torch.uint8, device=device)
+    base = (work.data_ptr() + 255) // 256 * 256
+    s = torch.cuda.current_stream().cuda_stream
+    for with_perm in (True, False):
+        ro.fill_(-1)
+        ci.fill_(-1)
+        call("nts_csr_from_csc", ptr(ro), ptr(ci), ptr(perm) if with_perm else 0, ptr(d_co), ptr(d_ri), Vd, Vs, E, base, s)
+        torch.cuda.synchronize()
+        assert np.array_equal(host_u32(ro), ro_want)
+        assert np.array_equal(host_u32(ci), ci_want)
+        if with_perm:
+            assert np.array_equal(host_u32(perm), order)
