@@ -89,9 +89,13 @@ def test_reference_gpu_operator_equals_its_cpu_operator_on_sampled_layers(arxiv_
     assert "worst_max_rel_err" in out
 
 
-def test_gcn_gpu_neighbor_toolkit_runs_unchanged(arxiv_shaped_files):
+@pytest.mark.parametrize("mode", ["pipeline", "explicit", "zerocopy"])
+def test_gcn_gpu_neighbor_toolkit_runs_unchanged(arxiv_shaped_files, mode):
+    """The toolkit's three batch loops (toolkits/GCN_GPU_NEIGHBOR.hpp:767-775): `pipeline` (stage threads),
+    `explicit` (features gathered on the host, then copied) and `zerocopy` (gathered by the device from
+    pinned host memory; this loop also fills the `graph` and `nn` columns of the log line)."""
     d = arxiv_shaped_files
-    out = run(NTS, write_cfg(d, "GCNNEIGHBORGPU"), cwd=d)
+    out = run(NTS, write_cfg(d, "GCNNEIGHBORGPU", MODE=mode), cwd=d)
     epochs = re.findall(r"Epoch (\d+) train_loss (\S+) train_acc (\S+) val_loss (\S+) val_acc (\S+) test_acc (\S+) "
                         r"train_time (\S+)\(sample (\S+) trans (\S+) graph (\S+) nn (\S+)\)", out)
     assert [e[0] for e in epochs] == ["000", "001"]
