@@ -127,3 +127,25 @@ def test_full_graph_toolkits_run_unchanged(arxiv_shaped_files, algorithm):
     print(f"{algorithm}: losses {losses}")
     assert len(losses) == 8 and all(math.isfinite(x) and 0 < x < 20 for x in losses)
     assert losses[-1] < losses[0]
+
+
+@pytest.mark.parametrize("algorithm,extra,expect", [
+    ("GCNNEIGHBORGPUEXP3", {}, r"Epoch 001 epoch_time \S+ sample_time \S+ gather_time \S+ trans_time \S+ train_time"),
+    ("GCNNEIGHBORGPUCACHEEXP", dict(CACHE_TYPE="rate", CACHE_POLICY="degree", CACHE_RATE_START=0.0, CACHE_RATE_END=0.3,
+                                    CACHE_RATE_NUM=3), r"cache_rate 0\.300 cache_hit_rate 0\.\d+"),
+    ("GCNNEIGHBORGPUTRANSEXP", dict(MODE="zerocopy", TRANS_THRESHOLD_START=0.0, TRANS_THRESHOLD_END=0.5,
+                                    TRANS_THRESHOLD_NUM=2), r"Epoch 001 epoch_time \S+ cache_rate"),
+    ("GCNEAGER", {}, r"Epoch\[1\]:loss\s+\S+"),
+    ("COMMNETGPU", {}, r"Epoch\[1\]:loss\s+\S+"),
+])
+def test_further_gpu_toolkits_of_the_reference_run_to_the_end(arxiv_shaped_files, algorithm, extra, expect):
+    """The other single-GPU entries of toolkits/main.cpp that reach this library: the experiment variants
+    of the sampled GCN (epoch breakdown, feature-cache sweep with the cached gather, transfer-threshold
+    sweep), the eager full-graph GCN and CommNet.  They must run to their end and print their epoch lines."""
+    d = arxiv_shaped_files
+    out = run(NTS, write_cfg(d, algorithm, **extra), cwd=d)
+    found = re.findall(expect, out)
+    print(f"{algorithm}: {found[-1] if found else None}")
+    assert found
+    if algorithm == "GCNNEIGHBORGPUCACHEEXP":  # the top 30 % of the vertices by degree serve most of the gathered rows
+        assert float(found[-1].split()[-1]) > 0.5
