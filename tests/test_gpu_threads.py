@@ -77,3 +77,58 @@ def test_two_host_threads_on_two_streams(device):
             assert torch.equal(got, want)
     for _, table in work:
         table.close()
+
+
+def test_two_host_threads_each_replaying_a_builder_graph(device):
+    """Two host threads, each with a batch builder of its own in graph mode on a stream of its own: the
+    graphs are recorded (thread-local capture) and replayed while the other thread does the same.  Every
+    batch equals what a launch-by-launch builder gives alone."""
+    from neutronbench_amd import synth
+    from neutronbench_amd.batch import BatchBuilder
+    from neutronbench_amd.layout import as_u32
+
+    V, E, fanouts, batch, n_batches = 30000, 600000, [12, 8], 1000, 12
+    src, dst = synth.rmat_edges(V, E, seed=91, device=device, sort=True)
+    co, ri = synth.build_csc(src, dst, V)
+    gco, gri = as_u32(co), as_u32(ri)
+    names = ("dev_source", "dev_column_offset", "dev_row_indices", "dev_row_offset", "dev_column_indices",
+             "dev_edge_weight_forward", "dev_edge_weight_backward")
+    perms = [as_u32(synth.permutation(V, 92 + k, device)) for k in range(2)]
+
+    def batches(builder, k, stream):
+        out = []
+        for b in range(n_batches):
+            ids = perms[k][b * batch:(b + 1) * batch - 7 * b]  # shrinking batches
+            builder.enqueue(ids, 500 * k + b, stream)
+            layers = builder.collect()
+            out.append([{n: getattr(l, n).cpu().numpy().copy() for n in names} for l in layers])
+        return out
+
+    s0 = torch.cuda.current_stream(device).cuda_stream
+    want = []
+    for k in range(2):
+        plain = BatchBuilder(gco, gri, fanouts, batch)
+        want.append(batches(plain, k, s0))
+        plain.close()
+    got, failures = [None, None], []
+
+    def worker(k):
+        try:
+            stream = torch.cuda.Stream(device=device)
+            builder = BatchBuilder(gco, gri, fanouts, batch, graph=True)
+            got[k] = batches(builder, k, stream.cuda_stream)
+            builder.close()
+        except BaseException as exc:
+            failures.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
+    for k in range(2):
+        for b in range(n_batches):
+            for lg, lw in zip(got[k][b], want[k][b]):
+                for n in names:
+                    assert lg[n].tobytes() == lw[n].tobytes(), f"thread {k} batch {b} {n}"
