@@ -323,6 +323,56 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     return out
 
 
+def run_native(name, scale=1.0, max_batches=0, warmup_batches=2, pipeline=1, quiet=False, graph=True, verify=False,
+               stage_sync=False, keep_dir=None):
+    """The same epoch driven from C++ (neutronbench_amd/host/epoch_driver.cpp -> lib/nts_epoch): the
+    arrays of the synthetic configuration are written to a directory, the program runs the batches
+    through the C ABI with no Python between the calls and prints one JSON line.  GCN configurations
+    only.  Same graph, train ids and seeds as `run`, so sampled_edges and gathered_rows are equal."""
+    import os
+    import shutil
+    import subprocess
+    import tempfile
+
+    cfg = dict(CONFIGS[name])
+    if cfg.get("heads"):
+        raise ValueError("the native driver runs the GCN configurations")
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "nts_epoch")
+    if not os.path.exists(exe):
+        raise RuntimeError(f"{exe} has not been built (make -C neutronbench_amd/csrc)")
+    dev = torch.device("cuda:0")
+    V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
+    n_train = int(cfg["train"] * scale)
+    src, dst = synth.rmat_edges(V, E, seed=cfg["seed"], device=dev, sort=True)
+    co, ri = synth.build_csc(src, dst, V)
+    del src, dst
+    d = keep_dir or tempfile.mkdtemp(prefix="nts_epoch_")
+    try:
+        as_u32(co).cpu().numpy().tofile(os.path.join(d, "co.bin"))
+        as_u32(ri).cpu().numpy().tofile(os.path.join(d, "ri.bin"))
+        synth.normal_features(V, cfg["F"], seed=cfg["seed"] + 40).numpy().tofile(os.path.join(d, "feat.bin"))
+        synth.uniform_labels(V, cfg["classes"], seed=cfg["seed"] + 41, device=dev).cpu().numpy().tofile(
+            os.path.join(d, "labels.bin"))
+        as_u32(synth.permutation(V, cfg["seed"] + 42, dev)[:n_train]).cpu().numpy().tofile(os.path.join(d, "train.bin"))
+        del co, ri
+        torch.cuda.empty_cache()
+        cmd = [exe, "--dir", d, "--V", str(V), "--F", str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch",
+               str(cfg["batch"]), "--fanout", ",".join(map(str, cfg["fanout"])), "--pipeline", str(pipeline), "--cache",
+               str(cfg["cache"]), "--graph", str(int(graph)), "--warmup", str(warmup_batches), "--max-batches",
+               str(max_batches), "--verify", str(int(verify)), "--stage-sync", str(int(stage_sync))]
+        p = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        if p.returncode != 0:
+            raise RuntimeError(f"nts_epoch failed ({p.returncode}): {p.stderr[-2000:]}")
+        out = json.loads(p.stdout.strip().splitlines()[-1])
+    finally:
+        if keep_dir is None:
+            shutil.rmtree(d, ignore_errors=True)
+    out.update(config=name, scale=scale, vertices=V, edges=E, fanout_output_side_first=cfg["fanout"])
+    if not quiet:
+        print(json.dumps(out))
+    return out
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", choices=sorted(CONFIGS), required=True)
@@ -341,6 +391,12 @@ if __name__ == "__main__":
     ap.add_argument("--graph", type=int, default=1, choices=[0, 1],
                     help="1 (default): each builder replays the launches of its hops as a HIP graph recorded at its "
                          "first batch; 0: the launches are enqueued one by one for every batch")
+    ap.add_argument("--native", action="store_true",
+                    help="drive the epoch from C++ (lib/nts_epoch) instead of this module's Python loop")
     a = ap.parse_args()
-    run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline,
-        stage_sync=None if a.stage_sync is None else bool(a.stage_sync), graph=bool(a.graph))
+    if a.native:
+        run_native(a.config, a.scale, a.max_batches, a.warmup_batches, a.pipeline, graph=bool(a.graph),
+                   stage_sync=bool(a.stage_sync))
+    else:
+        run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline,
+            stage_sync=None if a.stage_sync is None else bool(a.stage_sync), graph=bool(a.graph))

@@ -1,0 +1,405 @@
+// One epoch of the sampled mini-batch path driven from C++ through the C ABI: the batch loop of
+// toolkits/GCN_GPU_NEIGHBOR.hpp (run(): 386-500; the PIPELINES mode: 1350-1363) with this library's own
+// sampler in place of the reference's CPU sampler, and without the dense layers.
+//
+// Per batch: nts_batch_builder_sample / _layers (all hops, relabelling, CSR, weights), the feature
+// gather (zero-copy from mapped pinned host memory, or through the HBM cache of the top out-degree
+// vertices), the label gather, and for every layer the aggregation forward (zeroed output,
+// accumulate, as SingleGPUSampleGraphOp does) and, in reverse order, backward.  Inputs of the layers
+// after the first and the incoming gradients stand in for the dense layers' results: constant
+// buffers of the right shape.
+//
+// --pipeline 1: everything on one stream.  --pipeline 2: the next batch is sampled on a second stream
+// while this one is gathered and aggregated.  --pipeline P >= 3: P - 2 batches are sampled ahead, each
+// chain of hops on a stream of its own, the next batch's features and labels are gathered on a gather
+// stream, the current one is aggregated; events order a batch's gather before its aggregation and
+// an arena's re-use after the aggregation that read it.  One host thread enqueues all of it.
+//
+// The program reads raw arrays written by neutronbench_amd/epoch.py (--native): co.bin, ri.bin (uint32
+// CSC of the whole graph), feat.bin (float32 [V, F]), labels.bin (int64 [V]), train.bin (uint32 ids),
+// and prints one JSON line.  --verify 1 adds a checksum of every aggregation output (a device-side
+// hash per batch, which waits for the stream: not for timing).
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <numeric>
+#include <string>
+#include <vector>
+
+#include "nts_hip.h"
+
+namespace {
+
+[[noreturn]] void die(const char *what) {
+  fprintf(stderr, "nts_epoch: %s: %s\n", what, nts_last_error());
+  exit(1);
+}
+#define NTS(call)                 \
+  do {                            \
+    if ((call) != NTS_OK) die(#call); \
+  } while (0)
+#define HIP(call)                                                              \
+  do {                                                                         \
+    hipError_t e_ = (call);                                                    \
+    if (e_ != hipSuccess) {                                                    \
+      fprintf(stderr, "nts_epoch: %s: %s\n", #call, hipGetErrorString(e_));    \
+      exit(1);                                                                 \
+    }                                                                          \
+  } while (0)
+
+double now() {
+  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+template <typename T>
+std::vector<T> read_file(const std::string &path, size_t expect = 0) {
+  FILE *f = fopen(path.c_str(), "rb");
+  if (!f) {
+    fprintf(stderr, "nts_epoch: cannot open %s\n", path.c_str());
+    exit(1);
+  }
+  fseek(f, 0, SEEK_END);
+  const size_t bytes = static_cast<size_t>(ftell(f));
+  fseek(f, 0, SEEK_SET);
+  std::vector<T> v(bytes / sizeof(T));
+  if (fread(v.data(), sizeof(T), v.size(), f) != v.size() || (expect && v.size() != expect)) {
+    fprintf(stderr, "nts_epoch: %s holds %zu elements, expected %zu\n", path.c_str(), v.size(), expect);
+    exit(1);
+  }
+  fclose(f);
+  return v;
+}
+
+template <typename T>
+T *to_device(const std::vector<T> &v) {
+  void *p = nullptr;
+  NTS(nts_malloc_device(&p, std::max<size_t>(v.size() * sizeof(T), 256)));
+  if (!v.empty()) NTS(nts_memcpy_h2d(p, v.data(), v.size() * sizeof(T), 1));
+  return static_cast<T *>(p);
+}
+
+void *device_bytes(size_t bytes) {
+  void *p = nullptr;
+  NTS(nts_malloc_device(&p, std::max<size_t>(bytes, 256)));
+  return p;
+}
+
+struct Args {
+  std::string dir;
+  std::vector<int32_t> fanout;
+  uint32_t V = 0, F = 0, hidden = 128, batch = 1024, pipeline = 1, warmup = 2, max_batches = 0;
+  double cache = 0.0;
+  int graph = 1, verify = 0, stage_sync = 0;
+};
+
+Args parse(int argc, char **argv) {
+  Args a;
+  for (int i = 1; i + 1 < argc; i += 2) {
+    const std::string k = argv[i], v = argv[i + 1];
+    if (k == "--dir") a.dir = v;
+    else if (k == "--V") a.V = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--F") a.F = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--hidden") a.hidden = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--batch") a.batch = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--pipeline") a.pipeline = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--warmup") a.warmup = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--max-batches") a.max_batches = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--cache") a.cache = std::stod(v);
+    else if (k == "--graph") a.graph = std::stoi(v);
+    else if (k == "--verify") a.verify = std::stoi(v);
+    else if (k == "--stage-sync") a.stage_sync = std::stoi(v);
+    else if (k == "--fanout") {
+      size_t at = 0;
+      while (at < v.size()) {
+        size_t end = v.find(',', at);
+        if (end == std::string::npos) end = v.size();
+        a.fanout.push_back(std::stoi(v.substr(at, end - at)));
+        at = end + 1;
+      }
+    } else {
+      fprintf(stderr, "nts_epoch: unknown option %s\n", k.c_str());
+      exit(2);
+    }
+  }
+  if (a.dir.empty() || !a.V || !a.F || a.fanout.empty() || a.pipeline < 1 || a.pipeline > 8) {
+    fprintf(stderr,
+            "usage: nts_epoch --dir D --V n --F n --fanout a,b[,c] [--batch n] [--hidden n] [--pipeline 1..8]\n"
+            "                 [--cache fraction] [--graph 0|1] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n");
+    exit(2);
+  }
+  return a;
+}
+
+struct Slot {  // one batch in flight
+  nts_batch_builder_t *builder = nullptr;
+  void *arena = nullptr;
+  nts_sampled_layer_t layers[8];
+  float *x = nullptr;       // gathered features [src_size of the input layer, F]
+  int64_t *labels = nullptr;
+  uint32_t *hits = nullptr;
+  hipEvent_t gathered = nullptr, trained = nullptr;
+  bool has_trained = false;
+};
+
+}  // namespace
+
+int main(int argc, char **argv) {
+  const Args a = parse(argc, argv);
+  const uint32_t hops = static_cast<uint32_t>(a.fanout.size());
+  const uint32_t V = a.V, F = a.F;
+  std::vector<uint32_t> co = read_file<uint32_t>(a.dir + "/co.bin", static_cast<size_t>(V) + 1);
+  std::vector<uint32_t> ri = read_file<uint32_t>(a.dir + "/ri.bin");
+  const uint32_t E = static_cast<uint32_t>(ri.size());
+  std::vector<int64_t> labels_h = read_file<int64_t>(a.dir + "/labels.bin", V);
+  std::vector<uint32_t> train = read_file<uint32_t>(a.dir + "/train.bin");
+  uint32_t *d_co = to_device(co), *d_ri = to_device(ri), *d_train = to_device(train);
+  int64_t *d_labels = to_device(labels_h);
+
+  // Feature table in mapped pinned host memory, read by the device over the link.
+  float *table = nullptr;
+  NTS(nts_malloc_pinned_mapped(reinterpret_cast<void **>(&table), static_cast<size_t>(V) * F * sizeof(float)));
+  {
+    std::vector<float> feat = read_file<float>(a.dir + "/feat.bin", static_cast<size_t>(V) * F);
+    memcpy(table, feat.data(), feat.size() * sizeof(float));
+  }
+  // HBM cache of the top out-degree vertices (descending out-degree, ties by ascending id).
+  const uint32_t n_cache = static_cast<uint32_t>(a.cache * V);
+  float *d_cache = nullptr;
+  uint32_t *d_hashmap = nullptr;
+  if (n_cache) {
+    std::vector<uint32_t> outdeg(V, 0);
+    for (uint32_t s : ri) ++outdeg[s];
+    std::vector<uint32_t> order(V);
+    std::iota(order.begin(), order.end(), 0u);
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return outdeg[x] > outdeg[y]; });
+    std::vector<uint32_t> hashmap(V, 0xFFFFFFFFu);
+    std::vector<float> rows(static_cast<size_t>(n_cache) * F);
+    for (uint32_t k = 0; k < n_cache; ++k) {
+      hashmap[order[k]] = k;
+      memcpy(rows.data() + static_cast<size_t>(k) * F, table + static_cast<size_t>(order[k]) * F, F * sizeof(float));
+    }
+    d_cache = to_device(rows);
+    d_hashmap = to_device(hashmap);
+  }
+
+  // Capacities: rows of a layer never exceed the graph or the product of the fanouts so far.
+  uint64_t max_rows = a.batch;
+  for (int32_t f : a.fanout) max_rows = f < 0 ? V : std::min<uint64_t>(V, max_rows * static_cast<uint32_t>(f));
+  const uint32_t maxw = std::max(F, a.hidden);
+  const uint32_t P = a.pipeline;
+  std::vector<Slot> slots(P);
+  const size_t arena_bytes = nts_batch_builder_arena_bytes(V, E, a.fanout.data(), hops, a.batch, 0);
+  if (!arena_bytes) die("nts_batch_builder_arena_bytes");
+  const uint32_t x_buffers = P >= 3 ? 2 : 1;  // the gather of the next batch overlaps this one's aggregation
+  std::vector<float *> xbuf(x_buffers);
+  std::vector<int64_t *> lbuf(x_buffers);
+  std::vector<uint32_t *> hbufs(x_buffers);
+  for (uint32_t k = 0; k < x_buffers; ++k) {
+    xbuf[k] = static_cast<float *>(device_bytes(max_rows * F * sizeof(float)));
+    lbuf[k] = static_cast<int64_t *>(device_bytes(static_cast<size_t>(a.batch) * sizeof(int64_t)));
+    hbufs[k] = static_cast<uint32_t *>(device_bytes(256));
+  }
+  for (Slot &s : slots) {
+    s.arena = device_bytes(arena_bytes);
+    NTS(nts_batch_builder_create(&s.builder, d_co, d_ri, V, E, a.fanout.data(), hops, a.batch, 0, s.arena, arena_bytes));
+    if (a.graph) NTS(nts_batch_builder_use_graph(s.builder, 1));
+    HIP(hipEventCreateWithFlags(&s.gathered, hipEventDisableTiming));
+    HIP(hipEventCreateWithFlags(&s.trained, hipEventDisableTiming));
+  }
+  // Stand-ins for what the dense layers would hand over, and the aggregation outputs.
+  std::vector<float> ones(max_rows * maxw, 1.0f);
+  float *d_ones = to_device(ones);
+  ones.clear();
+  ones.shrink_to_fit();
+  float *d_out = static_cast<float *>(device_bytes(max_rows * maxw * sizeof(float)));
+  float *d_gin = static_cast<float *>(device_bytes(max_rows * maxw * sizeof(float)));
+
+  hipStream_t main_stream = nullptr, gather_stream = nullptr;
+  HIP(hipStreamCreateWithFlags(&main_stream, hipStreamNonBlocking));
+  std::vector<hipStream_t> sample_streams;
+  if (P >= 2) {
+    const uint32_t chains = P >= 3 ? P - 2 : 1;
+    sample_streams.resize(chains);
+    for (hipStream_t &s : sample_streams) HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  }
+  if (P >= 3) HIP(hipStreamCreateWithFlags(&gather_stream, hipStreamNonBlocking));
+
+  const uint32_t n_train = static_cast<uint32_t>(train.size());
+  uint32_t n_batches = (n_train + a.batch - 1) / a.batch;
+  if (a.max_batches && a.max_batches < n_batches) n_batches = a.max_batches;
+  uint64_t edges_total = 0, rows_total = 0, checksum = 0;
+  std::vector<uint32_t *> hit_words;  // device words read at the end of the epoch
+  double t_sample = 0, t_gather = 0, t_fwd = 0, t_bwd = 0;
+
+  auto sample = [&](Slot &s, uint32_t b, hipStream_t stream) {
+    const uint32_t n = std::min(a.batch, n_train - b * a.batch);
+    NTS(nts_batch_builder_sample(s.builder, d_train + static_cast<size_t>(b) * a.batch, n, 1000ull * b, stream));
+  };
+  auto gather = [&](Slot &s, uint32_t buffer, hipStream_t stream) {
+    const nts_sampled_layer_t &in = s.layers[0], &top = s.layers[hops - 1];
+    s.x = xbuf[buffer];
+    s.labels = lbuf[buffer];
+    s.hits = hbufs[buffer];
+    if (n_cache)
+      NTS(nts_gather_rows_cached_f32(s.x, table, d_cache, in.source, d_hashmap, in.src_size, F, s.hits, stream));
+    else
+      NTS(nts_gather_rows_f32(s.x, table, in.source, nullptr, nullptr, in.src_size, F, stream));
+    NTS(nts_gather_labels_i64(s.labels, d_labels, top.destination, top.v_size, 1, stream));
+  };
+  uint64_t hits_total = 0;
+  auto aggregate = [&](Slot &s, hipStream_t stream) {
+    double t0 = now();
+    for (uint32_t l = 0; l < hops; ++l) {
+      const nts_sampled_layer_t &L = s.layers[l];
+      const uint32_t w = l == 0 ? F : a.hidden;
+      const float *in = l == 0 ? s.x : d_ones;
+      NTS(nts_memset_zero(d_out, static_cast<size_t>(L.v_size) * w * sizeof(float), stream));
+      NTS(nts_spmm_gather(in, d_out, L.edge_weight_forward, L.column_offset, L.row_indices, 0, L.v_size, L.e_size, w, 1,
+                          stream));
+      if (a.verify) {
+        uint64_t fp = 0;
+        NTS(nts_fingerprint_u32(&fp, reinterpret_cast<const uint32_t *>(d_out), static_cast<uint64_t>(L.v_size) * w,
+                                nullptr, 0, stream));
+        checksum ^= fp * (2 * l + 1);
+      }
+      if (a.stage_sync) HIP(hipStreamSynchronize(stream));
+    }
+    if (a.stage_sync) t_fwd += now() - t0;
+    t0 = now();
+    for (uint32_t k = hops; k-- > 0;) {
+      const nts_sampled_layer_t &L = s.layers[k];
+      const uint32_t w = k == 0 ? F : a.hidden;
+      NTS(nts_memset_zero(d_gin, static_cast<size_t>(L.src_size) * w * sizeof(float), stream));
+      NTS(nts_spmm_gather(d_ones, d_gin, L.edge_weight_backward, L.row_offset, L.column_indices, 0, L.src_size, L.e_size,
+                          w, 1, stream));
+      if (a.verify) {
+        uint64_t fp = 0;
+        NTS(nts_fingerprint_u32(&fp, reinterpret_cast<const uint32_t *>(d_gin), static_cast<uint64_t>(L.src_size) * w,
+                                nullptr, 0, stream));
+        checksum ^= fp * (2 * k + 2);
+      }
+      if (a.stage_sync) HIP(hipStreamSynchronize(stream));
+    }
+    if (a.stage_sync) t_bwd += now() - t0;
+  };
+  auto account = [&](Slot &s) {
+    for (uint32_t l = 0; l < hops; ++l) edges_total += s.layers[l].e_size;
+    rows_total += s.layers[0].src_size;
+  };
+  auto read_hits = [&](Slot &s, hipStream_t stream) {  // serial modes: after the gather has been waited for
+    if (!n_cache) return;
+    uint32_t h = 0;
+    NTS(nts_memcpy_d2h_async(&h, s.hits, sizeof(h), stream));
+    HIP(hipStreamSynchronize(stream));
+    hits_total += h;
+  };
+
+  auto run_batches = [&](uint32_t count) {
+    if (!count) return;
+    if (P == 1) {
+      Slot &s = slots[0];
+      for (uint32_t b = 0; b < count; ++b) {
+        double t0 = now();
+        sample(s, b, main_stream);
+        NTS(nts_batch_builder_layers(s.builder, s.layers));
+        t_sample += now() - t0;
+        t0 = now();
+        gather(s, 0, main_stream);
+        if (a.stage_sync) HIP(hipStreamSynchronize(main_stream));
+        t_gather += now() - t0;
+        account(s);
+        aggregate(s, main_stream);
+        if (a.stage_sync || a.verify) read_hits(s, main_stream);
+      }
+      return;
+    }
+    if (P == 2) {
+      auto start = [&](uint32_t b) {
+        Slot &s = slots[b % 2];
+        if (s.has_trained) HIP(hipStreamWaitEvent(sample_streams[0], s.trained, 0));
+        sample(s, b, sample_streams[0]);
+      };
+      start(0);
+      for (uint32_t b = 0; b < count; ++b) {
+        Slot &s = slots[b % 2];
+        NTS(nts_batch_builder_layers(s.builder, s.layers));
+        if (b + 1 < count) start(b + 1);
+        gather(s, 0, main_stream);
+        account(s);
+        aggregate(s, main_stream);
+        HIP(hipEventRecord(s.trained, main_stream));
+        s.has_trained = true;
+      }
+      return;
+    }
+    const uint32_t chains = static_cast<uint32_t>(sample_streams.size());
+    uint32_t started = 0;
+    auto sample_through = [&](uint32_t last) {
+      while (started <= std::min(last, count - 1)) {
+        Slot &s = slots[started % P];
+        hipStream_t stream = sample_streams[started % chains];
+        if (s.has_trained) HIP(hipStreamWaitEvent(stream, s.trained, 0));  // the arena's last batch is still being read
+        sample(s, started, stream);
+        ++started;
+      }
+    };
+    auto start_gather = [&](uint32_t b) {
+      Slot &s = slots[b % P];
+      NTS(nts_batch_builder_layers(s.builder, s.layers));
+      // the x buffer this gather writes was read by the aggregation two batches back
+      if (b >= 2 && slots[(b - 2) % P].has_trained) HIP(hipStreamWaitEvent(gather_stream, slots[(b - 2) % P].trained, 0));
+      gather(s, b % 2, gather_stream);
+      HIP(hipEventRecord(s.gathered, gather_stream));
+    };
+    sample_through(chains - 1);
+    start_gather(0);
+    sample_through(chains);
+    for (uint32_t b = 0; b < count; ++b) {
+      Slot &s = slots[b % P];
+      if (b + 1 < count) start_gather(b + 1);
+      sample_through(b + P - 1);
+      HIP(hipStreamWaitEvent(main_stream, s.gathered, 0));
+      account(s);
+      aggregate(s, main_stream);
+      HIP(hipEventRecord(s.trained, main_stream));
+      s.has_trained = true;
+    }
+  };
+
+  const uint32_t n_warm = std::min(a.warmup, n_batches);
+  run_batches(n_warm);
+  HIP(hipDeviceSynchronize());
+  for (Slot &s : slots) s.has_trained = false;
+  edges_total = rows_total = checksum = hits_total = 0;
+  t_sample = t_gather = t_fwd = t_bwd = 0;
+  const double t0 = now();
+  run_batches(n_batches);
+  HIP(hipDeviceSynchronize());
+  const double epoch_s = now() - t0;
+
+  printf("{\"driver\": \"native\", \"batches\": %u, \"batch_size\": %u, \"pipeline\": %u, \"hop_launches_as_graph\": %s, "
+         "\"stage_sync\": %s, \"epoch_s\": %.4f, \"sampled_edges\": %llu, \"gathered_rows\": %llu, \"cache_rows\": %u",
+         n_batches, a.batch, P, a.graph ? "true" : "false", a.stage_sync ? "true" : "false", epoch_s,
+         static_cast<unsigned long long>(edges_total), static_cast<unsigned long long>(rows_total), n_cache);
+  if (P == 1 && a.stage_sync)
+    printf(", \"stage_s\": {\"sample\": %.4f, \"gather\": %.4f, \"aggregate_fwd\": %.4f, \"aggregate_bwd\": %.4f}", t_sample,
+           t_gather, t_fwd, t_bwd);
+  if (n_cache && P == 1 && (a.stage_sync || a.verify))
+    printf(", \"cache_hit_rate\": %.4f", rows_total ? static_cast<double>(hits_total) / rows_total : 0.0);
+  if (a.verify) printf(", \"checksum\": \"%016llx\"", static_cast<unsigned long long>(checksum));
+  printf("}\n");
+
+  for (Slot &s : slots) {
+    NTS(nts_batch_builder_destroy(s.builder));
+    NTS(nts_free_device(s.arena));
+    HIP(hipEventDestroy(s.gathered));
+    HIP(hipEventDestroy(s.trained));
+  }
+  NTS(nts_free_pinned(table));
+  return 0;
+}

@@ -71,3 +71,22 @@ def test_stream_wrapper_can_leave_batch_assembly_unsynchronised():
     torch.cuda.current_stream().wait_event(done)
     assert torch.equal(out, table[ids.long()])
     assert CudaStream(side.cuda_stream).synchronize is True
+
+
+@pytest.mark.parametrize("config,scale", [("arxiv", 0.25), ("products", 0.02)])
+def test_native_epoch_driver(config, scale):
+    """The epoch driven from C++ (lib/nts_epoch, neutronbench_amd/host/epoch_driver.cpp): same graph,
+    train ids and seeds as the Python loop, so it samples the same edges, gathers the same rows and
+    hits the cache as often; its checksum of every aggregation output (a device-side hash per layer
+    and direction) is the same for every number of batches in flight, with and without graph replay."""
+    from neutronbench_amd import epoch
+
+    py = epoch.run(config, scale=scale, max_batches=7, warmup_batches=1, quiet=True)
+    runs = [epoch.run_native(config, scale=scale, max_batches=7, warmup_batches=1, pipeline=p, graph=g, quiet=True,
+                             verify=True) for p, g in ((1, True), (1, False), (2, True), (3, True), (5, True))]
+    for r in runs:
+        assert r["batches"] == py["batches"]
+        assert r["sampled_edges"] == py["sampled_edges"] and r["gathered_rows"] == py["gathered_rows"]
+        assert r["checksum"] == runs[0]["checksum"]
+    if py["cache_hit_rate"] is not None:
+        assert abs(runs[0]["cache_hit_rate"] - py["cache_hit_rate"]) < 1e-4
