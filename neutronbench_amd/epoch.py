@@ -327,16 +327,14 @@ def run_native(name, scale=1.0, max_batches=0, warmup_batches=2, pipeline=1, qui
                stage_sync=False, keep_dir=None):
     """The same epoch driven from C++ (neutronbench_amd/host/epoch_driver.cpp -> lib/nts_epoch): the
     arrays of the synthetic configuration are written to a directory, the program runs the batches
-    through the C ABI with no Python between the calls and prints one JSON line.  GCN configurations
-    only.  Same graph, train ids and seeds as `run`, so sampled_edges and gathered_rows are equal."""
+    through the C ABI with no Python between the calls and prints one JSON line.  Same graph, train
+    ids and seeds as `run`, so sampled_edges and gathered_rows are equal."""
     import os
     import shutil
     import subprocess
     import tempfile
 
     cfg = dict(CONFIGS[name])
-    if cfg.get("heads"):
-        raise ValueError("the native driver runs the GCN configurations")
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "nts_epoch")
     if not os.path.exists(exe):
         raise RuntimeError(f"{exe} has not been built (make -C neutronbench_amd/csrc)")
@@ -357,7 +355,8 @@ def run_native(name, scale=1.0, max_batches=0, warmup_batches=2, pipeline=1, qui
         del co, ri
         torch.cuda.empty_cache()
         cmd = [exe, "--dir", d, "--V", str(V), "--F", str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch",
-               str(cfg["batch"]), "--fanout", ",".join(map(str, cfg["fanout"])), "--pipeline", str(pipeline), "--cache",
+               str(cfg["batch"]), "--fanout", ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)),
+               "--pipeline", str(pipeline), "--cache",
                str(cfg["cache"]), "--graph", str(int(graph)), "--warmup", str(warmup_batches), "--max-batches",
                str(max_batches), "--verify", str(int(verify)), "--stage-sync", str(int(stage_sync))]
         p = subprocess.run(cmd, capture_output=True, text=True, timeout=600)

@@ -5,9 +5,13 @@
 // Per batch: nts_batch_builder_sample / _layers (all hops, relabelling, CSR, weights), the feature
 // gather (zero-copy from mapped pinned host memory, or through the HBM cache of the top out-degree
 // vertices), the label gather, and for every layer the aggregation forward (zeroed output,
-// accumulate, as SingleGPUSampleGraphOp does) and, in reverse order, backward.  Inputs of the layers
-// after the first and the incoming gradients stand in for the dense layers' results: constant
-// buffers of the right shape.
+// accumulate, as SingleGPUSampleGraphOp does) and, in reverse order, backward.  With --heads H every
+// layer is a GAT layer instead: fused attention (nts_gat_attention_fwd) and attention-weighted
+// aggregation (nts_spmm_gather_heads) forward; backward the aggregation over the CSR, the per-edge
+// gradient of alpha (nts_sddmm_heads), the fused attention backward and the sum of the edge
+// gradients per source (nts_gather_edge_to_src).  Inputs of the layers after the first, the attention
+// terms and the incoming gradients stand in for the dense layers' results: constant buffers of the
+// right shape, filled once with pseudo-random values.
 //
 // --pipeline 1: everything on one stream.  --pipeline 2: the next batch is sampled on a second stream
 // while this one is gathered and aggregated.  --pipeline P >= 3: P - 2 batches are sampled ahead, each
@@ -92,7 +96,7 @@ void *device_bytes(size_t bytes) {
 struct Args {
   std::string dir;
   std::vector<int32_t> fanout;
-  uint32_t V = 0, F = 0, hidden = 128, batch = 1024, pipeline = 1, warmup = 2, max_batches = 0;
+  uint32_t V = 0, F = 0, hidden = 128, batch = 1024, pipeline = 1, warmup = 2, max_batches = 0, heads = 0;
   double cache = 0.0;
   int graph = 1, verify = 0, stage_sync = 0;
 };
@@ -109,6 +113,7 @@ Args parse(int argc, char **argv) {
     else if (k == "--pipeline") a.pipeline = static_cast<uint32_t>(std::stoul(v));
     else if (k == "--warmup") a.warmup = static_cast<uint32_t>(std::stoul(v));
     else if (k == "--max-batches") a.max_batches = static_cast<uint32_t>(std::stoul(v));
+    else if (k == "--heads") a.heads = static_cast<uint32_t>(std::stoul(v));
     else if (k == "--cache") a.cache = std::stod(v);
     else if (k == "--graph") a.graph = std::stoi(v);
     else if (k == "--verify") a.verify = std::stoi(v);
@@ -126,9 +131,10 @@ Args parse(int argc, char **argv) {
       exit(2);
     }
   }
-  if (a.dir.empty() || !a.V || !a.F || a.fanout.empty() || a.pipeline < 1 || a.pipeline > 8) {
+  if (a.dir.empty() || !a.V || !a.F || a.fanout.empty() || a.pipeline < 1 || a.pipeline > 8 ||
+      (a.heads && a.hidden % a.heads)) {
     fprintf(stderr,
-            "usage: nts_epoch --dir D --V n --F n --fanout a,b[,c] [--batch n] [--hidden n] [--pipeline 1..8]\n"
+            "usage: nts_epoch --dir D --V n --F n --fanout a,b[,c] [--batch n] [--hidden n] [--heads n] [--pipeline 1..8]\n"
             "                 [--cache fraction] [--graph 0|1] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n");
     exit(2);
   }
@@ -191,9 +197,23 @@ int main(int argc, char **argv) {
   uint64_t max_rows = a.batch;
   for (int32_t f : a.fanout) max_rows = f < 0 ? V : std::min<uint64_t>(V, max_rows * static_cast<uint32_t>(f));
   const uint32_t maxw = std::max(F, a.hidden);
+  const uint32_t H = a.heads, Fh = H ? a.hidden / H : 0;
+  // Edge capacity of every hop, as the builder lays it out (hop 0 = the batch's own hop).
+  std::vector<uint64_t> e_cap(hops);
+  {
+    uint64_t vd = a.batch;
+    for (uint32_t h = 0; h < hops; ++h) {
+      uint64_t e = a.fanout[h] < 0 ? E : vd * static_cast<uint32_t>(a.fanout[h]);
+      if (e > E && (h > 0 || a.fanout[h] < 0)) e = E;
+      e_cap[h] = e;
+      vd = std::min<uint64_t>(e, V);
+    }
+  }
+  const uint64_t max_edges = *std::max_element(e_cap.begin(), e_cap.end());
   const uint32_t P = a.pipeline;
   std::vector<Slot> slots(P);
-  const size_t arena_bytes = nts_batch_builder_arena_bytes(V, E, a.fanout.data(), hops, a.batch, 0);
+  const int want_perm = H ? 1 : 0;  // GAT layers walk the CSR through csr_to_csc
+  const size_t arena_bytes = nts_batch_builder_arena_bytes(V, E, a.fanout.data(), hops, a.batch, want_perm);
   if (!arena_bytes) die("nts_batch_builder_arena_bytes");
   const uint32_t x_buffers = P >= 3 ? 2 : 1;  // the gather of the next batch overlaps this one's aggregation
   std::vector<float *> xbuf(x_buffers);
@@ -206,16 +226,37 @@ int main(int argc, char **argv) {
   }
   for (Slot &s : slots) {
     s.arena = device_bytes(arena_bytes);
-    NTS(nts_batch_builder_create(&s.builder, d_co, d_ri, V, E, a.fanout.data(), hops, a.batch, 0, s.arena, arena_bytes));
+    NTS(nts_batch_builder_create(&s.builder, d_co, d_ri, V, E, a.fanout.data(), hops, a.batch, want_perm, s.arena,
+                                 arena_bytes));
     if (a.graph) NTS(nts_batch_builder_use_graph(s.builder, 1));
     HIP(hipEventCreateWithFlags(&s.gathered, hipEventDisableTiming));
     HIP(hipEventCreateWithFlags(&s.trained, hipEventDisableTiming));
   }
   // Stand-ins for what the dense layers would hand over, and the aggregation outputs.
-  std::vector<float> ones(max_rows * maxw, 1.0f);
+  std::vector<float> ones(max_rows * maxw + 64);  // the stand-ins start a few (whole 16-byte) words apart
+  {
+    uint32_t state = 12345u;  // values in [-1, 1)
+    for (float &v : ones) {
+      state = state * 1664525u + 1013904223u;
+      v = static_cast<float>(static_cast<int32_t>(state)) * (1.0f / 2147483648.0f);
+    }
+  }
   float *d_ones = to_device(ones);
   ones.clear();
   ones.shrink_to_fit();
+  // GAT: alpha of every layer is kept until its backward; er is zero as in the Python loop
+  std::vector<float *> d_alpha(hops, nullptr);
+  float *d_er = nullptr, *d_galpha = nullptr, *d_gs = nullptr, *d_ger = nullptr, *d_gel = nullptr;
+  if (H) {
+    for (uint32_t l = 0; l < hops; ++l) d_alpha[l] = static_cast<float *>(device_bytes(e_cap[hops - 1 - l] * H * sizeof(float)));
+    d_er = static_cast<float *>(device_bytes(max_rows * H * sizeof(float)));
+    NTS(nts_memset_zero(d_er, max_rows * H * sizeof(float), nullptr));
+    HIP(hipDeviceSynchronize());
+    d_galpha = static_cast<float *>(device_bytes(max_edges * H * sizeof(float)));
+    d_gs = static_cast<float *>(device_bytes(max_edges * H * sizeof(float)));
+    d_ger = static_cast<float *>(device_bytes(max_rows * H * sizeof(float)));
+    d_gel = static_cast<float *>(device_bytes(max_rows * H * sizeof(float)));
+  }
   float *d_out = static_cast<float *>(device_bytes(max_rows * maxw * sizeof(float)));
   float *d_gin = static_cast<float *>(device_bytes(max_rows * maxw * sizeof(float)));
 
@@ -252,7 +293,49 @@ int main(int argc, char **argv) {
     NTS(nts_gather_labels_i64(s.labels, d_labels, top.destination, top.v_size, 1, stream));
   };
   uint64_t hits_total = 0;
+  auto hash = [&](const float *p, uint64_t n, uint64_t salt, hipStream_t stream) {
+    uint64_t fp = 0;
+    NTS(nts_fingerprint_u32(&fp, reinterpret_cast<const uint32_t *>(p), n, nullptr, 0, stream));
+    checksum ^= fp * (2 * salt + 1);
+  };
+  auto aggregate_gat = [&](Slot &s, hipStream_t stream) {
+    const float slope = 0.2f;
+    double t0 = now();
+    for (uint32_t l = 0; l < hops; ++l) {
+      const nts_sampled_layer_t &L = s.layers[l];
+      const float *x = d_ones;  // [src_size, H * Fh]: stands in for the projected features of the layer
+      const float *el = d_ones + 8;  // [src_size, H]
+      NTS(nts_gat_attention_fwd(d_alpha[l], el, d_er, L.column_offset, L.row_indices, L.v_size, H, slope, stream));
+      NTS(nts_spmm_gather_heads(x, d_out, d_alpha[l], nullptr, L.column_offset, L.row_indices, L.v_size, L.e_size, H, Fh, 0,
+                                stream));
+      if (a.verify) {
+        hash(d_alpha[l], static_cast<uint64_t>(L.e_size) * H, 10 + l, stream);
+        hash(d_out, static_cast<uint64_t>(L.v_size) * H * Fh, 20 + l, stream);
+      }
+      if (a.stage_sync) HIP(hipStreamSynchronize(stream));
+    }
+    if (a.stage_sync) t_fwd += now() - t0;
+    t0 = now();
+    for (uint32_t k = hops; k-- > 0;) {
+      const nts_sampled_layer_t &L = s.layers[k];
+      const float *x = d_ones, *el = d_ones + 8, *g_out = d_ones + 4;  // g_out: [v_size, H * Fh]
+      NTS(nts_spmm_gather_heads(g_out, d_gin, d_alpha[k], L.csr_to_csc, L.row_offset, L.column_indices, L.src_size,
+                                L.e_size, H, Fh, 0, stream));
+      NTS(nts_sddmm_heads(d_galpha, x, g_out, L.column_offset, L.row_indices, L.v_size, H, Fh, stream));
+      NTS(nts_gat_attention_bwd(d_gs, d_ger, d_galpha, d_alpha[k], el, d_er, L.column_offset, L.row_indices, L.v_size, H,
+                                slope, stream));
+      NTS(nts_gather_edge_to_src(d_gel, d_gs, L.row_offset, L.csr_to_csc, L.src_size, H, 0, stream));
+      if (a.verify) {
+        hash(d_gin, static_cast<uint64_t>(L.src_size) * H * Fh, 30 + k, stream);
+        hash(d_ger, static_cast<uint64_t>(L.v_size) * H, 40 + k, stream);
+        hash(d_gel, static_cast<uint64_t>(L.src_size) * H, 50 + k, stream);
+      }
+      if (a.stage_sync) HIP(hipStreamSynchronize(stream));
+    }
+    if (a.stage_sync) t_bwd += now() - t0;
+  };
   auto aggregate = [&](Slot &s, hipStream_t stream) {
+    if (H) return aggregate_gat(s, stream);
     double t0 = now();
     for (uint32_t l = 0; l < hops; ++l) {
       const nts_sampled_layer_t &L = s.layers[l];

@@ -73,7 +73,7 @@ def test_stream_wrapper_can_leave_batch_assembly_unsynchronised():
     assert CudaStream(side.cuda_stream).synchronize is True
 
 
-@pytest.mark.parametrize("config,scale", [("arxiv", 0.25), ("products", 0.02)])
+@pytest.mark.parametrize("config,scale", [("arxiv", 0.25), ("products", 0.02), ("gat", 0.02)])
 def test_native_epoch_driver(config, scale):
     """The epoch driven from C++ (lib/nts_epoch, neutronbench_amd/host/epoch_driver.cpp): same graph,
     train ids and seeds as the Python loop, so it samples the same edges, gathers the same rows and
