@@ -1,4 +1,4 @@
-"""The reference's own toolkit program, unchanged, over this library (SURVEY section 8 f3).
+"""The reference's own toolkit program, unchanged, over this library.
 
 oracle/build_toolkits.sh compiles toolkits/main.cpp, core/GraphSegment.cpp and comm/network.cpp from the
 reference tree with CUDA_ENABLE against neutronbench_amd/host/compat (the veneer in place of cuda/) and
