@@ -84,9 +84,93 @@ def measured_traffic(workload):
             return None
         return {"traffic": int(fields["traffic_bytes_per_launch"]), "fetch": int(fields["fetch_bytes_per_launch"]),
                 "write": int(fields["write_bytes_per_launch"]), "kernel": fields.get("kernel"),
-                "l2_hit_rate": float(fields["l2_hit_rate"]) if "l2_hit_rate" in fields else None}
+                "l2_hit_rate": float(fields["l2_hit_rate"]) if "l2_hit_rate" in fields else None,
+                "l2_request_bytes": int(fields["l2_request_bytes_per_launch"]) if "l2_request_bytes_per_launch" in fields else None}
     except (OSError, KeyError, ValueError):
         return None
+
+
+def reddit_graph(torch, V, E, distinct, chunk, slabs, dev):
+    """The Reddit-shaped chunk: R-MAT a=.57 b=.19 c=.19, seed 3, ids permuted, edge list in (src, dst)
+    order.  distinct=True: the first E distinct pairs of the draw sequence (a simple graph, as the Reddit
+    graph itself is); False: the first E draws, parallel edges kept."""
+    from neutronbench_amd import synth
+    from neutronbench_amd.layout import FullGraphChunk
+
+    src, dst = synth.rmat_edges(V, E, 0.57, 0.19, 0.19, seed=3, device=dev, sort=True, distinct=distinct)
+    chunk_obj = FullGraphChunk.from_edges(src, dst, V, chunk, slabs)
+    del src, dst
+    return chunk_obj
+
+
+def time_steps(torch, chunk, tensors, steps, warmup):
+    """`warmup` untimed and `steps` timed steps (fwd F=602, fwd F=128, bwd F=128, bwd F=602) of the
+    operator mirror over `chunk`.  Returns (seconds for the timed steps, per-pass gather-kernel ms from
+    HIP events recorded by the library around its main kernel, the last step's four outputs)."""
+    from neutronbench_amd.abi import call
+    from neutronbench_amd.ops import ForwardSingleGPUfuseOp
+
+    x0, h1, g1, g0 = tensors
+    op = ForwardSingleGPUfuseOp(chunk, with_weight=True)
+    chunk.plan_forward.reserve(F_IN)
+    chunk.plan_backward.reserve(F_IN)
+    for _ in range(warmup):
+        op.forward(x0), op.forward(h1), op.backward(g1), op.backward(g0)
+    torch.cuda.synchronize()
+    # One HIP event pair per aggregation launch of the timed region (4 per step).  The library records
+    # them on the launch stream immediately before and after its main gather kernel; nothing waits on
+    # them until the timed region is over.
+    events = []
+    for _ in range(4 * steps):
+        a, b = ctypes.c_void_p(), ctypes.c_void_p()
+        call("nts_event_create", ctypes.byref(a))
+        call("nts_event_create", ctypes.byref(b))
+        events.append((a, b))
+    fwd, bwd = chunk.plan_forward.handle, chunk.plan_backward.handle
+    outs = [None] * 4
+
+    def timed_step(i):
+        call("nts_spmm_plan_set_events", fwd, *events[4 * i + 0])
+        outs[0] = op.forward(x0)    # layer 0: aggregate the 602-wide input features
+        call("nts_spmm_plan_set_events", fwd, *events[4 * i + 1])
+        outs[1] = op.forward(h1)    # layer 1: aggregate the 128-wide hidden features
+        call("nts_spmm_plan_set_events", bwd, *events[4 * i + 2])
+        outs[2] = op.backward(g1)   # layer 1 backward: gradient gather over the CSR
+        call("nts_spmm_plan_set_events", bwd, *events[4 * i + 3])
+        outs[3] = op.backward(g0)   # layer 0 backward
+
+    # Timed region: exactly `steps` steps between two synchronisations.
+    torch.cuda.synchronize()
+    t_start = time.perf_counter()
+    for i in range(steps):
+        timed_step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t_start
+    call("nts_spmm_plan_set_events", fwd, None, None)
+    call("nts_spmm_plan_set_events", bwd, None, None)
+    durs = []
+    for a, b in events:
+        ms = ctypes.c_float()
+        call("nts_event_elapsed_ms", ctypes.byref(ms), a, b)
+        durs.append(ms.value)
+        call("nts_event_destroy", a)
+        call("nts_event_destroy", b)
+    per_pass = [sum(durs[k::4]) / steps for k in range(4)]  # fwd602, fwd128, bwd128, bwd602
+    # Whole passes (padded copy where there is one, gather, second stage of the cut rows), each timed
+    # alone with events on the launch stream, outside the timed region.
+    whole = []
+    for run, x in ((op.forward, x0), (op.forward, h1), (op.backward, g1), (op.backward, g0)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            run(x)
+        e1.record()
+        torch.cuda.synchronize()
+        whole.append(e0.elapsed_time(e1) / 5)
+    return elapsed, per_pass, whole, list(outs)
+
+
+PASS_NAMES = ("fwd_F602", "fwd_F128", "bwd_F128", "bwd_F602")
 
 
 def main():
@@ -99,9 +183,15 @@ def main():
     ap.add_argument("--chunk", type=int, default=512, help="largest number of edges in one piece of a split hub row")
     ap.add_argument("--slabs", type=int, default=32,
                     help="source ranges of the cache-aware schedule (1 = split hub rows by edge count only)")
+    ap.add_argument("--graph", choices=["simple", "multigraph"], default="simple",
+                    help="simple (default): the first E distinct R-MAT pairs, a simple graph like the Reddit graph; "
+                         "multigraph: the first E draws with parallel edges kept (timed beside the headline anyway)")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip everything that runs on the host after the timed region: the check of the timed "
                          "outputs against the CPU oracle, the CPU baselines and the reference operator's time")
+    ap.add_argument("--no-epochs", action="store_true",
+                    help="skip the three sampled mini-batch epochs (BASELINE.json configs 2, 4, 5) of the default run")
+    ap.add_argument("--no-other-graph", action="store_true", help="skip the steps on the other kind of graph")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB row copy (identity gather) so that HBM byte counters can be scaled")
     ap.add_argument("--cpu-reps", type=int, default=5, help="timed repetitions of each CPU baseline (median reported)")
@@ -109,8 +199,8 @@ def main():
                     help="edges of the graph the reference's own operators are timed on (0 = the whole graph; a "
                          "smaller number takes the edges of the lowest-numbered source vertices)")
     ap.add_argument("--workload", choices=["reddit", "arxiv", "products", "gat"], default="reddit",
-                    help="reddit (default): the aggregation workload above; arxiv / products / gat: per-epoch time of "
-                         "that sampled mini-batch configuration (BASELINE.json configs 2, 4, 5) instead")
+                    help="reddit (default): the aggregation workload above, with the three epochs beside it; arxiv / "
+                         "products / gat: only the per-epoch time of that sampled mini-batch configuration")
     ap.add_argument("--cpu-batches", type=int, default=3, help="mini-batch workloads: batches the CPU oracle is timed on")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -122,35 +212,25 @@ def main():
 
     from neutronbench_amd import synth
     from neutronbench_amd.abi import call, ptr
-    from neutronbench_amd.layout import FullGraphChunk
-    from neutronbench_amd.ops import ForwardSingleGPUfuseOp
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (the HIP library has no CPU fallback)")
     dev = torch.device("cuda:0")
     V, E = args.vertices, args.edges
+    simple = args.graph == "simple"
 
     t0 = time.time()
-    src, dst = synth.rmat_edges(V, E, 0.57, 0.19, 0.19, seed=3, device=dev, sort=True)
-    chunk = FullGraphChunk.from_edges(src, dst, V, args.chunk, args.slabs)
-    del src, dst
+    chunk = reddit_graph(torch, V, E, simple, args.chunk, args.slabs, dev)
     x0 = synth.normal_features(V, F_IN, seed=31, device=dev)
     h1 = synth.normal_features(V, F_HID, seed=32, device=dev)
     g1 = synth.normal_features(V, F_HID, seed=33, device=dev)
     g0 = synth.normal_features(V, F_IN, seed=34, device=dev)
+    tensors = (x0, h1, g1, g0)
     torch.cuda.synchronize()
     setup_s = time.time() - t0
-    op = ForwardSingleGPUfuseOp(chunk, with_weight=True)
     chunk.plan_forward.reserve(F_IN)
     chunk.plan_backward.reserve(F_IN)
     scratch = [p.scratch_info(F_IN) for p in (chunk.plan_forward, chunk.plan_backward)]
-
-    def step():
-        y0 = op.forward(x0)    # layer 0: aggregate the 602-wide input features
-        y1 = op.forward(h1)    # layer 1: aggregate the 128-wide hidden features
-        d1 = op.backward(g1)   # layer 1 backward: gradient gather over the CSR
-        d0 = op.backward(g0)   # layer 0 backward
-        return y0, y1, d1, d0
 
     if args.calibrate:
         # Plain copy of known size: 2^18 rows of 1024 floats = 1 GiB read + 1 GiB written (+ 1 MiB of ids).
@@ -163,95 +243,62 @@ def main():
         torch.cuda.synchronize()
         del cal_src, cal_dst, cal_ids
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-
-    # One HIP event pair per aggregation launch of the timed region (4 per step).  The library records
-    # them on the launch stream immediately before and after its main gather kernel; nothing waits on
-    # them until the timed region is over.
-    n_ev = 4 * args.steps
-    events = []
-    for _ in range(n_ev):
-        a, b = ctypes.c_void_p(), ctypes.c_void_p()
-        call("nts_event_create", ctypes.byref(a))
-        call("nts_event_create", ctypes.byref(b))
-        events.append((a, b))
-    fwd, bwd = chunk.plan_forward.handle, chunk.plan_backward.handle
-    outs = [None] * 4
-
-    def timed_step(i):
-        call("nts_spmm_plan_set_events", fwd, *events[4 * i + 0])
-        outs[0] = op.forward(x0)
-        call("nts_spmm_plan_set_events", fwd, *events[4 * i + 1])
-        outs[1] = op.forward(h1)
-        call("nts_spmm_plan_set_events", bwd, *events[4 * i + 2])
-        outs[2] = op.backward(g1)
-        call("nts_spmm_plan_set_events", bwd, *events[4 * i + 3])
-        outs[3] = op.backward(g0)
-
-    # Timed region: exactly `steps` steps between two synchronisations.
-    torch.cuda.synchronize()
-    t_start = time.perf_counter()
-    for i in range(args.steps):
-        timed_step(i)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t_start
+    elapsed, per_pass, whole, outs = time_steps(torch, chunk, tensors, args.steps, args.warmup)
     ms_per_step = elapsed * 1e3 / args.steps
     edges_per_s = 4.0 * E / (elapsed / args.steps)
-    call("nts_spmm_plan_set_events", fwd, None, None)
-    call("nts_spmm_plan_set_events", bwd, None, None)
 
-    durs = []
-    for a, b in events:
-        ms = ctypes.c_float()
-        call("nts_event_elapsed_ms", ctypes.byref(ms), a, b)
-        durs.append(ms.value)
-        call("nts_event_destroy", a)
-        call("nts_event_destroy", b)
-    per_pass = [sum(durs[k::4]) / args.steps for k in range(4)]  # fwd602, fwd128, bwd128, bwd602
     # Dominant kernel: the F=602 gather (spmm_wave_kernel), launched twice per step: forward over the
     # CSC and backward over the CSR.  Same algorithmic bytes per launch for both.
     kernel_ms = (per_pass[0] + per_pass[3]) / 2
     algo = algorithmic_bytes(E, V, F_IN)
+    compulsory = compulsory_bytes(E, V, V, F_IN)
     model_gbs = algo / (kernel_ms * 1e-3) / 1e9
-    workload_key = f"V={V} E={E} chunk={args.chunk} slabs={args.slabs} F={F_IN}"
+    workload_key = f"V={V} E={E} graph={args.graph} chunk={args.chunk} slabs={args.slabs} F={F_IN}"
     measured = measured_traffic(workload_key)
     padded = scratch[0]["padded_input_bytes"] > 0
+    fabric_gbs = measured["traffic"] / (kernel_ms * 1e-3) / 1e9 if measured else None
     roofline = {
-        # `achieved` and `frac` are the bytes rocprofv3 counts between the L2 and the fabric (Infinity
-        # Cache / HBM) per launch over this run's kernel time: the figure the 60 %-of-peak target is
-        # judged on.  null when no counter summary matches the kernel sources of this run.
-        "bound": "hbm",
+        # What bounds the kernel: the path behind the L2 -- Infinity Cache and HBM together.  No counter of
+        # this GPU tells an Infinity Cache hit from an HBM read, so `traffic` (FETCH_SIZE + WRITE_SIZE of
+        # rocprofv3, counted where the L2 talks to the fabric) is an upper bound of the HBM bytes, and
+        # `achieved` / `frac` are that traffic over this run's kernel time against the HBM peak.
+        "bound": "l2+fabric",
         "kernel": (measured or {}).get("kernel") or
         ("spmm_wave_kernel<4,3,...> over a padded input copy" if padded else "spmm_wave_kernel<1,10,...>")
         + " (F=602 gather, forward and backward launches)",
-        "achieved": round(measured["traffic"] / (kernel_ms * 1e-3) / 1e9, 1) if measured else None,
+        "achieved": round(fabric_gbs, 1) if measured else None,
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
-        "frac": round(measured["traffic"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if measured else None,
+        "frac": round(fabric_gbs / HBM_PEAK_GBS, 4) if measured else None,
         "traffic": measured["traffic"] if measured else None,
+        "traffic_source": ("profiles/spmm_wave_f602_reddit_shaped_pmc.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per "
+                           "launch of this kernel on this workload, each scaled by the same counter's reading for a "
+                           "plain copy; quoted only while the sha256 of the kernel sources recorded there matches the "
+                           "sources of this run") if measured else "no counter summary matches this run's kernel sources",
+        "l2_request_bytes": (measured or {}).get("l2_request_bytes"),
+        "l2_hit_rate": (measured or {}).get("l2_hit_rate"),
         "target_frac": 0.6,
-        "target_met": bool(measured and measured["traffic"] / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS >= 0.6),
-        "limited_by": "L2 misses through the fabric: this library's plain streaming kernels move 4.9-6.1 TB/s by the "
-                      "same counters, and the gather fetches many times its compulsory bytes because one source "
-                      f"range does not fit a 4 MB L2 (L2 hit rate {(measured or {}).get('l2_hit_rate')})",
+        "target_met": bool(measured and fabric_gbs / HBM_PEAK_GBS >= 0.6),
+        "target_basis": "L2-miss traffic (Infinity Cache hits included: an upper bound of the HBM bytes) over the HBM peak",
+        # every array once, over the same kernel time: the share of the HBM peak spent on bytes that must move
+        "compulsory_bytes": compulsory,
+        "compulsory_frac": round(compulsory / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         # the edge-gather model (one source row per edge) counts every re-read served by L2 as a byte
         # moved; it exceeds the HBM peak and is reported for comparison only
+        "algorithmic_bytes": algo,
         "model_gbs": round(model_gbs, 1),
         "model_frac": round(model_gbs / HBM_PEAK_GBS, 4),
-        "algorithmic_bytes": algo,
-        "compulsory_bytes": compulsory_bytes(E, V, V, F_IN),
         "kernel_ms": round(kernel_ms, 3),
-        "per_pass_ms": {"fwd_F602": round(per_pass[0], 3), "fwd_F128": round(per_pass[1], 3),
-                        "bwd_F128": round(per_pass[2], 3), "bwd_F602": round(per_pass[3], 3)},
+        "per_pass_ms": {n: round(v, 3) for n, v in zip(PASS_NAMES, per_pass)},
+        # the whole call: padded copy where there is one + gather + second stage of the cut rows
+        "pass_ms": {n: round(v, 3) for n, v in zip(PASS_NAMES, whole)},
     }
 
     check = cpu_baseline = None
     reference_operator = None
     if not args.no_cpu_baseline:
-        inputs = dict(fwd_F602=x0, fwd_F128=h1, bwd_F128=g1, bwd_F602=g0)
-        check = check_against_oracle(torch, chunk, inputs, dict(zip(inputs, outs)), V)
+        inputs = dict(zip(PASS_NAMES, tensors))
+        check = check_against_oracle(torch, chunk, inputs, dict(zip(PASS_NAMES, outs)), V)
         if not check["ok"]:
             print(json.dumps({"error": "timed outputs differ from the CPU oracle", "check": check}))
             sys.exit(1)
@@ -263,6 +310,43 @@ def main():
             cpu_baseline["other_thread_setting"] = port.pop("reference_default_threads")
         else:
             cpu_baseline["port"] = port
+    plan_info = dict(chunk.plan_forward.info(), chunk_edges=args.chunk, slabs=args.slabs)
+    plan_build_s = chunk.plan_build_s
+    del chunk, outs
+    torch.cuda.empty_cache()
+
+    # The same step on the other kind of graph, outside the headline: the same R-MAT draws with parallel
+    # edges kept (a multigraph: the kernel then loads a source row once per run of equal neighbours).
+    other = None
+    if not args.no_other_graph:
+        chunk2 = reddit_graph(torch, V, E, not simple, args.chunk, args.slabs, dev)
+        el2, pp2, whole2, _ = time_steps(torch, chunk2, tensors, max(3, args.steps // 2), 2)
+        n2 = max(3, args.steps // 2)
+        sc2 = chunk2.plan_forward.scratch_info(F_IN)
+        other = {
+            "graph": ("the first E R-MAT draws, parallel edges kept" if simple else "the first E distinct R-MAT pairs"),
+            "ms_per_step": round(el2 * 1e3 / n2, 3),
+            "edges_per_s": round(4.0 * E / (el2 / n2), 1),
+            "per_pass_ms": {n: round(v, 3) for n, v in zip(PASS_NAMES, pp2)},
+            "pass_ms": {n: round(v, 3) for n, v in zip(PASS_NAMES, whole2)},
+            "repeated_edges": sc2["repeated_edges"],
+            "loads_once_per_run": sc2["loads_once_per_run"],
+            "note": "edges that repeat the neighbour of the edge before them in their row are parallel edges; with "
+                    "at least 1 in 20 such edges the kernel loads a row once per run and adds it once per edge, "
+                    "which is where a multigraph's higher rate comes from -- it does not apply to a simple graph",
+        }
+        del chunk2
+        torch.cuda.empty_cache()
+    del x0, h1, g1, g0, tensors
+    torch.cuda.empty_cache()
+
+    epochs = None
+    if not args.no_epochs:
+        epochs = run_epochs(torch, ("arxiv", "products", "gat"), not args.no_cpu_baseline, args.cpu_batches)
+        bad = [n for n, e in epochs.items() if e.get("check") and not e["check"]["ok"]]
+        if bad:
+            print(json.dumps({"error": f"epoch batch of {bad} differs from the CPU oracle", "epochs": epochs}))
+            sys.exit(1)
 
     out = {
         "metric": "edges aggregated/s (fwd+bwd)",
@@ -281,15 +365,15 @@ def main():
             "workload": "Reddit-shaped full-graph 2-layer GCN aggregation fwd+bwd (F=602,128)",
             "vertices": V,
             "edges": E,
-            "graph": "R-MAT a=.57 b=.19 c=.19, seed 3, ids permuted, edge list in (src, dst) order, duplicates kept",
+            "graph": "R-MAT a=.57 b=.19 c=.19, seed 3, ids permuted, edge list in (src, dst) order; "
+                     + ("the first E distinct pairs of the draw sequence: a simple graph, as the Reddit graph is"
+                        if simple else "the first E draws, parallel edges kept"),
             "parallel_edges": {"forward": scratch[0]["repeated_edges"], "backward": scratch[1]["repeated_edges"],
-                               "note": "edges that repeat the source (forward) / destination (backward) of the edge "
-                                       "before them in their row; the kernel loads such a row once per run and adds "
-                                       "it once per edge (NTS_SPMM_RUNS=0 NTS_SPMM_PAD=0 times the kernel without that)",
                                "loads_once_per_run": scratch[0]["loads_once_per_run"]},
+            "other_graph": other,
             "passes_per_step": 4,
-            "plan": dict(chunk.plan_forward.info(), chunk_edges=args.chunk, slabs=args.slabs),
-            "plan_build_s": round(chunk.plan_build_s, 3),
+            "plan": plan_info,
+            "plan_build_s": round(plan_build_s, 3),
             "plan_scratch_bytes": {"forward": scratch[0]["partial_bytes"] + scratch[0]["padded_input_bytes"],
                                    "backward": scratch[1]["partial_bytes"] + scratch[1]["padded_input_bytes"],
                                    "of_which_padded_input_copy": scratch[0]["padded_input_bytes"]},
@@ -300,6 +384,7 @@ def main():
         "roofline": roofline,
         "check": check,
         "cpu_baseline": cpu_baseline,
+        "epochs": epochs,
     }
     print(json.dumps(out))
 
@@ -484,64 +569,109 @@ def run_cpu_port_baseline(torch, chunk, x0, h1, g1, g0, V, reps):
     return out
 
 
-def run_epoch_workload(args):
-    """Per-epoch time of a sampled mini-batch configuration through the library (every stage through
-    the C ABI, see neutronbench_amd/epoch.py), next to the CPU oracle on a few batches of the same
-    epoch.  One JSON line; `value` is the epoch time with the stages run one after the other, as the
-    reference's default mode does, and config.pipelined_epoch_s the time with four batches in flight
-    (two being sampled, one gathered, one aggregated, each stage on streams of its own)."""
-    import torch
+def run_epochs(torch, names, with_cpu, cpu_batches):
+    """One epoch of each sampled mini-batch configuration, driven from C++ through the C ABI
+    (neutronbench_amd/host/epoch_driver.cpp -> lib/nts_epoch; sampling, layer construction,
+    feature/label gather, aggregation forward + backward of every layer; dense layers are not part of
+    this library).  Per configuration: the serial epoch -- one stream, a wait after every stage, the
+    figure and the stage columns of the reference's log line (toolkits/GCN_GPU_NEIGHBOR.hpp:1498-1506) --
+    the same epoch with four batches in flight, a check of every array of one batch of the epoch
+    against the CPU oracle (oracle/epoch_check.py), and the CPU oracle timed on a few batches."""
+    import shutil
+    import tempfile
 
     from neutronbench_amd import epoch
+    from oracle import epoch_check
+
+    records = {}
+    written = {}  # inputs on disk, shared by the configurations on the same graph (products, gat)
+    try:
+        for name in names:
+            cfg = epoch.CONFIGS[name]
+            key = tuple(cfg[k] for k in ("V", "E", "F", "seed", "classes", "train"))
+            if key not in written:
+                for d, _ in written.values():
+                    shutil.rmtree(d, ignore_errors=True)
+                written.clear()
+                d = tempfile.mkdtemp(prefix="nts_epoch_")
+                written[key] = (d, epoch.write_native_inputs(name, d, keep_host=True))
+            d, host = written[key]
+            dump = tempfile.mkdtemp(prefix="nts_dump_")
+            try:
+                serial = epoch.run_native_on(d, name, host["V"], pipeline=1, stage_sync=True, dump_dir=dump,
+                                             dump_batch=1)
+                piped = epoch.run_native_on(d, name, host["V"], pipeline=4, stage_sync=False)
+                check = epoch_check.check_dump(dump, host["co"], host["ri"], host["feat"], host["labels"], cfg["fanout"],
+                                               cfg["cache"]) if with_cpu else None
+            finally:
+                shutil.rmtree(dump, ignore_errors=True)
+            cpu = epoch_cpu_baseline(torch, name, host, serial["batches"], cpu_batches) if with_cpu else None
+            records[name] = {
+                "epoch_s": serial["epoch_s"], "stage_s": serial.get("stage_s"), "batches": serial["batches"],
+                "batch_size": cfg["batch"], "fanout_output_side_first": cfg["fanout"], "heads": cfg.get("heads", 0),
+                "vertices": host["V"], "edges": host["E"], "sampled_edges": serial["sampled_edges"],
+                "gathered_rows": serial["gathered_rows"], "cache_hit_rate": serial.get("cache_hit_rate"),
+                "ms_per_batch": round(1e3 * serial["epoch_s"] / max(serial["batches"], 1), 4),
+                "pipelined_epoch_s": piped["epoch_s"], "pipeline_depth": piped["pipeline"],
+                "driver": "lib/nts_epoch (C++ over the C ABI), one stream, a wait after every stage; 2 untimed batches first",
+                "check": check, "cpu_baseline": cpu,
+            }
+    finally:
+        for d, _ in written.values():
+            shutil.rmtree(d, ignore_errors=True)
+    return records
+
+
+def run_epoch_workload(args):
+    """Per-epoch time of one sampled mini-batch configuration (see run_epochs) as a JSON line of its own:
+    `value` is the serial epoch time, config.pipelined_epoch_s the time with four batches in flight."""
+    import torch
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (the HIP library has no CPU fallback)")
-    serial = epoch.run(args.workload, pipeline=1, quiet=True)
-    piped = epoch.run(args.workload, pipeline=4, quiet=True)
-    cpu = None
-    if not args.no_cpu_baseline and args.workload != "gat":
-        cpu = epoch_cpu_baseline(torch, args.workload, serial["batches"], args.cpu_batches)
-    cfg = epoch.CONFIGS[args.workload]
+    rec = run_epochs(torch, (args.workload,), not args.no_cpu_baseline, args.cpu_batches)[args.workload]
+    if rec["check"] is not None and not rec["check"]["ok"]:
+        print(json.dumps({"error": "a batch of the epoch differs from the CPU oracle", "check": rec["check"]}))
+        sys.exit(1)
     line = {
-        "metric": "epoch time", "value": serial["epoch_s"], "unit": "s", "n_gpus": 1, "steps": serial["batches"],
-        "warmup": serial["warmup_batches"], "ms_per_step": round(1e3 * serial["epoch_s"] / serial["batches"], 4),
+        "metric": "epoch time", "value": rec["epoch_s"], "unit": "s", "n_gpus": 1, "steps": rec["batches"],
+        "warmup": 2, "ms_per_step": rec["ms_per_batch"],
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}-shaped sampled mini-batch epoch, fanout (output side first) "
-                               f"{cfg['fanout']}, batch {cfg['batch']}, {serial['batches']} batches; a step = one batch: "
-                               "sampling, layer construction, feature/label gather, aggregation fwd+bwd of every layer",
-                   "vertices": serial["vertices"], "edges": serial["edges"], "stage_s": serial["stage_s"],
-                   "sampled_edges": serial["sampled_edges"], "gathered_rows": serial["gathered_rows"],
-                   "cache_hit_rate": serial["cache_hit_rate"], "pipelined_epoch_s": piped["epoch_s"],
-                   "pipeline_depth": piped["pipeline"]},
+                               f"{rec['fanout_output_side_first']}, batch {rec['batch_size']}, {rec['batches']} batches; "
+                               "a step = one batch: sampling, layer construction, feature/label gather, aggregation "
+                               "fwd+bwd of every layer",
+                   **{k: rec[k] for k in ("vertices", "edges", "stage_s", "sampled_edges", "gathered_rows",
+                                          "cache_hit_rate", "pipelined_epoch_s", "pipeline_depth", "driver")}},
         "roofline": None,
-        "cpu_baseline": cpu,
+        "check": rec["check"],
+        "cpu_baseline": rec["cpu_baseline"],
     }
     print(json.dumps(line))
 
 
-def epoch_cpu_baseline(torch, name, n_batches, k_batches):
+def epoch_cpu_baseline(torch, name, host, n_batches, k_batches):
     """The CPU oracle (restatement of the reference's host steps: sampCSC::postprocessing,
     generate_csr_from_csc, update_degree + compute_weight_*, get_feature, MiniBatchFuseOp forward and
-    backward) on the first k batches of the epoch, extrapolated to the epoch.  The neighbour pick
-    itself is an input here (the lists the library sampled are used), so the reference's CPU
-    sampling time is not part of the figure."""
+    backward; for the GAT configuration the chain of the reference's CPU edge operators,
+    toolkits/GAT_CPU.hpp:178-204) on the first k batches of the epoch, extrapolated to the epoch.  The
+    neighbour pick itself is an input here (the lists the library sampled are used), so the reference's
+    CPU sampling time is not part of the figure."""
     import numpy as np
 
     import oracle
-    from neutronbench_amd import epoch, synth
+    from neutronbench_amd import epoch
     from neutronbench_amd.batch import BatchBuilder
-    from neutronbench_amd.layout import as_u32
 
     cfg = epoch.CONFIGS[name]
     dev = torch.device("cuda:0")
-    V, E = cfg["V"], cfg["E"]
-    src, dst = synth.rmat_edges(V, E, seed=cfg["seed"], device=dev, sort=True)
-    co, ri = synth.build_csc(src, dst, V)
-    del src, dst
-    gco, gri = as_u32(co), as_u32(ri)
-    feat = synth.normal_features(V, cfg["F"], seed=cfg["seed"] + 40).numpy()
-    train32 = as_u32(synth.permutation(V, cfg["seed"] + 42, dev)[:cfg["train"]])
-    builder = BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"])
+    V = host["V"]
+    gco = torch.from_numpy(host["co"].view(np.int32)).to(dev)
+    gri = torch.from_numpy(host["ri"].view(np.int32)).to(dev)
+    feat = host["feat"]
+    train32 = torch.from_numpy(host["train"].view(np.int32)).to(dev)
+    heads = cfg.get("heads", 0)
+    builder = BatchBuilder(gco, gri, cfg["fanout"], cfg["batch"], want_perm=heads > 0)
     threads = oracle.max_threads()
     rng = np.random.default_rng(1)
     t = {"structure": 0.0, "gather": 0.0, "aggregate": 0.0}
@@ -553,12 +683,12 @@ def epoch_cpu_baseline(torch, name, n_batches, k_batches):
         if turn == 1:
             t = dict.fromkeys(t, 0.0)
         layers = builder.sample(train32[b * cfg["batch"]:(b + 1) * cfg["batch"]], 1000 * b)
-        host = [dict(dst=u32(l.dev_destination), co=u32(l.dev_column_offset), src=u32(l.dev_source),
-                     glob=u32(l.dev_source)[u32(l.dev_row_indices)]) for l in layers]
+        hostl = [dict(dst=u32(l.dev_destination), co=u32(l.dev_column_offset), src=u32(l.dev_source),
+                      glob=u32(l.dev_source)[u32(l.dev_row_indices)]) for l in layers]
         outd, ind = np.ones(V, np.uint32), np.ones(V, np.uint32)
         built = []
         t0 = time.perf_counter()
-        for h in host[::-1]:  # hop order: the batch's own hop first
+        for h in hostl[::-1]:  # hop order: the batch's own hop first
             local, source, n = oracle.postprocess(h["glob"], V)
             ro, ci = oracle.csr_from_csc(h["co"], local, n)
             ewf, ewb = oracle.layer_weights(h["co"], local, ro, ci, source, h["dst"], outd, ind)
@@ -566,10 +696,30 @@ def epoch_cpu_baseline(torch, name, n_batches, k_batches):
         t["structure"] += time.perf_counter() - t0
         built = built[::-1]  # input side first
         t0 = time.perf_counter()
-        x = oracle.get_feature(feat, host[0]["src"])
+        x = oracle.get_feature(feat, hostl[0]["src"])
         t["gather"] += time.perf_counter() - t0
         widths = [cfg["F"]] + [cfg["hidden"]] * (len(built) - 1)
         for (lco, local, ro, ci, ewf, ewb, Vd, Vs), F in zip(built, widths):
+            if heads:
+                H, Fh = heads, cfg["hidden"] // heads
+                E = local.size
+                xin = rng.standard_normal((Vs, H * Fh)).astype(np.float32)
+                el = rng.standard_normal((Vs, H)).astype(np.float32)
+                er = np.zeros((Vd, H), np.float32)
+                g = rng.standard_normal((Vd, H * Fh)).astype(np.float32)
+                t0 = time.perf_counter()
+                pre = oracle.scatter_src(el, lco, local) + oracle.scatter_dst(er, lco, E)
+                alpha = oracle.edge_softmax(np.where(pre > 0, pre, np.float32(0.2) * pre), lco)
+                msg = oracle.scatter_src(xin, lco, local)
+                x = oracle.aggregate_dst((msg.reshape(E, H, Fh) * alpha[:, :, None]).reshape(E, H * Fh), lco)
+                gmsg = oracle.scatter_dst(g, lco, E)
+                oracle.gather_to_src((gmsg.reshape(E, H, Fh) * alpha[:, :, None]).reshape(E, H * Fh), lco, local, Vs)
+                galpha = (msg.reshape(E, H, Fh) * gmsg.reshape(E, H, Fh)).sum(2)
+                gs = oracle.edge_softmax_bwd(galpha, alpha, lco) * np.where(pre > 0, np.float32(1), np.float32(0.2))
+                oracle.aggregate_dst(gs, lco)
+                oracle.gather_to_src(gs, lco, local, Vs)
+                t["aggregate"] += time.perf_counter() - t0
+                continue
             xin = x if x.shape == (Vs, F) else rng.standard_normal((Vs, F)).astype(np.float32)
             g = rng.standard_normal((Vd, F)).astype(np.float32)
             t0 = time.perf_counter()
@@ -577,6 +727,7 @@ def epoch_cpu_baseline(torch, name, n_batches, k_batches):
             oracle.spmm(g, ewb, ro, ci, Vs, threads=threads)
             t["aggregate"] += time.perf_counter() - t0
     builder.close()
+    del gco, gri
     per_batch = sum(t.values()) / k_batches
     return {
         "value": round(per_batch * n_batches, 4), "unit": "s", "cores": threads, "kind": "port",

@@ -159,6 +159,18 @@ int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t 
                     const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
                     uint32_t F, int accumulate, nts_stream_t stream);
 
+/* nts_spmm_gather with a bound the caller knows: no row has more than max_row_edges edges (a sampled
+ * layer's forward pass: a destination keeps at most `fanout` neighbours, core/ntsSampler.hpp:936-1042;
+ * nts_batch_builder_layers reports the bound as nts_sampled_layer_t::max_in_degree).  With
+ * 0 < max_row_edges <= 256 the call is ONE launch -- a wavefront or lane group per row, nothing to cut,
+ * no scratch -- whatever the edge count; with 0 (unknown) or a larger bound it is nts_spmm_gather.
+ * The bound only selects the launch: a row longer than stated is still summed correctly, by one
+ * wavefront.  Replaces the same reference calls as nts_spmm_gather (cuda/ntsCUDA.hpp:124-143), as
+ * reached from SingleGPUSampleGraphOp::forward (core/ntsMiniBatchGraphOp.hpp:288-318). */
+int nts_spmm_gather_bounded(const float *in, float *out, const float *w, const uint32_t *offsets,
+                            const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
+                            uint32_t F, int accumulate, uint32_t max_row_edges, nts_stream_t stream);
+
 /* nts_spmm_gather for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * Same arguments, same kernels and bit-identical results; the scratch of calls that cut long rows
@@ -333,6 +345,12 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
 int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const uint32_t *perm,
                           const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
                           uint32_t edges, uint32_t H, uint32_t Fh, int accumulate, nts_stream_t stream);
+/* nts_spmm_gather_heads with the caller's bound on the longest row, as nts_spmm_gather_bounded: one
+ * launch when 0 < max_row_edges <= 256 (a sampled GAT layer's forward pass). */
+int nts_spmm_gather_heads_bounded(const float *in, float *out, const float *alpha, const uint32_t *perm,
+                                  const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
+                                  uint32_t edges, uint32_t H, uint32_t Fh, int accumulate,
+                                  uint32_t max_row_edges, nts_stream_t stream);
 /* The same through a schedule built by nts_spmm_plan_create[_slabs] for `offsets` (full-graph GAT:
  * hub rows are split and the sum order of split rows is the plan's). */
 int nts_spmm_gather_heads_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *alpha,
@@ -453,7 +471,9 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
  * stream, or the earlier batch is waited for first (nts_batch_builder_layers does). */
 typedef struct nts_batch_builder nts_batch_builder_t;
 typedef struct nts_sampled_layer {
-  uint32_t v_size, e_size, src_size, reserved; /* destinations, edges, distinct sources */
+  uint32_t v_size, e_size, src_size;           /* destinations, edges, distinct sources */
+  uint32_t max_in_degree;                      /* no destination has more edges than this (the hop's
+                                                  fanout); 0 = no bound known (fanout -1)          */
   uint32_t *destination;                       /* [v_size]   global ids                        */
   uint32_t *source;                            /* [src_size] global ids, ascending             */
   uint32_t *column_offset;                     /* [v_size+1]                                   */

@@ -54,6 +54,7 @@ SIGNATURES = {
     "nts_event_elapsed_ms": [ctypes.POINTER(_f32), _vp, _vp],
     "nts_spmm_plan_set_events": [_vp, _vp, _vp],
     "nts_spmm_gather": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
+    "nts_spmm_gather_bounded": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, _vp],
     "nts_spmm_gather_static_scratch": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
     "nts_spmm_plan_create": [ctypes.POINTER(_vp), _vp, _u32, _u32, _u32, _vp],
     "nts_spmm_plan_create_slabs": [ctypes.POINTER(_vp), _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _vp],
@@ -76,6 +77,7 @@ SIGNATURES = {
     "nts_gat_attention_fwd": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp],
     "nts_gat_attention_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp],
     "nts_spmm_gather_heads": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
+    "nts_spmm_gather_heads_bounded": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, _vp],
     "nts_spmm_gather_heads_planned": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _int, _vp],
     "nts_sddmm_heads": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp],
     "nts_gather_rows_f32": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _vp],
@@ -121,7 +123,7 @@ _NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_trace_ranges_emitted", "
 
 class SampledLayerDesc(ctypes.Structure):
     """nts_sampled_layer_t of include/nts_hip.h."""
-    _fields_ = [("v_size", _u32), ("e_size", _u32), ("src_size", _u32), ("reserved", _u32),
+    _fields_ = [("v_size", _u32), ("e_size", _u32), ("src_size", _u32), ("max_in_degree", _u32),
                 ("destination", _vp), ("source", _vp), ("column_offset", _vp), ("row_indices", _vp),
                 ("row_offset", _vp), ("column_indices", _vp), ("csr_to_csc", _vp),
                 ("edge_weight_forward", _vp), ("edge_weight_backward", _vp)]
@@ -173,6 +175,8 @@ def last_error():
 
 def call(name, *args):
     """Calls an entry point and raises NtsError on a non-zero status."""
+    if name not in SIGNATURES:
+        raise KeyError(f"{name} has no entry in abi.SIGNATURES (arguments would be passed untyped)")
     fn = getattr(lib(), name)
     rc = fn(*args)
     if name not in _NO_STATUS and rc != NTS_OK:

@@ -191,6 +191,7 @@ class BatchBuilder:
             layer = SampledLayer()
             Vd, E, Vs = d.v_size, d.e_size, d.src_size
             layer.v_size, layer.e_size, layer.src_size = Vd, E, Vs
+            layer.max_in_degree = d.max_in_degree
             layer.dev_destination = self._array(d.destination, Vd, i32)
             layer.dev_source = self._array(d.source, Vs, i32)
             layer.dev_column_offset = self._array(d.column_offset, Vd + 1, i32)

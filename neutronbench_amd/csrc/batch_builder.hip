@@ -336,7 +336,7 @@ int nts_batch_builder_layers(nts_batch_builder_t *b, nts_sampled_layer_t *layers
     out.v_size = s[0];
     out.e_size = s[1];
     out.src_size = s[2];
-    out.reserved = 0;
+    out.max_in_degree = b->fanout[h] > 0 ? static_cast<uint32_t>(b->fanout[h]) : 0u;
     out.destination = reinterpret_cast<uint32_t *>(A + (h == 0 ? b->L.dst0 : b->L.hop[h - 1].source));
     out.source = reinterpret_cast<uint32_t *>(A + H.source);
     out.column_offset = reinterpret_cast<uint32_t *>(A + H.co);

@@ -1054,6 +1054,24 @@ int nts_spmm_gather(const float *in, float *out, const float *w, const uint32_t 
   return NTS_OK;
 }
 
+int nts_spmm_gather_bounded(const float *in, float *out, const float *w, const uint32_t *offsets,
+                            const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges, uint32_t F,
+                            int accumulate, uint32_t max_row_edges, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_gather_bounded");
+  if (int rc = nts::check_common(in, out, offsets, indices, rows, edges, F, "nts_spmm_gather_bounded: null pointer"))
+    return rc;
+  if (rows == 0) return NTS_OK;
+  nts::LaunchArgs a{in, out, w, offsets, indices, index_base, rows, F, nullptr, nullptr, accumulate, stream};
+  if (max_row_edges != 0 && max_row_edges <= nts::kAutoChunk) {
+    // No row can need cutting: one launch, a wavefront (or lane group) per row, no scratch.
+    nts::launch_spmm(a);
+  } else if (int rc = nts::launch_spmm_balanced(a, edges)) {
+    return rc;
+  }
+  NTS_LAUNCH_CHECK("nts_spmm_gather_bounded");
+  return NTS_OK;
+}
+
 int nts_spmm_gather_static_scratch(const float *in, float *out, const float *w, const uint32_t *offsets,
                                    const uint32_t *indices, uint32_t index_base, uint32_t rows, uint32_t edges,
                                    uint32_t F, int accumulate, nts_stream_t stream) {
@@ -1500,6 +1518,25 @@ int nts_spmm_gather_heads(const float *in, float *out, const float *alpha, const
   a.heads = nts::HeadArgs{perm, H, Fh};
   if (int rc = nts::launch_spmm_balanced(a, edges)) return rc;
   NTS_LAUNCH_CHECK("nts_spmm_gather_heads");
+  return NTS_OK;
+}
+
+int nts_spmm_gather_heads_bounded(const float *in, float *out, const float *alpha, const uint32_t *perm,
+                                  const uint32_t *offsets, const uint32_t *indices, uint32_t rows, uint32_t edges,
+                                  uint32_t H, uint32_t Fh, int accumulate, uint32_t max_row_edges, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_spmm_gather_heads_bounded");
+  if (int rc = check_heads(alpha, H, Fh, "nts_spmm_gather_heads_bounded: bad H / Fh / alpha")) return rc;
+  if (rows == 0) return NTS_OK;
+  if (!in || !out || !offsets || !indices)
+    return nts::fail(NTS_ERR_INVALID, "nts_spmm_gather_heads_bounded: null pointer");
+  nts::LaunchArgs a{in, out, alpha, offsets, indices, 0u, rows, H * Fh, nullptr, nullptr, accumulate, stream};
+  a.heads = nts::HeadArgs{perm, H, Fh};
+  if (max_row_edges != 0 && max_row_edges <= nts::kAutoChunk) {
+    nts::launch_spmm(a);
+  } else if (int rc = nts::launch_spmm_balanced(a, edges)) {
+    return rc;
+  }
+  NTS_LAUNCH_CHECK("nts_spmm_gather_heads_bounded");
   return NTS_OK;
 }
 

@@ -323,50 +323,78 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
     return out
 
 
-def run_native(name, scale=1.0, max_batches=0, warmup_batches=2, pipeline=1, quiet=False, graph=True, verify=False,
-               stage_sync=False, keep_dir=None):
-    """The same epoch driven from C++ (neutronbench_amd/host/epoch_driver.cpp -> lib/nts_epoch): the
-    arrays of the synthetic configuration are written to a directory, the program runs the batches
-    through the C ABI with no Python between the calls and prints one JSON line.  Same graph, train
-    ids and seeds as `run`, so sampled_edges and gathered_rows are equal."""
+def write_native_inputs(name, directory, scale=1.0, keep_host=False):
+    """Writes the arrays of a configuration for lib/nts_epoch: co.bin, ri.bin (uint32 CSC of the whole
+    graph), feat.bin (float32 [V, F]), labels.bin (int64 [V]), train.bin (uint32 ids).  Same graph, train
+    ids and seeds as `run`.  The products and gat configurations share every file.  Returns the shape
+    (and, with keep_host, the host arrays, for a checker)."""
     import os
-    import shutil
-    import subprocess
-    import tempfile
 
     cfg = dict(CONFIGS[name])
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "nts_epoch")
-    if not os.path.exists(exe):
-        raise RuntimeError(f"{exe} has not been built (make -C neutronbench_amd/csrc)")
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
     n_train = int(cfg["train"] * scale)
     src, dst = synth.rmat_edges(V, E, seed=cfg["seed"], device=dev, sort=True)
     co, ri = synth.build_csc(src, dst, V)
     del src, dst
+    host = dict(co=as_u32(co).cpu().numpy(), ri=as_u32(ri).cpu().numpy(),
+                feat=synth.normal_features(V, cfg["F"], seed=cfg["seed"] + 40).numpy(),
+                labels=synth.uniform_labels(V, cfg["classes"], seed=cfg["seed"] + 41, device=dev).cpu().numpy(),
+                train=as_u32(synth.permutation(V, cfg["seed"] + 42, dev)[:n_train]).cpu().numpy())
+    del co, ri
+    torch.cuda.empty_cache()
+    for key, arr in host.items():
+        arr.tofile(os.path.join(directory, f"{key}.bin"))
+    out = dict(V=V, E=E, n_train=n_train)
+    if keep_host:
+        import numpy as np
+
+        out.update(co=host["co"].view(np.uint32), ri=host["ri"].view(np.uint32), feat=host["feat"], labels=host["labels"],
+                   train=host["train"].view(np.uint32))
+    return out
+
+
+def run_native_on(directory, name, V, max_batches=0, warmup_batches=2, pipeline=1, graph=True, verify=False,
+                  stage_sync=False, dump_dir=None, dump_batch=0):
+    """Runs lib/nts_epoch on the arrays `write_native_inputs` left in `directory`; returns its JSON line."""
+    import os
+    import subprocess
+
+    cfg = dict(CONFIGS[name])
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "nts_epoch")
+    if not os.path.exists(exe):
+        raise RuntimeError(f"{exe} has not been built (make -C neutronbench_amd/csrc)")
+    cmd = [exe, "--dir", directory, "--V", str(V), "--F", str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch",
+           str(cfg["batch"]), "--fanout", ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)),
+           "--pipeline", str(pipeline), "--cache", str(cfg["cache"]), "--graph", str(int(graph)), "--warmup",
+           str(warmup_batches), "--max-batches", str(max_batches), "--verify", str(int(verify)), "--stage-sync",
+           str(int(stage_sync))]
+    if dump_dir:
+        cmd += ["--dump-dir", dump_dir, "--dump-batch", str(dump_batch)]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    if p.returncode != 0:
+        raise RuntimeError(f"nts_epoch failed ({p.returncode}): {p.stderr[-2000:]}")
+    return json.loads(p.stdout.strip().splitlines()[-1])
+
+
+def run_native(name, scale=1.0, max_batches=0, warmup_batches=2, pipeline=1, quiet=False, graph=True, verify=False,
+               stage_sync=False, keep_dir=None):
+    """The same epoch driven from C++ (neutronbench_amd/host/epoch_driver.cpp -> lib/nts_epoch): the
+    arrays of the synthetic configuration are written to a directory, the program runs the batches
+    through the C ABI with no Python between the calls and prints one JSON line.  Same graph, train
+    ids and seeds as `run`, so sampled_edges and gathered_rows are equal."""
+    import shutil
+    import tempfile
+
+    cfg = dict(CONFIGS[name])
     d = keep_dir or tempfile.mkdtemp(prefix="nts_epoch_")
     try:
-        as_u32(co).cpu().numpy().tofile(os.path.join(d, "co.bin"))
-        as_u32(ri).cpu().numpy().tofile(os.path.join(d, "ri.bin"))
-        synth.normal_features(V, cfg["F"], seed=cfg["seed"] + 40).numpy().tofile(os.path.join(d, "feat.bin"))
-        synth.uniform_labels(V, cfg["classes"], seed=cfg["seed"] + 41, device=dev).cpu().numpy().tofile(
-            os.path.join(d, "labels.bin"))
-        as_u32(synth.permutation(V, cfg["seed"] + 42, dev)[:n_train]).cpu().numpy().tofile(os.path.join(d, "train.bin"))
-        del co, ri
-        torch.cuda.empty_cache()
-        cmd = [exe, "--dir", d, "--V", str(V), "--F", str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch",
-               str(cfg["batch"]), "--fanout", ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)),
-               "--pipeline", str(pipeline), "--cache",
-               str(cfg["cache"]), "--graph", str(int(graph)), "--warmup", str(warmup_batches), "--max-batches",
-               str(max_batches), "--verify", str(int(verify)), "--stage-sync", str(int(stage_sync))]
-        p = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
-        if p.returncode != 0:
-            raise RuntimeError(f"nts_epoch failed ({p.returncode}): {p.stderr[-2000:]}")
-        out = json.loads(p.stdout.strip().splitlines()[-1])
+        shape = write_native_inputs(name, d, scale)
+        out = run_native_on(d, name, shape["V"], max_batches, warmup_batches, pipeline, graph, verify, stage_sync)
     finally:
         if keep_dir is None:
             shutil.rmtree(d, ignore_errors=True)
-    out.update(config=name, scale=scale, vertices=V, edges=E, fanout_output_side_first=cfg["fanout"])
+    out.update(config=name, scale=scale, vertices=shape["V"], edges=shape["E"], fanout_output_side_first=cfg["fanout"])
     if not quiet:
         print(json.dumps(out))
     return out

@@ -4,8 +4,10 @@
 //
 // Per batch: nts_batch_builder_sample / _layers (all hops, relabelling, CSR, weights), the feature
 // gather (zero-copy from mapped pinned host memory, or through the HBM cache of the top out-degree
-// vertices), the label gather, and for every layer the aggregation forward (zeroed output,
-// accumulate, as SingleGPUSampleGraphOp does) and, in reverse order, backward.  With --heads H every
+// vertices), the label gather, and for every layer the aggregation forward (one launch: the hop's
+// fanout bounds every destination's edges, nts_spmm_gather_bounded) and, in reverse order, backward
+// (sources can be hubs: nts_spmm_gather cuts long rows on the device).  Outputs are written, not added
+// to, so no buffer is cleared first.  With --heads H every
 // layer is a GAT layer instead: fused attention (nts_gat_attention_fwd) and attention-weighted
 // aggregation (nts_spmm_gather_heads) forward; backward the aggregation over the CSR, the per-edge
 // gradient of alpha (nts_sddmm_heads), the fused attention backward and the sum of the edge
@@ -22,7 +24,10 @@
 // The program reads raw arrays written by neutronbench_amd/epoch.py (--native): co.bin, ri.bin (uint32
 // CSC of the whole graph), feat.bin (float32 [V, F]), labels.bin (int64 [V]), train.bin (uint32 ids),
 // and prints one JSON line.  --verify 1 adds a checksum of every aggregation output (a device-side
-// hash per batch, which waits for the stream: not for timing).
+// hash per batch, which waits for the stream: not for timing).  --dump-dir D [--dump-batch b]: after the
+// timed epoch, batch b runs once more through the same calls and every array it produced -- the
+// layers' structure, the gathered features and labels, each aggregation's input and output -- is
+// written to D as raw files with a meta.json, for a checker to compare with the CPU oracle.
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -94,7 +99,8 @@ void *device_bytes(size_t bytes) {
 }
 
 struct Args {
-  std::string dir;
+  std::string dir, dump_dir;
+  uint32_t dump_batch = 0;
   std::vector<int32_t> fanout;
   uint32_t V = 0, F = 0, hidden = 128, batch = 1024, pipeline = 1, warmup = 2, max_batches = 0, heads = 0;
   double cache = 0.0;
@@ -118,6 +124,8 @@ Args parse(int argc, char **argv) {
     else if (k == "--graph") a.graph = std::stoi(v);
     else if (k == "--verify") a.verify = std::stoi(v);
     else if (k == "--stage-sync") a.stage_sync = std::stoi(v);
+    else if (k == "--dump-dir") a.dump_dir = v;
+    else if (k == "--dump-batch") a.dump_batch = static_cast<uint32_t>(std::stoul(v));
     else if (k == "--fanout") {
       size_t at = 0;
       while (at < v.size()) {
@@ -135,7 +143,8 @@ Args parse(int argc, char **argv) {
       (a.heads && a.hidden % a.heads)) {
     fprintf(stderr,
             "usage: nts_epoch --dir D --V n --F n --fanout a,b[,c] [--batch n] [--hidden n] [--heads n] [--pipeline 1..8]\n"
-            "                 [--cache fraction] [--graph 0|1] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n");
+            "                 [--cache fraction] [--graph 0|1] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n"
+            "                 [--dump-dir D [--dump-batch b]]\n");
     exit(2);
   }
   return a;
@@ -298,6 +307,20 @@ int main(int argc, char **argv) {
     NTS(nts_fingerprint_u32(&fp, reinterpret_cast<const uint32_t *>(p), n, nullptr, 0, stream));
     checksum ^= fp * (2 * salt + 1);
   };
+  // Dump mode (after the timed epoch): every array of the batch goes to a file as the stages produce it.
+  bool dumping = false;
+  auto dump = [&](const std::string &name, const void *dev, size_t bytes, hipStream_t stream) {
+    HIP(hipStreamSynchronize(stream));
+    std::vector<char> host(bytes);
+    if (bytes) HIP(hipMemcpy(host.data(), dev, bytes, hipMemcpyDeviceToHost));
+    FILE *f = fopen((a.dump_dir + "/" + name).c_str(), "wb");
+    if (!f || (bytes && fwrite(host.data(), 1, bytes, f) != bytes)) {
+      fprintf(stderr, "nts_epoch: cannot write %s/%s\n", a.dump_dir.c_str(), name.c_str());
+      exit(1);
+    }
+    fclose(f);
+  };
+  auto tag = [](const char *what, uint32_t layer) { return "L" + std::to_string(layer) + "_" + what + ".bin"; };
   auto aggregate_gat = [&](Slot &s, hipStream_t stream) {
     const float slope = 0.2f;
     double t0 = now();
@@ -306,11 +329,18 @@ int main(int argc, char **argv) {
       const float *x = d_ones;  // [src_size, H * Fh]: stands in for the projected features of the layer
       const float *el = d_ones + 8;  // [src_size, H]
       NTS(nts_gat_attention_fwd(d_alpha[l], el, d_er, L.column_offset, L.row_indices, L.v_size, H, slope, stream));
-      NTS(nts_spmm_gather_heads(x, d_out, d_alpha[l], nullptr, L.column_offset, L.row_indices, L.v_size, L.e_size, H, Fh, 0,
-                                stream));
+      NTS(nts_spmm_gather_heads_bounded(x, d_out, d_alpha[l], nullptr, L.column_offset, L.row_indices, L.v_size, L.e_size,
+                                        H, Fh, 0, L.max_in_degree, stream));
       if (a.verify) {
         hash(d_alpha[l], static_cast<uint64_t>(L.e_size) * H, 10 + l, stream);
         hash(d_out, static_cast<uint64_t>(L.v_size) * H * Fh, 20 + l, stream);
+      }
+      if (dumping) {
+        dump(tag("x", l), x, static_cast<size_t>(L.src_size) * H * Fh * 4, stream);
+        dump(tag("el", l), el, static_cast<size_t>(L.src_size) * H * 4, stream);
+        dump(tag("er", l), d_er, static_cast<size_t>(L.v_size) * H * 4, stream);
+        dump(tag("alpha", l), d_alpha[l], static_cast<size_t>(L.e_size) * H * 4, stream);
+        dump(tag("out", l), d_out, static_cast<size_t>(L.v_size) * H * Fh * 4, stream);
       }
       if (a.stage_sync) HIP(hipStreamSynchronize(stream));
     }
@@ -330,6 +360,14 @@ int main(int argc, char **argv) {
         hash(d_ger, static_cast<uint64_t>(L.v_size) * H, 40 + k, stream);
         hash(d_gel, static_cast<uint64_t>(L.src_size) * H, 50 + k, stream);
       }
+      if (dumping) {
+        dump(tag("gout", k), g_out, static_cast<size_t>(L.v_size) * H * Fh * 4, stream);
+        dump(tag("gin", k), d_gin, static_cast<size_t>(L.src_size) * H * Fh * 4, stream);
+        dump(tag("galpha", k), d_galpha, static_cast<size_t>(L.e_size) * H * 4, stream);
+        dump(tag("gs", k), d_gs, static_cast<size_t>(L.e_size) * H * 4, stream);
+        dump(tag("ger", k), d_ger, static_cast<size_t>(L.v_size) * H * 4, stream);
+        dump(tag("gel", k), d_gel, static_cast<size_t>(L.src_size) * H * 4, stream);
+      }
       if (a.stage_sync) HIP(hipStreamSynchronize(stream));
     }
     if (a.stage_sync) t_bwd += now() - t0;
@@ -341,14 +379,17 @@ int main(int argc, char **argv) {
       const nts_sampled_layer_t &L = s.layers[l];
       const uint32_t w = l == 0 ? F : a.hidden;
       const float *in = l == 0 ? s.x : d_ones;
-      NTS(nts_memset_zero(d_out, static_cast<size_t>(L.v_size) * w * sizeof(float), stream));
-      NTS(nts_spmm_gather(in, d_out, L.edge_weight_forward, L.column_offset, L.row_indices, 0, L.v_size, L.e_size, w, 1,
-                          stream));
+      NTS(nts_spmm_gather_bounded(in, d_out, L.edge_weight_forward, L.column_offset, L.row_indices, 0, L.v_size, L.e_size,
+                                  w, 0, L.max_in_degree, stream));
       if (a.verify) {
         uint64_t fp = 0;
         NTS(nts_fingerprint_u32(&fp, reinterpret_cast<const uint32_t *>(d_out), static_cast<uint64_t>(L.v_size) * w,
                                 nullptr, 0, stream));
         checksum ^= fp * (2 * l + 1);
+      }
+      if (dumping) {
+        dump(tag("in", l), in, static_cast<size_t>(L.src_size) * w * 4, stream);
+        dump(tag("out", l), d_out, static_cast<size_t>(L.v_size) * w * 4, stream);
       }
       if (a.stage_sync) HIP(hipStreamSynchronize(stream));
     }
@@ -357,14 +398,17 @@ int main(int argc, char **argv) {
     for (uint32_t k = hops; k-- > 0;) {
       const nts_sampled_layer_t &L = s.layers[k];
       const uint32_t w = k == 0 ? F : a.hidden;
-      NTS(nts_memset_zero(d_gin, static_cast<size_t>(L.src_size) * w * sizeof(float), stream));
       NTS(nts_spmm_gather(d_ones, d_gin, L.edge_weight_backward, L.row_offset, L.column_indices, 0, L.src_size, L.e_size,
-                          w, 1, stream));
+                          w, 0, stream));
       if (a.verify) {
         uint64_t fp = 0;
         NTS(nts_fingerprint_u32(&fp, reinterpret_cast<const uint32_t *>(d_gin), static_cast<uint64_t>(L.src_size) * w,
                                 nullptr, 0, stream));
         checksum ^= fp * (2 * k + 2);
+      }
+      if (dumping) {
+        dump(tag("gout", k), d_ones, static_cast<size_t>(L.v_size) * w * 4, stream);
+        dump(tag("gin", k), d_gin, static_cast<size_t>(L.src_size) * w * 4, stream);
       }
       if (a.stage_sync) HIP(hipStreamSynchronize(stream));
     }
@@ -464,14 +508,52 @@ int main(int argc, char **argv) {
   run_batches(n_batches);
   HIP(hipDeviceSynchronize());
   const double epoch_s = now() - t0;
+  const double stage_sample = t_sample, stage_gather = t_gather, stage_fwd = t_fwd, stage_bwd = t_bwd;
+
+  if (!a.dump_dir.empty() && a.dump_batch < n_batches) {
+    // The batch once more, through the same calls, with every array written out.
+    Slot &s = slots[0];
+    const uint32_t b = a.dump_batch;
+    sample(s, b, main_stream);
+    NTS(nts_batch_builder_layers(s.builder, s.layers));
+    gather(s, 0, main_stream);
+    HIP(hipStreamSynchronize(main_stream));
+    FILE *meta = fopen((a.dump_dir + "/meta.json").c_str(), "w");
+    if (!meta) die("cannot write meta.json");
+    fprintf(meta, "{\"batch\": %u, \"hops\": %u, \"F\": %u, \"hidden\": %u, \"heads\": %u, \"layers\": [", b, hops, F, a.hidden, H);
+    for (uint32_t l = 0; l < hops; ++l) {
+      const nts_sampled_layer_t &L = s.layers[l];
+      fprintf(meta, "%s{\"v_size\": %u, \"e_size\": %u, \"src_size\": %u, \"max_in_degree\": %u, \"width\": %u}", l ? ", " : "",
+              L.v_size, L.e_size, L.src_size, L.max_in_degree, H ? a.hidden : (l == 0 ? F : a.hidden));
+      dump(tag("destination", l), L.destination, static_cast<size_t>(L.v_size) * 4, main_stream);
+      dump(tag("source", l), L.source, static_cast<size_t>(L.src_size) * 4, main_stream);
+      dump(tag("column_offset", l), L.column_offset, (static_cast<size_t>(L.v_size) + 1) * 4, main_stream);
+      dump(tag("row_indices", l), L.row_indices, static_cast<size_t>(L.e_size) * 4, main_stream);
+      dump(tag("row_offset", l), L.row_offset, (static_cast<size_t>(L.src_size) + 1) * 4, main_stream);
+      dump(tag("column_indices", l), L.column_indices, static_cast<size_t>(L.e_size) * 4, main_stream);
+      dump(tag("edge_weight_forward", l), L.edge_weight_forward, static_cast<size_t>(L.e_size) * 4, main_stream);
+      dump(tag("edge_weight_backward", l), L.edge_weight_backward, static_cast<size_t>(L.e_size) * 4, main_stream);
+      if (L.csr_to_csc) dump(tag("csr_to_csc", l), L.csr_to_csc, static_cast<size_t>(L.e_size) * 4, main_stream);
+    }
+    uint32_t hits = 0;
+    if (n_cache) HIP(hipMemcpy(&hits, s.hits, sizeof(hits), hipMemcpyDeviceToHost));
+    fprintf(meta, "], \"cache_rows\": %u, \"cache_hits\": %u}\n", n_cache, hits);
+    fclose(meta);
+    dump("x.bin", s.x, static_cast<size_t>(s.layers[0].src_size) * F * 4, main_stream);
+    dump("labels.bin", s.labels, static_cast<size_t>(s.layers[hops - 1].v_size) * 8, main_stream);
+    dumping = true;
+    aggregate(s, main_stream);
+    dumping = false;
+    HIP(hipDeviceSynchronize());
+  }
 
   printf("{\"driver\": \"native\", \"batches\": %u, \"batch_size\": %u, \"pipeline\": %u, \"hop_launches_as_graph\": %s, "
          "\"stage_sync\": %s, \"epoch_s\": %.4f, \"sampled_edges\": %llu, \"gathered_rows\": %llu, \"cache_rows\": %u",
          n_batches, a.batch, P, a.graph ? "true" : "false", a.stage_sync ? "true" : "false", epoch_s,
          static_cast<unsigned long long>(edges_total), static_cast<unsigned long long>(rows_total), n_cache);
   if (P == 1 && a.stage_sync)
-    printf(", \"stage_s\": {\"sample\": %.4f, \"gather\": %.4f, \"aggregate_fwd\": %.4f, \"aggregate_bwd\": %.4f}", t_sample,
-           t_gather, t_fwd, t_bwd);
+    printf(", \"stage_s\": {\"sample\": %.4f, \"gather\": %.4f, \"aggregate_fwd\": %.4f, \"aggregate_bwd\": %.4f}", stage_sample,
+           stage_gather, stage_fwd, stage_bwd);
   if (n_cache && P == 1 && (a.stage_sync || a.verify))
     printf(", \"cache_hit_rate\": %.4f", rows_total ? static_cast<double>(hits_total) / rows_total : 0.0);
   if (a.verify) printf(", \"checksum\": \"%016llx\"", static_cast<unsigned long long>(checksum));

@@ -149,6 +149,7 @@ class SampledLayer:
 
     def __init__(self):
         self.v_size = self.e_size = self.src_size = 0
+        self.max_in_degree = 0  # bound on a destination's edges where the sampler knows one (its fanout), else 0
         self.dev_destination = self.dev_source = None
         self.dev_column_offset = self.dev_row_indices = None
         self.dev_row_offset = self.dev_column_indices = None

@@ -58,8 +58,13 @@ class SingleGPUSampleGraphOp:
         sg = self.sg
         F = f_input.shape[1]
         out = torch.zeros(sg.v_size, F, dtype=torch.float32, device=f_input.device)
-        self.cs.Gather_By_Dst_From_Src(f_input, out, sg.dev_ewf(), sg.dev_r_i(), sg.dev_c_o(), 0, 0, 0, 0, sg.e_size,
-                                       sg.v_size, F, True, False)
+        if 0 < sg.max_in_degree <= 256:
+            # the sampler bounded every destination's edges by its fanout: one launch, nothing to cut
+            call("nts_spmm_gather_bounded", ptr(f_input), ptr(out), ptr(sg.dev_ewf()), ptr(sg.dev_c_o()),
+                 ptr(sg.dev_r_i()), 0, sg.v_size, sg.e_size, F, 1, sg.max_in_degree, self.cs.stream)
+        else:
+            self.cs.Gather_By_Dst_From_Src(f_input, out, sg.dev_ewf(), sg.dev_r_i(), sg.dev_c_o(), 0, 0, 0, 0,
+                                           sg.e_size, sg.v_size, F, True, False)
         if self.sync:
             self.cs.CUDA_DEVICE_SYNCHRONIZE()
         return out
@@ -219,8 +224,8 @@ class GATAggregateOp:
         Fh = x.shape[1] // self.H
         out = torch.empty(sg.v_size, x.shape[1], dtype=torch.float32, device=x.device)
         stream = torch.cuda.current_stream(x.device).cuda_stream
-        call("nts_spmm_gather_heads", ptr(x), ptr(out), ptr(alpha), 0, ptr(sg.dev_c_o()), ptr(sg.dev_r_i()), sg.v_size,
-             sg.e_size, self.H, Fh, 0, stream)
+        call("nts_spmm_gather_heads_bounded", ptr(x), ptr(out), ptr(alpha), 0, ptr(sg.dev_c_o()), ptr(sg.dev_r_i()),
+             sg.v_size, sg.e_size, self.H, Fh, 0, getattr(sg, "max_in_degree", 0), stream)
         self.x, self.alpha = x, alpha
         return out
 

@@ -47,15 +47,53 @@ def permutation(n, seed, device="cpu"):
     return torch.argsort(keys, stable=True)
 
 
-def rmat_edges(V, E, a=0.57, b=0.19, c=0.19, seed=1, device="cpu", permute=True, sort=False):
+def rmat_edges(V, E, a=0.57, b=0.19, c=0.19, seed=1, device="cpu", permute=True, sort=False, distinct=False):
     """R-MAT directed edge list (src, dst) as int64 tensors of length E.  sort=True returns the list
-    in (source, destination) order, the order of an edge file exported from sorted adjacency lists;
-    duplicates are kept either way."""
+    in (source, destination) order, the order of an edge file exported from sorted adjacency lists.
+    Duplicates are kept unless distinct=True: then the list holds the first E distinct (src, dst)
+    pairs of the same draw sequence (a simple graph, as the social-network datasets are), in draw
+    order or, with sort=True, in (source, destination) order."""
+    if distinct:
+        return _rmat_distinct(V, E, a, b, c, seed, device, permute, sort)
+    return _rmat_draws(V, 0, E, a, b, c, seed, device, permute, sort)
+
+
+def _rmat_distinct(V, E, a, b, c, seed, device, permute, sort):
+    if E > V * V:
+        raise ValueError("more distinct edges asked for than vertex pairs exist")
+    draws = E + E // 2 + 16
+    while True:
+        src, dst = _rmat_draws(V, 0, draws, a, b, c, seed, device, permute, False)
+        key = src * V + dst
+        del src, dst
+        skey, order = torch.sort(key, stable=True)  # equal pairs stay in draw order: the first is the earliest draw
+        del key
+        first = torch.ones(draws, dtype=torch.bool, device=device)
+        first[1:] = skey[1:] != skey[:-1]
+        n_distinct = int(first.sum())
+        if n_distinct >= E:
+            break
+        del skey, order, first
+        draws = draws + draws // 3  # the same draw sequence, longer
+    skey, drawn_at = skey[first], order[first]
+    del order, first
+    if n_distinct > E:  # keep the E pairs that were drawn first
+        limit = torch.sort(drawn_at).values[E - 1]
+        keep = drawn_at <= limit
+        skey, drawn_at = skey[keep], drawn_at[keep]
+    if not sort:
+        skey = skey[torch.sort(drawn_at).indices]
+    return skey // V, skey % V
+
+
+def _rmat_draws(V, first, count, a, b, c, seed, device, permute, sort):
+    """Draws first .. first + count - 1 of the seeded R-MAT sequence."""
+    E = count
     scale = max(1, math.ceil(math.log2(V)))
     ta = int(a * (1 << 24))
     tb = int((a + b) * (1 << 24))
     tc = int((a + b + c) * (1 << 24))
-    idx = torch.arange(E, dtype=torch.int64, device=device)
+    idx = torch.arange(first, first + E, dtype=torch.int64, device=device)
     src = torch.zeros(E, dtype=torch.int64, device=device)
     dst = torch.zeros(E, dtype=torch.int64, device=device)
     for level in range(scale):

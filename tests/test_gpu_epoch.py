@@ -90,3 +90,29 @@ def test_native_epoch_driver(config, scale):
         assert r["checksum"] == runs[0]["checksum"]
     if py["cache_hit_rate"] is not None:
         assert abs(runs[0]["cache_hit_rate"] - py["cache_hit_rate"]) < 1e-4
+
+
+@pytest.mark.parametrize("config,scale", [("arxiv", 0.25), ("products", 0.02), ("gat", 0.02)])
+def test_native_epoch_batch_against_the_oracle(config, scale, tmp_path):
+    """Every array of one batch of the native epoch -- sampled layers, CSR, weights, gathered features
+    and labels, each aggregation's (or GAT operator's) input and output, as written by --dump-dir after
+    the timed epoch -- against the CPU oracle: structure and gathers bit for bit, sums within 1e-4."""
+    from neutronbench_amd import epoch
+    from oracle import epoch_check
+
+    data, dump = tmp_path / "data", tmp_path / "dump"
+    data.mkdir()
+    dump.mkdir()
+    host = epoch.write_native_inputs(config, str(data), scale, keep_host=True)
+    cfg = epoch.CONFIGS[config]
+    n_batches = min(4, -(-host["n_train"] // cfg["batch"]))
+    out = epoch.run_native_on(str(data), config, host["V"], max_batches=4, warmup_batches=1, stage_sync=True,
+                              dump_dir=str(dump), dump_batch=n_batches - 1)
+    assert out["batches"] == n_batches
+    assert set(out["stage_s"]) == {"sample", "gather", "aggregate_fwd", "aggregate_bwd"}
+    res = epoch_check.check_dump(str(dump), host["co"], host["ri"], host["feat"], host["labels"], cfg["fanout"],
+                                 cfg["cache"])
+    assert res["ok"], res
+    assert res["sampled_edges"] > 0 and res["checked_rows"] > 0 and res["max_rel_err"] <= 1e-4
+    if not cfg.get("heads"):
+        assert res["bit_exact_rows"] > 0
