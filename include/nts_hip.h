@@ -224,6 +224,12 @@ int nts_spmm_plan_schedule_host(const uint32_t *offsets_host, const uint32_t *in
                                 uint64_t items_cap, uint32_t *n_items, uint32_t *n_split_rows,
                                 uint32_t *n_partials);
 int nts_spmm_plan_destroy(nts_spmm_plan_t *plan);
+/* Copies a plan's schedule to the host: items_out (nullable; items_cap items of four words, as
+ * nts_spmm_plan_schedule_host writes them) and splits_out (nullable; splits_cap entries of four words:
+ * row, first partial slot, slot count, 0 -- the split rows in the order the second stage visits them).
+ * For tests and for inspecting a schedule; the counts come from nts_spmm_plan_info. */
+int nts_spmm_plan_copy_schedule(const nts_spmm_plan_t *plan, uint32_t *items_out, uint64_t items_cap,
+                                uint32_t *splits_out, uint64_t splits_cap);
 /* Number of work items, split rows and partial-sum slots of a plan (for tests and reports). */
 int nts_spmm_plan_info(const nts_spmm_plan_t *plan, uint32_t *items, uint32_t *split_rows,
                        uint32_t *partials);

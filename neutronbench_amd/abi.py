@@ -61,6 +61,7 @@ SIGNATURES = {
     "nts_spmm_plan_schedule_host": [_vp, _vp, _u32, _u32, _u32, _u32, _vp, _u64, ctypes.POINTER(_u32),
                                     ctypes.POINTER(_u32), ctypes.POINTER(_u32)],
     "nts_spmm_plan_destroy": [_vp],
+    "nts_spmm_plan_copy_schedule": [_vp, _vp, _u64, _vp, _u64],
     "nts_spmm_plan_info": [_vp, ctypes.POINTER(_u32), ctypes.POINTER(_u32), ctypes.POINTER(_u32)],
     "nts_spmm_plan_scratch_info": [_vp, _u32, ctypes.POINTER(_sz), ctypes.POINTER(_sz), ctypes.POINTER(_u64),
                                    ctypes.POINTER(_int)],

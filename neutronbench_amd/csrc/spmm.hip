@@ -975,6 +975,182 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
   return NTS_OK;
 }
 
+// ---- the same schedule built on the device -----------------------------------------------------------
+//
+// nts_spmm_plan_create_slabs needs the index array to cut rows at source-range boundaries; copying it
+// to the host and scheduling there costs seconds per 10^8 edges.  The kernels below build the item
+// list of make_schedule -- the same pieces, slots, order of pieces, order of whole rows and order of
+// split rows, entry for entry -- from the arrays where they lie:
+//   plan_cut_rows_kernel      one thread per row: the row's range count by its length, a lower_bound per
+//                             range boundary, pieces per (row, range) into a [rows, n_slabs] table
+//   exclusive scan of the table = first partial slot of every (row, range); its total = slots
+//   plan_emit_pieces_kernel   one thread per non-empty (row, range): its pieces and their sort keys
+//                             (range id, then longer pieces first); slot order is creation order, so a
+//                             stable radix sort by key reproduces the host's stable_sort
+//   plan_row_keys_kernel      per row: key of the whole rows (descending length, stable by row) and of
+//                             the split rows (descending slot count, stable by row)
+//   plan_finish_kernel        whole rows behind the pieces; the split-row table
+// Rows long enough to be cut must ascend; plan_scan_edges_kernel lists every descent idx[k-1] > idx[k]
+// (in a sorted graph these sit at row starts only) and plan_check_descents_kernel flags one inside such
+// a row -- then the host path, which sorts those rows in a copy of its own, takes over.
+
+struct PlanShape {
+  uint32_t chunk, n_slabs, wide_ranges;
+  uint64_t fine_width;
+  // Ranges a row of `deg` edges is cut at (0 = the row stays whole): see make_schedule.
+  __host__ __device__ uint32_t ranges_for(uint32_t deg) const {
+    if (deg <= chunk) return (wide_ranges && deg > chunk / 4) ? wide_ranges : 0u;
+    return (wide_ranges && deg <= 4ull * chunk) ? n_slabs / 2 : n_slabs;
+  }
+};
+
+struct PlanCounters {  // device words read back once
+  unsigned long long repeated_raw;  // k in [1, E) with idx[k] == idx[k-1], row starts included
+  uint32_t boundary_equal;          // of those, the ones at a row start
+  uint32_t n_descents;
+  uint32_t descent_overflow;
+  uint32_t unsorted_long_row;
+  uint32_t n_splits;
+  uint32_t pad;
+};
+
+__device__ __forceinline__ uint32_t lower_bound_index(const uint32_t *__restrict__ idx, uint32_t lo, uint32_t hi,
+                                                      uint64_t lim, uint32_t base) {
+  while (lo < hi) {
+    const uint32_t mid = lo + (hi - lo) / 2;
+    if (static_cast<uint64_t>(idx[mid] - base) < lim) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(256) void plan_cut_rows_kernel(uint32_t *__restrict__ counts, uint32_t *__restrict__ stops,
+                                                            const uint32_t *__restrict__ off,
+                                                            const uint32_t *__restrict__ idx, uint32_t index_base,
+                                                            uint32_t rows, PlanShape sh) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  const uint32_t b = off[r], e = off[r + 1], deg = e - b;
+  const uint32_t R = sh.ranges_for(deg);
+  if (R == 0) return;  // the table was cleared: a whole row has no pieces
+  uint32_t *cnt = counts + static_cast<size_t>(r) * sh.n_slabs;
+  uint32_t *stp = stops + static_cast<size_t>(r) * sh.n_slabs;
+  const uint32_t per = sh.n_slabs / R;
+  uint32_t cut = b, nonempty = 0;
+  for (uint32_t c = 0; c < R; ++c) {
+    const uint64_t hi = static_cast<uint64_t>(c + 1) * per * sh.fine_width;  // first index of the next range
+    const uint32_t stop = (c + 1 == R || cut >= e) ? e : lower_bound_index(idx, cut, e, hi, index_base);
+    const uint32_t n = stop - cut;
+    cnt[c] = deg > sh.chunk ? (n + sh.chunk - 1) / sh.chunk : (n ? 1u : 0u);
+    stp[c] = stop;
+    nonempty += n ? 1u : 0u;
+    cut = stop;
+  }
+  if (deg <= sh.chunk && nonempty <= 1)  // all edges in one wide range: the row stays whole
+    for (uint32_t c = 0; c < R; ++c) cnt[c] = 0;
+}
+
+__global__ __launch_bounds__(256) void plan_emit_pieces_kernel(Item *__restrict__ pieces, uint32_t *__restrict__ keys,
+                                                               const uint32_t *__restrict__ counts,
+                                                               const uint32_t *__restrict__ stops,
+                                                               const uint32_t *__restrict__ slot_base,
+                                                               const uint32_t *__restrict__ off, uint32_t rows,
+                                                               PlanShape sh) {
+  const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= static_cast<uint64_t>(rows) * sh.n_slabs) return;
+  const uint32_t n = counts[i];
+  if (!n) return;
+  const uint32_t r = static_cast<uint32_t>(i / sh.n_slabs), c = static_cast<uint32_t>(i % sh.n_slabs);
+  const uint32_t b = off[r], deg = off[r + 1] - b;
+  const uint32_t per = sh.n_slabs / sh.ranges_for(deg);
+  const uint32_t lo = c ? stops[i - 1] : b, hi = stops[i];
+  const uint32_t first = slot_base[i];
+  for (uint32_t j = 0; j < n; ++j) {
+    const uint32_t e0 = lo + j * sh.chunk, e1 = min(hi, e0 + sh.chunk);
+    pieces[first + j] = make_uint4(r, e0, e1, first + j);
+    keys[first + j] = c * per * (sh.chunk + 1) + (sh.chunk - (e1 - e0));
+  }
+}
+
+__global__ __launch_bounds__(256) void plan_row_keys_kernel(uint32_t *__restrict__ whole_key,
+                                                            uint32_t *__restrict__ split_key,
+                                                            const uint32_t *__restrict__ slot_base,
+                                                            const uint32_t *__restrict__ off, uint32_t rows,
+                                                            PlanShape sh, PlanCounters *__restrict__ counters) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  uint32_t split = 0;
+  if (r < rows) {
+    const uint32_t P = slot_base[static_cast<size_t>(r + 1) * sh.n_slabs] - slot_base[static_cast<size_t>(r) * sh.n_slabs];
+    const uint32_t deg = off[r + 1] - off[r];
+    whole_key[r] = P == 0 ? sh.chunk - deg : sh.chunk + 1;  // whole rows by descending length, cut rows last
+    split_key[r] = ~P;                                      // split rows by descending slot count, whole rows last
+    split = P ? 1u : 0u;
+  }
+  const uint32_t n = __popcll(__ballot(split));
+  if ((threadIdx.x & (kWave - 1)) == 0 && n) atomicAdd(&counters->n_splits, n);
+}
+
+__global__ __launch_bounds__(256) void plan_finish_kernel(Item *__restrict__ items, uint4 *__restrict__ splits,
+                                                          const uint32_t *__restrict__ whole_order,
+                                                          const uint32_t *__restrict__ split_order,
+                                                          const uint32_t *__restrict__ slot_base,
+                                                          const uint32_t *__restrict__ off, uint32_t n_pieces,
+                                                          uint32_t n_whole, uint32_t n_splits, uint32_t n_slabs) {
+  const uint32_t j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j < n_whole) {
+    const uint32_t r = whole_order[j];
+    items[n_pieces + j] = make_uint4(r, off[r], off[r + 1], kNoSlot);
+  }
+  if (j < n_splits) {
+    const uint32_t r = split_order[j];
+    const uint32_t first = slot_base[static_cast<size_t>(r) * n_slabs];
+    splits[j] = make_uint4(r, first, slot_base[static_cast<size_t>(r + 1) * n_slabs] - first, 0u);
+  }
+}
+
+__global__ __launch_bounds__(256) void plan_scan_edges_kernel(const uint32_t *__restrict__ idx, uint32_t edges,
+                                                              uint32_t *__restrict__ descents, uint32_t descent_cap,
+                                                              PlanCounters *__restrict__ counters) {
+  unsigned long long equal = 0;
+  for (uint64_t k = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x + 1; k < edges;
+       k += static_cast<uint64_t>(gridDim.x) * blockDim.x) {
+    const uint32_t a = idx[k - 1], b = idx[k];
+    equal += a == b ? 1u : 0u;
+    if (a > b) {
+      const uint32_t at = atomicAdd(&counters->n_descents, 1u);  // list order does not matter
+      if (at < descent_cap) descents[at] = static_cast<uint32_t>(k); else counters->descent_overflow = 1u;
+    }
+  }
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) equal += __shfl_xor(equal, m, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0 && equal) atomicAdd(&counters->repeated_raw, equal);
+}
+
+__global__ __launch_bounds__(256) void plan_row_starts_kernel(const uint32_t *__restrict__ off,
+                                                              const uint32_t *__restrict__ idx, uint32_t rows,
+                                                              uint32_t edges, PlanCounters *__restrict__ counters) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x + 1;
+  uint32_t hit = 0;
+  if (r < rows) {
+    const uint32_t p = off[r];
+    // every edge position that starts a row is met once: at the first row that starts there
+    hit = (off[r - 1] < p && p < edges && idx[p] == idx[p - 1]) ? 1u : 0u;
+  }
+  const uint32_t n = __popcll(__ballot(hit));
+  if ((threadIdx.x & (kWave - 1)) == 0 && n) atomicAdd(&counters->boundary_equal, n);
+}
+
+__global__ __launch_bounds__(256) void plan_check_descents_kernel(const uint32_t *__restrict__ descents,
+                                                                  const uint32_t *__restrict__ off, uint32_t rows,
+                                                                  uint32_t cut_above, uint32_t descent_cap,
+                                                                  PlanCounters *__restrict__ counters) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t n = min(counters->n_descents, descent_cap);
+  if (i >= n) return;
+  const uint32_t k = descents[i];
+  const uint32_t r = owner_of(off, rows, k);
+  if (k != off[r] && off[r + 1] - off[r] > cut_above) counters->unsorted_long_row = 1u;
+}
+
 int check_common(const float *in, float *out, const uint32_t *offsets, const uint32_t *indices, uint32_t rows,
                  uint32_t edges, uint32_t F, const char *who) {
   if (F == 0) return fail(NTS_ERR_INVALID, "spmm: feature width F is 0");
@@ -1308,6 +1484,154 @@ int build_plan(nts_spmm_plan_t **plan_out, const uint32_t *offsets_dev, const st
   return NTS_OK;
 }
 
+// Builds the schedule of make_schedule on the device (kernels above).  *fell_back is set, and nothing
+// built, when a row that would be cut does not ascend (the host path sorts such rows in a copy).
+int build_plan_device(nts_spmm_plan_t **plan_out, const uint32_t *offsets, const uint32_t *indices,
+                      uint32_t index_base, uint32_t n_index, uint32_t rows, uint32_t edges, uint32_t chunk,
+                      uint32_t n_slabs, hipStream_t stream, bool *fell_back) {
+  using nts::Item;
+  *fell_back = false;
+  nts::PlanShape sh;
+  sh.chunk = chunk;
+  sh.n_slabs = n_slabs;
+  sh.wide_ranges = n_slabs >= 8 ? n_slabs / 4 : 0;
+  sh.fine_width = (static_cast<uint64_t>(n_index) + n_slabs - 1) / n_slabs;
+  const size_t cells = static_cast<size_t>(rows) * n_slabs;
+  const uint32_t descent_cap = rows + 1;
+  unsigned key_bits = 1;
+  while ((1ull << key_bits) < static_cast<uint64_t>(n_slabs) * (chunk + 1)) ++key_bits;
+  unsigned whole_bits = 1;
+  while ((1ull << whole_bits) < static_cast<uint64_t>(chunk) + 2) ++whole_bits;
+
+  size_t scan_bytes = 0, sort_rows_bytes = 0;
+  uint32_t *nul = nullptr;
+  NTS_HIP_TRY(rocprim::exclusive_scan(nullptr, scan_bytes, nul, nul, 0u, cells + 1, rocprim::plus<uint32_t>(), stream,
+                                      false));
+  NTS_HIP_TRY(rocprim::radix_sort_pairs(nullptr, sort_rows_bytes, nul, nul, rocprim::counting_iterator<uint32_t>(0u), nul,
+                                        rows, 0u, 32u, stream, false));
+  const size_t tmp1_bytes = nts::up256(std::max(scan_bytes, sort_rows_bytes));
+  const size_t cell_words = nts::up256((cells + 1) * sizeof(uint32_t));
+  const size_t row_words = nts::up256((static_cast<size_t>(rows) + 1) * sizeof(uint32_t));
+  struct Block {  // freed on every path out
+    unsigned char *p = nullptr;
+    ~Block() {
+      if (p) (void)hipFree(p);
+    }
+  } work, work2;
+  NTS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&work.p), 3 * cell_words + 7 * row_words + 256 + tmp1_bytes));
+  unsigned char *cursor = work.p;
+  auto take = [&cursor](size_t bytes) {
+    unsigned char *q = cursor;
+    cursor += bytes;
+    return q;
+  };
+  uint32_t *counts = reinterpret_cast<uint32_t *>(take(cell_words));
+  uint32_t *stops = reinterpret_cast<uint32_t *>(take(cell_words));
+  uint32_t *slot_base = reinterpret_cast<uint32_t *>(take(cell_words));
+  uint32_t *whole_key = reinterpret_cast<uint32_t *>(take(row_words));
+  uint32_t *split_key = reinterpret_cast<uint32_t *>(take(row_words));
+  uint32_t *key_sorted = reinterpret_cast<uint32_t *>(take(row_words));
+  uint32_t *whole_order = reinterpret_cast<uint32_t *>(take(row_words));
+  uint32_t *split_order = reinterpret_cast<uint32_t *>(take(row_words));
+  uint32_t *descents = reinterpret_cast<uint32_t *>(take(2 * row_words));
+  nts::PlanCounters *counters = reinterpret_cast<nts::PlanCounters *>(take(256));
+  void *tmp1 = take(tmp1_bytes);
+
+  NTS_HIP_TRY(hipMemsetAsync(counts, 0, (cells + 1) * sizeof(uint32_t), stream));
+  NTS_HIP_TRY(hipMemsetAsync(counters, 0, sizeof(nts::PlanCounters), stream));
+  const uint32_t row_blocks = nts::ceil_div(static_cast<uint64_t>(rows) + 1, 256);
+  if (edges > 1) {
+    const uint32_t edge_blocks = static_cast<uint32_t>(std::min<uint64_t>((static_cast<uint64_t>(edges) + 255) / 256, 1u << 14));
+    hipLaunchKernelGGL(nts::plan_scan_edges_kernel, dim3(edge_blocks), dim3(256), 0, stream, indices, edges, descents,
+                       descent_cap, counters);
+    hipLaunchKernelGGL(nts::plan_row_starts_kernel, dim3(row_blocks), dim3(256), 0, stream, offsets, indices, rows, edges,
+                       counters);
+    hipLaunchKernelGGL(nts::plan_check_descents_kernel, dim3(row_blocks), dim3(256), 0, stream, descents, offsets, rows,
+                       sh.wide_ranges ? chunk / 4 : chunk, descent_cap, counters);
+  }
+  hipLaunchKernelGGL(nts::plan_cut_rows_kernel, dim3(row_blocks), dim3(256), 0, stream, counts, stops, offsets, indices,
+                     index_base, rows, sh);
+  NTS_LAUNCH_CHECK("plan_cut_rows_kernel");
+  NTS_HIP_TRY(rocprim::exclusive_scan(tmp1, scan_bytes, counts, slot_base, 0u, cells + 1, rocprim::plus<uint32_t>(),
+                                      stream, false));
+  hipLaunchKernelGGL(nts::plan_row_keys_kernel, dim3(row_blocks), dim3(256), 0, stream, whole_key, split_key, slot_base,
+                     offsets, rows, sh, counters);
+  NTS_LAUNCH_CHECK("plan_row_keys_kernel");
+  nts::PlanCounters host_counters;
+  uint32_t n_pieces = 0;
+  NTS_HIP_TRY(hipMemcpyAsync(&host_counters, counters, sizeof(host_counters), hipMemcpyDeviceToHost, stream));
+  NTS_HIP_TRY(hipMemcpyAsync(&n_pieces, slot_base + cells, sizeof(n_pieces), hipMemcpyDeviceToHost, stream));
+  NTS_HIP_TRY(hipStreamSynchronize(stream));
+  if (host_counters.unsorted_long_row || host_counters.descent_overflow) {
+    *fell_back = true;
+    return NTS_OK;
+  }
+  const uint32_t n_splits = host_counters.n_splits, n_whole = rows - n_splits;
+  const uint64_t n_items64 = static_cast<uint64_t>(n_pieces) + n_whole;
+  if (n_items64 > 0xFFFFFFF0ull) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create_slabs: too many work items");
+
+  nts_spmm_plan *p = new (std::nothrow) nts_spmm_plan();
+  if (!p) return nts::fail(NTS_ERR_NOMEM, "nts_spmm_plan_create_slabs: host allocation failed");
+  p->rows = rows;
+  p->edges = edges;
+  p->chunk = chunk;
+  p->offsets = offsets;
+  p->n_items = static_cast<uint32_t>(n_items64);
+  p->n_splits = n_splits;
+  p->n_partials = n_pieces;
+  p->n_index = n_index;
+  p->repeated_edges = host_counters.repeated_raw - host_counters.boundary_equal;
+  p->dup_runs = edges > 0 && p->repeated_edges * 20 >= edges;
+  auto bail = [&](hipError_t err, const char *what) {
+    nts_spmm_plan_destroy(p);
+    return nts::fail_hip(err, what);
+  };
+  hipError_t err = hipEventCreateWithFlags(&p->done, hipEventDisableTiming);
+  if (err == hipSuccess && p->n_items) err = hipMalloc(reinterpret_cast<void **>(&p->items), p->n_items * sizeof(uint4));
+  if (err == hipSuccess && n_splits) err = hipMalloc(reinterpret_cast<void **>(&p->splits), n_splits * sizeof(uint4));
+  if (err != hipSuccess) return bail(err, "nts_spmm_plan_create_slabs: device allocation");
+
+  if (n_pieces) {
+    size_t sort_pieces_bytes = 0;
+    err = rocprim::radix_sort_pairs(nullptr, sort_pieces_bytes, nul, nul, rocprim::counting_iterator<uint32_t>(0u), nul,
+                                    n_pieces, 0u, key_bits, stream, false);
+    if (err != hipSuccess) return bail(err, "nts_spmm_plan_create_slabs: sort size");
+    const size_t piece_items = nts::up256(static_cast<size_t>(n_pieces) * sizeof(Item));
+    const size_t piece_words = nts::up256(static_cast<size_t>(n_pieces) * sizeof(uint32_t));
+    err = hipMalloc(reinterpret_cast<void **>(&work2.p), piece_items + 3 * piece_words + nts::up256(sort_pieces_bytes));
+    if (err != hipSuccess) return bail(err, "nts_spmm_plan_create_slabs: device allocation");
+    Item *pieces = reinterpret_cast<Item *>(work2.p);
+    uint32_t *keys = reinterpret_cast<uint32_t *>(work2.p + piece_items);
+    uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(work2.p + piece_items + piece_words);
+    uint32_t *order = reinterpret_cast<uint32_t *>(work2.p + piece_items + 2 * piece_words);
+    void *tmp2 = work2.p + piece_items + 3 * piece_words;
+    hipLaunchKernelGGL(nts::plan_emit_pieces_kernel, dim3(nts::ceil_div(cells, 256)), dim3(256), 0, stream, pieces, keys,
+                       counts, stops, slot_base, offsets, rows, sh);
+    err = hipGetLastError();
+    if (err == hipSuccess)
+      err = rocprim::radix_sort_pairs(tmp2, sort_pieces_bytes, keys, keys_sorted, rocprim::counting_iterator<uint32_t>(0u),
+                                      order, n_pieces, 0u, key_bits, stream, false);
+    if (err != hipSuccess) return bail(err, "nts_spmm_plan_create_slabs: ordering of the pieces");
+    hipLaunchKernelGGL(nts::auto_order_items_kernel, dim3(nts::ceil_div(n_pieces, 256)), dim3(256), 0, stream, p->items,
+                       pieces, order, n_pieces);
+  }
+  err = rocprim::radix_sort_pairs(tmp1, sort_rows_bytes, whole_key, key_sorted, rocprim::counting_iterator<uint32_t>(0u),
+                                  whole_order, rows, 0u, whole_bits, stream, false);
+  if (err == hipSuccess)
+    err = rocprim::radix_sort_pairs(tmp1, sort_rows_bytes, split_key, key_sorted, rocprim::counting_iterator<uint32_t>(0u),
+                                    split_order, rows, 0u, 32u, stream, false);
+  if (err != hipSuccess) return bail(err, "nts_spmm_plan_create_slabs: ordering of the rows");
+  if (n_whole || n_splits)
+    hipLaunchKernelGGL(nts::plan_finish_kernel, dim3(nts::ceil_div(std::max(n_whole, n_splits), 256)), dim3(256), 0, stream,
+                       p->items, p->splits, whole_order, split_order, slot_base, offsets, n_pieces, n_whole, n_splits,
+                       n_slabs);
+  err = hipGetLastError();
+  if (err == hipSuccess) err = hipStreamSynchronize(stream);
+  if (err != hipSuccess) return bail(err, "nts_spmm_plan_create_slabs: device schedule");
+  *plan_out = p;
+  return NTS_OK;
+}
+
 int read_offsets(std::vector<uint32_t> &off, const uint32_t *offsets, uint32_t rows, uint32_t edges,
                  hipStream_t stream) {
   off.assign(static_cast<size_t>(rows) + 1, 0u);
@@ -1343,6 +1667,22 @@ int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan_out, const uint32_t *offse
   if (edges != 0 && !indices) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_create_slabs: null indices");
   std::vector<uint32_t> off;
   if (int rc = read_offsets(off, offsets, rows, edges, stream)) return rc;
+  const uint32_t chunk = chunk_edges ? chunk_edges : 512u, slabs = n_slabs ? n_slabs : 32u;
+  // The schedule is built on the device where that reproduces the host's (source ranges in use, sizes
+  // within the 32-bit sort keys and the range table); NTS_SPMM_PLAN_HOST=1 forces the host path.
+  static const bool force_host = [] {
+    const char *e = getenv("NTS_SPMM_PLAN_HOST");
+    return e && e[0] != '0';
+  }();
+  if (!force_host && slabs > 1 && n_index > 0 && rows > 0 && edges > 0 &&
+      static_cast<uint64_t>(slabs) * (static_cast<uint64_t>(chunk) + 1) < (1ull << 32) && slabs <= 4096 &&
+      static_cast<uint64_t>(rows) * slabs < (1ull << 31)) {
+    bool fell_back = false;
+    if (int rc = build_plan_device(plan_out, offsets, indices, index_base, n_index, rows, edges, chunk, slabs, stream,
+                                   &fell_back))
+      return rc;
+    if (!fell_back) return NTS_OK;
+  }
   std::vector<uint32_t> idx(edges);
   if (edges) {
     NTS_HIP_TRY(hipMemcpyAsync(idx.data(), indices, idx.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
@@ -1350,8 +1690,7 @@ int nts_spmm_plan_create_slabs(nts_spmm_plan_t **plan_out, const uint32_t *offse
     if (index_base)
       for (uint32_t &v : idx) v -= index_base;
   }
-  return build_plan(plan_out, offsets, off, idx.data(), rows, edges, chunk_edges ? chunk_edges : 512u,
-                    n_slabs ? n_slabs : 32u, n_index);
+  return build_plan(plan_out, offsets, off, idx.data(), rows, edges, chunk, slabs, n_index);
 }
 
 int nts_spmm_plan_schedule_host(const uint32_t *offsets_host, const uint32_t *indices_host, uint32_t n_index,
@@ -1393,6 +1732,24 @@ int nts_spmm_plan_destroy(nts_spmm_plan_t *plan) {
   if (e1 != hipSuccess) return nts::fail_hip(e1, "nts_spmm_plan_destroy");
   if (e2 != hipSuccess) return nts::fail_hip(e2, "nts_spmm_plan_destroy");
   if (e3 != hipSuccess) return nts::fail_hip(e3, "nts_spmm_plan_destroy");
+  return NTS_OK;
+}
+
+int nts_spmm_plan_copy_schedule(const nts_spmm_plan_t *plan, uint32_t *items_out, uint64_t items_cap,
+                                uint32_t *splits_out, uint64_t splits_cap) {
+  NTS_TRACE_RANGE("nts_spmm_plan_copy_schedule");
+  if (!plan) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_copy_schedule: null plan");
+  if (items_out) {
+    if (items_cap < plan->n_items) return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_copy_schedule: items_out too small");
+    if (plan->n_items)
+      NTS_HIP_TRY(hipMemcpy(items_out, plan->items, plan->n_items * sizeof(uint4), hipMemcpyDeviceToHost));
+  }
+  if (splits_out) {
+    if (splits_cap < plan->n_splits)
+      return nts::fail(NTS_ERR_INVALID, "nts_spmm_plan_copy_schedule: splits_out too small");
+    if (plan->n_splits)
+      NTS_HIP_TRY(hipMemcpy(splits_out, plan->splits, plan->n_splits * sizeof(uint4), hipMemcpyDeviceToHost));
+  }
   return NTS_OK;
 }
 
