@@ -48,9 +48,12 @@ SIGNATURES = {
     "nts_device_sync": [],
     "nts_mem_info": [ctypes.POINTER(_sz), ctypes.POINTER(_sz)],
     "nts_fingerprint_u32": [ctypes.POINTER(_u64), _vp, _u64, _vp, _u64, _vp],
+    "nts_fingerprint_u32_async": [_vp, _vp, _u64, _vp, _u64, _vp],
+    "nts_fingerprint_finish": [_u64, _u64, _u64],
     "nts_event_create": [ctypes.POINTER(_vp)],
     "nts_event_destroy": [_vp],
     "nts_event_record": [_vp, _vp],
+    "nts_stream_wait_event": [_vp, _vp],
     "nts_event_elapsed_ms": [ctypes.POINTER(_f32), _vp, _vp],
     "nts_spmm_plan_set_events": [_vp, _vp, _vp],
     "nts_spmm_gather": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
@@ -113,12 +116,12 @@ SIGNATURES = {
     "nts_table_bin_info": [_str, ctypes.POINTER(_u64), ctypes.POINTER(_u64), ctypes.POINTER(_u32)],
     "nts_table_bin_read": [_str, _vp, _u64, _u64],
 }
-_RESTYPES = {"nts_last_error": ctypes.c_char_p, "nts_csr_from_csc_work_bytes": _sz,
+_RESTYPES = {"nts_last_error": ctypes.c_char_p, "nts_fingerprint_finish": _u64, "nts_csr_from_csc_work_bytes": _sz,
              "nts_relabel_sources_work_bytes": _sz, "nts_sample_hop_work_bytes": _sz,
              "nts_chunk_from_edges_work_bytes": _sz, "nts_batch_builder_arena_bytes": _sz,
              "nts_trace_ranges_emitted": ctypes.c_long}
 # Entry points whose int result is a value, not a status.
-_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_trace_ranges_emitted", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
+_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_fingerprint_finish", "nts_trace_ranges_emitted", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
               "nts_sample_hop_work_bytes", "nts_chunk_from_edges_work_bytes", "nts_batch_builder_arena_bytes"}
 
 

@@ -39,23 +39,49 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned char *p, size_t
   if (tid < tail) p[head + body16 * 16 + tid] = 0;
 }
 
-// Position-dependent 64-bit checksum of a uint32 array: the sum over i of a 64-bit mix of
-// (value, salt + i).  A sum, so that blocks can add their shares in any order (integer atomics).
-__device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
-  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-  return z ^ (z >> 31);
+// Position-dependent 64-bit checksum of a uint32 array: the sum over i of (a[i] + c) * k(salt + i) in
+// 64 bits, k an odd 32-bit word hashed from the position -- one 32 x 32 -> 64 multiply-add per element,
+// so the kernel runs at the rate the array can be read.  An element that changes changes the sum (an odd
+// multiplier times a non-zero 32-bit difference is never 0 mod 2^64); elements that move change it unless
+// their multipliers collide.  A sum, so that blocks can add their shares in any order (integer atomics).
+__device__ __forceinline__ unsigned long long checksum_term(uint32_t v, unsigned long long pos) {
+  uint32_t k = static_cast<uint32_t>(pos) * 0x9E3779B1u + static_cast<uint32_t>(pos >> 32) * 0x85EBCA77u;
+  k ^= k >> 15;
+  k *= 0x2C1B3C6Du;
+  k ^= k >> 12;
+  return static_cast<unsigned long long>(v + 0x632BE5ABu) * (k | 1u);
 }
+
 __global__ __launch_bounds__(256) void fingerprint_kernel(unsigned long long *__restrict__ out,
                                                           const uint32_t *__restrict__ a, unsigned long long n,
                                                           unsigned long long salt) {
   unsigned long long acc = 0;
+  const unsigned long long tid = static_cast<unsigned long long>(blockIdx.x) * blockDim.x + threadIdx.x;
   const unsigned long long stride = static_cast<unsigned long long>(gridDim.x) * blockDim.x;
-  for (unsigned long long i = static_cast<unsigned long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
-    acc += mix64((static_cast<unsigned long long>(a[i]) << 32) ^ ((salt + i) * 0x9E3779B97F4A7C15ull));
+  // elements before the first 16-byte boundary, then 16-byte loads, then the rest
+  unsigned long long head = ((16 - (reinterpret_cast<uintptr_t>(a) & 15)) & 15) / 4;
+  if (head > n) head = n;
+  const unsigned long long quads = (n - head) / 4;
+  const uint4 *body = reinterpret_cast<const uint4 *>(a + head);
+  for (unsigned long long q = tid; q < quads; q += stride) {
+    const uint4 v = body[q];
+    const unsigned long long at = salt + head + 4 * q;
+    acc += checksum_term(v.x, at) + checksum_term(v.y, at + 1) + checksum_term(v.z, at + 2) + checksum_term(v.w, at + 3);
+  }
+  if (tid < head) acc += checksum_term(a[tid], salt + tid);
+  const unsigned long long tail0 = head + 4 * quads;
+  if (tid < n - tail0) acc += checksum_term(a[tail0 + tid], salt + tail0 + tid);
 #pragma unroll
   for (int m = kWave / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, kWave);
-  if ((threadIdx.x & (kWave - 1)) == 0 && acc) atomicAdd(out, acc);
+  // one atomic per block: thousands of atomics on one word would take longer than reading the array
+  __shared__ unsigned long long wave_sum[256 / kWave];
+  if ((threadIdx.x & (kWave - 1)) == 0) wave_sum[threadIdx.x / kWave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long total = 0;
+    for (int k = 0; k < 256 / kWave; ++k) total += wave_sum[k];
+    if (total) atomicAdd(out, total);
+  }
 }
 
 }  // namespace
@@ -251,23 +277,36 @@ int nts_memset_zero(void *dev_ptr, size_t bytes, nts_stream_t stream) {
   return NTS_OK;
 }
 
+namespace {
+// Enqueues the checksum kernels for (a, b) on `stream`, accumulating into the zeroed device word `word`.
+int enqueue_fingerprint(unsigned long long *word, const uint32_t *a, uint64_t n_a, const uint32_t *b, uint64_t n_b,
+                        hipStream_t stream) {
+  if (int rc = nts_memset_zero(word, 16, stream)) return rc;
+  const uint64_t lens[2] = {n_a, n_b};
+  const uint32_t *arrays[2] = {a, b};
+  for (int k = 0; k < 2; ++k) {
+    if (!lens[k]) continue;
+    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((lens[k] / 4 + 255) / 256 + 1, 2048));
+    hipLaunchKernelGGL(nts::fingerprint_kernel, dim3(blocks), dim3(256), 0, stream, word, arrays[k],
+                       static_cast<unsigned long long>(lens[k]), k ? 0x5851F42D4C957F2Dull + n_a : 0ull);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return nts::fail_hip(err, "fingerprint_kernel");
+  }
+  return NTS_OK;
+}
+// lengths are part of the value, so that a prefix of an array does not collide with the array
+inline uint64_t fingerprint_value(uint64_t sum, uint64_t n_a, uint64_t n_b) {
+  return sum ^ (n_a * 0xD6E8FEB86659FD93ull) ^ (n_b * 0xA0761D6478BD642Full);
+}
+}  // namespace
+
 int nts_fingerprint_u32(uint64_t *fingerprint, const uint32_t *a, uint64_t n_a, const uint32_t *b, uint64_t n_b,
                         nts_stream_t stream) {
   if (!fingerprint) return fail(NTS_ERR_INVALID, "nts_fingerprint_u32: null out-pointer");
   if ((n_a && !a) || (n_b && !b)) return fail(NTS_ERR_INVALID, "nts_fingerprint_u32: null array");
   unsigned long long *word = nullptr;
   NTS_HIP_TRY(nts::scratch_alloc(reinterpret_cast<void **>(&word), 16, stream));
-  int rc = nts_memset_zero(word, 16, stream);
-  const uint64_t lens[2] = {n_a, n_b};
-  const uint32_t *arrays[2] = {a, b};
-  for (int k = 0; k < 2 && rc == NTS_OK; ++k) {
-    if (!lens[k]) continue;
-    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((lens[k] + 255) / 256, 8192));
-    hipLaunchKernelGGL(nts::fingerprint_kernel, dim3(blocks), dim3(256), 0, stream, word, arrays[k],
-                       static_cast<unsigned long long>(lens[k]), k ? 0x5851F42D4C957F2Dull + n_a : 0ull);
-    const hipError_t err = hipGetLastError();
-    if (err != hipSuccess) rc = nts::fail_hip(err, "fingerprint_kernel");
-  }
+  int rc = enqueue_fingerprint(word, a, n_a, b, n_b, stream);
   unsigned long long host = 0;
   if (rc == NTS_OK) {
     hipError_t err = hipMemcpyAsync(&host, word, sizeof(host), hipMemcpyDeviceToHost, stream);
@@ -276,10 +315,27 @@ int nts_fingerprint_u32(uint64_t *fingerprint, const uint32_t *a, uint64_t n_a, 
   }
   const hipError_t ferr = nts::scratch_free(word, stream);
   if (rc == NTS_OK && ferr != hipSuccess) rc = nts::fail_hip(ferr, "nts_fingerprint_u32: scratch_free");
-  // lengths are part of the value, so that a prefix of an array does not collide with the array
-  *fingerprint = host ^ (n_a * 0xD6E8FEB86659FD93ull) ^ (n_b * 0xA0761D6478BD642Full);
+  *fingerprint = fingerprint_value(host, n_a, n_b);
   return rc;
 }
+
+int nts_fingerprint_u32_async(uint64_t *pinned_sum, const uint32_t *a, uint64_t n_a, const uint32_t *b, uint64_t n_b,
+                              nts_stream_t stream) {
+  if (!pinned_sum) return fail(NTS_ERR_INVALID, "nts_fingerprint_u32_async: null out-pointer");
+  if ((n_a && !a) || (n_b && !b)) return fail(NTS_ERR_INVALID, "nts_fingerprint_u32_async: null array");
+  unsigned long long *word = nullptr;
+  NTS_HIP_TRY(nts::scratch_alloc(reinterpret_cast<void **>(&word), 16, stream));
+  int rc = enqueue_fingerprint(word, a, n_a, b, n_b, stream);
+  if (rc == NTS_OK) {
+    const hipError_t err = hipMemcpyAsync(pinned_sum, word, sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
+    if (err != hipSuccess) rc = nts::fail_hip(err, "nts_fingerprint_u32_async: read-back");
+  }
+  const hipError_t ferr = nts::scratch_free(word, stream);
+  if (rc == NTS_OK && ferr != hipSuccess) rc = nts::fail_hip(ferr, "nts_fingerprint_u32_async: scratch_free");
+  return rc;
+}
+
+uint64_t nts_fingerprint_finish(uint64_t sum, uint64_t n_a, uint64_t n_b) { return fingerprint_value(sum, n_a, n_b); }
 
 int nts_stream_create(nts_stream_t *stream) {
   if (!stream) return fail(NTS_ERR_INVALID, "nts_stream_create: null out-pointer");
@@ -318,6 +374,12 @@ int nts_event_destroy(nts_event_t event) {
 int nts_event_record(nts_event_t event, nts_stream_t stream) {
   if (!event) return fail(NTS_ERR_INVALID, "nts_event_record: null event");
   NTS_HIP_TRY(hipEventRecord(event, stream));
+  return NTS_OK;
+}
+
+int nts_stream_wait_event(nts_stream_t stream, nts_event_t event) {
+  if (!event) return fail(NTS_ERR_INVALID, "nts_stream_wait_event: null event");
+  NTS_HIP_TRY(hipStreamWaitEvent(stream, event, 0));
   return NTS_OK;
 }
 

@@ -83,7 +83,23 @@ struct State {
   long plans_built = 0;
   long planned_calls = 0;
   long plans_dropped_by_checksum = 0;
+  long deferred_checks = 0;
   int enabled = -1;
+  // A checksum taken on a side stream while the scheduled aggregation it guards runs (see plan_for):
+  // at most one is outstanding; it is settled at the next call through this header.
+  nts_stream_t verify_stream = NULL;
+  nts_event_t verify_fork = NULL;
+  uint64_t *pinned_sum = NULL;
+  int async_verify = -1;
+  struct Pending {
+    bool active;
+    uintptr_t key;
+    const float *input, *weight;
+    float *output;
+    const uint32_t *offsets, *indices;
+    uint32_t index_base, rows, edges, F;
+    nts_stream_t stream;
+  } pending = {false, 0, NULL, NULL, NULL, NULL, NULL, 0, 0, 0, 0, NULL};
 };
 inline State &state() {
   static State s;
@@ -91,6 +107,42 @@ inline State &state() {
 }
 const uint32_t kPlanMinEdges = 1u << 22;
 
+// The buffer this host thread cleared last through zero_buffer, until anything else is written through
+// this header: the reference clears an output and then aggregates into it (Nts->ZeroVarMem + GatherBy*,
+// core/graph.hpp:3443-3445, 3469-3471); an aggregation that finds its output in this record writes the
+// sums instead of adding them to the zeros -- the same values, without reading the output back.  Only
+// writes made through this header are seen: a caller that clears a buffer here, fills it by other means
+// and then aggregates into it must switch this off (NTS_VENEER_ZERO_TRACKING=0 in the environment).
+struct ZeroRecord {
+  const void *ptr;
+  size_t floats;
+};
+inline ZeroRecord &zero_record() {
+  static thread_local ZeroRecord r = {NULL, 0};
+  return r;
+}
+inline bool zero_tracking_enabled() {
+  static const int on = [] {
+    const char *e = getenv("NTS_VENEER_ZERO_TRACKING");
+    return (e && e[0] == '0') ? 0 : 1;
+  }();
+  return on != 0;
+}
+inline void note_zeroed(const void *p, size_t floats) {
+  ZeroRecord &r = zero_record();
+  r.ptr = p;
+  r.floats = floats;
+}
+// True when `p` is exactly the buffer cleared last and `floats` of it are still known to be zero.
+inline bool take_zeroed(const void *p, size_t floats) {
+  ZeroRecord &r = zero_record();
+  const bool hit = zero_tracking_enabled() && r.ptr != NULL && r.ptr == p && floats <= r.floats;
+  r.ptr = NULL;
+  r.floats = 0;
+  return hit;
+}
+
+inline void settle_pending_locked(State &st);
 inline std::map<uintptr_t, Region>::iterator region_of(State &st, const void *p) {
   const uintptr_t a = (uintptr_t)p;
   std::map<uintptr_t, Region>::iterator it = st.regions.upper_bound(a);
@@ -120,25 +172,67 @@ inline void note_free(void *p) {
   if (!p) return;
   State &st = state();
   std::lock_guard<std::mutex> lock(st.mu);
+  settle_pending_locked(st);
   std::map<uintptr_t, Region>::iterator it = st.regions.find((uintptr_t)p);
   if (it == st.regions.end()) return;
   drop_plans_touching(st, it->first, it->second.bytes);
   st.regions.erase(it);
 }
+// Settles the outstanding side-stream checksum, if any: waits for it, and when the arrays no longer
+// hold what the schedule was built from, drops the schedule and computes the aggregation again without
+// one (the output had been cleared before the call, so it is cleared again and rewritten).  Caller
+// holds st.mu.  Every entry of this header that writes, synchronises or copies results out comes
+// through here first, so a result computed with a stale schedule never leaves this header.
+inline void settle_pending_locked(State &st) {
+  if (!st.pending.active) return;
+  State::Pending p = st.pending;
+  st.pending.active = false;
+  bool stale = nts_stream_sync(st.verify_stream) != NTS_OK;
+  std::map<uintptr_t, CachedPlan>::iterator it = st.plans.find(p.key);
+  if (!stale && it != st.plans.end() && it->second.plan)
+    stale = nts_fingerprint_finish(*st.pinned_sum, (uint64_t)p.rows + 1, p.edges) != it->second.fingerprint;
+  if (!stale) return;
+  if (it != st.plans.end() && it->second.plan) {
+    nts_stream_sync(p.stream);  // the call that used the schedule has finished before the schedule goes
+    nts_spmm_plan_destroy(it->second.plan);
+    it->second.plan = NULL;
+    it->second.seen = 1;
+  }
+  ++st.plans_dropped_by_checksum;
+  --st.planned_calls;  // the call is not one that a schedule served
+  if (nts_spmm_gather(p.input, p.output, p.weight, p.offsets, p.indices, p.index_base, p.rows, p.edges, p.F, 0,
+                      p.stream) != NTS_OK) {
+    printf("HIP call while recomputing an aggregation returned an error: %s\n", nts_last_error());
+    exit(1);
+  }
+}
+inline void settle_pending() {
+  State &st = state();
+  std::lock_guard<std::mutex> lock(st.mu);
+  settle_pending_locked(st);
+}
 // A write into device memory at p (an upload, a zeroing, a kernel output).
 inline void note_write(const void *p) {
   if (!p) return;
+  zero_record().ptr = NULL;  // something was written through this header since the last zero_buffer
   State &st = state();
   std::lock_guard<std::mutex> lock(st.mu);
+  settle_pending_locked(st);
   std::map<uintptr_t, Region>::iterator it = region_of(st, p);
   if (it != st.regions.end()) it->second.generation = st.clock++;
 }
 // The schedule for this (offsets, indices) pair if the structure has proved static, else NULL.
+// may_defer: the caller's output is known to be all zeros, so the call can be computed again if needed;
+// then the checksum runs on a side stream next to the aggregation and *deferred is set -- the caller
+// registers the call with defer_check once it is enqueued.
 inline nts_spmm_plan_t *plan_for(const uint32_t *offsets, const uint32_t *indices, uint32_t index_base,
-                                 uint32_t n_index, uint32_t rows, uint32_t edges, nts_stream_t stream) {
+                                 uint32_t n_index, uint32_t rows, uint32_t edges, nts_stream_t stream,
+                                 bool may_defer = false, bool *deferred = NULL) {
+  if (deferred) *deferred = false;
   if (edges < kPlanMinEdges || n_index == 0) return NULL;
   State &st = state();
   std::lock_guard<std::mutex> lock(st.mu);
+  settle_pending_locked(st);
   if (st.enabled < 0) {
     const char *e = getenv("NTS_VENEER_PLAN_CACHE");
     st.enabled = (e && e[0] == '0') ? 0 : 1;
@@ -169,6 +263,24 @@ inline nts_spmm_plan_t *plan_for(const uint32_t *offsets, const uint32_t *indice
     }
     ++st.plans_built;
   }
+  if (may_defer && deferred) {
+    if (st.async_verify < 0) {
+      const char *e = getenv("NTS_VENEER_ASYNC_VERIFY");
+      st.async_verify = (e && e[0] == '0') ? 0 : 1;
+      if (st.async_verify && (nts_stream_create(&st.verify_stream) != NTS_OK || nts_event_create(&st.verify_fork) != NTS_OK ||
+                              nts_malloc_pinned_mapped((void **)&st.pinned_sum, 64) != NTS_OK))
+        st.async_verify = 0;
+    }
+    // the side stream sees the arrays as the caller's stream has left them so far
+    if (st.async_verify && nts_event_record(st.verify_fork, stream) == NTS_OK &&
+        nts_stream_wait_event(st.verify_stream, st.verify_fork) == NTS_OK &&
+        nts_fingerprint_u32_async(st.pinned_sum, offsets, (uint64_t)rows + 1, indices, edges, st.verify_stream) == NTS_OK) {
+      *deferred = true;
+      ++st.planned_calls;
+      ++st.deferred_checks;
+      return c.plan;
+    }
+  }
   if (nts_fingerprint_u32(&now, offsets, (uint64_t)rows + 1, indices, edges, stream) != NTS_OK || now != c.fingerprint) {
     // the arrays were written behind this header's back: forget the schedule and start counting again
     nts_spmm_plan_destroy(c.plan);
@@ -180,6 +292,17 @@ inline nts_spmm_plan_t *plan_for(const uint32_t *offsets, const uint32_t *indice
   ++st.planned_calls;
   return c.plan;
 }
+// Registers the scheduled call that was just enqueued on `stream` with the side-stream checksum started
+// by plan_for: settled at the next entry of this header.
+inline void defer_check(const uint32_t *offsets, const uint32_t *indices, uint32_t index_base, uint32_t rows,
+                        uint32_t edges, uint32_t F, const float *input, float *output, const float *weight,
+                        nts_stream_t stream) {
+  State &st = state();
+  std::lock_guard<std::mutex> lock(st.mu);
+  State::Pending p = {true, (uintptr_t)offsets, input, weight, output, offsets, indices, index_base, rows, edges, F, stream};
+  st.pending = p;
+}
+inline long deferred_checks() { return state().deferred_checks; }
 inline long plans_built() { return state().plans_built; }
 inline long planned_calls() { return state().planned_calls; }
 inline long plans_dropped_by_checksum() { return state().plans_dropped_by_checksum; }
@@ -248,6 +371,7 @@ inline void allocate_gpu_edge_async(VertexId_CUDA **input, int size, cudaStream_
   nts_veneer::note_alloc(*input, sizeof(VertexId_CUDA) * (size_t)size);
 }
 inline void move_result_out(float *output, float *input, int src, int dst, int feature_size, bool sync = true) {
+  nts_veneer::settle_pending();
   NTS_VENEER_CHECK(nts_memcpy_d2h(output, input, (size_t)(dst - src) * feature_size * sizeof(float), sync));
 }
 inline void move_data_in(float *d_pointer, float *h_pointer, int start, int end, int feature_size, bool sync = true) {
@@ -272,8 +396,12 @@ inline void zero_buffer(float *buffer, int size) {
   nts_veneer::note_write(buffer);
   NTS_VENEER_CHECK(nts_memset_zero(buffer, sizeof(float) * (size_t)size, (cudaStream_t)0));
   NTS_VENEER_CHECK(nts_device_sync());
+  nts_veneer::note_zeroed(buffer, (size_t)size);
 }
-inline void CUDA_DEVICE_SYNCHRONIZE() { NTS_VENEER_CHECK(nts_device_sync()); }
+inline void CUDA_DEVICE_SYNCHRONIZE() {
+  nts_veneer::settle_pending();
+  NTS_VENEER_CHECK(nts_device_sync());
+}
 // The few raw runtime names that core/ and comm/ call outside cuda/ (core/ntsMiniBatchGraphOp.hpp:283,
 // core/coocsc.hpp:673-773, comm/network.cpp:53, 84).
 inline int cudaFree(void *p) {
@@ -281,7 +409,10 @@ inline int cudaFree(void *p) {
   return nts_free_device(p);
 }
 inline int cudaFreeHost(void *p) { return nts_free_pinned(p); }
-inline int cudaStreamSynchronize(cudaStream_t s) { return nts_stream_sync(s); }
+inline int cudaStreamSynchronize(cudaStream_t s) {
+  nts_veneer::settle_pending();
+  return nts_stream_sync(s);
+}
 
 // cudaMallocManaged as the data loader uses it (core/ntsDataloador.hpp:66-73): memory that both the
 // host and the device address.  Page-locked mapped host memory has that property; the device reads
@@ -354,11 +485,15 @@ class Cuda_Stream {
     destory_Stream();
     stream = cudaStream;
   }
-  void CUDA_DEVICE_SYNCHRONIZE() { NTS_VENEER_CHECK(nts_stream_sync(stream)); }
+  void CUDA_DEVICE_SYNCHRONIZE() {
+    nts_veneer::settle_pending();
+    NTS_VENEER_CHECK(nts_stream_sync(stream));
+  }
 
   void move_result_out(float *output, float *input, VertexId_CUDA src, VertexId_CUDA dst, int feature_size,
                        bool sync = true) {
     (void)sync;
+    nts_veneer::settle_pending();
     NTS_VENEER_CHECK(nts_memcpy_d2h_async(output, input, (size_t)(dst - src) * feature_size * sizeof(float), stream));
   }
   void move_data_in(float *d_pointer, float *h_pointer, VertexId_CUDA start, VertexId_CUDA end, int feature_size,
@@ -385,15 +520,22 @@ class Cuda_Stream {
                               bool tensor_weight = false) {
     (void)dst_start; (void)dst_end;
     reject_tensor_weight(with_weight && tensor_weight);
+    // output += sum; on an output this thread has just cleared with zero_buffer that is output = sum
+    const int accumulate = nts_veneer::take_zeroed(output, (size_t)batch_size * feature_size) ? 0 : 1;
     nts_veneer::note_write(output);
-    nts_spmm_plan_t *plan = nts_veneer::plan_for(column_offset, row_indices, src_start,
-                                                  src_end > src_start ? src_end - src_start : 0, batch_size, edges, stream);
-    if (plan)
+    bool deferred = false;
+    nts_spmm_plan_t *plan =
+        nts_veneer::plan_for(column_offset, row_indices, src_start, src_end > src_start ? src_end - src_start : 0,
+                             batch_size, edges, stream, accumulate == 0, &deferred);
+    if (plan) {
       NTS_VENEER_CHECK(nts_spmm_gather_planned(plan, input, output, with_weight ? weight_forward : NULL, column_offset,
-                                               row_indices, src_start, feature_size, 1, stream));
-    else
+                                               row_indices, src_start, feature_size, accumulate, stream));
+      if (deferred)
+        nts_veneer::defer_check(column_offset, row_indices, src_start, batch_size, edges, feature_size, input, output,
+                                with_weight ? weight_forward : NULL, stream);
+    } else
       NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_forward : NULL, column_offset, row_indices,
-                                       src_start, batch_size, edges, feature_size, 1, stream));
+                                       src_start, batch_size, edges, feature_size, accumulate, stream));
   }
   void Gather_By_Dst_From_Src_Optim(float *input, float *output, float *weight_forward, VertexId_CUDA *row_indices,
                                     VertexId_CUDA *column_offset, VertexId_CUDA src_start, VertexId_CUDA src_end,
@@ -410,15 +552,21 @@ class Cuda_Stream {
                               bool tensor_weight = false) {
     (void)src_start; (void)src_end;
     reject_tensor_weight(with_weight && tensor_weight);
+    const int accumulate = nts_veneer::take_zeroed(output, (size_t)batch_size * feature_size) ? 0 : 1;
     nts_veneer::note_write(output);
-    nts_spmm_plan_t *plan = nts_veneer::plan_for(row_offset, column_indices, dst_start,
-                                                  dst_end > dst_start ? dst_end - dst_start : 0, batch_size, edges, stream);
-    if (plan)
+    bool deferred = false;
+    nts_spmm_plan_t *plan =
+        nts_veneer::plan_for(row_offset, column_indices, dst_start, dst_end > dst_start ? dst_end - dst_start : 0,
+                             batch_size, edges, stream, accumulate == 0, &deferred);
+    if (plan) {
       NTS_VENEER_CHECK(nts_spmm_gather_planned(plan, input, output, with_weight ? weight_backward : NULL, row_offset,
-                                               column_indices, dst_start, feature_size, 1, stream));
-    else
+                                               column_indices, dst_start, feature_size, accumulate, stream));
+      if (deferred)
+        nts_veneer::defer_check(row_offset, column_indices, dst_start, batch_size, edges, feature_size, input, output,
+                                with_weight ? weight_backward : NULL, stream);
+    } else
       NTS_VENEER_CHECK(nts_spmm_gather(input, output, with_weight ? weight_backward : NULL, row_offset, column_indices,
-                                       dst_start, batch_size, edges, feature_size, 1, stream));
+                                       dst_start, batch_size, edges, feature_size, accumulate, stream));
   }
   void Gather_By_Src_From_Dst_Optim(float *input, float *output, float *weight_backward, VertexId_CUDA *row_offset,
                                     VertexId_CUDA *column_indices, VertexId_CUDA src_start, VertexId_CUDA src_end,

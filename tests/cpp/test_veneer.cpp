@@ -65,6 +65,28 @@ int main() {
   for (size_t i = 0; i < got.size(); ++i) twice = twice && fabsf(got[i] - 2.f * ref[i]) <= 1e-5f * (1.f + fabsf(ref[i]));
   EXPECT(twice);
 
+  // An output that was cleared with zero_buffer and then written through this header before the call is
+  // not taken for zeros: the call still adds to what the buffer holds.
+  {
+    std::vector<float> ones(got.size(), 1.f);
+    zero_buffer(dout, (int)got.size());
+    move_data_in(dout, ones.data(), 0, Vd, F);
+    cs.Gather_By_Dst_From_Src(dx, dout, dw, csc.row_indices, csc.column_offset, 0, 0, 0, 0, E, Vd, F, true, false);
+    cs.CUDA_DEVICE_SYNCHRONIZE();
+    move_result_out(got.data(), dout, 0, Vd, F);
+    bool added = true;
+    for (size_t i = 0; i < got.size(); ++i) added = added && fabsf(got[i] - (1.f + ref[i])) <= 1e-5f * (1.f + fabsf(ref[i]));
+    EXPECT(added);
+    // and a cleared output of another size or address is not confused with this one
+    zero_buffer(dx, 4);
+    move_data_in(dx, x.data(), 0, Vs, F);
+    zero_buffer(dout, (int)got.size());
+    cs.Gather_By_Src_From_Dst(dx, dout, dw, csc.column_offset, csc.row_indices, 0, 0, 0, 0, E, Vd, F, true, false);
+    cs.CUDA_DEVICE_SYNCHRONIZE();
+    move_result_out(got.data(), dout, 0, Vd, F);
+    EXPECT(memcmp(got.data(), ref.data(), got.size() * sizeof(float)) == 0);
+  }
+
   // zero-copy feature gather from mapped pinned host memory + label gather
   float *pinned = (float *)cudaMallocPinned((long)x.size() * sizeof(float));
   memcpy(pinned, x.data(), x.size() * sizeof(float));
@@ -195,6 +217,7 @@ int main() {
     EXPECT(run_and_check(want));  // correct on the new contents ...
     EXPECT(nts_veneer::planned_calls() == planned2);  // ... because the schedule was not used
     EXPECT(nts_veneer::plans_dropped_by_checksum() == dropped0 + 1);
+    EXPECT(nts_veneer::deferred_checks() > 0);  // the checksums ran on the side stream, next to the aggregation
     EXPECT(run_and_check(want));
     EXPECT(run_and_check(want));  // and a new schedule follows once the new contents have repeated
     EXPECT(run_and_check(want));
