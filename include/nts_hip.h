@@ -353,6 +353,21 @@ int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const floa
                           const float *el, const float *er, const uint32_t *co, const uint32_t *ri,
                           uint32_t Vd, uint32_t H, float slope, nts_stream_t stream);
 
+/* nts_gat_attention_fwd / _bwd with the caller's bound on a destination's edges (a sampled layer: the
+ * hop's fanout, nts_sampled_layer_t::max_in_degree).  When max_degree * H is at most 128 (and H a power
+ * of two up to 16) the call is ONE launch, a lane group per destination with the segment in registers;
+ * up to 32,768 values the launches that look for hub destinations and handle them are left out (three
+ * launches instead of eleven for a layer of 16,384 destinations or more); 0 = no bound known = the calls
+ * above.  The bound only selects the launches: a longer segment than stated is still computed -- by one
+ * lane group or wavefront, slowly. */
+int nts_gat_attention_fwd_bounded(float *alpha, const float *el, const float *er, const uint32_t *co,
+                                  const uint32_t *ri, uint32_t Vd, uint32_t H, float slope,
+                                  uint32_t max_degree, nts_stream_t stream);
+int nts_gat_attention_bwd_bounded(float *gs, float *ger, const float *galpha, const float *alpha,
+                                  const float *el, const float *er, const uint32_t *co, const uint32_t *ri,
+                                  uint32_t Vd, uint32_t H, float slope, uint32_t max_degree,
+                                  nts_stream_t stream);
+
 /* Attention-weighted aggregation, multi-head (DistAggregateDstFuseWeight::forward,
  * core/ntsDistCPUGraphOp.hpp:401-440; composition E_msg*alpha -> SingleCPUDstAggregateOp of
  * toolkits/GAT_CPU.hpp:196-201):

@@ -80,6 +80,8 @@ SIGNATURES = {
     "nts_edge_softmax_bwd": [_vp, _vp, _vp, _vp, _u32, _u32, _vp],
     "nts_gat_attention_fwd": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp],
     "nts_gat_attention_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _vp],
+    "nts_gat_attention_fwd_bounded": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _u32, _vp],
+    "nts_gat_attention_bwd_bounded": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _f32, _u32, _vp],
     "nts_spmm_gather_heads": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _vp],
     "nts_spmm_gather_heads_bounded": [_vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, _vp],
     "nts_spmm_gather_heads_planned": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _int, _vp],

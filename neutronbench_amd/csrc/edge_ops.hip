@@ -194,6 +194,48 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
       my_e1 = off[base + lane + 1];
       mine = my_e1 - my_e0 <= long_limit;  // longer rows belong to the block kernels
     }
+    if (G == 1) {
+      // Rows one vector wide (the per-head values of an attention layer): a lane sums its own row when
+      // the row has at most eight edges -- most rows of a sampled layer's transposed structure -- with
+      // the eight loads in flight at once, added in edge order like everywhere else; only the longer
+      // rows go through the sharing scheme below.
+      const uint32_t deg = my_e1 - my_e0;
+      if (mine && deg <= 8u) {
+        V v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          v[u] = V{};
+          if (static_cast<uint32_t>(u) < deg) {
+            const uint32_t e = perm ? perm[my_e0 + u] : my_e0 + u;
+            v[u] = msg[e];
+          }
+        }
+        float s1[NF];
+#pragma unroll
+        for (int t = 0; t < NF; ++t) s1[t] = 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (static_cast<uint32_t>(u) < deg) {
+            const float *vf = reinterpret_cast<const float *>(&v[u]);
+#pragma unroll
+            for (int t = 0; t < NF; ++t) s1[t] += vf[t];
+          }
+        }
+        V *p = out + (base + lane);
+        if (accumulate) {
+          const V o = *p;
+          const float *of = reinterpret_cast<const float *>(&o);
+#pragma unroll
+          for (int t = 0; t < NF; ++t) s1[t] += of[t];
+        }
+        V res;
+        float *rf = reinterpret_cast<float *>(&res);
+#pragma unroll
+        for (int t = 0; t < NF; ++t) rf[t] = s1[t];
+        *p = res;
+        mine = false;
+      }
+    }
     uint64_t pending = __ballot(mine);  // rows of this set not handed out yet (wave-uniform)
     bool have = false;
     uint32_t row = 0, k = 0, e1 = 0;
@@ -297,7 +339,8 @@ constexpr uint32_t kPieceCap = 8192;
 constexpr uint32_t kGiantMinPiece = 4096;  // edges
 
 // hdr: [0] giant rows seen (may exceed kGiantCap until the plan kernel clamps it), [1] pieces,
-//      [2] edges per piece, [4..5] edges of the listed giant rows (64-bit).
+//      [2] edges per piece, [4..5] edges of the listed giant rows (64-bit), [6] the long-row counter
+//      (`count` points here, so that one fill clears all of them).
 // list[0 .. *count) = rows r with (off[r+1] - off[r]) * width > limit that are not listed as giant
 // (any order); giant_rows[0 .. min(hdr[0], kGiantCap)) = rows above giant_limit values.
 __global__ __launch_bounds__(256) void collect_long_rows_kernel(uint32_t *__restrict__ list,
@@ -731,7 +774,52 @@ __device__ __forceinline__ bool any_lane(bool pred) { return __ballot(pred) != 0
 
 // Short segments (n <= kShortValues; power-of-two H <= kShortG): a group of kShortG lanes per
 // destination, striding over the destinations.  BWD selects the backward formula.
+// A segment of any length by one group of kShortG lanes, with plain strided passes (the safety net of a
+// launch that was told no segment exceeds the short class: correct, not fast).
 template <bool FUSED, bool BWD>
+__device__ void softmax_group_any(float *__restrict__ outs, float *__restrict__ ger, const float *__restrict__ xs,
+                                  const float *__restrict__ ys, const float *__restrict__ el,
+                                  const float *__restrict__ er, const uint32_t *__restrict__ ri, uint32_t d,
+                                  uint32_t e0, uint64_t n, uint32_t H, float slope, uint32_t gl) {
+  const uint32_t h = gl & (H - 1);
+  const float erv = FUSED ? er[static_cast<size_t>(d) * H + h] : 0.f;
+  auto score = [&](uint64_t i) {
+    if (!FUSED) return xs[i];
+    return leaky(el[static_cast<size_t>(ri[e0 + i / H]) * H + h] + erv, slope);
+  };
+  if (!BWD) {
+    float mx = -INFINITY;
+    for (uint64_t i = gl; i < n; i += kShortG) mx = fmaxf(mx, score(i));
+    mx = head_reduce_w<0, kShortG>(mx, H);
+    float sum = 0.f;
+    for (uint64_t i = gl; i < n; i += kShortG) sum += softmax_exp(score(i) - mx);
+    sum = head_reduce_w<1, kShortG>(sum, H);
+    const float inv = 1.f / sum;
+    for (uint64_t i = gl; i < n; i += kShortG) outs[i] = softmax_exp(score(i) - mx) * inv;
+  } else {
+    float dot = 0.f;
+    for (uint64_t i = gl; i < n; i += kShortG) dot += xs[i] * ys[i];
+    dot = head_reduce_w<1, kShortG>(dot, H);
+    float gsum = 0.f;
+    for (uint64_t i = gl; i < n; i += kShortG) {
+      float g = ys[i] * (xs[i] - dot);
+      if (FUSED) {
+        const float pre = el[static_cast<size_t>(ri[e0 + i / H]) * H + h] + erv;
+        g *= pre > 0.f ? 1.f : slope;
+        gsum += g;
+      }
+      outs[i] = g;
+    }
+    if (FUSED) {
+      gsum = head_reduce_w<1, kShortG>(gsum, H);
+      if (gl < H) ger[static_cast<size_t>(d) * H + gl] = gsum;
+    }
+  }
+}
+
+// ALL: the launch is the only one of its call (the caller bounded every segment by the short class), so
+// a segment beyond the class is not skipped but computed by the group with plain strided passes.
+template <bool FUSED, bool BWD, bool ALL = false>
 __global__ __launch_bounds__(256) void edge_softmax_short_kernel(float *__restrict__ out, float *__restrict__ ger,
                                                                  const float *__restrict__ x_or_gy,
                                                                  const float *__restrict__ y,
@@ -746,9 +834,14 @@ __global__ __launch_bounds__(256) void edge_softmax_short_kernel(float *__restri
     const uint32_t d = static_cast<uint32_t>(d64);
     const uint32_t e0 = co[d], e1 = co[d + 1];
     const uint64_t n64 = static_cast<uint64_t>(e1 - e0) * H;
-    if (n64 > kShortValues) continue;  // the whole group skips together
-    const uint32_t n = static_cast<uint32_t>(n64);
     const size_t base = static_cast<size_t>(e0) * H;
+    if (n64 > kShortValues) {  // the whole group takes the same way
+      if (ALL)
+        softmax_group_any<FUSED, BWD>(out + base, ger, x_or_gy ? x_or_gy + base : nullptr, y ? y + base : nullptr, el, er,
+                                      ri, d, e0, n64, H, slope, gl);
+      continue;
+    }
+    const uint32_t n = static_cast<uint32_t>(n64);
     if (BWD) {
       if (FUSED) {  // the four instances together would cost this kernel a wavefront per SIMD
         softmax_bwd_regs<FUSED, kShortG, kShortK>(out + base, ger, x_or_gy + base, y + base, el, er, ri, d, e0, n, H,
@@ -1506,18 +1599,17 @@ struct LongRows {
 int collect_long_rows(LongRows &lr, const uint32_t *off, uint32_t rows, uint32_t width, uint32_t limit,
                       uint64_t giant_limit, hipStream_t stream) {
   if (rows < kLongMinVertices) return NTS_OK;
-  const size_t list_bytes = (static_cast<size_t>(rows) + 1 + 7) / 8 * 8 * sizeof(uint32_t);  // list + counter, 32-byte multiple
-  const size_t small_bytes = (8 + kGiantCap + kGiantCap + 8) * sizeof(uint32_t);             // hdr, rows, first
+  const size_t list_bytes = (static_cast<size_t>(rows) + 7) / 8 * 8 * sizeof(uint32_t);  // list, 32-byte multiple
+  const size_t small_bytes = (8 + kGiantCap + kGiantCap + 8) * sizeof(uint32_t);         // hdr (with the counter), rows, first
   NTS_HIP_TRY(lr.block.alloc(list_bytes + small_bytes + kPieceCap * sizeof(uint4), stream));
   unsigned char *buf = static_cast<unsigned char *>(lr.block.ptr);
   lr.list = reinterpret_cast<uint32_t *>(buf);
-  lr.count = lr.list + rows;
   lr.hdr = reinterpret_cast<uint32_t *>(buf + list_bytes);
+  lr.count = lr.hdr + 6;
   lr.giant_rows = lr.hdr + 8;
   lr.first = lr.giant_rows + kGiantCap;
   lr.pieces = reinterpret_cast<uint4 *>(buf + list_bytes + small_bytes);
-  if (int rc = nts_memset_zero(lr.count, sizeof(uint32_t), stream)) return rc;
-  if (int rc = nts_memset_zero(lr.hdr, 8 * sizeof(uint32_t), stream)) return rc;
+  if (int rc = nts_memset_zero(lr.hdr, 8 * sizeof(uint32_t), stream)) return rc;  // counters and the ticket
   hipLaunchKernelGGL(collect_long_rows_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, stream, lr.list, lr.count,
                      lr.giant_rows, lr.hdr, off, rows, width, limit, giant_limit);
   NTS_LAUNCH_CHECK("collect_long_rows_kernel");
@@ -1625,10 +1717,14 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
 // null where the variant does not use them.
 int softmax_impl(bool backward, bool fused, float *out, float *ger, const float *x_or_gy, const float *y,
                  const float *el, const float *er, const uint32_t *co, const uint32_t *ri, uint32_t Vd, uint32_t H,
-                 float slope, hipStream_t stream, const char *who) {
+                 float slope, hipStream_t stream, const char *who, uint32_t max_degree = 0) {
   const bool pow2 = is_pow2(H) && H <= kWave;
   LongRows lr;
-  if (pow2)
+  // A caller that bounds every segment below the block kernels' class (a sampled layer: at most `fanout`
+  // edges per destination) needs none of the launches that look for hub rows; a longer segment than
+  // stated is still computed, by one wavefront.
+  const bool no_hubs = max_degree != 0 && static_cast<uint64_t>(max_degree) * H <= kLongRowValues;
+  if (pow2 && !no_hubs)
     if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, kGiantValues, stream)) return rc;
   const uint32_t max_values = lr.list ? kLongRowValues : kNoLimit;
   // 16-byte lanes for the segments that do not fit the register paths: whole heads per lane and
@@ -1643,6 +1739,18 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   const dim3 short_grid(short_blocks < 16384u ? short_blocks : 16384u);
   const uint32_t wave_blocks = ceil_div(Vd, 4);  // at most one destination per wavefront
   const dim3 grid(wave_blocks < 8192u ? wave_blocks : 8192u);
+  if (use_short && fused && max_degree != 0 && static_cast<uint64_t>(max_degree) * H <= kShortValues) {
+    // Every segment fits the short class by the caller's word: one launch (which still computes a
+    // longer segment, slowly, should there be one).
+    if (backward)
+      hipLaunchKernelGGL((edge_softmax_short_kernel<true, true, true>), short_grid, block, 0, stream, out, ger, x_or_gy,
+                         y, el, er, co, ri, Vd, H, slope);
+    else
+      hipLaunchKernelGGL((edge_softmax_short_kernel<true, false, true>), short_grid, block, 0, stream, out, ger, x_or_gy,
+                         y, el, er, co, ri, Vd, H, slope);
+    NTS_LAUNCH_CHECK(who);
+    return NTS_OK;
+  }
   if (use_short) {
 #define NTS_SHORT(FU, BW)                                                                                          \
   hipLaunchKernelGGL((edge_softmax_short_kernel<FU, BW>), short_grid, block, 0, stream, out, ger, x_or_gy, y, el, er, \
@@ -1810,6 +1918,29 @@ int nts_gat_attention_fwd(float *alpha, const float *el, const float *er, const 
   if (!alpha || !el || !er || !co || !ri) return fail(NTS_ERR_INVALID, "nts_gat_attention_fwd: null pointer");
   return softmax_impl(false, true, alpha, nullptr, nullptr, nullptr, el, er, co, ri, Vd, H, slope, stream,
                       "nts_gat_attention_fwd");
+}
+
+int nts_gat_attention_fwd_bounded(float *alpha, const float *el, const float *er, const uint32_t *co,
+                                  const uint32_t *ri, uint32_t Vd, uint32_t H, float slope, uint32_t max_degree,
+                                  nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gat_attention_fwd_bounded");
+  if (H == 0) return fail(NTS_ERR_INVALID, "nts_gat_attention_fwd_bounded: H is 0");
+  if (Vd == 0) return NTS_OK;
+  if (!alpha || !el || !er || !co || !ri) return fail(NTS_ERR_INVALID, "nts_gat_attention_fwd_bounded: null pointer");
+  return softmax_impl(false, true, alpha, nullptr, nullptr, nullptr, el, er, co, ri, Vd, H, slope, stream,
+                      "nts_gat_attention_fwd_bounded", max_degree);
+}
+
+int nts_gat_attention_bwd_bounded(float *gs, float *ger, const float *galpha, const float *alpha, const float *el,
+                                  const float *er, const uint32_t *co, const uint32_t *ri, uint32_t Vd, uint32_t H,
+                                  float slope, uint32_t max_degree, nts_stream_t stream) {
+  NTS_TRACE_RANGE("nts_gat_attention_bwd_bounded");
+  if (H == 0) return fail(NTS_ERR_INVALID, "nts_gat_attention_bwd_bounded: H is 0");
+  if (Vd == 0) return NTS_OK;
+  if (!gs || !ger || !galpha || !alpha || !el || !er || !co || !ri)
+    return fail(NTS_ERR_INVALID, "nts_gat_attention_bwd_bounded: null pointer");
+  return softmax_impl(true, true, gs, ger, galpha, alpha, el, er, co, ri, Vd, H, slope, stream,
+                      "nts_gat_attention_bwd_bounded", max_degree);
 }
 
 int nts_gat_attention_bwd(float *gs, float *ger, const float *galpha, const float *alpha, const float *el,

@@ -37,20 +37,30 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(V *__restrict__ out, c
 // table.  Blocks stride over the rows and count their hits locally; one integer atomic per block
 // adds the block's count (one atomic per hit row on a single address was measured at 1.3 ms of a
 // 1.9 ms launch for 337 k rows).
+// miss_blocks > 0 (table in host memory): the first miss_blocks blocks copy only the rows that miss
+// the cache -- they wait for the link -- and the blocks after them only the rows that hit, from HBM;
+// every block walks all row ids of its stride and skips the rows of the other kind.  The few blocks
+// that keep the link full are then not also the ones that move the (many more) cached rows.
 template <typename V, int G>
 __global__ __launch_bounds__(256) void gather_rows_cached_kernel(V *__restrict__ out, const V *__restrict__ table,
                                                                  const V *__restrict__ cache,
                                                                  const uint32_t *__restrict__ row_ids,
                                                                  const uint32_t *__restrict__ hashmap, uint32_t n,
-                                                                 uint32_t Fv, uint32_t *__restrict__ hits) {
+                                                                 uint32_t Fv, uint32_t *__restrict__ hits,
+                                                                 uint32_t miss_blocks) {
   constexpr uint32_t kRowsPerBlock = 256 / G;
   const uint32_t gl = threadIdx.x & (G - 1);
   uint32_t my_hits = 0;
-  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / G; i < n;
-       i += static_cast<uint64_t>(gridDim.x) * kRowsPerBlock) {
+  // blocks of this block's kind, and its rank among them
+  const bool split = miss_blocks != 0, miss_side = blockIdx.x < miss_blocks;
+  const uint32_t peers = !split ? gridDim.x : (miss_side ? miss_blocks : gridDim.x - miss_blocks);
+  const uint32_t rank = (!split || miss_side) ? blockIdx.x : blockIdx.x - miss_blocks;
+  for (uint64_t i = static_cast<uint64_t>(rank) * kRowsPerBlock + threadIdx.x / G; i < n;
+       i += static_cast<uint64_t>(peers) * kRowsPerBlock) {
     const uint32_t g = row_ids[i];
     const uint32_t slot = hashmap[g];
     const bool hit = slot != kMiss;
+    if (split && hit == miss_side) continue;  // the other kind of block copies this row
     const V *src = hit ? cache + static_cast<size_t>(slot) * Fv : table + static_cast<size_t>(g) * Fv;
     V *dst = out + static_cast<size_t>(i) * Fv;
     for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
@@ -113,6 +123,7 @@ struct RowsArgs {
 // instead of parking wavefronts that wait for the link on every compute unit.
 constexpr uint32_t kHostTableBlocks = 128;
 constexpr uint32_t kCachedBlocks = 16384;  // table in device memory: fill the chip several times over
+constexpr uint32_t kHitBlocks = 1024;      // table in host memory: blocks that copy the rows the HBM cache holds
 
 // Whether `p` is host memory the device reads over the link.  The answer for the last table asked
 // about is kept per thread (one query costs microseconds, and a caller gathers from the same table
@@ -139,13 +150,19 @@ void launch_rows(const RowsArgs &a, uint32_t Fv) {
   const bool host_table = table_in_host_memory(a.table);
   // Both kernels stride over the rows, so any grid covers them.
   const uint32_t cap = host_table ? kHostTableBlocks : (a.cache ? kCachedBlocks : blocks);
+  const uint32_t wanted = blocks;
   if (blocks > cap) blocks = cap;
-  const dim3 grid(blocks);
-  if (a.cache)
-    hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), grid, dim3(256), 0, a.stream,
+  if (a.cache) {
+    // table in host memory: kHostTableBlocks blocks for the rows that miss, and beside them blocks for
+    // the rows the cache holds (enough to move them at HBM speed, still a fraction of the chip)
+    const uint32_t miss_blocks = (host_table && wanted > kHostTableBlocks) ? kHostTableBlocks : 0u;
+    const uint32_t hit_blocks = miss_blocks ? std::min<uint32_t>(wanted, kHitBlocks) : 0u;
+    hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), dim3(blocks + hit_blocks), dim3(256), 0, a.stream,
                        reinterpret_cast<V *>(a.out), reinterpret_cast<const V *>(a.table),
-                       reinterpret_cast<const V *>(a.cache), a.row_ids, a.remap, a.n, Fv, a.hits);
-  else
+                       reinterpret_cast<const V *>(a.cache), a.row_ids, a.remap, a.n, Fv, a.hits, miss_blocks);
+    return;
+  }
+  const dim3 grid(blocks);
     hipLaunchKernelGGL((gather_rows_kernel<V, G>), grid, dim3(256), 0, a.stream, reinterpret_cast<V *>(a.out),
                        reinterpret_cast<const V *>(a.table), a.row_ids, a.sel, a.remap, a.n, Fv);
 }

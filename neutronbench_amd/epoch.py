@@ -420,8 +420,22 @@ if __name__ == "__main__":
                          "first batch; 0: the launches are enqueued one by one for every batch")
     ap.add_argument("--native", action="store_true",
                     help="drive the epoch from C++ (lib/nts_epoch) instead of this module's Python loop")
+    ap.add_argument("--write-inputs", metavar="DIR", default=None,
+                    help="only write the configuration's arrays for lib/nts_epoch to DIR and print the command line "
+                         "that runs the epoch on them (to run the program under a profiler)")
     a = ap.parse_args()
-    if a.native:
+    if a.write_inputs:
+        import os
+
+        os.makedirs(a.write_inputs, exist_ok=True)
+        shape = write_native_inputs(a.config, a.write_inputs, a.scale)
+        cfg = CONFIGS[a.config]
+        print(" ".join(["neutronbench_amd/lib/nts_epoch", "--dir", a.write_inputs, "--V", str(shape["V"]), "--F",
+                        str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch", str(cfg["batch"]), "--fanout",
+                        ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)), "--cache",
+                        str(cfg["cache"]), "--pipeline", str(a.pipeline), "--stage-sync",
+                        str(int(bool(a.stage_sync)) if a.stage_sync is not None else 1)]))
+    elif a.native:
         run_native(a.config, a.scale, a.max_batches, a.warmup_batches, a.pipeline, graph=bool(a.graph),
                    stage_sync=bool(a.stage_sync))
     else:

@@ -328,7 +328,8 @@ int main(int argc, char **argv) {
       const nts_sampled_layer_t &L = s.layers[l];
       const float *x = d_ones;  // [src_size, H * Fh]: stands in for the projected features of the layer
       const float *el = d_ones + 8;  // [src_size, H]
-      NTS(nts_gat_attention_fwd(d_alpha[l], el, d_er, L.column_offset, L.row_indices, L.v_size, H, slope, stream));
+      NTS(nts_gat_attention_fwd_bounded(d_alpha[l], el, d_er, L.column_offset, L.row_indices, L.v_size, H, slope,
+                                        L.max_in_degree, stream));
       NTS(nts_spmm_gather_heads_bounded(x, d_out, d_alpha[l], nullptr, L.column_offset, L.row_indices, L.v_size, L.e_size,
                                         H, Fh, 0, L.max_in_degree, stream));
       if (a.verify) {
@@ -352,8 +353,8 @@ int main(int argc, char **argv) {
       NTS(nts_spmm_gather_heads(g_out, d_gin, d_alpha[k], L.csr_to_csc, L.row_offset, L.column_indices, L.src_size,
                                 L.e_size, H, Fh, 0, stream));
       NTS(nts_sddmm_heads(d_galpha, x, g_out, L.column_offset, L.row_indices, L.v_size, H, Fh, stream));
-      NTS(nts_gat_attention_bwd(d_gs, d_ger, d_galpha, d_alpha[k], el, d_er, L.column_offset, L.row_indices, L.v_size, H,
-                                slope, stream));
+      NTS(nts_gat_attention_bwd_bounded(d_gs, d_ger, d_galpha, d_alpha[k], el, d_er, L.column_offset, L.row_indices,
+                                        L.v_size, H, slope, L.max_in_degree, stream));
       NTS(nts_gather_edge_to_src(d_gel, d_gs, L.row_offset, L.csr_to_csc, L.src_size, H, 0, stream));
       if (a.verify) {
         hash(d_gin, static_cast<uint64_t>(L.src_size) * H * Fh, 30 + k, stream);

@@ -185,8 +185,8 @@ class GATAttentionOp:
         H = el.shape[1]
         alpha = torch.empty(sg.e_size, H, dtype=torch.float32, device=el.device)
         stream = torch.cuda.current_stream(el.device).cuda_stream
-        call("nts_gat_attention_fwd", ptr(alpha), ptr(el), ptr(er), ptr(sg.dev_c_o()), ptr(sg.dev_r_i()), sg.v_size, H,
-             self.slope, stream)
+        call("nts_gat_attention_fwd_bounded", ptr(alpha), ptr(el), ptr(er), ptr(sg.dev_c_o()), ptr(sg.dev_r_i()),
+             sg.v_size, H, self.slope, getattr(sg, "max_in_degree", 0), stream)
         self.alpha, self.el, self.er = alpha, el, er
         return alpha
 
@@ -198,8 +198,9 @@ class GATAttentionOp:
         stream = torch.cuda.current_stream(dev).cuda_stream
         gs = torch.empty_like(g_alpha)
         self.ger = torch.empty(sg.v_size, H, dtype=torch.float32, device=dev)
-        call("nts_gat_attention_bwd", ptr(gs), ptr(self.ger), ptr(g_alpha), ptr(self.alpha), ptr(self.el),
-             ptr(self.er), ptr(sg.dev_c_o()), ptr(sg.dev_r_i()), sg.v_size, H, self.slope, stream)
+        call("nts_gat_attention_bwd_bounded", ptr(gs), ptr(self.ger), ptr(g_alpha), ptr(self.alpha), ptr(self.el),
+             ptr(self.er), ptr(sg.dev_c_o()), ptr(sg.dev_r_i()), sg.v_size, H, self.slope,
+             getattr(sg, "max_in_degree", 0), stream)
         gel = torch.empty(sg.src_size, H, dtype=torch.float32, device=dev)
         call("nts_gather_edge_to_src", ptr(gel), ptr(gs), ptr(sg.dev_r_o()), ptr(sg.dev_csr_to_csc), sg.src_size, H, 0,
              stream)
