@@ -458,7 +458,10 @@ int nts_message_rows_add(float *rows, const float *records, uint32_t n_records, 
  *                            nts_sample_hop_work_bytes(n) bytes of 256-byte-aligned device scratch.
  *   nts_sample_hop_neighbors ri_global[co[i] .. co[i+1]) = all in-neighbours of dst[i] in CSC order when none is
  *                            dropped, otherwise that many DISTINCT positions of its CSC segment chosen uniformly
- *                            from a hash of (seed, i, dst[i]), in ascending position order.
+ *                            from a hash of (seed, i, dst[i]), in ascending position order.  Any fanout, as the
+ *                            reference's sampler (core/ntsSampler.hpp:936-1042): up to 64 by Floyd's sampling inside
+ *                            a lane group, up to 1,024 by a keyed permutation of the positions, above that the
+ *                            positions with the `fanout` smallest keyed hashes (a radix select per destination).
  * Which neighbours the reference picks depends on its RNG, thread count and container iteration
  * order, so the pick is specified here by these properties, not by equality with the reference. */
 size_t nts_sample_hop_work_bytes(uint32_t n);

@@ -231,8 +231,6 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
     return fail(NTS_ERR_INVALID, "nts_batch_builder_create: empty graph or batch");
   for (uint32_t h = 0; h < hops; ++h) {
     if (fanouts[h] == 0) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: fanout 0");
-    if (fanouts[h] > kWidestFanout)
-      return fail(NTS_ERR_UNSUPPORTED, "nts_batch_builder_create: fanouts above 1,024 are not supported");
   }
   if (!aligned_to(arena, 256)) return fail(NTS_ERR_INVALID, "nts_batch_builder_create: arena must be 256-byte aligned");
   nts_batch_builder *b = new (std::nothrow) nts_batch_builder();

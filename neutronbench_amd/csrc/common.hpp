@@ -127,8 +127,9 @@ struct DevSeed {
 inline DevSeed host_seed(uint64_t v) { return DevSeed{nullptr, v}; }
 inline DevSeed device_seed(const uint64_t *base, uint64_t add) { return DevSeed{base, add}; }
 
-// Largest finite fanout of the neighbour pick (distinct uniform positions: up to 64 inside lane
-// groups with Floyd's algorithm, up to this many by a keyed permutation of the positions).
+// Distinct uniform positions of the neighbour pick: up to 64 inside lane groups with Floyd's algorithm,
+// up to this many by a keyed permutation of the positions staged in LDS, above it by a radix select
+// of keyed hashes (any fanout).
 constexpr int32_t kWidestFanout = 1024;
 
 // Steps of a sampled layer's construction with sizes that may live on the device (sampler.hip,

@@ -6,8 +6,9 @@
 // The reference draws positions with a per-thread mt19937 and iterates an unordered_set, so which
 // neighbours it picks (and in which order) is implementation-defined; here positions come from a
 // counter-based hash of (seed, destination slot) through Floyd's sampling (fanouts up to 64) or a
-// keyed permutation of the positions (up to 1,024) and are emitted in ascending position order, which keeps source ids ascending inside a destination for graphs with
-// sorted adjacency.  Results depend only on the arguments: the same seed gives the same sample.
+// keyed permutation of the positions (up to 1,024) or the positions with the smallest keyed hashes (any
+// larger fanout) and are emitted in ascending position order, which keeps source ids ascending inside a
+// destination for graphs with sorted adjacency.  Results depend only on the arguments: the same seed gives the same sample.
 #include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
 #include <rocprim/iterator/transform_iterator.hpp>
@@ -175,6 +176,91 @@ __global__ __launch_bounds__(256) void hop_pick_wide_kernel(uint32_t *__restrict
   }
 }
 
+// Fanouts above 1,024: one block per destination that has more neighbours than the fanout.  Every
+// position p of the neighbourhood gets a 32-bit key hashed from (seed, destination slot, p); the
+// sample is the `take` positions with the smallest keys -- a uniform subset without replacement,
+// distinct by construction -- and ties at the largest chosen key are broken by position.  The take-th
+// smallest key is found by a radix select (four passes over the positions, one byte of the key each,
+// a 256-bin histogram in LDS; keys are recomputed, not stored), then one more pass copies the chosen
+// neighbours in ascending position order, their output slots coming from a block-wide count of the
+// chosen positions before them.  Any fanout and any degree; the work is five hashes per neighbour of
+// the destinations that need it.  Blocks stride over the destinations.
+__global__ __launch_bounds__(256) void hop_pick_select_kernel(uint32_t *__restrict__ ri_out,
+                                                              const uint32_t *__restrict__ co,
+                                                              const uint32_t *__restrict__ graph_co,
+                                                              const uint32_t *__restrict__ graph_ri,
+                                                              const uint32_t *__restrict__ dst, DevCount n,
+                                                              uint32_t edge_cap, DevSeed seed,
+                                                              uint32_t *__restrict__ mark) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t sh_prefix, sh_k, wave_less[4], wave_eq[4];
+  const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const uint32_t live = n.get();
+  for (uint32_t i = blockIdx.x; i < live; i += gridDim.x) {
+    const uint32_t d = dst[i];
+    const uint32_t base = graph_co[d];
+    const uint32_t deg = graph_co[d + 1] - base;
+    const uint32_t out = co[i];
+    const uint32_t take = co[i + 1] - out;
+    if (co[i + 1] > edge_cap || take == deg || take <= static_cast<uint32_t>(kWidestFanout)) continue;  // block-uniform
+    const uint64_t key = mix64(seed.get() ^ (static_cast<uint64_t>(i) << 32) ^ d);
+    auto key_of = [&](uint32_t p) { return static_cast<uint32_t>(mix64(key ^ (static_cast<uint64_t>(p) * 0x9E3779B97F4A7C15ull)) >> 32); };
+    // radix select: the take-th smallest key (1-based rank k among the keys that share the prefix)
+    if (threadIdx.x == 0) {
+      sh_prefix = 0;
+      sh_k = take;
+    }
+    for (int pass = 0; pass < 4; ++pass) {
+      const uint32_t shift = 24 - 8 * pass;
+      hist[threadIdx.x] = 0;
+      __syncthreads();
+      const uint32_t prefix = sh_prefix;
+      for (uint32_t p = threadIdx.x; p < deg; p += 256) {
+        const uint32_t h = key_of(p);
+        if (pass == 0 || (h >> (shift + 8)) == prefix) atomicAdd(&hist[(h >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        uint32_t k = sh_k, digit = 0;
+        while (digit < 255u && hist[digit] < k) k -= hist[digit++];
+        sh_k = k;
+        sh_prefix = (prefix << 8) | digit;
+      }
+      __syncthreads();
+    }
+    const uint32_t threshold = sh_prefix, ties_wanted = sh_k;  // keys below are all chosen; of the equal ones the first few
+    uint32_t less_before = 0, eq_before = 0;                   // chosen / tied positions before this chunk (block-uniform)
+    for (uint32_t p0 = 0; p0 < deg; p0 += 256) {
+      const uint32_t p = p0 + threadIdx.x;
+      const uint32_t h = p < deg ? key_of(p) : 0xFFFFFFFFu;
+      const bool less = p < deg && h < threshold, eq = p < deg && h == threshold;
+      const uint64_t less_mask = __ballot(less), eq_mask = __ballot(eq);
+      const uint64_t below = (1ull << lane) - 1ull;
+      if (lane == 0) {
+        wave_less[wave] = __popcll(less_mask);
+        wave_eq[wave] = __popcll(eq_mask);
+      }
+      __syncthreads();
+      uint32_t my_less = less_before + __popcll(less_mask & below), my_eq = eq_before + __popcll(eq_mask & below);
+      uint32_t chunk_less = 0, chunk_eq = 0;
+      for (uint32_t w = 0; w < 4; ++w) {
+        if (w < wave) {
+          my_less += wave_less[w];
+          my_eq += wave_eq[w];
+        }
+        chunk_less += wave_less[w];
+        chunk_eq += wave_eq[w];
+      }
+      // ties are taken in position order, so the number taken before this position is min(my_eq, wanted)
+      const uint32_t ties_before = my_eq < ties_wanted ? my_eq : ties_wanted;
+      if (less || (eq && my_eq < ties_wanted)) emit(ri_out, mark, out + my_less + ties_before, graph_ri[base + p]);
+      less_before += chunk_less;
+      eq_before += chunk_eq;
+      __syncthreads();
+    }
+  }
+}
+
 hipError_t scan_bytes(uint32_t n, size_t *bytes) {
   size_t tmp = 0;
   uint32_t *nul = nullptr;
@@ -226,9 +312,12 @@ int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph
   }
 #undef NTS_LAUNCH_PICK
   NTS_LAUNCH_CHECK("hop_pick_kernel");
-  if (fanout > kMaxFanout) {
-    if (fanout > kWidestFanout)
-      return fail(NTS_ERR_UNSUPPORTED, "neighbour pick: fanouts above 1,024 are not supported");
+  if (fanout > kWidestFanout) {
+    const uint32_t blocks = n.cap < 4096u ? n.cap : 4096u;
+    hipLaunchKernelGGL(hop_pick_select_kernel, dim3(blocks ? blocks : 1u), dim3(256), 0, stream, ri_global, co, graph_co,
+                       graph_ri, dst, n, edge_cap, seed, mark_bits);
+    NTS_LAUNCH_CHECK("hop_pick_select_kernel");
+  } else if (fanout > kMaxFanout) {
     hipLaunchKernelGGL(hop_pick_wide_kernel, dim3(ceil_div(static_cast<uint64_t>(n.cap) * kWave, 256)), dim3(256), 0,
                        stream, ri_global, co, graph_co, graph_ri, dst, n, edge_cap, seed, mark_bits);
     NTS_LAUNCH_CHECK("hop_pick_wide_kernel");

@@ -12,7 +12,7 @@ from neutronbench_amd import abi
 from neutronbench_amd.abi import call, ptr
 from neutronbench_amd.batch import (FeatureCache, MappedHostTable, load_feature_gpu, load_feature_gpu_cache,
                                     load_label_gpu, sample_hop)
-from neutronbench_amd.layout import SampledLayer
+from neutronbench_amd.layout import SampledLayer, as_u32
 from neutronbench_amd.stream import CudaStream, get_gpu_mem
 from util import brute_csr, random_block
 
@@ -310,9 +310,65 @@ def test_wide_fanouts_pick_spread_positions_uniformly(device):
     # pairs of positions are not tied together: positions 0 and 1 are picked together about (fanout/deg)^2 of the time
     both = np.mean((picks == 0).any(1) & (picks == 1).any(1))
     assert both < 3 * (fanout / deg) ** 2 + 0.01
-    # fanouts beyond the supported width are refused
-    assert abi.status("nts_sample_hop_neighbors", ptr(ri), ptr(co), ptr(gco), ptr(gri), ptr(dst), n, 2000, 1,
-                      torch.cuda.current_stream().cuda_stream) == abi.NTS_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("deg,fanout,n", [(20000, 1500, 300), (70001, 5000, 60), (1025, 1025, 8), (1100, 1025, 200)])
+def test_fanouts_above_1024_pick_the_smallest_keyed_hashes(device, deg, fanout, n):
+    """Any larger fanout (the reference's sampler takes any, core/ntsSampler.hpp:936-1042): the positions
+    with the `fanout` smallest keyed hashes, found by a radix select -- exactly `fanout` distinct positions
+    of the neighbourhood in ascending order, every position about equally often, the same picks for the
+    same seed; destinations with at most `fanout` neighbours keep all of them in CSC order."""
+    small = 700  # a second vertex with fewer neighbours than the fanout
+    gco = torch.tensor([0, deg, deg + small], dtype=torch.int32, device=device)
+    gri = torch.cat([torch.arange(deg, dtype=torch.int32), 5 * torch.arange(small, dtype=torch.int32)]).to(device)
+    dst = torch.zeros(n + 1, dtype=torch.int32, device=device)
+    dst[n] = 1
+    co, ri = sample_hop(gco, gri, dst, fanout, 21)
+    take = min(deg, fanout)
+    assert int(co[-1]) == n * take + small
+    flat = ri.cpu().numpy()
+    assert np.array_equal(flat[n * take:], 5 * np.arange(small))
+    picks = flat[:n * take].reshape(n, take)
+    assert picks.min() >= 0 and picks.max() < deg
+    assert np.all(np.diff(picks, axis=1) > 0)  # ascending, hence distinct
+    if take < deg:
+        counts = np.bincount(picks.ravel(), minlength=deg)
+        expect = n * take / deg
+        assert np.all(np.abs(counts - expect) < 6 * np.sqrt(expect) + 1), (counts.min(), counts.max(), expect)
+        assert np.unique(picks, axis=0).shape[0] > n // 2  # destinations do not share one sample
+        co2, ri2 = sample_hop(gco, gri, dst, fanout, 21)
+        assert torch.equal(ri, ri2)
+        _, ri3 = sample_hop(gco, gri, dst, fanout, 22)
+        assert not torch.equal(ri, ri3)
+
+
+def test_batch_builder_with_a_fanout_above_1024(device):
+    """The whole-batch builder with a hop of fanout 2,000 on a graph with a 6,000-neighbour hub: layers
+    equal to the per-hop entry points, the hub's destination keeps 2,000 distinct neighbours."""
+    from neutronbench_amd.batch import BatchBuilder
+
+    V = 8000
+    rng = np.random.default_rng(4)
+    deg = rng.integers(1, 30, V)
+    deg[17] = 6000
+    gco_h = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+    gri_h = np.concatenate([np.sort(rng.choice(V, d, replace=False)) for d in deg]).astype(np.int64)
+    gco = as_u32(torch.from_numpy(gco_h)).to(device)
+    gri = as_u32(torch.from_numpy(gri_h)).to(device)
+    batch = as_u32(torch.tensor([17, 5, 900, 17], dtype=torch.int64)).to(device)
+    builder = BatchBuilder(gco, gri, [2000, 3], 16)
+    layers = builder.sample(batch, 99)
+    top = layers[-1]
+    co = top.dev_column_offset.cpu().numpy()
+    assert co[1] - co[0] == 2000 and co[4] - co[3] == 2000 and co[2] - co[1] == deg[5]
+    src = top.dev_source.cpu().numpy()
+    local = top.dev_row_indices.cpu().numpy()[co[0]:co[1]]
+    glob = src[local]
+    assert np.unique(glob).size == 2000 and np.all(np.isin(glob, gri_h[gco_h[17]:gco_h[18]]))
+    off, rows = sample_hop(gco, gri, batch, 2000, 99)
+    assert np.array_equal(off.cpu().numpy(), co)
+    assert np.array_equal(np.sort(np.unique(rows.cpu().numpy())), src)
+    builder.close()
 
 
 @pytest.mark.parametrize("Vs,E,skew", [

@@ -430,3 +430,64 @@ def test_edge_parallel_kernels_over_runs_of_empty_rows(device):
     want = (hs[ri].reshape(E, H, Fh).astype(np.float64) * xd[seg].reshape(E, H, Fh)).sum(2)
     scale = np.abs(hs[ri].reshape(E, H, Fh).astype(np.float64) * xd[seg].reshape(E, H, Fh)).sum(2)
     check(galpha.cpu().numpy(), want.astype(np.float32), scale=scale.astype(np.float32))
+
+
+@pytest.mark.parametrize("Vd,fanout", [(3000, 10), (20000, 25)])
+def test_bounded_attention_and_aggregation_equal_the_unbounded_calls(device, Vd, fanout):
+    """The entry points that take the caller's bound on a destination's edges (a sampled layer's fanout)
+    choose fewer launches, never other values: with an honest bound, with a bound far too small (the
+    launch that was told every segment is short computes the longer ones by its slow path) and with a
+    bound of 0 they match the unbounded calls -- exactly where the same kernel serves the segment, within
+    1e-5 where another one does."""
+    H, Fh, Vs = 4, 8, 5000
+    rng = np.random.default_rng(Vd)
+    deg = rng.integers(0, fanout + 1, Vd)
+    deg[5] = 700  # far beyond the bound: 2,800 values in one segment
+    co = np.concatenate([[0], np.cumsum(deg)]).astype(np.uint32)
+    E = int(co[-1])
+    ri = rng.integers(0, Vs, E).astype(np.uint32)
+    el = rng.standard_normal((Vs, H)).astype(np.float32)
+    er = rng.standard_normal((Vd, H)).astype(np.float32)
+    x = rng.standard_normal((Vs, H * Fh)).astype(np.float32)
+    gal = rng.standard_normal((E, H)).astype(np.float32)
+    dco, dri, del_, der, dx, dgal = (dev(t, device) for t in (co, ri, el, er, x, gal))
+    s = stream()
+
+    def attention(bound):
+        alpha = torch.full((E, H), float("nan"), device=device)
+        gs = torch.full((E, H), float("nan"), device=device)
+        ger = torch.full((Vd, H), float("nan"), device=device)
+        out = torch.full((Vd, H * Fh), float("nan"), device=device)
+        if bound is None:
+            call("nts_gat_attention_fwd", ptr(alpha), ptr(del_), ptr(der), ptr(dco), ptr(dri), Vd, H, 0.2, s)
+            call("nts_gat_attention_bwd", ptr(gs), ptr(ger), ptr(dgal), ptr(alpha), ptr(del_), ptr(der), ptr(dco),
+                 ptr(dri), Vd, H, 0.2, s)
+            call("nts_spmm_gather_heads", ptr(dx), ptr(out), ptr(alpha), 0, ptr(dco), ptr(dri), Vd, E, H, Fh, 0, s)
+        else:
+            call("nts_gat_attention_fwd_bounded", ptr(alpha), ptr(del_), ptr(der), ptr(dco), ptr(dri), Vd, H, 0.2,
+                 bound, s)
+            call("nts_gat_attention_bwd_bounded", ptr(gs), ptr(ger), ptr(dgal), ptr(alpha), ptr(del_), ptr(der),
+                 ptr(dco), ptr(dri), Vd, H, 0.2, bound, s)
+            call("nts_spmm_gather_heads_bounded", ptr(dx), ptr(out), ptr(alpha), 0, ptr(dco), ptr(dri), Vd, E, H, Fh, 0,
+                 bound, s)
+        return [t.cpu().numpy() for t in (alpha, gs, ger, out)]
+
+    want = attention(None)
+    assert all(np.isfinite(t).all() for t in want)
+    for bound in (0, fanout, 2, 1000, 100000):
+        got = attention(bound)
+        for a, b in zip(got, want):
+            assert np.isfinite(a).all()
+            np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
+    # the plain aggregation with a bound: same values as without, bit for bit on rows within the bound
+    w = rng.random(E).astype(np.float32)
+    dw = dev(w, device)
+    xin = dev(rng.standard_normal((Vs, 100)).astype(np.float32), device)
+    ref = torch.empty(Vd, 100, device=device)
+    call("nts_spmm_gather", ptr(xin), ptr(ref), ptr(dw), ptr(dco), ptr(dri), 0, Vd, E, 100, 0, s)
+    for bound in (0, fanout, 3, 5000):
+        out = torch.full((Vd, 100), float("nan"), device=device)
+        call("nts_spmm_gather_bounded", ptr(xin), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, Vd, E, 100, 0, bound, s)
+        rows = torch.from_numpy(np.flatnonzero(deg <= 256)).to(device)
+        assert torch.equal(out[rows], ref[rows])
+        assert torch.allclose(out, ref, rtol=1e-5, atol=1e-5)
