@@ -62,6 +62,9 @@ long nts_trace_ranges_emitted(void);
  * call, cuda/ntsCUDAGraphOP.cu:595-653).  nts_scratch_trim returns the current device's unused
  * scratch to the driver; work queued earlier is not affected. */
 int nts_scratch_trim(void);
+/* Scratch blocks the library has taken from its pool so far in this process (every call that needs
+ * scratch takes one or two): lets a caller check that a code path allocates nothing. */
+long nts_scratch_alloc_count(void);
 
 /* ---------------------------------------------------------------------------------------------
  * Memory, copies, streams
@@ -194,7 +197,9 @@ int nts_spmm_gather_bounded(const float *in, float *out, const float *w, const u
  * both sizes in nts_last_error() and launches nothing; calls below 65,536 edges need no scratch.
  * Every call on a device uses the same array: calls that overlap on one device (two streams, two
  * host threads) race, so a caller serialises them.  Nothing in the array has to be zero on entry:
- * each call writes every word before it reads it. */
+ * each call writes every word before it reads it.  Under stream capture: calls below 2^22 edges record
+ * kernel launches only; from 2^22 edges up the pieces are ordered with the runtime library's radix sort,
+ * which may record fill nodes, so such a call is not for capture. */
 #define NTS_SPMM_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int nts_spmm_gather_static_scratch(const float *in, float *out, const float *w, const uint32_t *offsets,
                                    const uint32_t *indices, uint32_t index_base, uint32_t rows,
@@ -269,7 +274,11 @@ int nts_spmm_plan_reserve(nts_spmm_plan_t *plan, uint32_t F);
  * serialised per plan, and a call on another stream than the previous one first waits, on the
  * device, for that call's last kernel; calls on one plan therefore never overlap on the device,
  * from however many streams or host threads they come (use one plan per stream for overlap).  The
- * caller must not destroy a plan while a call on it is being made. */
+ * caller must not destroy a plan while a call on it is being made.  A call on a stream that is being
+ * captured is recorded without that ordering (no event is waited for or recorded under capture): the
+ * caller orders replays of the captured call against eager calls and other streams that use the plan.
+ * `in` must hold all n_index rows the plan was built for: a plan that gathers from a padded copy of
+ * the input (see below) copies every row of `in` on each call. */
 int nts_spmm_gather_planned(nts_spmm_plan_t *plan, const float *in, float *out, const float *w,
                             const uint32_t *offsets, const uint32_t *indices, uint32_t index_base,
                             uint32_t F, int accumulate, nts_stream_t stream);

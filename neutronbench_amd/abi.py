@@ -29,6 +29,7 @@ SIGNATURES = {
     "nts_abi_version": [],
     "nts_trace_ranges_emitted": [],
     "nts_scratch_trim": [],
+    "nts_scratch_alloc_count": [],
     "nts_malloc_device": [ctypes.POINTER(_vp), _sz],
     "nts_free_device": [_vp],
     "nts_malloc_device_async": [ctypes.POINTER(_vp), _sz, _vp],
@@ -121,9 +122,9 @@ SIGNATURES = {
 _RESTYPES = {"nts_last_error": ctypes.c_char_p, "nts_fingerprint_finish": _u64, "nts_csr_from_csc_work_bytes": _sz,
              "nts_relabel_sources_work_bytes": _sz, "nts_sample_hop_work_bytes": _sz,
              "nts_chunk_from_edges_work_bytes": _sz, "nts_batch_builder_arena_bytes": _sz,
-             "nts_trace_ranges_emitted": ctypes.c_long}
+             "nts_trace_ranges_emitted": ctypes.c_long, "nts_scratch_alloc_count": ctypes.c_long}
 # Entry points whose int result is a value, not a status.
-_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_fingerprint_finish", "nts_trace_ranges_emitted", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
+_NO_STATUS = {"nts_last_error", "nts_abi_version", "nts_fingerprint_finish", "nts_scratch_alloc_count", "nts_trace_ranges_emitted", "nts_csr_from_csc_work_bytes", "nts_relabel_sources_work_bytes",
               "nts_sample_hop_work_bytes", "nts_chunk_from_edges_work_bytes", "nts_batch_builder_arena_bytes"}
 
 

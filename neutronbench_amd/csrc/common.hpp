@@ -64,6 +64,7 @@ struct TraceRange {
 hipError_t scratch_alloc(void **ptr, size_t bytes, hipStream_t stream);
 hipError_t scratch_free(void *ptr, hipStream_t stream);
 hipError_t scratch_trim();  // gives the current device's unused scratch back to the driver
+long scratch_alloc_count();  // scratch blocks handed out so far by this process
 
 // A scratch block that is returned to the pool when its scope ends, whichever way the function is
 // left (the error paths included); release() frees it early and reports the result.

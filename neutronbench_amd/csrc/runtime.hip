@@ -137,7 +137,13 @@ hipError_t scratch_pool(hipMemPool_t *pool) {
 }
 }  // namespace
 
+namespace {
+std::atomic<long> g_scratch_allocs{0};
+}
+long scratch_alloc_count() { return g_scratch_allocs.load(); }
+
 hipError_t scratch_alloc(void **ptr, size_t bytes, hipStream_t stream) {
+  g_scratch_allocs.fetch_add(1);
   hipMemPool_t pool = nullptr;
   if (scratch_pool(&pool) != hipSuccess) {
     (void)hipGetLastError();                   // a device without pool support: the device's default pool
@@ -168,6 +174,8 @@ extern "C" {
 
 const char *nts_last_error(void) { return nts::g_last_error; }
 long nts_trace_ranges_emitted(void) { return nts::trace_ranges_emitted(); }
+long nts_scratch_alloc_count(void) { return nts::scratch_alloc_count(); }
+
 int nts_scratch_trim(void) {
   hipError_t err = nts::scratch_trim();
   return err == hipSuccess ? NTS_OK : nts::fail_hip(err, "nts_scratch_trim");

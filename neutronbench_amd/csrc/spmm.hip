@@ -1821,11 +1821,25 @@ int reserve_locked(nts_spmm_plan *plan, uint32_t F, bool heads) {
 
 // A call on `stream` is about to use the plan's scratch: if the previous call ran on another stream,
 // `stream` first waits for it (in stream order, the host does not block).  Caller holds plan->mu.
+// A stream that is being captured records its launches instead of running them: a call under capture
+// neither waits for the plan's event (that would pull the other stream's work into the capture, or
+// fail) nor records it, and leaves the plan's bookkeeping alone -- replays of the captured call are
+// ordered against other uses of the plan by the caller.
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
 int enter_stream(nts_spmm_plan *plan, hipStream_t stream) {
+  if (stream_is_capturing(stream)) return NTS_OK;
   if (plan->in_flight && plan->last_stream != stream) NTS_HIP_TRY(hipStreamWaitEvent(stream, plan->done, 0));
   return NTS_OK;
 }
 int leave_stream(nts_spmm_plan *plan, hipStream_t stream) {
+  if (stream_is_capturing(stream)) return NTS_OK;
   NTS_HIP_TRY(hipEventRecord(plan->done, stream));
   plan->last_stream = stream;
   plan->in_flight = true;

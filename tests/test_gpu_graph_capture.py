@@ -55,4 +55,18 @@ def test_planned_aggregation_and_softmax_in_a_hip_graph(device):
         assert torch.equal(got_out, out), f"replay {rep}: aggregation differs from the eager launch"
         assert torch.equal(got_alpha, alpha), f"replay {rep}: softmax differs from the eager launch"
         assert float(out.abs().sum()) > 0
+    # An eager call on another stream after the capture: the captured call left no event behind that
+    # this one would wait on (a wait on an event recorded under capture is an error), and once the
+    # caller has ordered the streams the result is the eager one again.
+    torch.cuda.synchronize()
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(other):
+        call("nts_spmm_gather_planned", plan.handle, ptr(x), ptr(out), ptr(w), ptr(dco), ptr(dri), 0, F, 0,
+             other.cuda_stream)
+    other.synchronize()
+    want = out.clone()
+    out.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
     plan.close()

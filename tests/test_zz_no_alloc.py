@@ -45,8 +45,17 @@ def _both(device, Vd, Vs, F, mean_deg, hubs, seed, accumulate=0):
     outs = []
     for name in ("nts_spmm_gather", "nts_spmm_gather_static_scratch"):
         out = dev(init, device) if accumulate else torch.full((Vd, F), float("nan"), device=device)
+        torch.cuda.synchronize()
+        blocks_before = call("nts_scratch_alloc_count")
+        free_before = torch.cuda.mem_get_info()[0]
         call(name, ptr(dx), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, Vd, E, F, accumulate, stream())
         torch.cuda.synchronize()
+        if name == "nts_spmm_gather_static_scratch":
+            # the property the entry point exists for: no scratch block taken, no device memory gone
+            assert call("nts_scratch_alloc_count") == blocks_before
+            assert torch.cuda.mem_get_info()[0] == free_before
+        elif E >= 65536:
+            assert call("nts_scratch_alloc_count") > blocks_before  # the pooled path does take scratch here
         outs.append(out.cpu().numpy())
     pooled, fixed = outs
     assert np.array_equal(pooled.view(np.uint32), fixed.view(np.uint32)), "static-scratch result differs"
@@ -103,3 +112,45 @@ def test_request_beyond_the_fixed_scratch_is_refused(device):
     assert "fixed scratch holds 67108864" in msg and "needs" in msg, msg
     torch.cuda.synchronize()
     assert bool((out == 7.0).all())
+
+
+def test_static_scratch_call_recorded_into_a_hip_graph(device):
+    """The use the entry point is advertised for: a call recorded into a HIP graph (kernel launches
+    only) and replayed with new inputs, eager work and synchronisations in between; every replay equals
+    nts_spmm_gather on the same inputs bit for bit."""
+    Vd, Vs, F = 20000, 30000, 64
+    co, ri = _block(Vd, Vs, 40, [50000, 4000, 300], seed=7)
+    E = ri.size
+    assert 65536 <= E < (1 << 22)
+    rng = np.random.default_rng(8)
+    dw, dco, dri = dev(rng.random(E).astype(np.float32), device), dev(co, device), dev(ri, device)
+    x = torch.zeros(Vs, F, device=device)
+    out = torch.zeros(Vd, F, device=device)
+    ref = torch.zeros(Vd, F, device=device)
+
+    def run(stream_handle):
+        call("nts_spmm_gather_static_scratch", ptr(x), ptr(out), ptr(dw), ptr(dco), ptr(dri), 0, Vd, E, F, 0,
+             stream_handle)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(side.cuda_stream)  # the first call on a device looks the scratch address up: before the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    blocks_before = call("nts_scratch_alloc_count")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(torch.cuda.current_stream().cuda_stream)
+    for rep in range(4):
+        x.copy_(torch.from_numpy(rng.standard_normal((Vs, F)).astype(np.float32)))
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        call("nts_spmm_gather", ptr(x), ptr(ref), ptr(dw), ptr(dco), ptr(dri), 0, Vd, E, F, 0, stream())
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref), f"replay {rep} differs from nts_spmm_gather"
+        assert float(ref.abs().sum()) > 0
+    # nothing but the comparison calls took scratch
+    assert call("nts_scratch_alloc_count") == blocks_before + 4
