@@ -38,6 +38,9 @@ F_IN, F_HID = 602, 128
 # its CPU operator, and its GPU operator class compiled against this library's host veneer.
 REFERENCE_PROGRAM = os.path.join(ROOT, "oracle", "_ref", "ref_fullgraph_cpu")
 REFERENCE_GPU_PROGRAM = os.path.join(ROOT, "oracle", "_ref", "ref_fullgraph_gpu")
+# The reference's own sampler and mini-batch CPU operator behind a small driver (oracle/ref_minibatch_driver.cpp,
+# built by oracle/build_toolkits.sh where the reference tree is present).
+REFERENCE_MINIBATCH_PROGRAM = os.path.join(ROOT, "oracle", "_ref", "ref_minibatch")
 HBM_PEAK_GBS = 8000.0
 # rocprofv3 counter summary of the dominant kernel on this workload; it names the kernel sources it was
 # measured with, and its traffic figure is only quoted while those sources are unchanged.
@@ -515,7 +518,8 @@ def run_reference_programs(torch, chunk, x0, h1, V, sample_edges, reps):
             rows = re.findall(pat, r.stdout)
             if r.returncode == 0 and len(rows) == 2:
                 gpu = {"what": "the reference's ForwardSingleGPUfuseOp class, unchanged, over the host veneer "
-                               "(torch::zeros output, accumulate=1, stream synchronisation per call); wall time per "
+                               "(torch::zeros output, zero_buffer, the aggregation, stream synchronisation per call; the veneer "
+                               "writes into the output it has just seen cleared and checks its schedule on a side stream); wall time per "
                                f"call, median of {reps} after 1 warm-up; the veneer builds its schedule on the third "
                                "identical call, so the best time is the steady state",
                        "edges": int(rows[0][0])}
@@ -606,6 +610,8 @@ def run_epochs(torch, names, with_cpu, cpu_batches):
             finally:
                 shutil.rmtree(dump, ignore_errors=True)
             cpu = epoch_cpu_baseline(torch, name, host, serial["batches"], cpu_batches) if with_cpu else None
+            if cpu is not None and not cfg.get("heads"):
+                cpu["reference_sampler_and_operator"] = epoch_reference_cpu(name, host, serial["batches"], cpu_batches)
             records[name] = {
                 "epoch_s": serial["epoch_s"], "stage_s": serial.get("stage_s"), "batches": serial["batches"],
                 "batch_size": cfg["batch"], "fanout_output_side_first": cfg["fanout"], "heads": cfg.get("heads", 0),
@@ -648,6 +654,59 @@ def run_epoch_workload(args):
         "cpu_baseline": rec["cpu_baseline"],
     }
     print(json.dumps(line))
+
+
+def epoch_reference_cpu(name, host, n_batches, k_batches):
+    """The reference's own host side of a mini-batch -- Sampler::sample_one (neighbour pick, relabelling,
+    CSR, weights) and MiniBatchFuseOp forward + backward of every layer -- timed by oracle/_ref/ref_minibatch
+    on k batches of the same graph (its loader reads the edge list this function writes), extrapolated to
+    the epoch.  None when the program has not been built (no reference tree) or fails."""
+    import re
+    import shutil
+    import subprocess
+    import tempfile
+
+    import numpy as np
+
+    from neutronbench_amd import epoch
+
+    if not os.path.exists(REFERENCE_MINIBATCH_PROGRAM):
+        return None
+    cfg = epoch.CONFIGS[name]
+    V = host["V"]
+    tmp = tempfile.mkdtemp(prefix="nts_refmb_")
+    try:
+        owner = np.repeat(np.arange(V, dtype=np.uint32), np.diff(host["co"].astype(np.int64)))
+        np.stack([host["ri"], owner], 1).astype(np.uint32).tofile(os.path.join(tmp, "g.edge"))
+        del owner
+        layers = "-".join(map(str, [cfg["F"]] + [cfg["hidden"]] * (len(cfg["fanout"]) - 1) + [cfg["classes"]]))
+        fan = ",".join(map(str, reversed(cfg["fanout"])))  # the reference reverses its FANOUT string
+        lines = dict(ALGORITHM="GCNNEIGHBORGPU", VERTICES=V, EPOCHS=1, LAYERS=layers, FANOUT=fan, VALFANOUT=fan,
+                     BATCH_SIZE=cfg["batch"], BATCH_TYPE="shuffle", EDGE_FILE=f"{tmp}/g.edge", FEATURE_FILE="none",
+                     LABEL_FILE="none", MASK_FILE="none", MINI_PULL=1, CACHE_TYPE="none", PIPELINES=1, MODE="pipeline",
+                     CLASSES=1, PROC_OVERLAP=0, PROC_LOCAL=0, PROC_CUDA=0, PROC_REP=0, LOCK_FREE=1, TIME_SKIP=0, RUNS=1,
+                     LEARN_RATE=0.01, WEIGHT_DECAY=0.0001, DECAY_RATE=0.97, DECAY_EPOCH=100, DROP_RATE=0.5)
+        with open(os.path.join(tmp, "g.cfg"), "w") as f:
+            f.write("".join(f"{k}:{v}\n" for k, v in lines.items()))
+        t0 = time.perf_counter()
+        r = subprocess.run([REFERENCE_MINIBATCH_PROGRAM, os.path.join(tmp, "g.cfg"), str(k_batches), "time"],
+                           capture_output=True, text=True, timeout=300, cwd=tmp)
+        wall = time.perf_counter() - t0
+        m = re.search(r"reference mini-batch cpu timing: batches=(\d+) sample_s=([0-9.]+) aggregate_s=([0-9.]+) "
+                      r"sampled_edges=(\d+) threads=(\d+)", r.stdout)
+        if r.returncode != 0 or not m or int(m.group(1)) == 0:
+            return None
+        k, ts, ta = int(m.group(1)), float(m.group(2)), float(m.group(3))
+        return {"value": round((ts + ta) / k * n_batches, 4), "unit": "s", "cores": int(m.group(5)), "kind": "reference",
+                "sample": f"the reference's Sampler::sample_one and MiniBatchFuseOp (forward + backward of every layer) on "
+                          f"{k} batches of {cfg['batch']} after one untimed batch, on its own loader's copy of the graph, "
+                          f"extrapolated to {n_batches} batches: per batch sampling {ts / k * 1e3:.2f} ms, aggregation "
+                          f"{ta / k * 1e3:.2f} ms ({int(m.group(4)) // k} sampled edges); the feature gather is not "
+                          f"included; built with the METIS shim of oracle/build_toolkits.sh; program wall time {wall:.1f} s"}
+    except (OSError, subprocess.SubprocessError):
+        return None
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
 
 
 def epoch_cpu_baseline(torch, name, host, n_batches, k_batches):

@@ -13,10 +13,15 @@
 // (sum|terms| from the CPU operator run on |input|; edge weights are positive) and how many output
 // rows are equal bit for bit.
 //
-//   usage: ref_minibatch <cfg file> <batches>
+//   usage: ref_minibatch <cfg file> <batches> [time]
+// With `time` nothing touches the device: after one untimed batch, the reference's Sampler::sample_one
+// (neighbour pick, relabelling, CSR, weights: its whole host side) and its CPU operator MiniBatchFuseOp
+// (forward and backward of every layer) are timed on <batches> batches and the totals printed -- the
+// reference's own CPU cost of the steps this library moves to the GPU.
 #include "core/neutronstar.hpp"  // what the toolkits include: graph, sampler, operators
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <string>
@@ -75,6 +80,42 @@ int main(int argc, char **argv) {
   std::vector<VertexId> train_nids;
   for (VertexId v = 0; v < graph->vertices; v += 2) train_nids.push_back(v);  // every other vertex trains
   Sampler *sampler = new Sampler(fully_rep_graph, train_nids, 1, false);
+  if (argc > 3 && std::string(argv[3]) == "time") {
+    auto now = [] { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); };
+    const int n_layers = graph->gnnctx->layer_size.size() - 1;
+    double t_sample = 0, t_aggregate = 0;
+    long edges = 0;
+    int timed = 0;
+    torch::manual_seed(1234);
+    for (int b = 0; b < batches + 1 && sampler->work_offset < sampler->work_range[1]; ++b) {
+      SampledSubgraph *ssg = sampler->subgraph_list[0];
+      double t0 = now();
+      sampler->sample_one(ssg, graph->config->batch_type, true);
+      const double ts = now() - t0;
+      double ta = 0;
+      for (int l = 0; l < n_layers; ++l) {
+        sampCSC *sg = ssg->sampled_sgs[l];
+        const long F = graph->gnnctx->layer_size[l];
+        NtsVar X = torch::randn({(long)sg->src_size, F});
+        NtsVar G = torch::randn({(long)sg->v_size, F});
+        nts::op::MiniBatchFuseOp op(ssg, graph, l);
+        t0 = now();
+        NtsVar Y = op.forward(X);
+        NtsVar D = op.backward(G);
+        ta += now() - t0;
+        if (b > 0) edges += sg->e_size;
+      }
+      if (b > 0) {  // the first batch starts the thread pools and touches the buffers for the first time
+        t_sample += ts;
+        t_aggregate += ta;
+        ++timed;
+      }
+      sampler->reverse_sgs(ssg);
+    }
+    printf("reference mini-batch cpu timing: batches=%d sample_s=%.6f aggregate_s=%.6f sampled_edges=%ld threads=%d\n", timed,
+           t_sample, t_aggregate, edges, omp_get_max_threads());
+    return 0;
+  }
   Cuda_Stream *cs = new Cuda_Stream();
   const int layers = graph->gnnctx->layer_size.size() - 1;
   torch::manual_seed(1234);
