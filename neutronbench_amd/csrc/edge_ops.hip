@@ -168,13 +168,25 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__
 // row: together they load 8 S consecutive edge rows at once, and every lane of the group then adds
 // those values in edge order, fetching each from the lane that loaded it.  The sum is the same
 // running fp32 sum, bit for bit; only the loads are spread.
+//
+// Rows of more than `coop_limit` edges (G <= 8 only) are taken by the whole wavefront after the
+// set's other rows: all 64 lanes load consecutive edge rows (256 values of type V per round), stage
+// them in a tile of LDS private to the wavefront, and request the next round's rows before the
+// lanes that each own one float of the output row add the staged values in edge order -- again the
+// same running fp32 sum (the tile is padded with zeros, and a sum that starts at +0 is never -0, so
+// the padding changes no bit).  A 1,000-edge row of 16-byte values is four such rounds instead of
+// sixteen dependent ones.
 template <typename V, int G, int S>
 __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__restrict__ out,
                                                                           const V *__restrict__ msg,
                                                                           const uint32_t *__restrict__ off,
                                                                           const uint32_t *__restrict__ perm,
                                                                           uint32_t rows, uint32_t Fv, int accumulate,
-                                                                          uint32_t long_limit) {
+                                                                          uint32_t long_limit, uint32_t coop_limit) {
+  constexpr bool kCoop = G <= 8;
+  constexpr int kCoopU = sizeof(V) == 16 ? 4 : 8;           // loads per lane and round on the cooperative path
+  constexpr uint32_t kCoopFloats = kWave * kCoopU * (sizeof(V) / 4);  // floats of a wavefront's tile
+  __shared__ float coop_tile[kCoop ? 4 : 1][kCoop ? kCoopFloats : 1];
   // Rows a wavefront takes at a time: eight per lane group, so that a wavefront with two groups
   // (128-byte-wide vectors) is not left with 32 rows per group while others have finished.
   constexpr uint32_t kSet = (kWave / (G * S)) * 8 < kWave ? (kWave / (G * S)) * 8 : kWave;
@@ -193,6 +205,12 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
       my_e0 = off[base + lane];
       my_e1 = off[base + lane + 1];
       mine = my_e1 - my_e0 <= long_limit;  // longer rows belong to the block kernels
+    }
+    uint64_t coop = 0;
+    if (kCoop) {
+      const bool shared = mine && my_e1 - my_e0 > coop_limit;
+      coop = __ballot(shared);
+      if (shared) mine = false;
     }
     if (G == 1) {
       // Rows one vector wide (the per-head values of an attention layer): a lane sums its own row when
@@ -322,6 +340,55 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
             *p = res;
           }
           have = false;
+        }
+      }
+    }
+    if (kCoop) {
+      // The long rows of this set, one after the other, by the whole wavefront.
+      constexpr uint32_t kSlots = kWave / G;           // edge rows per load of the wavefront
+      constexpr uint32_t kRound = kSlots * kCoopU;     // edge rows per round
+      constexpr uint32_t kPitch = G * NF;              // floats of an edge row in the tile
+      float *tile = coop_tile[threadIdx.x / kWave];
+      const uint32_t slot = lane / G;
+      const uint32_t comps = Fv * NF;                  // floats of an output row: lane c < comps owns float c
+      while (coop) {
+        const uint32_t j = static_cast<uint32_t>(__builtin_ctzll(coop));
+        coop &= coop - 1;
+        const uint32_t r0 = wave_read(my_e0, j), r1 = wave_read(my_e1, j);
+        V cur[kCoopU];
+        auto load_round = [&](uint32_t k) {
+#pragma unroll
+          for (int u = 0; u < kCoopU; ++u) {
+            cur[u] = V{};
+            const uint32_t idx = k + u * kSlots + slot;
+            if (idx < r1 && col_live) {
+              const uint32_t e = perm ? perm[idx] : idx;
+              cur[u] = msg[static_cast<size_t>(e) * Fv + col];
+            }
+          }
+        };
+        load_round(r0);
+        float acc = 0.f;
+        for (uint32_t k = r0; k < r1; k += kRound) {
+          __builtin_amdgcn_wave_barrier();  // the previous round's reads of the tile are done
+#pragma unroll
+          for (int u = 0; u < kCoopU; ++u) reinterpret_cast<V *>(tile)[u * kWave + lane] = cur[u];
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          if (k + kRound < r1) load_round(k + kRound);  // in flight while this round is added up
+          const uint32_t n = r1 - k < kRound ? r1 - k : kRound;
+          if (lane < comps) {
+            for (uint32_t i = 0; i < n; i += 8) {  // whole groups of eight: the tile's tail holds zeros
+#pragma unroll
+              for (uint32_t t = 0; t < 8; ++t) acc += tile[(i + t) * kPitch + lane];
+            }
+          }
+        }
+        if (lane < comps) {
+          float *p = reinterpret_cast<float *>(out) + static_cast<size_t>(base + j) * comps + lane;
+          if (accumulate) acc += *p;
+          *p = acc;
         }
       }
     }
@@ -1626,6 +1693,18 @@ int release_long_rows(LongRows &lr) {
 
 constexpr unsigned kLongGrid = 512;  // blocks of the long-row kernels; they stride over the list
 
+// Edges of a row above which the whole wavefront takes it (rows up to eight lanes wide); NTS_EDGE_SUM_COOP
+// in the environment overrides it (0 = never).
+uint32_t coop_limit() {
+  static const uint32_t value = [] {
+    const char *env = getenv("NTS_EDGE_SUM_COOP");
+    if (!env) return 64u;
+    const long v = atol(env);
+    return v <= 0 ? kNoLimit : static_cast<uint32_t>(v);
+  }();
+  return value;
+}
+
 template <typename V>
 void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_t *perm, uint32_t rows, uint32_t Fv,
                         int accumulate, uint32_t limit, hipStream_t stream) {
@@ -1636,7 +1715,7 @@ void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_
     const uint32_t set = (kWave / ((GG) * (SS))) * 8 < kWave ? (kWave / ((GG) * (SS))) * 8 : kWave;            \
     const uint32_t blocks = ceil_div(rows, 4 * set); /* at most `set` rows per wavefront at a time */          \
     hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG, SS>), dim3(blocks < 16384u ? blocks : 16384u), \
-                       dim3(256), 0, stream, out, msg, off, perm, rows, Fv, accumulate, limit);                 \
+                       dim3(256), 0, stream, out, msg, off, perm, rows, Fv, accumulate, limit, coop_limit());   \
   } while (0)
     switch (lanes_for(Fv)) {  // rows narrower than eight lanes are shared by eight lanes all the same
       case 1: NTS_BALANCED(1, 8); break;

@@ -5,6 +5,9 @@
 //   gather_sum  every wavefront reads 512 rows of 602 floats picked by a hash from a table of the given
 //               size with 4-byte lanes, ten loads per row and four rows in flight -- the access pattern
 //               of the F = 602 aggregation without its arithmetic, indices or output
+//   gather16    every lane reads 16-byte rows picked by a hash from a table of the given size, eight in
+//               flight per lane, either one row per lane (16-byte loads) or one row per four lanes (4-byte
+//               loads) -- the el[src] reads of the fused attention kernels without anything else
 // Prints GB/s per case.  A measuring tool: nothing in the library calls it.
 #include <hip/hip_runtime.h>
 #include <cstdio>
@@ -43,6 +46,27 @@ __global__ __launch_bounds__(256) void gather_sum(const float* __restrict__ p, u
   float s = 0; for (int k = 0; k < 10; ++k) s += acc[k];
   if (s == 12345.678f) out[0] = s;
 }
+// random 16-byte rows: QUAD = false: one row per lane; true: one row per four adjacent lanes, 4 bytes each
+template <bool QUAD>
+__global__ __launch_bounds__(256) void gather16(const float* __restrict__ p, uint32_t n_rows, uint32_t per_lane, float* out) {
+  const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+  uint32_t state = (QUAD ? t >> 2 : t) * 2654435761u + 12345u;
+  float acc = 0.f;
+  for (uint32_t r = 0; r < per_lane; r += 8) {
+    uint32_t row[8];
+    for (int u = 0; u < 8; ++u) { state = state * 1664525u + 1013904223u; row[u] = (uint32_t)(((uint64_t)(state >> 4) * n_rows) >> 28); }
+    if (QUAD) {
+      float v[8];
+      for (int u = 0; u < 8; ++u) v[u] = p[(size_t)row[u] * 4 + (t & 3)];
+      for (int u = 0; u < 8; ++u) acc += v[u];
+    } else {
+      float4 v[8];
+      for (int u = 0; u < 8; ++u) v[u] = reinterpret_cast<const float4*>(p)[row[u]];
+      for (int u = 0; u < 8; ++u) acc += v[u].x + v[u].y + v[u].z + v[u].w;
+    }
+  }
+  if (acc == 12345.678f) out[0] = acc;
+}
 int main() {
   float* out; CK(hipMalloc(&out, 256));
   size_t sizes[] = {2ull<<20, 8ull<<20, 24ull<<20, 64ull<<20, 128ull<<20, 200ull<<20, 512ull<<20, 2048ull<<20, 8192ull<<20};
@@ -76,6 +100,28 @@ int main() {
     double gb = (double)waves * rpw * F * 4 / 1e9;
     printf("gather_sum table %6u rows (%7.1f MiB): %8.1f GB/s (%.3f ms per %.1f GB)\n", n_rows, bytes / 1048576.0, gb * 3 / ms * 1e3, ms / 3, gb);
     fflush(stdout);
+    CK(hipFree(p));
+  }
+  // random gathers of 16-byte rows (2.449 M rows = the el table of a Products-shaped graph with four heads)
+  for (uint32_t n_rows : {65536u, 262144u, 2449029u, 16777216u, 134217728u}) {
+    float* p; size_t bytes = (size_t)n_rows * 16; CK(hipMalloc(&p, bytes)); CK(hipMemset(p, 0, bytes));
+    for (int quad = 0; quad < 2; ++quad) {
+      const uint32_t lanes = 256 * 2048 * (quad ? 4 : 1), per_lane = 256;  // 134 M row reads per launch
+      auto launch = [&] {
+        if (quad) hipLaunchKernelGGL(gather16<true>, dim3(lanes / 256), dim3(256), 0, 0, p, n_rows, per_lane, out);
+        else hipLaunchKernelGGL(gather16<false>, dim3(lanes / 256), dim3(256), 0, 0, p, n_rows, per_lane, out);
+      };
+      launch();
+      CK(hipEventRecord(e0));
+      for (int r = 0; r < 3; ++r) launch();
+      CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+      float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+      const double rows = 256.0 * 2048 * per_lane;
+      printf("gather16 table %9u rows (%7.1f MiB) %s: %7.1f G rows/s = %7.1f GB/s of rows (%.3f ms per %.0f M rows)\n", n_rows,
+             bytes / 1048576.0, quad ? "4-byte lanes, 4 per row" : "16-byte lanes, 1 per row", rows * 3 / ms / 1e6,
+             rows * 16 * 3 / ms / 1e6, ms / 3, rows / 1e6);
+      fflush(stdout);
+    }
     CK(hipFree(p));
   }
   return 0;

@@ -491,3 +491,50 @@ def test_bounded_attention_and_aggregation_equal_the_unbounded_calls(device, Vd,
         rows = torch.from_numpy(np.flatnonzero(deg <= 256)).to(device)
         assert torch.equal(out[rows], ref[rows])
         assert torch.allclose(out, ref, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("F", [1, 4, 8, 12, 32, 100])
+def test_long_rows_of_narrow_messages_are_the_edge_order_sum(device, F):
+    """Rows of 65 .. 1,024 edges, which a whole wavefront adds up when the row is at most eight lanes wide
+    (F <= 8 floats, or <= 32 in 16-byte vectors), next to short rows that lane groups take: the same bits as
+    the running fp32 sum in edge order, with and without accumulation; the 5,000-edge row goes to the block
+    kernel (slices added in a fixed order: within rounding)."""
+    print(f"case F={F}", flush=True)
+    Vs = 20000
+    rng = np.random.default_rng(300 + F)
+    deg = rng.integers(0, 12, Vs)
+    deg[[3, 77, 1234, 19999]] = [65, 256, 1000, 5000]
+    deg[5000:5040] = rng.integers(60, 700, 40)
+    deg[5040:5044] = [1024, 1023, 257, 513]
+    ro = np.concatenate([[0], np.cumsum(deg)]).astype(np.uint32)
+    E = int(ro[-1])
+    perm = rng.permutation(E).astype(np.uint32)
+    msg = rng.standard_normal((E, F)).astype(np.float32)
+    init = rng.standard_normal((Vs, F)).astype(np.float32)
+    want = np.zeros((Vs, F), np.float32)
+    for r in np.flatnonzero(deg):
+        acc = np.zeros(F, np.float32)
+        for k in range(int(ro[r]), int(ro[r + 1])):
+            acc = acc + msg[perm[k]]
+        want[r] = acc
+    dro, dperm, dmsg = dev(ro, device), dev(perm, device), dev(msg, device)
+    s = stream()
+    chains = deg <= 1024
+    out = torch.full((Vs, F), float("nan"), device=device)
+    call("nts_gather_edge_to_src", ptr(out), ptr(dmsg), ptr(dro), ptr(dperm), Vs, F, 0, s)
+    got = out.cpu().numpy()
+    assert np.array_equal(got[chains], want[chains])
+    np.testing.assert_allclose(got[~chains], want[~chains], rtol=1e-4, atol=1e-4)
+    acc = dev(init, device)
+    call("nts_gather_edge_to_src", ptr(acc), ptr(dmsg), ptr(dro), ptr(dperm), Vs, F, 1, s)
+    assert np.array_equal(acc.cpu().numpy()[chains], (want + init)[chains])
+    # the same rows as destinations of the edge list in its own order (no permutation)
+    out = torch.full((Vs, F), float("nan"), device=device)
+    call("nts_gather_edge_to_dst", ptr(out), ptr(dmsg), ptr(dro), Vs, F, 0, s)
+    ident = np.zeros((Vs, F), np.float32)
+    for r in np.flatnonzero(chains & (deg > 0)):
+        a = np.zeros(F, np.float32)
+        for k in range(int(ro[r]), int(ro[r + 1])):
+            a = a + msg[k]
+        ident[r] = a
+    assert np.array_equal(out.cpu().numpy()[chains], ident[chains])
