@@ -28,7 +28,7 @@ struct HopLayout {
 
 struct Layout {
   HopLayout hop[kMaxHops];
-  size_t dst0, sizes, seed, ri_global, relabel_work, csr_work, scan_work, total;
+  size_t dst0, sizes, seed, ri_global, owner, relabel_work, csr_work, scan_work, total;
   size_t relabel_bytes, csr_bytes, scan_bytes;
 };
 
@@ -70,6 +70,7 @@ bool plan_layout(Layout *L, uint32_t V, uint32_t graph_edges, const int32_t *fan
     vd = H.vs_cap;
   }
   L->ri_global = take(static_cast<size_t>(e_max) * sizeof(uint32_t));
+  L->owner = take(static_cast<size_t>(e_max) * sizeof(uint32_t));  // destination slot of every edge of the hop in work
   L->relabel_bytes = nts_relabel_sources_work_bytes(V);
   // The sort and scan scratch is shared by the hops: the largest any of them asks for (a library
   // routine may pick another algorithm, with other needs, for a smaller input).
@@ -139,6 +140,9 @@ int enqueue_hops(nts_batch_builder *b, hipStream_t stream) {
   const uint64_t *seed_word = reinterpret_cast<const uint64_t *>(A + b->L.seed);
   uint32_t *dst = reinterpret_cast<uint32_t *>(A + b->L.dst0);
   uint32_t *ri_global = reinterpret_cast<uint32_t *>(A + b->L.ri_global);
+  uint32_t *owner = reinterpret_cast<uint32_t *>(A + b->L.owner);
+  // where csr_from_csc leaves the sorted keys: the source of every CSR edge
+  const uint32_t *csr_owner = reinterpret_cast<const uint32_t *>(A + b->L.csr_work);
   uint32_t *bits = reinterpret_cast<uint32_t *>(A + b->L.relabel_work);
   const uint32_t words = (b->V + 31) / 32;
   for (uint32_t h = 0; h < b->hops; ++h) {
@@ -158,7 +162,7 @@ int enqueue_hops(nts_batch_builder *b, hipStream_t stream) {
     if (int rc = hop_offsets(co, b->graph_co, dst, Vd, b->fanout[h], A + b->L.scan_work, b->L.scan_bytes, stream))
       return rc;
     if (int rc = hop_neighbors(ri_global, co, b->graph_co, b->graph_ri, dst, Vd, H.e_cap, b->fanout[h],
-                               device_seed(seed_word, h), bits, stream))
+                               device_seed(seed_word, h), bits, owner, stream))
       return rc;
     // Local ids; the unused tail of the edge array is padded with a key that sorts after every
     // source.
@@ -166,9 +170,9 @@ int enqueue_hops(nts_batch_builder *b, hipStream_t stream) {
                                  hop_sizes + 1, b->V, A + b->L.relabel_work, true, stream))
       return rc;
     if (int rc = csr_from_csc(ro, ci, perm, co, ri, Vd, Vs, E, H.e_cap, bits_for(H.vs_cap + 1), A + b->L.csr_work,
-                              stream))
+                              owner, stream))
       return rc;
-    if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, bits, words, stream)) return rc;
+    if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, bits, words, owner, csr_owner, stream)) return rc;
     dst = source;  // the next hop's destinations are this hop's sources (init_dst)
   }
   const size_t size_bytes = (b->hops + 1) * kSizeWords * sizeof(uint32_t);

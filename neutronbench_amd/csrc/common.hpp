@@ -139,7 +139,7 @@ int hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, Dev
                 size_t scan_tmp_bytes, hipStream_t stream);
 int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co, const uint32_t *graph_ri,
                   const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, DevSeed seed, uint32_t *mark_bits,
-                  hipStream_t stream);
+                  uint32_t *owner, hipStream_t stream);  // owner (nullable): [edge_cap] destination slot of every edge
 size_t hop_scan_bytes(uint32_t n);
 // fill_to > E: local[E .. fill_to) = fill_value (padding for a sort over a fixed capacity);
 // n_source_copy / e_out (nullable) receive the source count again / the edge count.  marked: the
@@ -147,13 +147,16 @@ size_t hop_scan_bytes(uint32_t n);
 int relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *n_source_copy, uint32_t *local,
                     const uint32_t *global_ids, DevCount E, uint32_t fill_to, uint32_t fill_value, uint32_t *e_out,
                     uint32_t V, void *work, bool marked, hipStream_t stream);
-// Sorts sort_n keys of key_bits bits (sort_n = E.cap, padded entries sort last).
+// Sorts sort_n keys of key_bits bits (sort_n = E.cap, padded entries sort last).  owner (nullable): the
+// destination slot of every CSC edge, which the neighbour pick can record; without it the slots are
+// searched for in co.  The sorted keys (the source of every CSR edge) stay at the start of `work`.
 int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, DevCount Vd,
-                 DevCount Vs, DevCount E, uint32_t sort_n, unsigned key_bits, void *work, hipStream_t stream);
+                 DevCount Vs, DevCount E, uint32_t sort_n, unsigned key_bits, void *work, const uint32_t *owner,
+                 hipStream_t stream);
 size_t csr_from_csc_bytes(uint32_t sort_n);
 int gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t *ri, const uint32_t *ro,
                      const uint32_t *ci, DevCount Vd, DevCount Vs, uint32_t *clear, uint32_t clear_words,
-                     hipStream_t stream);
+                     const uint32_t *csc_owner, const uint32_t *csr_owner, hipStream_t stream);  // owners nullable
 
 #if defined(__HIPCC__)
 // Value of `v` held by wavefront lane `lane` (lane must be wave-uniform); result is an SGPR.

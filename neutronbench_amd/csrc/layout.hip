@@ -32,12 +32,32 @@ __global__ __launch_bounds__(256) void offsets_from_sorted_kernel(uint32_t *__re
 // Both halves of the transposed structure from the sorted (source, CSC edge id) pairs in one launch:
 // thread t writes ro[t] (as above) when t <= Vs, and ci[t] = the destination that owns CSC edge
 // perm[t] when t < E.  perm may alias ci: each thread reads its own element before writing it.
+// owner (nullable): the destination slot of every CSC edge; with it ci is a gather instead of a
+// search, and ro comes from the places where the sorted keys change (thread t writes the offsets of
+// the sources keys[t-1]+1 .. keys[t], a loop of one step when every source has an edge) instead of a
+// search per source.
 __global__ __launch_bounds__(256) void csr_finish_kernel(uint32_t *__restrict__ ro, uint32_t *ci,
                                                          const uint32_t *__restrict__ keys, const uint32_t *perm,
                                                          const uint32_t *__restrict__ co, DevCount Vd, DevCount Vs,
-                                                         DevCount edges) {
+                                                         DevCount edges, const uint32_t *__restrict__ owner) {
   const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
   const uint32_t E = edges.get();
+  if (owner) {
+    const uint32_t vs = Vs.get();
+    if (E == 0) {
+      if (t <= vs) ro[t] = 0;
+      return;
+    }
+    if (t < E) {
+      const uint32_t here = keys[t] < vs ? keys[t] : vs;
+      const uint32_t from = t ? (keys[t - 1] < vs ? keys[t - 1] : vs) + 1 : 0u;
+      for (uint32_t s = from; s <= here; ++s) ro[s] = t;
+      if (t + 1 == E)
+        for (uint32_t s = here + 1; s <= vs; ++s) ro[s] = E;
+      ci[t] = owner[perm[t]];
+    }
+    return;
+  }
   if (t <= Vs.get()) {
     uint32_t lo = 0, hi = E;
     while (lo < hi) {
@@ -60,14 +80,18 @@ __device__ __forceinline__ float norm_weight(uint32_t out_deg, uint32_t in_deg) 
 // blockIdx.y (+ first) = 0: CSC edges e, owner = destination, other end = ri[e] (a source)   -> ewf
 //                        1: CSR edges k, owner = source, other end = ci[k] (a destination)    -> ewb
 // The edge count is read on the device (own_off[n_own]); threads stride over the edges.  `clear`
-// (nullable): `clear_words` words zeroed on the side for the caller's next step.
+// (nullable): `clear_words` words zeroed on the side for the caller's next step.  csc_owner / csr_owner
+// (nullable): the owner of every CSC / CSR edge where the caller has them (the neighbour pick's record
+// and the sorted keys of the transposition); without them the owner is searched for in the offsets.
 __global__ __launch_bounds__(256) void edge_weights_kernel(float *__restrict__ ewf, float *__restrict__ ewb,
                                                            const uint32_t *__restrict__ co,
                                                            const uint32_t *__restrict__ ri,
                                                            const uint32_t *__restrict__ ro,
                                                            const uint32_t *__restrict__ ci, DevCount Vd, DevCount Vs,
                                                            int first, uint32_t *__restrict__ clear,
-                                                           uint32_t clear_words) {
+                                                           uint32_t clear_words,
+                                                           const uint32_t *__restrict__ csc_owner,
+                                                           const uint32_t *__restrict__ csr_owner) {
   const int which = first + static_cast<int>(blockIdx.y);
   const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
   const uint64_t start = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -77,11 +101,12 @@ __global__ __launch_bounds__(256) void edge_weights_kernel(float *__restrict__ e
   const uint32_t *other_off = which == 0 ? ro : co;
   const uint32_t *other_idx = which == 0 ? ri : ci;
   float *wout = which == 0 ? ewf : ewb;
+  const uint32_t *known = which == 0 ? csc_owner : csr_owner;
   if (!wout) return;
   const uint32_t n_own = which == 0 ? Vd.get() : Vs.get();
   const uint32_t E = own_off[n_own];
   for (uint64_t e = start; e < E; e += stride) {
-    const uint32_t o = owner_of(own_off, n_own, static_cast<uint32_t>(e));
+    const uint32_t o = known ? known[e] : owner_of(own_off, n_own, static_cast<uint32_t>(e));
     const uint32_t own_deg = own_off[o + 1] - own_off[o];
     const uint32_t t = other_idx[e];
     const uint32_t other_deg = other_off[t + 1] - other_off[t];
@@ -399,7 +424,8 @@ size_t csr_from_csc_bytes(uint32_t sort_n) {
 }
 
 int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co, const uint32_t *ri, DevCount Vd,
-                 DevCount Vs, DevCount E, uint32_t sort_n, unsigned key_bits, void *work, hipStream_t stream) {
+                 DevCount Vs, DevCount E, uint32_t sort_n, unsigned key_bits, void *work, const uint32_t *owner,
+                 hipStream_t stream) {
   unsigned char *w = static_cast<unsigned char *>(work);
   const size_t arr = align_up(static_cast<size_t>(sort_n ? sort_n : 1) * sizeof(uint32_t), 256);
   uint32_t *keys_sorted = reinterpret_cast<uint32_t *>(w);
@@ -433,7 +459,7 @@ int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co,
   }
   const uint64_t span = static_cast<uint64_t>(Vs.cap) + 1 > E.cap ? static_cast<uint64_t>(Vs.cap) + 1 : E.cap;
   hipLaunchKernelGGL(csr_finish_kernel, dim3(ceil_div(span, 256)), dim3(256), 0, stream, ro, ci, keys_sorted, perm_out,
-                     co, Vd, Vs, E);
+                     co, Vd, Vs, E, owner);
   NTS_LAUNCH_CHECK("csr_finish_kernel");
   return NTS_OK;
 }
@@ -465,7 +491,7 @@ int relabel_sources(uint32_t *source, uint32_t *n_source, uint32_t *n_source_cop
 
 int gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t *ri, const uint32_t *ro,
                      const uint32_t *ci, DevCount Vd, DevCount Vs, uint32_t *clear, uint32_t clear_words,
-                     hipStream_t stream) {
+                     const uint32_t *csc_owner, const uint32_t *csr_owner, hipStream_t stream) {
   // The edge count lives on the device: the grid is sized from the vertex counts and the kernel
   // strides over co[Vd] edges, so the call neither needs the count nor synchronises.  Forward and
   // backward weights share one launch (grid.y).
@@ -476,7 +502,7 @@ int gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint32_t 
   const int first = ewf ? 0 : 1;
   const unsigned passes = (ewf && ewb) ? 2u : 1u;
   hipLaunchKernelGGL(edge_weights_kernel, dim3(static_cast<unsigned>(blocks), passes), dim3(256), 0, stream, ewf, ewb, co,
-                     ri, ro, ci, Vd, Vs, first, clear, clear_words);
+                     ri, ro, ci, Vd, Vs, first, clear, clear_words, csc_owner, csr_owner);
   NTS_LAUNCH_CHECK("edge_weights_kernel");
   return NTS_OK;
 }
@@ -502,7 +528,8 @@ int nts_csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t 
   }
   if (!ci || !co || !ri || !work) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: null pointer");
   if (!aligned_to(work, 256)) return fail(NTS_ERR_INVALID, "nts_csr_from_csc: work must be 256-byte aligned");
-  return csr_from_csc(ro, ci, perm, co, ri, host_count(Vd), host_count(Vs), host_count(E), E, bits_for(Vs), work, stream);
+  return csr_from_csc(ro, ci, perm, co, ri, host_count(Vd), host_count(Vs), host_count(E), E, bits_for(Vs), work, nullptr,
+                      stream);
 }
 
 size_t nts_chunk_from_edges_work_bytes(uint32_t V, uint32_t E) {
@@ -611,7 +638,7 @@ int nts_gcn_edge_weights(float *ewf, float *ewb, const uint32_t *co, const uint3
   if (Vd == 0 || Vs == 0) return NTS_OK;
   if (ewf && !ri) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ri");
   if (ewb && !ci) return fail(NTS_ERR_INVALID, "nts_gcn_edge_weights: null ci");
-  return gcn_edge_weights(ewf, ewb, co, ri, ro, ci, host_count(Vd), host_count(Vs), nullptr, 0, stream);
+  return gcn_edge_weights(ewf, ewb, co, ri, ro, ci, host_count(Vd), host_count(Vs), nullptr, 0, nullptr, nullptr, stream);
 }
 
 }  // extern "C"

@@ -60,10 +60,13 @@ __device__ __forceinline__ bool group_any(bool pred) {
 }
 
 // Stores one sampled source id; with `mark` also sets its bit in the bitmap of sampled sources
-// (integer OR: the result does not depend on the order), which saves the relabelling a pass.
-__device__ __forceinline__ void emit(uint32_t *__restrict__ ri_out, uint32_t *__restrict__ mark, uint32_t pos,
-                                     uint32_t g) {
+// (integer OR: the result does not depend on the order), which saves the relabelling a pass; with
+// `owner` also records the destination slot the edge belongs to, which saves the construction of the
+// transposed structure a search per edge.
+__device__ __forceinline__ void emit(uint32_t *__restrict__ ri_out, uint32_t *__restrict__ mark,
+                                     uint32_t *__restrict__ owner, uint32_t pos, uint32_t g, uint32_t slot) {
   ri_out[pos] = g;
+  if (owner) owner[pos] = slot;
   if (mark) atomicOr(&mark[g >> 5], 1u << (g & 31));
 }
 
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
                                                        const uint32_t *__restrict__ graph_ri,
                                                        const uint32_t *__restrict__ dst, DevCount n,
                                                        uint32_t edge_cap, int32_t fanout, DevSeed seed,
-                                                       uint32_t *__restrict__ mark) {
+                                                       uint32_t *__restrict__ mark, uint32_t *__restrict__ owner) {
   const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) / G;
   if (i >= n.get()) return;  // whole groups leave together
   const uint32_t gl = threadIdx.x & (G - 1);
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
   const uint32_t take = co[i + 1] - out;
   if (co[i + 1] > edge_cap) return;  // never past the edge array (a full-neighbourhood batch that repeats vertices)
   if (take == deg) {  // full neighbourhood, in CSC order
-    for (uint32_t k = gl; k < deg; k += G) emit(ri_out, mark, out + k, graph_ri[base + k]);
+    for (uint32_t k = gl; k < deg; k += G) emit(ri_out, mark, owner, out + k, graph_ri[base + k], i);
     return;
   }
   const uint64_t state0 = mix64(seed.get() ^ (static_cast<uint64_t>(i) << 32) ^ d);
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(256) void hop_pick_kernel(uint32_t *__restrict__ ri
   if (gl < take) {
     uint32_t rank = 0;
     for (uint32_t q = 0; q < take; ++q) rank += __shfl(v, q, G) < v ? 1u : 0u;
-    emit(ri_out, mark, out + rank, graph_ri[base + v]);
+    emit(ri_out, mark, owner, out + rank, graph_ri[base + v], i);
   }
 }
 
@@ -132,7 +135,7 @@ __global__ __launch_bounds__(256) void hop_pick_wide_kernel(uint32_t *__restrict
                                                             const uint32_t *__restrict__ graph_ri,
                                                             const uint32_t *__restrict__ dst, DevCount n,
                                                             uint32_t edge_cap, DevSeed seed,
-                                                            uint32_t *__restrict__ mark) {
+                                                            uint32_t *__restrict__ mark, uint32_t *__restrict__ owner) {
   __shared__ uint32_t picked[4][kWidestFanout];
   const uint32_t lane = threadIdx.x & (kWave - 1);
   uint32_t *mine = picked[threadIdx.x / kWave];
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(256) void hop_pick_wide_kernel(uint32_t *__restrict
     const uint32_t v = mine[k];
     uint32_t rank = 0;
     for (uint32_t q = 0; q < take; ++q) rank += mine[q] < v ? 1u : 0u;
-    emit(ri_out, mark, out + rank, graph_ri[base + v]);
+    emit(ri_out, mark, owner, out + rank, graph_ri[base + v], i);
   }
 }
 
@@ -191,7 +194,8 @@ __global__ __launch_bounds__(256) void hop_pick_select_kernel(uint32_t *__restri
                                                               const uint32_t *__restrict__ graph_ri,
                                                               const uint32_t *__restrict__ dst, DevCount n,
                                                               uint32_t edge_cap, DevSeed seed,
-                                                              uint32_t *__restrict__ mark) {
+                                                              uint32_t *__restrict__ mark,
+                                                              uint32_t *__restrict__ owner) {
   __shared__ uint32_t hist[256];
   __shared__ uint32_t sh_prefix, sh_k, wave_less[4], wave_eq[4];
   const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -253,7 +257,8 @@ __global__ __launch_bounds__(256) void hop_pick_select_kernel(uint32_t *__restri
       }
       // ties are taken in position order, so the number taken before this position is min(my_eq, wanted)
       const uint32_t ties_before = my_eq < ties_wanted ? my_eq : ties_wanted;
-      if (less || (eq && my_eq < ties_wanted)) emit(ri_out, mark, out + my_less + ties_before, graph_ri[base + p]);
+      if (less || (eq && my_eq < ties_wanted))
+        emit(ri_out, mark, owner, out + my_less + ties_before, graph_ri[base + p], i);
       less_before += chunk_less;
       eq_before += chunk_eq;
       __syncthreads();
@@ -292,7 +297,7 @@ int hop_offsets(uint32_t *co, const uint32_t *graph_co, const uint32_t *dst, Dev
 
 int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph_co, const uint32_t *graph_ri,
                   const uint32_t *dst, DevCount n, uint32_t edge_cap, int32_t fanout, DevSeed seed, uint32_t *mark_bits,
-                  hipStream_t stream) {
+                  uint32_t *owner, hipStream_t stream) {
   // Lanes per destination: the fanout rounded up to a power of two (full neighbourhoods and
   // fanouts above one wavefront are strided copies, for which a quarter wavefront serves well).
   int g = 8;
@@ -303,7 +308,7 @@ int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph
   const dim3 grid(ceil_div(static_cast<uint64_t>(n.cap) * g, 256));
 #define NTS_LAUNCH_PICK(G)                                                                                      \
   hipLaunchKernelGGL(hop_pick_kernel<G>, grid, dim3(256), 0, stream, ri_global, co, graph_co, graph_ri, dst, n, \
-                     edge_cap, fanout, seed, mark_bits)
+                     edge_cap, fanout, seed, mark_bits, owner)
   switch (g) {
     case 8: NTS_LAUNCH_PICK(8); break;
     case 16: NTS_LAUNCH_PICK(16); break;
@@ -315,11 +320,11 @@ int hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint32_t *graph
   if (fanout > kWidestFanout) {
     const uint32_t blocks = n.cap < 4096u ? n.cap : 4096u;
     hipLaunchKernelGGL(hop_pick_select_kernel, dim3(blocks ? blocks : 1u), dim3(256), 0, stream, ri_global, co, graph_co,
-                       graph_ri, dst, n, edge_cap, seed, mark_bits);
+                       graph_ri, dst, n, edge_cap, seed, mark_bits, owner);
     NTS_LAUNCH_CHECK("hop_pick_select_kernel");
   } else if (fanout > kMaxFanout) {
     hipLaunchKernelGGL(hop_pick_wide_kernel, dim3(ceil_div(static_cast<uint64_t>(n.cap) * kWave, 256)), dim3(256), 0,
-                       stream, ri_global, co, graph_co, graph_ri, dst, n, edge_cap, seed, mark_bits);
+                       stream, ri_global, co, graph_co, graph_ri, dst, n, edge_cap, seed, mark_bits, owner);
     NTS_LAUNCH_CHECK("hop_pick_wide_kernel");
   }
   return NTS_OK;
@@ -357,7 +362,7 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
   if (!ri_global || !co || !graph_co || !graph_ri || !dst)
     return fail(NTS_ERR_INVALID, "nts_sample_hop_neighbors: null pointer");
   return hop_neighbors(ri_global, co, graph_co, graph_ri, dst, host_count(n), 0xFFFFFFFFu, fanout, host_seed(seed), nullptr,
-                       stream);
+                       nullptr, stream);
 }
 
 }  // extern "C"
