@@ -213,6 +213,30 @@ __device__ __forceinline__ uint32_t owners_of_step(const uint32_t *__restrict__ 
   return last <= e ? owner_of(off, n, e) : d0 + pos;
 }
 
+// Exclusive prefix of `mine` over the THREADS threads of a block, in thread order; *total = the sum.
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_prefix(uint32_t mine, uint32_t *wave_sums, uint32_t *total) {
+  const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  uint32_t incl = mine;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t up = __shfl_up(incl, d, kWave);
+    if (lane >= static_cast<uint32_t>(d)) incl += up;
+  }
+  __syncthreads();  // wave_sums may still be read from an earlier call
+  if (lane == kWave - 1) wave_sums[wave] = incl;
+  __syncthreads();
+  uint32_t before = 0, all = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < THREADS / kWave; ++w) {
+    const uint32_t v = wave_sums[w];
+    if (w < wave) before += v;
+    all += v;
+  }
+  *total = all;
+  return before + incl - mine;
+}
+
 // Butterfly reductions over the `width` lanes of an aligned lane group (width = power of two <= 64).
 template <int WIDTH>
 __device__ __forceinline__ float group_max(float v) {

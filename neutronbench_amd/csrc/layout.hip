@@ -4,7 +4,6 @@
 // algorithms; everything is order-independent, so the outputs are deterministic.
 #include <string.h>
 
-#include <rocprim/block/block_radix_sort.hpp>
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/device/device_scan.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
@@ -229,15 +228,15 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 //   hop_sort_rows     one block per digit: exclusive scan of that digit's row over the blocks, and
 //                     the digit's total
 //   hop_sort_scatter  block b turns the totals into the digits' first positions, adds its entries of
-//                     the table, sorts its 2,048 (digit, position) pairs with the block-wide stable
-//                     sort, so that equal digits lie next to each other in their original order, and
-//                     writes every edge to start[digit] + its rank inside the chunk's run of that digit
+//                     the table, ranks each of its 2,048 edges among the chunk's edges of the same
+//                     digit (ballots inside a wavefront, per-wavefront histograms across them) and
+//                     writes every edge to start[digit] + that rank
 // Equal keys keep their order in every pass: the result is the stable order, bit for bit.  Only
 // blocks below ceil(E / 2048) of the launched ceil(capacity / 2048) do anything.
 constexpr int kHopSortThreads = 256;
 constexpr int kHopSortItems = 8;
 constexpr uint32_t kHopSortChunk = kHopSortThreads * kHopSortItems;  // 2,048 edges
-constexpr unsigned kHopSortMaxDigitBits = 10;
+constexpr unsigned kHopSortMaxDigitBits = 10;  // 11 (two passes for 22-bit keys) measured slower: 2,048-bin tables
 constexpr uint32_t kHopSortMaxBins = 1u << kHopSortMaxDigitBits;
 
 struct HopSortShape {
@@ -252,30 +251,6 @@ inline HopSortShape hop_sort_shape(uint32_t capacity, unsigned key_bits) {
   sh.passes = (key_bits + kHopSortMaxDigitBits - 1) / kHopSortMaxDigitBits;
   sh.digit_bits = (key_bits + sh.passes - 1) / sh.passes;
   return sh;
-}
-
-// Exclusive prefix of `mine` over the THREADS threads of a block, in thread order; *total = the sum.
-template <int THREADS>
-__device__ __forceinline__ uint32_t block_prefix(uint32_t mine, uint32_t *wave_sums, uint32_t *total) {
-  const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  uint32_t incl = mine;
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const uint32_t up = __shfl_up(incl, d, kWave);
-    if (lane >= static_cast<uint32_t>(d)) incl += up;
-  }
-  __syncthreads();  // wave_sums may still be read from an earlier call
-  if (lane == kWave - 1) wave_sums[wave] = incl;
-  __syncthreads();
-  uint32_t before = 0, all = 0;
-#pragma unroll
-  for (uint32_t w = 0; w < THREADS / kWave; ++w) {
-    const uint32_t v = wave_sums[w];
-    if (w < wave) before += v;
-    all += v;
-  }
-  *total = all;
-  return before + incl - mine;
 }
 
 __global__ __launch_bounds__(kHopSortThreads) void hop_sort_count_kernel(uint32_t *__restrict__ table,
@@ -317,8 +292,12 @@ __global__ __launch_bounds__(kHopSortThreads) void hop_sort_rows_kernel(uint32_t
   if (threadIdx.x == 0) totals[blockIdx.x] = total;
 }
 
-// vals_in == nullptr: the value of edge e is e.  THREADS x ITEMS = 2,048: the block-wide sort ranks a
-// thread's items one after the other, so more threads with fewer items each shorten the chain.
+// vals_in == nullptr: the value of edge e is e.  THREADS x ITEMS = 2,048 edges per block.  Wavefront w
+// takes the edges [512 w, 512 (w + 1)) of the chunk, 64 consecutive ones per round: the lanes that hold
+// the same digit find each other with one ballot per digit bit, an edge's rank is the number of equal
+// digits the wavefront has seen in earlier rounds (a histogram of its own in LDS) plus the equal digits
+// on lower lanes, and the wavefronts' histograms, added up in wavefront order, give the rest -- the
+// stable rank of every edge without sorting the chunk.
 template <int THREADS, int ITEMS>
 __global__ __launch_bounds__(THREADS) void hop_sort_scatter_kernel(uint32_t *__restrict__ keys_out,
                                                                            uint32_t *__restrict__ vals_out,
@@ -328,20 +307,31 @@ __global__ __launch_bounds__(THREADS) void hop_sort_scatter_kernel(uint32_t *__r
                                                                            const uint32_t *__restrict__ totals,
                                                                            DevCount edges, unsigned shift,
                                                                            unsigned digit_bits) {
-  // one ranking round over the whole digit (the library's default is eight bits per round)
-  using Sort = rocprim::block_radix_sort<uint32_t, THREADS, ITEMS, uint32_t, 1, 1, kHopSortMaxDigitBits>;
-  __shared__ typename Sort::storage_type sort_storage;
-  __shared__ uint32_t start[kHopSortMaxBins];     // output position of the first edge of each digit from this block
-  __shared__ uint32_t first_at[kHopSortMaxBins];  // where the chunk's run of each digit begins
-  __shared__ uint32_t chunk_keys[kHopSortChunk], chunk_vals[kHopSortChunk];
-  __shared__ uint16_t sorted_digit[kHopSortChunk];
-  __shared__ uint32_t wave_sums[THREADS / kWave];
+  constexpr int kWaves = THREADS / kWave;
+  __shared__ uint32_t start[kHopSortMaxBins];  // output position of the first edge of each digit from this block
+  __shared__ uint32_t wave_hist[kWaves][kHopSortMaxBins];
+  __shared__ uint32_t wave_sums[kWaves];
   static_assert(THREADS * ITEMS == static_cast<int>(kHopSortChunk), "one chunk per block");
   const uint32_t E = edges.get();
   const uint64_t c0 = static_cast<uint64_t>(blockIdx.x) * kHopSortChunk;
   if (c0 >= E) return;
   const uint32_t n = static_cast<uint32_t>(E - c0 < kHopSortChunk ? E - c0 : kHopSortChunk);
   const uint32_t bins = 1u << digit_bits, mask = bins - 1u;
+  const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  uint32_t key[ITEMS], val[ITEMS], rank[ITEMS];
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {  // coalesced: round j of this wavefront
+    const uint32_t p = wave * (kWave * ITEMS) + j * kWave + lane;
+    key[j] = 0;
+    val[j] = 0;
+    if (p < n) {
+      key[j] = keys_in[c0 + p];
+      val[j] = vals_in ? vals_in[c0 + p] : static_cast<uint32_t>(c0 + p);
+    }
+  }
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w)
+    for (uint32_t d = threadIdx.x; d < bins; d += THREADS) wave_hist[w][d] = 0;
   {  // first position of every digit: exclusive scan of the totals, plus this block's entry of the table
     const uint32_t per = (bins + THREADS - 1) / THREADS;
     const uint32_t b = threadIdx.x * per, e = b + per < bins ? b + per : bins;
@@ -354,41 +344,48 @@ __global__ __launch_bounds__(THREADS) void hop_sort_scatter_kernel(uint32_t *__r
       run += totals[d];
     }
   }
-  uint32_t digit[ITEMS], idx[ITEMS];
+  __syncthreads();
+  uint32_t *hist = wave_hist[wave];
+  const uint64_t below = (1ull << lane) - 1ull;
 #pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {  // coalesced load into LDS
-    const uint32_t p = j * THREADS + threadIdx.x;
-    if (p < n) {
-      chunk_keys[p] = keys_in[c0 + p];
-      chunk_vals[p] = vals_in ? vals_in[c0 + p] : static_cast<uint32_t>(c0 + p);
+  for (int j = 0; j < ITEMS; ++j) {
+    const uint32_t p = wave * (kWave * ITEMS) + j * kWave + lane;
+    const bool active = p < n;
+    const uint32_t d = (key[j] >> shift) & mask;
+    uint64_t peers = __ballot(active);  // for an active lane: the active lanes with the same digit
+    for (unsigned b = 0; b < digit_bits; ++b) {
+      const bool one = (d >> b) & 1u;
+      const uint64_t votes = __ballot(one);
+      peers &= one ? votes : ~votes;
+    }
+    const uint32_t seen = active ? hist[d] : 0u;
+    rank[j] = seen + __popcll(peers & below);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();  // every lane has read its count before a leader raises it
+    if (active && (peers & below) == 0) hist[d] = seen + __popcll(peers);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  __syncthreads();
+  for (uint32_t d = threadIdx.x; d < bins; d += THREADS) {  // counts -> edges of the digit in earlier wavefronts
+    uint32_t run = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const uint32_t v = wave_hist[w][d];
+      wave_hist[w][d] = run;
+      run += v;
     }
   }
   __syncthreads();
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
-    const uint32_t p = threadIdx.x * ITEMS + j;  // blocked arrangement keeps the input order
-    idx[j] = p;
-    // The chunk's unused tail takes the largest digit: it comes last in the input, so the stable
-    // sort leaves it behind every edge, at positions n and above.
-    digit[j] = p < n ? ((chunk_keys[p] >> shift) & mask) : mask;
-  }
-  Sort().sort(digit, idx, sort_storage, 0, digit_bits);
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) sorted_digit[threadIdx.x * ITEMS + j] = static_cast<uint16_t>(digit[j]);
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {  // the first element of every run records where the run begins
-    const uint32_t p = threadIdx.x * ITEMS + j;
-    if (p < n && (p == 0 || sorted_digit[p - 1] != sorted_digit[p])) first_at[digit[j]] = p;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    const uint32_t p = threadIdx.x * ITEMS + j;
+    const uint32_t p = wave * (kWave * ITEMS) + j * kWave + lane;
     if (p < n) {
-      const uint32_t pos = start[digit[j]] + (p - first_at[digit[j]]);
-      keys_out[pos] = chunk_keys[idx[j]];
-      vals_out[pos] = chunk_vals[idx[j]];
+      const uint32_t d = (key[j] >> shift) & mask;
+      const uint32_t pos = start[d] + hist[d] + rank[j];
+      keys_out[pos] = key[j];
+      vals_out[pos] = val[j];
     }
   }
 }
@@ -450,7 +447,6 @@ int csr_from_csc(uint32_t *ro, uint32_t *ci, uint32_t *perm, const uint32_t *co,
                        sh.digit_bits);
     hipLaunchKernelGGL(hop_sort_rows_kernel, dim3(1u << sh.digit_bits), dim3(kHopSortThreads), 0, stream, table, totals,
                        sh.blocks, E);
-    // (512 x 4 and 1,024 x 2 were measured as well: the same within 3 %)
     hipLaunchKernelGGL((hop_sort_scatter_kernel<kHopSortThreads, kHopSortItems>), dim3(sh.blocks), dim3(kHopSortThreads), 0,
                        stream, kout, vout, kin, vin, table, totals, E, shift, sh.digit_bits);
     NTS_LAUNCH_CHECK("hop_sort kernels");
