@@ -1519,33 +1519,38 @@ __global__ __launch_bounds__(256) void sddmm_edge_kernel(float *__restrict__ gal
     const uint64_t e = base + lane;
     const uint32_t own = owners_of_step(co, Vd, static_cast<uint32_t>(base), d0);
     const uint32_t src = e < E ? ri[e] : 0u;
-    // Four edges at a time: their gathered rows are requested before the first is used.
+    // Four edges at a time: their gathered rows -- and the destination rows of the edges at which the
+    // destination changes -- are requested before the first is used.
     constexpr uint32_t U = 4;
     for (uint32_t j0 = 0; j0 < G; j0 += U) {
       uint32_t d[U];
-      bool valid[U];
-      float4 x4[U];
-      float x1[U];
+      bool valid[U], fresh[U];
+      float4 x4[U], w4[U];
+      float x1[U], w1[U];
 #pragma unroll
       for (uint32_t u = 0; u < U; ++u) {
         const uint32_t holder = grp * G + j0 + u;
         const uint32_t s = __shfl(src, holder & (kWave - 1), kWave);
         d[u] = __shfl(own, holder & (kWave - 1), kWave);
         valid[u] = j0 + u < G && base + holder < E;
-        x4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        x1[u] = 0.f;
+        fresh[u] = valid[u] && d[u] != (u ? d[u - 1] : d_held);  // an edge is valid only if the one before it is
+        x4[u] = w4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        x1[u] = w1[u] = 0.f;
         if (valid[u]) {
           const float *a = in + static_cast<size_t>(s) * F + gl * VEC;
           if (VEC == 4) x4[u] = *reinterpret_cast<const float4 *>(a); else x1[u] = a[0];
+        }
+        if (fresh[u]) {
+          const float *b = gout + static_cast<size_t>(d[u]) * F + gl * VEC;
+          if (VEC == 4) w4[u] = *reinterpret_cast<const float4 *>(b); else w1[u] = b[0];
         }
       }
 #pragma unroll
       for (uint32_t u = 0; u < U; ++u) {
         float p = 0.f;
         if (valid[u]) {
-          if (d[u] != d_held) {
-            const float *b = gout + static_cast<size_t>(d[u]) * F + gl * VEC;
-            if (VEC == 4) y4 = *reinterpret_cast<const float4 *>(b); else y1 = b[0];
+          if (fresh[u]) {
+            if (VEC == 4) y4 = w4[u]; else y1 = w1[u];
             d_held = d[u];
           }
           p = VEC == 4 ? fmaf(x4[u].w, y4.w, fmaf(x4[u].z, y4.z, fmaf(x4[u].y, y4.y, x4[u].x * y4.x))) : x1[u] * y1;
