@@ -34,16 +34,13 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(V *__restrict__ out, c
 }
 
 // Cached gather: a row comes from the HBM cache when its id has a slot, else from the (mapped host)
-// table.  A wavefront looks at 64 rows at a time -- one coalesced load of their ids and 64 look-ups of
-// their slots side by side -- and its lane groups then copy the rows of that set one after the other,
-// so that a group never waits for a look-up per row.  Hits are counted per wavefront from the look-up
-// mask; one integer atomic per block adds the block's count (one atomic per hit row on a single
-// address was measured at 1.3 ms of a 1.9 ms launch for 337 k rows).
+// table.  Blocks stride over the rows and count their hits locally; one integer atomic per block
+// adds the block's count (one atomic per hit row on a single address was measured at 1.3 ms of a
+// 1.9 ms launch for 337 k rows).
 // miss_blocks > 0 (table in host memory): the first miss_blocks blocks copy only the rows that miss
 // the cache -- they wait for the link -- and the blocks after them only the rows that hit, from HBM;
-// every wavefront looks up all rows of its stride and copies the ones of its kind.  The few blocks
-// that keep the link full are then not also the ones that move the (many more) cached rows, and
-// because their groups only ever hold rows that miss, every group has a request on the link.
+// every block walks all row ids of its stride and skips the rows of the other kind.  The few blocks
+// that keep the link full are then not also the ones that move the (many more) cached rows.
 template <typename V, int G>
 __global__ __launch_bounds__(256) void gather_rows_cached_kernel(V *__restrict__ out, const V *__restrict__ table,
                                                                  const V *__restrict__ cache,
@@ -51,57 +48,34 @@ __global__ __launch_bounds__(256) void gather_rows_cached_kernel(V *__restrict__
                                                                  const uint32_t *__restrict__ hashmap, uint32_t n,
                                                                  uint32_t Fv, uint32_t *__restrict__ hits,
                                                                  uint32_t miss_blocks) {
-  constexpr uint32_t kGroups = kWave / G;
-  constexpr uint32_t kWaves = 256 / kWave;
-  const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint32_t gl = lane & (G - 1), grp = lane / G;
+  constexpr uint32_t kRowsPerBlock = 256 / G;
+  const uint32_t gl = threadIdx.x & (G - 1);
   uint32_t my_hits = 0;
   // blocks of this block's kind, and its rank among them
   const bool split = miss_blocks != 0, miss_side = blockIdx.x < miss_blocks;
   const uint32_t peers = !split ? gridDim.x : (miss_side ? miss_blocks : gridDim.x - miss_blocks);
   const uint32_t rank = (!split || miss_side) ? blockIdx.x : blockIdx.x - miss_blocks;
-  const uint64_t wave = static_cast<uint64_t>(rank) * kWaves + threadIdx.x / kWave;
-  const uint64_t n_waves = static_cast<uint64_t>(peers) * kWaves;
-  for (uint64_t base = wave * kWave; base < n; base += n_waves * kWave) {
-    uint32_t g = 0, slot = kMiss;
-    const bool have = base + lane < n;
-    if (have) {
-      g = row_ids[base + lane];
-      slot = hashmap[g];
-    }
-    const bool hit = have && slot != kMiss;
-    const uint64_t hit_mask = __ballot(hit);
-    uint64_t todo = !split ? __ballot(have) : (miss_side ? __ballot(have && !hit) : hit_mask);
-    if (lane == 0 && (!split || !miss_side)) my_hits += __popcll(hit_mask);
-    while (todo) {
-      // the next kGroups rows of the set, one per lane group
-      uint32_t pick = kWave;
-      uint64_t m = todo;
-#pragma unroll
-      for (uint32_t t = 0; t < kGroups; ++t) {
-        if (m) {
-          if (t == grp) pick = static_cast<uint32_t>(__builtin_ctzll(m));
-          m &= m - 1;
-        }
-      }
-      todo = m;
-      const uint32_t from = pick < kWave ? pick : 0u;
-      const uint32_t row_g = __shfl(g, from, kWave), row_slot = __shfl(slot, from, kWave);
-      if (pick < kWave) {
-        const V *src = row_slot != kMiss ? cache + static_cast<size_t>(row_slot) * Fv : table + static_cast<size_t>(row_g) * Fv;
-        V *dst = out + (base + pick) * Fv;
-        for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
-      }
-    }
+  for (uint64_t i = static_cast<uint64_t>(rank) * kRowsPerBlock + threadIdx.x / G; i < n;
+       i += static_cast<uint64_t>(peers) * kRowsPerBlock) {
+    const uint32_t g = row_ids[i];
+    const uint32_t slot = hashmap[g];
+    const bool hit = slot != kMiss;
+    if (split && hit == miss_side) continue;  // the other kind of block copies this row
+    const V *src = hit ? cache + static_cast<size_t>(slot) * Fv : table + static_cast<size_t>(g) * Fv;
+    V *dst = out + static_cast<size_t>(i) * Fv;
+    for (uint32_t c = gl; c < Fv; c += G) dst[c] = src[c];
+    my_hits += (hit && gl == 0) ? 1u : 0u;
   }
   if (!hits) return;  // uniform across the block
-  __shared__ uint32_t wave_hits[kWaves];
-  if (lane == 0) wave_hits[threadIdx.x / kWave] = my_hits;
+  __shared__ uint32_t wave_hits[256 / kWave];
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) my_hits += __shfl_xor(my_hits, m, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) wave_hits[threadIdx.x / kWave] = my_hits;
   __syncthreads();
   if (threadIdx.x == 0) {
     uint32_t total = 0;
 #pragma unroll
-    for (uint32_t k = 0; k < kWaves; ++k) total += wave_hits[k];
+    for (int k = 0; k < 256 / kWave; ++k) total += wave_hits[k];
     if (total) atomicAdd(hits, total);  // integer count: order-independent
   }
 }
@@ -179,15 +153,12 @@ void launch_rows(const RowsArgs &a, uint32_t Fv) {
   const uint32_t wanted = blocks;
   if (blocks > cap) blocks = cap;
   if (a.cache) {
-    // A wavefront of the cached kernel takes 64 rows at a time: 256 per block and round.
-    const uint32_t sets = ceil_div(a.n, 256);
-    const uint32_t side_cap = host_table ? kHostTableBlocks : kCachedBlocks;
     // table in host memory: kHostTableBlocks blocks for the rows that miss, and beside them blocks for
     // the rows the cache holds (enough to move them at HBM speed, still a fraction of the chip)
-    const uint32_t miss_blocks = (host_table && sets > kHostTableBlocks) ? kHostTableBlocks : 0u;
-    const uint32_t hit_blocks = miss_blocks ? std::min<uint32_t>(sets, kHitBlocks) : 0u;
-    hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), dim3(std::min(sets, side_cap) + hit_blocks), dim3(256), 0,
-                       a.stream, reinterpret_cast<V *>(a.out), reinterpret_cast<const V *>(a.table),
+    const uint32_t miss_blocks = (host_table && wanted > kHostTableBlocks) ? kHostTableBlocks : 0u;
+    const uint32_t hit_blocks = miss_blocks ? std::min<uint32_t>(wanted, kHitBlocks) : 0u;
+    hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), dim3(blocks + hit_blocks), dim3(256), 0, a.stream,
+                       reinterpret_cast<V *>(a.out), reinterpret_cast<const V *>(a.table),
                        reinterpret_cast<const V *>(a.cache), a.row_ids, a.remap, a.n, Fv, a.hits, miss_blocks);
     return;
   }
