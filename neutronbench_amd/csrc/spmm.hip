@@ -873,6 +873,113 @@ __global__ __launch_bounds__(256) void auto_reduce_wide_kernel(float *__restrict
 
 inline size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 
+// Calls below kAutoLargeEdges (sampled layers) need no order among the pieces, so they need no scan
+// either: a long row takes its consecutive partial slots from a counter (integer atomic: which slots a
+// row gets varies from call to call, the order of its pieces inside them and therefore every sum does
+// not), and lists itself for the second stage.
+//   ctr[0] = slots handed out, ctr[1] = rows listed.  Items are pre-filled as empty, so the slots beyond
+//   the live count cost a wavefront that writes zeros to a slot nobody reads.
+__global__ __launch_bounds__(256) void auto_fill_kernel(Item *__restrict__ items, uint32_t *__restrict__ ctr,
+                                                        uint32_t p_max) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < 2) ctr[i] = 0;
+  if (i < p_max) items[i] = make_uint4(0u, 0u, 0u, i);
+}
+
+__global__ __launch_bounds__(256) void auto_cut_kernel(Item *__restrict__ items, uint4 *__restrict__ splits,
+                                                       uint32_t *__restrict__ ctr, const uint32_t *__restrict__ off,
+                                                       uint32_t rows, uint32_t chunk, uint32_t p_max, uint32_t s_max) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  const uint32_t b = off[r], e = off[r + 1], deg = e - b;
+  if (deg <= chunk) return;
+  uint32_t n = (deg + chunk - 1) / chunk;
+  const uint32_t first = atomicAdd(&ctr[0], n);
+  // Slots at or beyond p_max do not exist (only possible when the caller's edge count is smaller than
+  // offsets[rows]): such pieces are not created and not read.
+  if (first >= p_max) return;
+  if (first + n > p_max) n = p_max - first;
+  for (uint32_t j = 0; j < n; ++j) {
+    const uint32_t e0 = b + j * chunk;
+    items[first + j] = make_uint4(r, e0, min(e, e0 + chunk), first + j);
+  }
+  const uint32_t s = atomicAdd(&ctr[1], 1u);
+  if (s < s_max) splits[s] = make_uint4(r, first, n, 0u);
+}
+
+// Block (x, y): adds the partials of listed row x in slot order into out (256 columns per block, tile y).
+__global__ __launch_bounds__(256) void auto_reduce_listed_kernel(float *__restrict__ out,
+                                                                 const float *__restrict__ partial,
+                                                                 const uint4 *__restrict__ splits,
+                                                                 const uint32_t *__restrict__ ctr, uint32_t F,
+                                                                 int accumulate, uint32_t s_max) {
+  const uint32_t live = ctr[1] < s_max ? ctr[1] : s_max;
+  if (blockIdx.x >= live) return;
+  const uint4 sp = splits[blockIdx.x];
+  const uint32_t c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= F || sp.z == 0) return;
+  const float *src = partial + static_cast<size_t>(sp.y) * F + c;
+  float a = src[0];
+  uint32_t k = 1;
+  for (; k + 8 <= sp.z; k += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[static_cast<size_t>(k + u) * F];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a += v[u];
+  }
+  for (; k < sp.z; ++k) a += src[static_cast<size_t>(k) * F];
+  float *dst = out + static_cast<size_t>(sp.x) * F + c;
+  if (accumulate) a += *dst;
+  *dst = a;
+}
+
+int launch_spmm_cut_small(const LaunchArgs &a, uint32_t edges, unsigned char *fixed, size_t fixed_cap) {
+  const uint32_t rows = a.n_items;
+  const uint32_t chunk = kAutoChunk;
+  const uint32_t by_edges = edges / chunk;
+  const uint32_t s_max = (rows < by_edges ? rows : by_edges) + 1;  // rows of more than `chunk` edges
+  const uint32_t p_max = by_edges + s_max;
+  const size_t n_items_b = up256(static_cast<size_t>(p_max) * sizeof(Item));
+  const size_t n_splits_b = up256(static_cast<size_t>(s_max) * sizeof(uint4));
+  const size_t n_partial = up256(static_cast<size_t>(p_max) * a.F * sizeof(float));
+  const size_t need = 256 + n_items_b + n_splits_b + n_partial;
+  unsigned char *buf = fixed;
+  if (fixed) {
+    if (need > fixed_cap) {
+      char msg[200];
+      snprintf(msg, sizeof msg, "spmm: the call needs %zu bytes of scratch, the fixed scratch holds %zu", need,
+               fixed_cap);
+      return fail(NTS_ERR_INVALID, msg);
+    }
+  } else {
+    NTS_HIP_TRY(scratch_alloc(reinterpret_cast<void **>(&buf), need, a.stream));
+  }
+  uint32_t *ctr = reinterpret_cast<uint32_t *>(buf);
+  Item *items = reinterpret_cast<Item *>(buf + 256);
+  uint4 *splits = reinterpret_cast<uint4 *>(buf + 256 + n_items_b);
+  float *partial = reinterpret_cast<float *>(buf + 256 + n_items_b + n_splits_b);
+  hipLaunchKernelGGL(auto_fill_kernel, dim3(ceil_div(p_max, 256)), dim3(256), 0, a.stream, items, ctr, p_max);
+  hipLaunchKernelGGL(auto_cut_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, a.stream, items, splits, ctr, a.offsets,
+                     rows, chunk, p_max, s_max);
+  LaunchArgs pc = a;
+  pc.n_items = p_max;
+  pc.items = items;
+  pc.partial = partial;
+  pc.rows_after_items = rows;
+  pc.row_edge_limit = chunk;
+  launch_spmm(pc);
+  hipLaunchKernelGGL(auto_reduce_listed_kernel, dim3(s_max, ceil_div(a.F, 256)), dim3(256), 0, a.stream, a.out, partial,
+                     splits, ctr, a.F, a.accumulate, s_max);
+  const hipError_t err = hipGetLastError();
+  if (!fixed) {
+    const hipError_t freed = scratch_free(buf, a.stream);
+    if (err == hipSuccess && freed != hipSuccess) return fail_hip(freed, "spmm: scratch");
+  }
+  if (err != hipSuccess) return fail_hip(err, "spmm: balanced launch");
+  return NTS_OK;
+}
+
 // `a` describes the whole-row launch (a.n_items = rows, no items).  Scratch comes from the library's
 // stream-ordered pool, or, when `fixed` is set, from that caller-held region of `fixed_cap` bytes
 // (nothing is allocated or freed then; a call that needs more is refused).
@@ -883,6 +990,7 @@ int launch_spmm_balanced(LaunchArgs a, uint32_t edges, unsigned char *fixed = nu
     return NTS_OK;
   }
   const bool large = edges >= kAutoLargeEdges;
+  if (!large) return launch_spmm_cut_small(a, edges, fixed, fixed_cap);
   const uint32_t chunk = kAutoChunk;
   const uint32_t by_edges = edges / chunk;
   const uint32_t p_max = by_edges + (rows < by_edges ? rows : by_edges) + 1;
