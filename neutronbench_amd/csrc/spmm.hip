@@ -741,7 +741,8 @@ void launch_spmm(const LaunchArgs &a) {
 // wavefronts write partial sums and a last kernel adds each long row's partials in slot order.
 // The number of pieces is not known on the host, so grids and buffers are sized for its upper bound
 // E/chunk + min(rows, E/chunk); surplus work items are empty.  Scratch is stream-ordered
-// (hipMallocAsync / hipFreeAsync).
+// (hipMallocAsync / hipFreeAsync).  Calls below kAutoLargeEdges take the pieces' slots from a counter
+// instead of a scan (launch_spmm_cut_small).
 
 constexpr uint32_t kAutoMinEdges = 1u << 16;  // below this a serial hub row costs less than the set-up
 // Piece length.  Shorter pieces mean more partial rows but also narrower index spans per piece
