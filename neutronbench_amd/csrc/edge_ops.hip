@@ -673,6 +673,7 @@ constexpr int kShortK = 8;         // values per lane held in registers there
 constexpr uint32_t kShortValues = kShortG * kShortK;
 constexpr int kWaveK = 8;          // values per lane the wave kernel can hold in registers
 constexpr uint32_t kWaveRegValues = kWave * kWaveK;
+constexpr uint32_t kWaveMidValues = kWave * 32;  // the fused forward's launch for the class above that: 32 per lane
 
 // One strided pass over a segment with U loads in flight: positions first, first + stride, ...
 // below n; `load(i)` fetches, `use(i, v)` consumes, in ascending position order.
@@ -947,10 +948,12 @@ __device__ __forceinline__ uint64_t wave_rows_in_class(const uint32_t *__restric
 // leaky_relu(el[ri[e],h] + er[d,h], slope); in the three-pass path y first holds the raw score, then
 // alpha.  Visits the destinations with min_values <= n <= max_values.
 // PART: 0 = every segment size in one launch; 1 = the register-resident segments only, 2 = the
-// longer ones only -- two launches, each instance allotted the registers of its own path.  The fused
-// form is launched in two parts: its longer segments read el[src] with 16-byte lanes, which costs
-// registers that the short ones should not pay for (Products-shaped graph: 3.05 -> 2.82 ms); for the
-// plain softmax one launch is as fast as two or three (every variant runs at the rate of a copy).
+// longer ones only, 3 = segments of 513 .. 2,048 values held 16 or 32 per lane in registers -- launches
+// of their own, each instance allotted the registers of its own path.  The fused form is launched in
+// parts: its longer segments read el[src] with 16-byte lanes, which costs registers that the short
+// ones should not pay for (Products-shaped graph: 3.05 -> 2.82 ms), and the class between them is
+// still one pass over memory instead of writing raw scores and reading them back (2.76 -> 2.65 ms); for
+// the plain softmax one launch is as fast as two or three (every variant runs at the rate of a copy).
 template <bool FUSED, bool POW2, int PART>
 __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict__ y, const float *__restrict__ x,
                                                                const float *__restrict__ el,
@@ -981,6 +984,11 @@ __global__ __launch_bounds__(256) void edge_softmax_fwd_kernel(float *__restrict
           continue;
         }
         if (PART == 1) continue;
+        if (PART == 3) {  // 513 .. 2,048 values: still one pass, 16 or 32 values per lane in registers
+          if (n <= 16u * kWave) softmax_fwd_regs<FUSED, kWave, 16>(ys, xs, el, er, ri, d, e0, n, H, slope, lane);
+          else softmax_fwd_regs<FUSED, kWave, 32>(ys, xs, el, er, ri, d, e0, n, H, slope, lane);
+          continue;
+        }
         if (PART == 2 && vec4 && n >= 2048u) {  // at least two full rounds of four vectors per lane
           const uint32_t h0 = (lane * 4u) & (H - 1);  // head of this lane's first value; 256 k = 0 mod H
           const uint32_t hq = H / 4;                  // lanes hq apart hold the same heads
@@ -1113,6 +1121,7 @@ __global__ __launch_bounds__(256) void edge_softmax_bwd_kernel(float *__restrict
           continue;
         }
         if (PART == 1) continue;
+
         if (PART == 2 && FUSED && vec4 && n >= 2048u) {
           // 16-byte lanes: four consecutive values = heads (4 lane mod H) .. +3 of one edge
           const uint32_t h0 = (lane * 4u) & (H - 1);
@@ -1852,7 +1861,13 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
       // the register-resident segments, then the longer ones
       const uint32_t regs_hi = max_values < kWaveRegValues ? max_values : kWaveRegValues;
       NTS_FWD(true, true, 1, min_values, regs_hi);
-      if (max_values > kWaveRegValues) NTS_FWD(true, true, 2, kWaveRegValues + 1, max_values);
+      // 513 .. 2,048 values in a launch of their own: 16 or 32 values per lane in registers, one pass over
+      // memory, and the registers that costs are not the other classes' (64 per lane measured slower)
+      if (max_values > kWaveRegValues) {
+        const uint32_t mid_hi = max_values < kWaveMidValues ? max_values : kWaveMidValues;
+        NTS_FWD(true, true, 3, kWaveRegValues + 1, mid_hi);
+        if (max_values > kWaveMidValues) NTS_FWD(true, true, 2, kWaveMidValues + 1, max_values);
+      }
     } else if (pow2) {
       NTS_FWD(false, true, 0, min_values, max_values);
     } else {
@@ -1876,6 +1891,8 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
     if (pow2 && fused) {
       const uint32_t regs_hi = max_values < kWaveRegValues ? max_values : kWaveRegValues;
       NTS_BWD(true, true, 1, min_values, regs_hi);
+      // (a launch of its own for 513 .. 1,024 values held in registers, as in the forward pass, measured no
+      // gain: the backward holds two arrays per lane, and that class has few edges)
       if (max_values > kWaveRegValues) NTS_BWD(true, true, 2, kWaveRegValues + 1, max_values);
     } else if (pow2) {
       NTS_BWD(false, true, 0, min_values, max_values);
