@@ -512,6 +512,11 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
  *                arena, none is a memset node); what changes is the host time per batch.  The
  *                recording is thread-local and runs on a stream the library creates for it; the
  *                graph is then launched on the caller's stream.  Off by default.
+ *                enable == 2: the same, and in the recorded graph each hop's transposition and edge
+ *                weights run on a side branch beside the next hop's sampling (same arrays; a batch
+ *                built on an otherwise idle device gets shorter, one built beside other batches in
+ *                flight does not -- use 1 there).  Any other non-zero value means 1.  Changing the
+ *                value after a graph was recorded discards it; the next batch records again.
  * Calls on one builder must not overlap: consecutive nts_batch_builder_sample calls go to the same
  * stream, or the earlier batch is waited for first (nts_batch_builder_layers does). */
 typedef struct nts_batch_builder nts_batch_builder_t;

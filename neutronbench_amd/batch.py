@@ -162,8 +162,8 @@ class BatchBuilder:
         call("nts_batch_builder_create", ctypes.byref(handle), ptr(graph_co), ptr(graph_ri), V, E, fan, self.hops,
              max_batch, int(want_perm), self.arena.data_ptr() + self._skew, nbytes)
         self.handle = handle.value
-        if graph:
-            call("nts_batch_builder_use_graph", self.handle, 1)
+        if graph:  # True/1: one recorded chain of launches; 2: hop transpositions on a side branch
+            call("nts_batch_builder_use_graph", self.handle, int(graph))
         self._desc = (SampledLayerDesc * self.hops)()
 
     def _array(self, address, count, dtype):

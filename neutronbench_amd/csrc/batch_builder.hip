@@ -23,12 +23,12 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct HopLayout {
   uint32_t vd_cap, e_cap, vs_cap;
-  size_t co, ri_local, source, ro, ci, perm, ewf, ewb;  // byte offsets into the arena
+  size_t co, ri_local, source, ro, ci, perm, ewf, ewb, owner;  // byte offsets into the arena
 };
 
 struct Layout {
   HopLayout hop[kMaxHops];
-  size_t dst0, sizes, seed, ri_global, owner, relabel_work, csr_work, scan_work, total;
+  size_t dst0, sizes, seed, ri_global, relabel_work, csr_work, scan_work, total;
   size_t relabel_bytes, csr_bytes, scan_bytes;
 };
 
@@ -66,11 +66,11 @@ bool plan_layout(Layout *L, uint32_t V, uint32_t graph_edges, const int32_t *fan
     H.perm = want_perm ? take(eb) : 0;
     H.ewf = take(eb);
     H.ewb = take(eb);
+    H.owner = take(eb);  // destination slot of every edge, recorded by the neighbour pick
     if (H.e_cap > e_max) e_max = H.e_cap;
     vd = H.vs_cap;
   }
   L->ri_global = take(static_cast<size_t>(e_max) * sizeof(uint32_t));
-  L->owner = take(static_cast<size_t>(e_max) * sizeof(uint32_t));  // destination slot of every edge of the hop in work
   L->relabel_bytes = nts_relabel_sources_work_bytes(V);
   // The sort and scan scratch is shared by the hops: the largest any of them asks for (a library
   // routine may pick another algorithm, with other needs, for a smaller input).
@@ -125,6 +125,7 @@ struct nts_batch_builder {
   bool pending;
   bool bitmap_clean;  // the bitmap of sampled sources is all zero (each hop's last kernel leaves it so)
   bool use_graph;     // replay the hops' launches as one HIP graph, captured at the first batch
+  bool fork_hops;     // in that graph, a hop's transposition and weights run on a branch beside the next hop's sampling
   hipGraph_t graph;
   hipGraphExec_t graph_exec;
 };
@@ -134,13 +135,18 @@ namespace {
 // Every launch of a batch after start_batch_kernel: the hops, then the copy of the size table to the
 // host.  All arguments are addresses inside the arena, capacities and device-resident counts, so the
 // sequence is the same for every batch of a builder.
-int enqueue_hops(nts_batch_builder *b, hipStream_t stream) {
+// side (only while recording a graph): a second stream of the recording.  A hop's transposition and
+// weights need nothing of the hops after it and the next hop's sampling needs only this hop's source
+// list, so with `side` the chain forks after the relabelling: sort, CSR and weights of hop h go to the
+// side stream (which takes them hop by hop: they share the sort scratch), the main stream goes on with
+// hop h + 1, and the two join before the size table is copied.  The bitmap of sampled sources, which the
+// weights launch otherwise clears on its way, is then cleared by a launch of its own on the main stream.
+int enqueue_hops(nts_batch_builder *b, hipStream_t stream, hipStream_t side = nullptr, hipEvent_t *events = nullptr) {
   unsigned char *A = b->arena;
   uint32_t *sizes = reinterpret_cast<uint32_t *>(A + b->L.sizes);
   const uint64_t *seed_word = reinterpret_cast<const uint64_t *>(A + b->L.seed);
   uint32_t *dst = reinterpret_cast<uint32_t *>(A + b->L.dst0);
   uint32_t *ri_global = reinterpret_cast<uint32_t *>(A + b->L.ri_global);
-  uint32_t *owner = reinterpret_cast<uint32_t *>(A + b->L.owner);
   // where csr_from_csc leaves the sorted keys: the source of every CSR edge
   const uint32_t *csr_owner = reinterpret_cast<const uint32_t *>(A + b->L.csr_work);
   uint32_t *bits = reinterpret_cast<uint32_t *>(A + b->L.relabel_work);
@@ -156,6 +162,7 @@ int enqueue_hops(nts_batch_builder *b, hipStream_t stream) {
     uint32_t *perm = b->want_perm ? reinterpret_cast<uint32_t *>(A + H.perm) : nullptr;
     float *ewf = reinterpret_cast<float *>(A + H.ewf);
     float *ewb = reinterpret_cast<float *>(A + H.ewb);
+    uint32_t *owner = reinterpret_cast<uint32_t *>(A + H.owner);
     const DevCount Vd = device_count(hop_sizes + 0, H.vd_cap);
     const DevCount Vs = device_count(hop_sizes + 2, H.vs_cap);
     const DevCount E = device_edge_count(co, hop_sizes + 0, H.vd_cap, H.e_cap);
@@ -169,11 +176,24 @@ int enqueue_hops(nts_batch_builder *b, hipStream_t stream) {
     if (int rc = relabel_sources(source, hop_sizes + 2, hop_sizes + kSizeWords, ri, ri_global, E, H.e_cap, H.vs_cap,
                                  hop_sizes + 1, b->V, A + b->L.relabel_work, true, stream))
       return rc;
+    hipStream_t rest = stream;
+    if (side) {
+      if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
+      NTS_HIP_TRY(hipEventRecord(events[h], stream));
+      NTS_HIP_TRY(hipStreamWaitEvent(side, events[h], 0));
+      rest = side;
+    }
     if (int rc = csr_from_csc(ro, ci, perm, co, ri, Vd, Vs, E, H.e_cap, bits_for(H.vs_cap + 1), A + b->L.csr_work,
-                              owner, stream))
+                              owner, rest))
       return rc;
-    if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, bits, words, owner, csr_owner, stream)) return rc;
+    if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, side ? nullptr : bits, side ? 0u : words, owner,
+                                  csr_owner, rest))
+      return rc;
     dst = source;  // the next hop's destinations are this hop's sources (init_dst)
+  }
+  if (side) {  // join
+    NTS_HIP_TRY(hipEventRecord(events[b->hops], side));
+    NTS_HIP_TRY(hipStreamWaitEvent(stream, events[b->hops], 0));
   }
   const size_t size_bytes = (b->hops + 1) * kSizeWords * sizeof(uint32_t);
   NTS_HIP_TRY(hipMemcpyAsync(b->host_sizes, sizes, size_bytes, hipMemcpyDeviceToHost, stream));
@@ -191,10 +211,22 @@ int capture_hops(nts_batch_builder *b) {
     (void)hipStreamDestroy(stream);
     return fail_hip(begin, "nts_batch_builder_sample: hipStreamBeginCapture");
   }
-  const int rc = enqueue_hops(b, stream);
+  hipStream_t side = nullptr;
+  hipEvent_t events[kMaxHops + 1] = {};
+  int rc = NTS_OK;
+  if (b->fork_hops) {
+    if (hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) rc = fail(NTS_ERR_INVALID, "nts_batch_builder_sample: side stream");
+    for (uint32_t h = 0; rc == NTS_OK && h <= b->hops; ++h)
+      if (hipEventCreateWithFlags(&events[h], hipEventDisableTiming) != hipSuccess)
+        rc = fail(NTS_ERR_INVALID, "nts_batch_builder_sample: event");
+  }
+  if (rc == NTS_OK) rc = enqueue_hops(b, stream, side, side ? events : nullptr);
   hipGraph_t graph = nullptr;
   const hipError_t end = hipStreamEndCapture(stream, &graph);  // always ends the recording, also after an error
   (void)hipStreamDestroy(stream);
+  if (side) (void)hipStreamDestroy(side);
+  for (uint32_t h = 0; h <= kMaxHops; ++h)
+    if (events[h]) (void)hipEventDestroy(events[h]);
   if (rc != NTS_OK) {
     if (graph) (void)hipGraphDestroy(graph);
     return rc;
@@ -255,6 +287,7 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
   b->pending = false;
   b->bitmap_clean = false;
   b->use_graph = false;
+  b->fork_hops = false;
   b->graph = nullptr;
   b->graph_exec = nullptr;
   hipError_t err = hipHostMalloc(reinterpret_cast<void **>(&b->host_sizes), (hops + 1) * kSizeWords * sizeof(uint32_t),
@@ -321,7 +354,15 @@ int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, 
 
 int nts_batch_builder_use_graph(nts_batch_builder_t *b, int enable) {
   if (!b) return fail(NTS_ERR_INVALID, "nts_batch_builder_use_graph: null builder");
+  if (b->graph_exec && (b->use_graph != (enable != 0) || b->fork_hops != (enable == 2))) {
+    // another shape of graph than the one recorded: record again at the next batch
+    (void)hipGraphExecDestroy(b->graph_exec);
+    (void)hipGraphDestroy(b->graph);
+    b->graph_exec = nullptr;
+    b->graph = nullptr;
+  }
   b->use_graph = enable != 0;
+  b->fork_hops = enable == 2;
   return NTS_OK;
 }
 

@@ -60,9 +60,20 @@ class Timer:
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
+def graph_mode(graph, pipeline):
+    """The value for nts_batch_builder_use_graph.  True picks by measurement: with one batch in flight
+    the hops' transpositions go to a side branch of the recorded graph (2: the chip is otherwise idle
+    beside the chain of small sampling launches); with several batches in flight the chains of the
+    other builders already fill it and the extra branch only costs (1)."""
+    if graph is True:
+        return 2 if pipeline == 1 else 1
+    return int(graph)
+
+
 def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False, checksum=False,
         stage_sync=None, graph=True):
     cfg = dict(CONFIGS[name])
+    graph = graph_mode(graph, pipeline)
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
     n_train = int(cfg["train"] * scale)
@@ -310,6 +321,7 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         "stage_s": {k: round(v, 4) for k, v in tm.t.items()},
         "library_s": round(sum(v for k, v in tm.t.items() if k != "sample" or sampler != "harness"), 4),
         "sampler": sampler, "hop_launches_as_graph": bool(graph and sampler == "builder"),
+        "hop_graph_mode": graph if sampler == "builder" else 0,
         "pipeline": pipeline if pipelined else 1, "stage_sync": stage_sync,
         "sampled_edges": edges_total, "gathered_rows": rows_total,
         "cache_hit_rate": round(hits_total / max(rows_total, 1), 4) if cache is not None else None,
@@ -366,7 +378,8 @@ def run_native_on(directory, name, V, max_batches=0, warmup_batches=2, pipeline=
         raise RuntimeError(f"{exe} has not been built (make -C neutronbench_amd/csrc)")
     cmd = [exe, "--dir", directory, "--V", str(V), "--F", str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch",
            str(cfg["batch"]), "--fanout", ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)),
-           "--pipeline", str(pipeline), "--cache", str(cfg["cache"]), "--graph", str(int(graph)), "--warmup",
+           "--pipeline", str(pipeline), "--cache", str(cfg["cache"]), "--graph", str(graph_mode(graph, pipeline)),
+           "--warmup",
            str(warmup_batches), "--max-batches", str(max_batches), "--verify", str(int(verify)), "--stage-sync",
            str(int(stage_sync))]
     if dump_dir:
@@ -415,9 +428,10 @@ if __name__ == "__main__":
                     help="1: wait for the stream after every stage (stage times are device times; default up to "
                          "--pipeline 2); 0: never wait for an aggregation, batches are ordered by events (stage times "
                          "are host enqueue times; default from --pipeline 3)")
-    ap.add_argument("--graph", type=int, default=1, choices=[0, 1],
-                    help="1 (default): each builder replays the launches of its hops as a HIP graph recorded at its "
-                         "first batch; 0: the launches are enqueued one by one for every batch")
+    ap.add_argument("--graph", type=int, default=None, choices=[0, 1, 2],
+                    help="1: each builder replays the launches of its hops as a HIP graph recorded at its first "
+                         "batch; 2: the same with each hop's transposition and weights on a side branch of the graph; "
+                         "0: the launches are enqueued one by one for every batch; default 2 for --pipeline 1, else 1")
     ap.add_argument("--native", action="store_true",
                     help="drive the epoch from C++ (lib/nts_epoch) instead of this module's Python loop")
     ap.add_argument("--write-inputs", metavar="DIR", default=None,
@@ -434,10 +448,12 @@ if __name__ == "__main__":
                         str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch", str(cfg["batch"]), "--fanout",
                         ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)), "--cache",
                         str(cfg["cache"]), "--pipeline", str(a.pipeline), "--stage-sync",
-                        str(int(bool(a.stage_sync)) if a.stage_sync is not None else 1)]))
+                        str(int(bool(a.stage_sync)) if a.stage_sync is not None else 1), "--graph",
+                        str(graph_mode(True if a.graph is None else a.graph, a.pipeline))]))
     elif a.native:
-        run_native(a.config, a.scale, a.max_batches, a.warmup_batches, a.pipeline, graph=bool(a.graph),
-                   stage_sync=bool(a.stage_sync))
+        run_native(a.config, a.scale, a.max_batches, a.warmup_batches, a.pipeline,
+                   graph=True if a.graph is None else a.graph, stage_sync=bool(a.stage_sync))
     else:
         run(a.config, a.scale, a.max_batches, a.sampler, a.warmup_batches, a.pipeline,
-            stage_sync=None if a.stage_sync is None else bool(a.stage_sync), graph=bool(a.graph))
+            stage_sync=None if a.stage_sync is None else bool(a.stage_sync),
+            graph=True if a.graph is None else a.graph)

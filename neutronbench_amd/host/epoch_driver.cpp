@@ -143,7 +143,7 @@ Args parse(int argc, char **argv) {
       (a.heads && a.hidden % a.heads)) {
     fprintf(stderr,
             "usage: nts_epoch --dir D --V n --F n --fanout a,b[,c] [--batch n] [--hidden n] [--heads n] [--pipeline 1..8]\n"
-            "                 [--cache fraction] [--graph 0|1] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n"
+            "                 [--cache fraction] [--graph 0|1|2] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n"
             "                 [--dump-dir D [--dump-batch b]]\n");
     exit(2);
   }
@@ -237,7 +237,7 @@ int main(int argc, char **argv) {
     s.arena = device_bytes(arena_bytes);
     NTS(nts_batch_builder_create(&s.builder, d_co, d_ri, V, E, a.fanout.data(), hops, a.batch, want_perm, s.arena,
                                  arena_bytes));
-    if (a.graph) NTS(nts_batch_builder_use_graph(s.builder, 1));
+    if (a.graph) NTS(nts_batch_builder_use_graph(s.builder, a.graph));
     HIP(hipEventCreateWithFlags(&s.gathered, hipEventDisableTiming));
     HIP(hipEventCreateWithFlags(&s.trained, hipEventDisableTiming));
   }
@@ -549,8 +549,8 @@ int main(int argc, char **argv) {
   }
 
   printf("{\"driver\": \"native\", \"batches\": %u, \"batch_size\": %u, \"pipeline\": %u, \"hop_launches_as_graph\": %s, "
-         "\"stage_sync\": %s, \"epoch_s\": %.4f, \"sampled_edges\": %llu, \"gathered_rows\": %llu, \"cache_rows\": %u",
-         n_batches, a.batch, P, a.graph ? "true" : "false", a.stage_sync ? "true" : "false", epoch_s,
+         "\"hop_graph_mode\": %d, \"stage_sync\": %s, \"epoch_s\": %.4f, \"sampled_edges\": %llu, \"gathered_rows\": %llu, \"cache_rows\": %u",
+         n_batches, a.batch, P, a.graph ? "true" : "false", a.graph, a.stage_sync ? "true" : "false", epoch_s,
          static_cast<unsigned long long>(edges_total), static_cast<unsigned long long>(rows_total), n_cache);
   if (P == 1 && a.stage_sync)
     printf(", \"stage_s\": {\"sample\": %.4f, \"gather\": %.4f, \"aggregate_fwd\": %.4f, \"aggregate_bwd\": %.4f}", stage_sample,

@@ -180,17 +180,19 @@ def test_two_builders_on_two_streams_overlap_without_interference(device):
         b.close()
 
 
+@pytest.mark.parametrize("mode", [1, 2])
 @pytest.mark.parametrize("fanouts,want_perm", [([25, 10], True), ([15, 10, 5], True), ([64, 100], True)])
-def test_builder_replaying_a_graph_equals_the_launch_by_launch_builder(device, fanouts, want_perm):
+def test_builder_replaying_a_graph_equals_the_launch_by_launch_builder(device, fanouts, want_perm, mode):
     """nts_batch_builder_use_graph: the hops' launches are recorded at the first batch and replayed
-    for every later one.  Replays are interleaved with eager work and synchronisations of the
+    for every later one (mode 1: as one chain; mode 2: each hop's transposition and weights on a
+    side branch of the graph, beside the next hop's sampling).  Replays are interleaved with eager work and synchronisations of the
     program's own (the per-hop path run for comparison, read-backs), batch sizes and seeds change
     from replay to replay, and every replay must give the arrays of the eager builder bit for bit."""
     V, E, cap = 30000, 700000, 1500
     gco, gri = graph(V, E, 61, device)
     perm = synth.permutation(V, 62, device)
     eager = BatchBuilder(gco, gri, fanouts, cap, want_perm=want_perm)
-    replay = BatchBuilder(gco, gri, fanouts, cap, want_perm=want_perm, graph=True)
+    replay = BatchBuilder(gco, gri, fanouts, cap, want_perm=want_perm, graph=mode)
     sizes = [1500, 1500, 640, 1, 0, 1499, 77, 1500]
     at = 0
     for k, n in enumerate(sizes):
