@@ -515,8 +515,23 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
  *                enable == 2: the same, and in the recorded graph each hop's transposition and edge
  *                weights run on a side branch beside the next hop's sampling (same arrays; a batch
  *                built on an otherwise idle device gets shorter, one built beside other batches in
- *                flight does not -- use 1 there).  Any other non-zero value means 1.  Changing the
- *                value after a graph was recorded discards it; the next batch records again.
+ *                flight does not -- use 1 there).
+ *                enable == 3: two graphs.  The first holds the sampling and relabelling of every hop
+ *                and the copy of the layer shapes and runs on the caller's stream; the second holds
+ *                every hop's transposition and edge weights and runs after it on a stream that the
+ *                builder owns.  nts_batch_builder_layers then returns as soon as the FIRST has
+ *                finished: destination, source, column_offset and row_indices of every layer are
+ *                complete, and the feature gather can start, while row_offset, column_indices,
+ *                csr_to_csc and both weight arrays are still being written.  A stream that reads
+ *                those must be passed to nts_batch_builder_join first (the host must wait for that
+ *                stream before it reads them itself).  The next nts_batch_builder_sample of the
+ *                builder waits for the second graph by itself.  Same arrays bit for bit.
+ *                Any other non-zero value means 1.  Changing the value after a graph was recorded
+ *                discards it (waiting for a second graph still running); the next batch records again.
+ *   nts_batch_builder_join  makes `stream` wait (on the device; the call returns at once) until every
+ *                array of the builder's current batch is complete.  Needed with enable == 3 only;
+ *                otherwise the arrays are complete when nts_batch_builder_layers returns and the call
+ *                does nothing.
  * Calls on one builder must not overlap: consecutive nts_batch_builder_sample calls go to the same
  * stream, or the earlier batch is waited for first (nts_batch_builder_layers does). */
 typedef struct nts_batch_builder nts_batch_builder_t;
@@ -542,6 +557,7 @@ int nts_batch_builder_create(nts_batch_builder_t **builder, const uint32_t *grap
 int nts_batch_builder_sample(nts_batch_builder_t *builder, const uint32_t *batch_ids, uint32_t n, uint64_t seed,
                              nts_stream_t stream);
 int nts_batch_builder_use_graph(nts_batch_builder_t *builder, int enable);
+int nts_batch_builder_join(nts_batch_builder_t *builder, nts_stream_t stream);
 int nts_batch_builder_layers(nts_batch_builder_t *builder, nts_sampled_layer_t *layers);
 int nts_batch_builder_destroy(nts_batch_builder_t *builder);
 

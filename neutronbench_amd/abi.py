@@ -101,6 +101,7 @@ SIGNATURES = {
     "nts_batch_builder_sample": [_vp, _vp, _u32, _u64, _vp],
     "nts_batch_builder_layers": [_vp, _vp],
     "nts_batch_builder_use_graph": [_vp, ctypes.c_int],
+    "nts_batch_builder_join": [_vp, _vp],
     "nts_batch_builder_destroy": [_vp],
     "nts_relabel_sources_work_bytes": [_u32],
     "nts_relabel_sources": [_vp, _vp, _vp, _vp, _u32, _u32, _vp, _vp],

@@ -162,7 +162,9 @@ class BatchBuilder:
         call("nts_batch_builder_create", ctypes.byref(handle), ptr(graph_co), ptr(graph_ri), V, E, fan, self.hops,
              max_batch, int(want_perm), self.arena.data_ptr() + self._skew, nbytes)
         self.handle = handle.value
-        if graph:  # True/1: one recorded chain of launches; 2: hop transpositions on a side branch
+        # True/1: one recorded chain of launches; 2: hop transpositions on a side branch; 3: sampling and
+        # transpositions as two graphs, the second on a stream of the builder's (see `join`)
+        if graph:
             call("nts_batch_builder_use_graph", self.handle, int(graph))
         self._desc = (SampledLayerDesc * self.hops)()
 
@@ -182,9 +184,21 @@ class BatchBuilder:
             stream = torch.cuda.current_stream(self.device).cuda_stream
         call("nts_batch_builder_sample", self.handle, ptr(batch_ids), batch_ids.numel(), seed, stream)
 
-    def collect(self):
-        """Waits for the batch started by `enqueue`; the layers are complete when this returns."""
+    def join(self, stream=None):
+        """Makes `stream` (a raw handle; default: torch's current stream) wait on the device for every
+        array of the current batch; only a builder created with graph=3 has anything to wait for."""
+        if stream is None:
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+        call("nts_batch_builder_join", self.handle, stream)
+
+    def collect(self, join=True):
+        """Waits for the batch started by `enqueue`.  The layers are complete when this returns --
+        for a builder created with graph=3: complete for work enqueued on torch's current stream
+        (join=True), or, with join=False, only the sampled half (destination, source, column_offset,
+        row_indices; the caller calls `join` before the first use of the other arrays)."""
         call("nts_batch_builder_layers", self.handle, ctypes.addressof(self._desc))
+        if join:
+            self.join()
         layers = []
         i32, f32 = torch.int32, torch.float32
         for d in self._desc:

@@ -126,8 +126,16 @@ struct nts_batch_builder {
   bool bitmap_clean;  // the bitmap of sampled sources is all zero (each hop's last kernel leaves it so)
   bool use_graph;     // replay the hops' launches as one HIP graph, captured at the first batch
   bool fork_hops;     // in that graph, a hop's transposition and weights run on a branch beside the next hop's sampling
+  bool defer;         // two graphs: sampling on the caller's stream, transpositions and weights on `side`
   hipGraph_t graph;
   hipGraphExec_t graph_exec;
+  // defer only: the second graph, the builder's own stream that runs it, and the event recorded
+  // after it (what nts_batch_builder_join makes a consumer's stream wait for)
+  hipGraph_t structure_graph;
+  hipGraphExec_t structure_exec;
+  hipStream_t side;
+  hipEvent_t structured;
+  bool structure_pending;
 };
 
 namespace {
@@ -141,7 +149,12 @@ namespace {
 // side stream (which takes them hop by hop: they share the sort scratch), the main stream goes on with
 // hop h + 1, and the two join before the size table is copied.  The bitmap of sampled sources, which the
 // weights launch otherwise clears on its way, is then cleared by a launch of its own on the main stream.
-int enqueue_hops(nts_batch_builder *b, hipStream_t stream, hipStream_t side = nullptr, hipEvent_t *events = nullptr) {
+// phase: kAllOfABatch, or one half of it for a builder that defers the structure -- kSampling (offsets,
+// pick, relabelling and bitmap clearing of every hop, then the size table) and kStructure (sort, CSR
+// and weights of every hop), recorded as graphs of their own.
+enum Phase { kAllOfABatch, kSampling, kStructure };
+int enqueue_hops(nts_batch_builder *b, hipStream_t stream, hipStream_t side = nullptr, hipEvent_t *events = nullptr,
+                 Phase phase = kAllOfABatch) {
   unsigned char *A = b->arena;
   uint32_t *sizes = reinterpret_cast<uint32_t *>(A + b->L.sizes);
   const uint64_t *seed_word = reinterpret_cast<const uint64_t *>(A + b->L.seed);
@@ -166,44 +179,53 @@ int enqueue_hops(nts_batch_builder *b, hipStream_t stream, hipStream_t side = nu
     const DevCount Vd = device_count(hop_sizes + 0, H.vd_cap);
     const DevCount Vs = device_count(hop_sizes + 2, H.vs_cap);
     const DevCount E = device_edge_count(co, hop_sizes + 0, H.vd_cap, H.e_cap);
-    if (int rc = hop_offsets(co, b->graph_co, dst, Vd, b->fanout[h], A + b->L.scan_work, b->L.scan_bytes, stream))
-      return rc;
-    if (int rc = hop_neighbors(ri_global, co, b->graph_co, b->graph_ri, dst, Vd, H.e_cap, b->fanout[h],
-                               device_seed(seed_word, h), bits, owner, stream))
-      return rc;
-    // Local ids; the unused tail of the edge array is padded with a key that sorts after every
-    // source.
-    if (int rc = relabel_sources(source, hop_sizes + 2, hop_sizes + kSizeWords, ri, ri_global, E, H.e_cap, H.vs_cap,
-                                 hop_sizes + 1, b->V, A + b->L.relabel_work, true, stream))
-      return rc;
+    // the weights launch clears the bitmap on its way unless it runs apart from the sampling
+    const bool clear_apart = side != nullptr || phase != kAllOfABatch;
+    if (phase != kStructure) {
+      if (int rc = hop_offsets(co, b->graph_co, dst, Vd, b->fanout[h], A + b->L.scan_work, b->L.scan_bytes, stream))
+        return rc;
+      if (int rc = hop_neighbors(ri_global, co, b->graph_co, b->graph_ri, dst, Vd, H.e_cap, b->fanout[h],
+                                 device_seed(seed_word, h), bits, owner, stream))
+        return rc;
+      // Local ids; the unused tail of the edge array is padded with a key that sorts after every
+      // source.
+      if (int rc = relabel_sources(source, hop_sizes + 2, hop_sizes + kSizeWords, ri, ri_global, E, H.e_cap, H.vs_cap,
+                                   hop_sizes + 1, b->V, A + b->L.relabel_work, true, stream))
+        return rc;
+      if (clear_apart)
+        if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
+    }
     hipStream_t rest = stream;
     if (side) {
-      if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
       NTS_HIP_TRY(hipEventRecord(events[h], stream));
       NTS_HIP_TRY(hipStreamWaitEvent(side, events[h], 0));
       rest = side;
     }
-    if (int rc = csr_from_csc(ro, ci, perm, co, ri, Vd, Vs, E, H.e_cap, bits_for(H.vs_cap + 1), A + b->L.csr_work,
-                              owner, rest))
-      return rc;
-    if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, side ? nullptr : bits, side ? 0u : words, owner,
-                                  csr_owner, rest))
-      return rc;
+    if (phase != kSampling) {
+      if (int rc = csr_from_csc(ro, ci, perm, co, ri, Vd, Vs, E, H.e_cap, bits_for(H.vs_cap + 1), A + b->L.csr_work,
+                                owner, rest))
+        return rc;
+      if (int rc = gcn_edge_weights(ewf, ewb, co, ri, ro, ci, Vd, Vs, clear_apart ? nullptr : bits,
+                                    clear_apart ? 0u : words, owner, csr_owner, rest))
+        return rc;
+    }
     dst = source;  // the next hop's destinations are this hop's sources (init_dst)
   }
   if (side) {  // join
     NTS_HIP_TRY(hipEventRecord(events[b->hops], side));
     NTS_HIP_TRY(hipStreamWaitEvent(stream, events[b->hops], 0));
   }
-  const size_t size_bytes = (b->hops + 1) * kSizeWords * sizeof(uint32_t);
-  NTS_HIP_TRY(hipMemcpyAsync(b->host_sizes, sizes, size_bytes, hipMemcpyDeviceToHost, stream));
+  if (phase != kStructure) {
+    const size_t size_bytes = (b->hops + 1) * kSizeWords * sizeof(uint32_t);
+    NTS_HIP_TRY(hipMemcpyAsync(b->host_sizes, sizes, size_bytes, hipMemcpyDeviceToHost, stream));
+  }
   return NTS_OK;
 }
 
 // Records enqueue_hops into a graph and instantiates it.  The recording runs on a stream created for
 // it (the caller's may be the null stream, which cannot record; nothing executes while recording)
 // in thread-local mode: other host threads keep using the device meanwhile.
-int capture_hops(nts_batch_builder *b) {
+int capture_hops(nts_batch_builder *b, Phase phase, hipGraph_t *graph_out, hipGraphExec_t *exec_out) {
   hipStream_t stream = nullptr;
   NTS_HIP_TRY(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
   hipError_t begin = hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal);
@@ -214,13 +236,14 @@ int capture_hops(nts_batch_builder *b) {
   hipStream_t side = nullptr;
   hipEvent_t events[kMaxHops + 1] = {};
   int rc = NTS_OK;
-  if (b->fork_hops) {
-    if (hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) rc = fail(NTS_ERR_INVALID, "nts_batch_builder_sample: side stream");
+  if (b->fork_hops && phase == kAllOfABatch) {
+    if (hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess)
+      rc = fail(NTS_ERR_INVALID, "nts_batch_builder_sample: side stream");
     for (uint32_t h = 0; rc == NTS_OK && h <= b->hops; ++h)
       if (hipEventCreateWithFlags(&events[h], hipEventDisableTiming) != hipSuccess)
         rc = fail(NTS_ERR_INVALID, "nts_batch_builder_sample: event");
   }
-  if (rc == NTS_OK) rc = enqueue_hops(b, stream, side, side ? events : nullptr);
+  if (rc == NTS_OK) rc = enqueue_hops(b, stream, side, side ? events : nullptr, phase);
   hipGraph_t graph = nullptr;
   const hipError_t end = hipStreamEndCapture(stream, &graph);  // always ends the recording, also after an error
   (void)hipStreamDestroy(stream);
@@ -238,9 +261,23 @@ int capture_hops(nts_batch_builder *b) {
     (void)hipGraphDestroy(graph);
     return fail_hip(inst, "nts_batch_builder_sample: hipGraphInstantiate");
   }
-  b->graph = graph;
-  b->graph_exec = exec;
+  *graph_out = graph;
+  *exec_out = exec;
   return NTS_OK;
+}
+
+// Drops the recorded graphs (after waiting for a structure graph still running): the next batch records again.
+void drop_graphs(nts_batch_builder *b) {
+  if (b->side) (void)hipStreamSynchronize(b->side);
+  b->structure_pending = false;
+  if (b->graph_exec) (void)hipGraphExecDestroy(b->graph_exec);
+  if (b->graph) (void)hipGraphDestroy(b->graph);
+  if (b->structure_exec) (void)hipGraphExecDestroy(b->structure_exec);
+  if (b->structure_graph) (void)hipGraphDestroy(b->structure_graph);
+  b->graph_exec = nullptr;
+  b->graph = nullptr;
+  b->structure_exec = nullptr;
+  b->structure_graph = nullptr;
 }
 
 }  // namespace
@@ -288,8 +325,14 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
   b->bitmap_clean = false;
   b->use_graph = false;
   b->fork_hops = false;
+  b->defer = false;
   b->graph = nullptr;
   b->graph_exec = nullptr;
+  b->structure_graph = nullptr;
+  b->structure_exec = nullptr;
+  b->side = nullptr;
+  b->structured = nullptr;
+  b->structure_pending = false;
   hipError_t err = hipHostMalloc(reinterpret_cast<void **>(&b->host_sizes), (hops + 1) * kSizeWords * sizeof(uint32_t),
                                  hipHostMallocDefault);
   if (err == hipSuccess) {
@@ -307,8 +350,9 @@ int nts_batch_builder_create(nts_batch_builder_t **out, const uint32_t *graph_co
 int nts_batch_builder_destroy(nts_batch_builder_t *b) {
   NTS_TRACE_RANGE("nts_batch_builder_destroy");
   if (!b) return NTS_OK;
-  if (b->graph_exec) (void)hipGraphExecDestroy(b->graph_exec);
-  if (b->graph) (void)hipGraphDestroy(b->graph);
+  drop_graphs(b);
+  if (b->structured) (void)hipEventDestroy(b->structured);
+  if (b->side) (void)hipStreamDestroy(b->side);
   hipError_t e1 = hipEventDestroy(b->done);
   hipError_t e2 = hipHostFree(b->host_sizes);
   delete b;
@@ -332,6 +376,8 @@ int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, 
   // hop's last kernel clears them again; only a first or an interrupted batch clears them up front.
   uint32_t *bits = reinterpret_cast<uint32_t *>(A + b->L.relabel_work);
   const uint32_t words = (b->V + 31) / 32;
+  // the structure graph of the batch before reads what this batch's sampling overwrites
+  if (b->structure_pending) NTS_HIP_TRY(hipStreamWaitEvent(stream, b->structured, 0));
   if (!b->bitmap_clean)
     if (int rc = nts_memset_zero(bits, static_cast<size_t>(words) * sizeof(uint32_t), stream)) return rc;
   b->bitmap_clean = false;
@@ -341,7 +387,9 @@ int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, 
   NTS_LAUNCH_CHECK("start_batch_kernel");
   if (b->use_graph) {
     if (!b->graph_exec)
-      if (int rc = capture_hops(b)) return rc;
+      if (int rc = capture_hops(b, b->defer ? kSampling : kAllOfABatch, &b->graph, &b->graph_exec)) return rc;
+    if (b->defer && !b->structure_exec)
+      if (int rc = capture_hops(b, kStructure, &b->structure_graph, &b->structure_exec)) return rc;
     NTS_HIP_TRY(hipGraphLaunch(b->graph_exec, stream));
   } else {
     if (int rc = enqueue_hops(b, stream)) return rc;
@@ -349,20 +397,37 @@ int nts_batch_builder_sample(nts_batch_builder_t *b, const uint32_t *batch_ids, 
   NTS_HIP_TRY(hipEventRecord(b->done, stream));
   b->pending = true;
   b->bitmap_clean = true;
+  if (b->use_graph && b->defer) {
+    NTS_HIP_TRY(hipStreamWaitEvent(b->side, b->done, 0));
+    NTS_HIP_TRY(hipGraphLaunch(b->structure_exec, b->side));
+    NTS_HIP_TRY(hipEventRecord(b->structured, b->side));
+    b->structure_pending = true;
+  }
   return NTS_OK;
 }
 
 int nts_batch_builder_use_graph(nts_batch_builder_t *b, int enable) {
   if (!b) return fail(NTS_ERR_INVALID, "nts_batch_builder_use_graph: null builder");
-  if (b->graph_exec && (b->use_graph != (enable != 0) || b->fork_hops != (enable == 2))) {
-    // another shape of graph than the one recorded: record again at the next batch
-    (void)hipGraphExecDestroy(b->graph_exec);
-    (void)hipGraphDestroy(b->graph);
-    b->graph_exec = nullptr;
-    b->graph = nullptr;
+  if (b->use_graph != (enable != 0) || b->fork_hops != (enable == 2) || b->defer != (enable == 3))
+    drop_graphs(b);  // another shape of graph than the one recorded: record again at the next batch
+  if (enable == 3 && !b->side) {
+    NTS_HIP_TRY(hipStreamCreateWithFlags(&b->side, hipStreamNonBlocking));
+    const hipError_t err = hipEventCreateWithFlags(&b->structured, hipEventDisableTiming);
+    if (err != hipSuccess) {
+      (void)hipStreamDestroy(b->side);
+      b->side = nullptr;
+      return fail_hip(err, "nts_batch_builder_use_graph: hipEventCreateWithFlags");
+    }
   }
   b->use_graph = enable != 0;
   b->fork_hops = enable == 2;
+  b->defer = enable == 3;
+  return NTS_OK;
+}
+
+int nts_batch_builder_join(nts_batch_builder_t *b, nts_stream_t stream) {
+  if (!b) return fail(NTS_ERR_INVALID, "nts_batch_builder_join: null builder");
+  if (b->structure_pending) NTS_HIP_TRY(hipStreamWaitEvent(stream, b->structured, 0));
   return NTS_OK;
 }
 

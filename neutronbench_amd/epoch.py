@@ -60,20 +60,25 @@ class Timer:
         self.t[key] = self.t.get(key, 0.0) + time.perf_counter() - t0
 
 
-def graph_mode(graph, pipeline):
-    """The value for nts_batch_builder_use_graph.  True picks by measurement: with one batch in flight
-    the hops' transpositions go to a side branch of the recorded graph (2: the chip is otherwise idle
-    beside the chain of small sampling launches); with several batches in flight the chains of the
-    other builders already fill it and the extra branch only costs (1)."""
+def graph_mode(graph, pipeline, cache=0.0):
+    """The value for nts_batch_builder_use_graph.  True picks by measurement.  With several batches in
+    flight: 1 (one recorded chain of launches; the chains of the other builders already fill the
+    chip, extra branches and streams only cost).  With one batch in flight the transpositions and
+    weights leave the chain: with an HBM feature cache they run as a second graph beside the gather
+    (3); a gather that reads every row over PCIe slows kernels running beside it several times over
+    (their memory requests queue behind the link's), so there they stay inside the batch's one graph,
+    on a side branch beside the next hop's sampling (2)."""
     if graph is True:
-        return 2 if pipeline == 1 else 1
+        if pipeline > 1:
+            return 1
+        return 3 if cache > 0 else 2
     return int(graph)
 
 
 def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pipeline=1, quiet=False, checksum=False,
         stage_sync=None, graph=True):
     cfg = dict(CONFIGS[name])
-    graph = graph_mode(graph, pipeline)
+    graph = graph_mode(graph, pipeline, cfg["cache"])
     dev = torch.device("cuda:0")
     V, E = int(cfg["V"] * scale), int(cfg["E"] * scale)
     n_train = int(cfg["train"] * scale)
@@ -212,13 +217,16 @@ def run(name, scale=1.0, max_batches=0, sampler="builder", warmup_batches=2, pip
         for b in sequence:
             if builder is not None:
                 t0 = time.perf_counter()
-                layers = builder.sample(batch_ids(b), 1000 * b)
+                builder.enqueue(batch_ids(b), 1000 * b)
+                layers = builder.collect(join=False)  # graph mode 3: the transposed structure is still being built
                 tm.add("sample", t0)
             else:
                 layers = sample_hop_by_hop(b)
             t0 = time.perf_counter()
             x, _, hits = gather(cs, layers)
             tm.add("gather", t0)
+            if builder is not None:
+                builder.join()  # the aggregation is the first to read the transposed structure and the weights
             finish_batch(layers, x, hits)
 
     def run_two_stage(sequence):
@@ -378,10 +386,9 @@ def run_native_on(directory, name, V, max_batches=0, warmup_batches=2, pipeline=
         raise RuntimeError(f"{exe} has not been built (make -C neutronbench_amd/csrc)")
     cmd = [exe, "--dir", directory, "--V", str(V), "--F", str(cfg["F"]), "--hidden", str(cfg["hidden"]), "--batch",
            str(cfg["batch"]), "--fanout", ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)),
-           "--pipeline", str(pipeline), "--cache", str(cfg["cache"]), "--graph", str(graph_mode(graph, pipeline)),
-           "--warmup",
-           str(warmup_batches), "--max-batches", str(max_batches), "--verify", str(int(verify)), "--stage-sync",
-           str(int(stage_sync))]
+           "--pipeline", str(pipeline), "--cache", str(cfg["cache"]), "--graph",
+           str(graph_mode(graph, pipeline, cfg["cache"])), "--warmup", str(warmup_batches), "--max-batches",
+           str(max_batches), "--verify", str(int(verify)), "--stage-sync", str(int(stage_sync))]
     if dump_dir:
         cmd += ["--dump-dir", dump_dir, "--dump-batch", str(dump_batch)]
     p = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
@@ -428,10 +435,12 @@ if __name__ == "__main__":
                     help="1: wait for the stream after every stage (stage times are device times; default up to "
                          "--pipeline 2); 0: never wait for an aggregation, batches are ordered by events (stage times "
                          "are host enqueue times; default from --pipeline 3)")
-    ap.add_argument("--graph", type=int, default=None, choices=[0, 1, 2],
+    ap.add_argument("--graph", type=int, default=None, choices=[0, 1, 2, 3],
                     help="1: each builder replays the launches of its hops as a HIP graph recorded at its first "
                          "batch; 2: the same with each hop's transposition and weights on a side branch of the graph; "
-                         "0: the launches are enqueued one by one for every batch; default 2 for --pipeline 1, else 1")
+                         "3: transpositions and weights as a second graph on the builder's own stream, beside the "
+                         "gather; 0: the launches are enqueued one by one for every batch; default for --pipeline 1: "
+                         "3 with a feature cache, 2 without; else 1")
     ap.add_argument("--native", action="store_true",
                     help="drive the epoch from C++ (lib/nts_epoch) instead of this module's Python loop")
     ap.add_argument("--write-inputs", metavar="DIR", default=None,
@@ -449,7 +458,7 @@ if __name__ == "__main__":
                         ",".join(map(str, cfg["fanout"])), "--heads", str(cfg.get("heads", 0)), "--cache",
                         str(cfg["cache"]), "--pipeline", str(a.pipeline), "--stage-sync",
                         str(int(bool(a.stage_sync)) if a.stage_sync is not None else 1), "--graph",
-                        str(graph_mode(True if a.graph is None else a.graph, a.pipeline))]))
+                        str(graph_mode(True if a.graph is None else a.graph, a.pipeline, cfg["cache"]))]))
     elif a.native:
         run_native(a.config, a.scale, a.max_batches, a.warmup_batches, a.pipeline,
                    graph=True if a.graph is None else a.graph, stage_sync=bool(a.stage_sync))

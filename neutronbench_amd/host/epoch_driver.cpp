@@ -143,7 +143,7 @@ Args parse(int argc, char **argv) {
       (a.heads && a.hidden % a.heads)) {
     fprintf(stderr,
             "usage: nts_epoch --dir D --V n --F n --fanout a,b[,c] [--batch n] [--hidden n] [--heads n] [--pipeline 1..8]\n"
-            "                 [--cache fraction] [--graph 0|1|2] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n"
+            "                 [--cache fraction] [--graph 0|1|2|3] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n"
             "                 [--dump-dir D [--dump-batch b]]\n");
     exit(2);
   }
@@ -374,6 +374,9 @@ int main(int argc, char **argv) {
     if (a.stage_sync) t_bwd += now() - t0;
   };
   auto aggregate = [&](Slot &s, hipStream_t stream) {
+    // --graph 3: the transposed structure and the weights are still being built on the builder's own
+    // stream while the features are gathered; the aggregation is the first to read them
+    NTS(nts_batch_builder_join(s.builder, stream));
     if (H) return aggregate_gat(s, stream);
     double t0 = now();
     for (uint32_t l = 0; l < hops; ++l) {
@@ -518,6 +521,7 @@ int main(int argc, char **argv) {
     sample(s, b, main_stream);
     NTS(nts_batch_builder_layers(s.builder, s.layers));
     gather(s, 0, main_stream);
+    NTS(nts_batch_builder_join(s.builder, main_stream));  // the transposed structure is written out below
     HIP(hipStreamSynchronize(main_stream));
     FILE *meta = fopen((a.dump_dir + "/meta.json").c_str(), "w");
     if (!meta) die("cannot write meta.json");

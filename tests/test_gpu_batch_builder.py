@@ -180,12 +180,13 @@ def test_two_builders_on_two_streams_overlap_without_interference(device):
         b.close()
 
 
-@pytest.mark.parametrize("mode", [1, 2])
+@pytest.mark.parametrize("mode", [1, 2, 3])
 @pytest.mark.parametrize("fanouts,want_perm", [([25, 10], True), ([15, 10, 5], True), ([64, 100], True)])
 def test_builder_replaying_a_graph_equals_the_launch_by_launch_builder(device, fanouts, want_perm, mode):
     """nts_batch_builder_use_graph: the hops' launches are recorded at the first batch and replayed
     for every later one (mode 1: as one chain; mode 2: each hop's transposition and weights on a
-    side branch of the graph, beside the next hop's sampling).  Replays are interleaved with eager work and synchronisations of the
+    side branch of the graph, beside the next hop's sampling; mode 3: the transpositions and weights
+    as a second graph on a stream of the builder's, which `sample` joins to the current stream).  Replays are interleaved with eager work and synchronisations of the
     program's own (the per-hop path run for comparison, read-backs), batch sizes and seeds change
     from replay to replay, and every replay must give the arrays of the eager builder bit for bit."""
     V, E, cap = 30000, 700000, 1500
@@ -233,3 +234,37 @@ def test_graph_builders_on_two_streams(device):
                 assert getattr(l, name).cpu().numpy().tobytes() == expect[name].tobytes(), f"batch {k} {name}"
     for b in builders:
         b.close()
+
+
+def test_deferred_structure_is_joined_by_the_stream_that_reads_it(device):
+    """Graph mode 3: nts_batch_builder_layers returns when the sampled half of the batch is complete
+    (ids, offsets, local row indices: readable at once from any stream) while the transposed structure
+    and the weights are still being built on the builder's own stream; a stream that reads those calls
+    nts_batch_builder_join first.  The next batch is enqueued without any wait for that second half
+    from the caller (the builder orders it); every array equals the launch-by-launch builder's."""
+    V, E, fanouts, cap = 40000, 900000, [12, 9, 6], 1200
+    gco, gri = graph(V, E, 81, device)
+    perm = as_u32(synth.permutation(V, 82, device))
+    eager = BatchBuilder(gco, gri, fanouts, cap, want_perm=True)
+    deferred = BatchBuilder(gco, gri, fanouts, cap, want_perm=True, graph=3)
+    sampled_half = ("dev_destination", "dev_source", "dev_column_offset", "dev_row_indices")
+    producer, reader = torch.cuda.Stream(device=device), torch.cuda.Stream(device=device)
+    at = 0
+    for k, n in enumerate([1200, 1200, 500, 0, 1199, 3, 1200]):
+        ids = perm[at:at + n]
+        at += n
+        want = eager.sample(ids, 300 + k)
+        torch.cuda.synchronize()
+        deferred.enqueue(ids, 300 + k, producer.cuda_stream)
+        layers = deferred.collect(join=False)
+        with torch.cuda.stream(reader):
+            first = [{name: getattr(l, name).tensor().clone() for name in sampled_half} for l in layers]
+            deferred.join(reader.cuda_stream)
+            rest = [{name: getattr(l, name).tensor().clone() for name in ARRAYS if name not in sampled_half}
+                    for l in layers]
+        reader.synchronize()
+        for l, a, b in zip(want, first, rest):
+            for name, got in {**a, **b}.items():
+                assert torch.equal(got, getattr(l, name).tensor()), f"batch {k} {name}"
+    eager.close()
+    deferred.close()

@@ -78,12 +78,15 @@ def test_native_epoch_driver(config, scale):
     """The epoch driven from C++ (lib/nts_epoch, neutronbench_amd/host/epoch_driver.cpp): same graph,
     train ids and seeds as the Python loop, so it samples the same edges, gathers the same rows and
     hits the cache as often; its checksum of every aggregation output (a device-side hash per layer
-    and direction) is the same for every number of batches in flight, with and without graph replay."""
+    and direction) is the same for every number of batches in flight, without graph replay and with each of its three
+    shapes (one chain; transpositions on a side branch; transpositions as a second graph on the builder's own
+    stream, joined before the aggregation)."""
     from neutronbench_amd import epoch
 
     py = epoch.run(config, scale=scale, max_batches=7, warmup_batches=1, quiet=True)
     runs = [epoch.run_native(config, scale=scale, max_batches=7, warmup_batches=1, pipeline=p, graph=g, quiet=True,
-                             verify=True) for p, g in ((1, True), (1, False), (2, True), (3, True), (5, True))]
+                             verify=True)
+            for p, g in ((1, True), (1, False), (1, 1), (1, 2), (1, 3), (2, True), (2, 3), (3, True), (5, True), (4, 3))]
     for r in runs:
         assert r["batches"] == py["batches"]
         assert r["sampled_edges"] == py["sampled_edges"] and r["gathered_rows"] == py["gathered_rows"]
