@@ -107,9 +107,10 @@ __global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, con
 // ---- edge -> vertex sums ----------------------------------------------------------------------
 //
 // Rows with at most `long_limit` edges: a group of G lanes per row (64/G rows per wavefront) adds
-// the row's edge rows in order.  Longer rows (power-law hubs) are left to the block kernel below,
-// which is handed the list of such rows; it spreads a row's edges over the slices of a 1024-thread
-// block and adds the slices' partial sums in a fixed order.
+// the row's edge rows in order.  Longer rows (power-law hubs) are listed first and summed by whole
+// blocks -- the first blocks of the same launch where the row launch is the balanced kernel, the
+// block kernels below otherwise -- which spread a row's edges over the slices of the block and add
+// the slices' partial sums in a fixed order.
 
 constexpr uint32_t kNoLimit = 0xFFFFFFFFu;
 constexpr uint32_t kLongRowEdges = 1024;    // edges of a row above which the block kernel takes over
@@ -174,6 +175,87 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_kernel(V *__restrict__
   }
 }
 
+// What the first blocks of a row launch do beside it when the rows above `long_limit` edges are summed
+// in the same launch: the list of those rows, the piece table of the giant ones, where the pieces' sums
+// go, the column tile of a 256-thread block and how many blocks are set aside (0: none).
+template <typename V>
+struct LongRowWork {
+  const uint32_t *list, *count, *hdr;
+  const uint4 *pieces;
+  V *partial;
+  uint32_t tile, blocks;
+};
+
+__device__ __forceinline__ void vadd(float &a, const float &b) { a += b; }
+__device__ __forceinline__ void vadd(float4 &a, const float4 &b) {
+  a.x += b.x;
+  a.y += b.y;
+  a.z += b.z;
+  a.w += b.w;
+}
+template <typename V>
+__device__ __forceinline__ V vnull();
+template <>
+__device__ __forceinline__ float vnull<float>() {
+  return 0.f;
+}
+template <>
+__device__ __forceinline__ float4 vnull<float4>() {
+  return make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// Sum of the edge rows [e0, e1) by one block of BLOCK threads, added into dst[0 .. Fv) (V = float, or
+// float4 when rows are 16-byte aligned: a quarter of the load instructions and of the rounds a row
+// takes).  Columns are taken in tiles of `tile` vectors (a power of two <= BLOCK); thread t owns
+// column t % tile of slice t / tile, a slice adds every (BLOCK/tile)-th edge of the range in ascending
+// order (eight loads in flight), and the slices' sums are then added pairwise in a fixed tree.
+template <typename V, int BLOCK>
+__device__ __forceinline__ void block_sum_edge_rows(V *__restrict__ dst, const V *__restrict__ msg,
+                                                    const uint32_t *__restrict__ perm, uint32_t e0, uint32_t e1,
+                                                    uint32_t Fv, uint32_t tile, int accumulate, V *part) {
+  const uint32_t c = threadIdx.x & (tile - 1);
+  const uint32_t slice = threadIdx.x / tile;
+  const uint32_t n_slices = BLOCK / tile;
+  for (uint32_t cb = 0; cb < Fv; cb += tile) {
+    const uint32_t col = cb + c;
+    V a = vnull<V>();
+    if (col < Fv) {
+      uint32_t k = e0 + slice;
+      for (; static_cast<uint64_t>(k) + 7ull * n_slices < e1; k += 8 * n_slices) {
+        V v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const uint32_t kk = k + u * n_slices;
+          const uint32_t e = perm ? perm[kk] : kk;
+          v[u] = msg[static_cast<size_t>(e) * Fv + col];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) vadd(a, v[u]);
+      }
+      for (; k < e1; k += n_slices) {
+        const uint32_t e = perm ? perm[k] : k;
+        vadd(a, msg[static_cast<size_t>(e) * Fv + col]);
+      }
+    }
+    part[threadIdx.x] = a;
+    __syncthreads();
+    for (uint32_t stride = n_slices / 2; stride >= 1; stride >>= 1) {
+      if (slice < stride) {
+        V lo = part[threadIdx.x];
+        vadd(lo, part[threadIdx.x + stride * tile]);
+        part[threadIdx.x] = lo;
+      }
+      __syncthreads();
+    }
+    if (slice == 0 && col < Fv) {
+      V total = part[c];
+      if (accumulate) vadd(total, dst[col]);
+      dst[col] = total;
+    }
+    __syncthreads();
+  }
+}
+
 // The same sums for rows that fit one group (Fv <= G), with the rows of a wavefront handed out
 // dynamically: a wavefront takes 64 consecutive rows, reads their offsets with one coalesced load,
 // and its 64/G groups then pull rows from that set one after the other -- a group that finishes a
@@ -200,7 +282,27 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
                                                                           const uint32_t *__restrict__ off,
                                                                           const uint32_t *__restrict__ perm,
                                                                           uint32_t rows, uint32_t Fv, int accumulate,
-                                                                          uint32_t long_limit, uint32_t coop_limit) {
+                                                                          uint32_t long_limit, uint32_t coop_limit,
+                                                                          LongRowWork<V> lw) {
+  if (blockIdx.x < lw.blocks) {
+    // The first blocks of the launch take the listed long rows, one block per row, and the pieces of
+    // the giant ones (their partial sums are combined by a launch of its own afterwards); the rows
+    // below fill the chip meanwhile.
+    __shared__ V long_part[256];
+    const uint32_t n_rows = *lw.count;
+    for (uint32_t i = blockIdx.x; i < n_rows; i += lw.blocks) {
+      const uint32_t r = lw.list[i];
+      block_sum_edge_rows<V, 256>(out + static_cast<size_t>(r) * Fv, msg, perm, off[r], off[r + 1], Fv, lw.tile,
+                                  accumulate, long_part);
+    }
+    const uint32_t n_pieces = lw.hdr[1];
+    for (uint32_t p = blockIdx.x; p < n_pieces; p += lw.blocks) {
+      const uint4 pc = lw.pieces[p];
+      block_sum_edge_rows<V, 256>(lw.partial + static_cast<size_t>(p) * Fv, msg, perm, pc.z, pc.w, Fv, lw.tile, 0,
+                                  long_part);
+    }
+    return;
+  }
   constexpr bool kCoop = G <= 8;
   constexpr int kCoopU = sizeof(V) == 16 ? 4 : 8;           // loads per lane and round on the cooperative path
   constexpr uint32_t kCoopFloats = kWave * kCoopU * (sizeof(V) / 4);  // floats of a wavefront's tile
@@ -213,8 +315,8 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
   constexpr int GG = G * S;  // lanes that share a row
   const uint32_t gl = lane & (GG - 1), grp = lane / GG;
   const uint32_t col = gl & (G - 1), slice = gl / G;
-  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
-  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * blockDim.x / kWave;
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x - lw.blocks) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x - lw.blocks) * blockDim.x / kWave;
   const bool col_live = col < Fv;
   for (uint64_t base = wave * kSet; base < rows; base += n_waves * kSet) {
     uint32_t my_e0 = 0, my_e1 = 0;
@@ -485,76 +587,6 @@ __global__ __launch_bounds__(256) void giant_plan_kernel(uint32_t *__restrict__ 
   }
 }
 
-__device__ __forceinline__ void vadd(float &a, const float &b) { a += b; }
-__device__ __forceinline__ void vadd(float4 &a, const float4 &b) {
-  a.x += b.x;
-  a.y += b.y;
-  a.z += b.z;
-  a.w += b.w;
-}
-template <typename V>
-__device__ __forceinline__ V vnull();
-template <>
-__device__ __forceinline__ float vnull<float>() {
-  return 0.f;
-}
-template <>
-__device__ __forceinline__ float4 vnull<float4>() {
-  return make_float4(0.f, 0.f, 0.f, 0.f);
-}
-
-// Sum of the edge rows [e0, e1) by one 1024-thread block, added into dst[0 .. Fv) (V = float, or
-// float4 when rows are 16-byte aligned: a quarter of the load instructions and of the rounds a row
-// takes).  Columns are taken in tiles of `tile` vectors (a power of two <= 1024); thread t owns
-// column t % tile of slice t / tile, a slice adds every (1024/tile)-th edge of the range in ascending
-// order (eight loads in flight), and the slices' sums are then added pairwise in a fixed tree.
-template <typename V>
-__device__ __forceinline__ void block_sum_edge_rows(V *__restrict__ dst, const V *__restrict__ msg,
-                                                    const uint32_t *__restrict__ perm, uint32_t e0, uint32_t e1,
-                                                    uint32_t Fv, uint32_t tile, int accumulate, V *part) {
-  const uint32_t c = threadIdx.x & (tile - 1);
-  const uint32_t slice = threadIdx.x / tile;
-  const uint32_t n_slices = kLongBlock / tile;
-  for (uint32_t cb = 0; cb < Fv; cb += tile) {
-    const uint32_t col = cb + c;
-    V a = vnull<V>();
-    if (col < Fv) {
-      uint32_t k = e0 + slice;
-      for (; static_cast<uint64_t>(k) + 7ull * n_slices < e1; k += 8 * n_slices) {
-        V v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const uint32_t kk = k + u * n_slices;
-          const uint32_t e = perm ? perm[kk] : kk;
-          v[u] = msg[static_cast<size_t>(e) * Fv + col];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) vadd(a, v[u]);
-      }
-      for (; k < e1; k += n_slices) {
-        const uint32_t e = perm ? perm[k] : k;
-        vadd(a, msg[static_cast<size_t>(e) * Fv + col]);
-      }
-    }
-    part[threadIdx.x] = a;
-    __syncthreads();
-    for (uint32_t stride = n_slices / 2; stride >= 1; stride >>= 1) {
-      if (slice < stride) {
-        V lo = part[threadIdx.x];
-        vadd(lo, part[threadIdx.x + stride * tile]);
-        part[threadIdx.x] = lo;
-      }
-      __syncthreads();
-    }
-    if (slice == 0 && col < Fv) {
-      V total = part[c];
-      if (accumulate) vadd(total, dst[col]);
-      dst[col] = total;
-    }
-    __syncthreads();
-  }
-}
-
 // One 1024-thread block per listed long row.
 template <typename V>
 __global__ __launch_bounds__(kLongBlock) void gather_edge_to_row_long_kernel(
@@ -565,7 +597,8 @@ __global__ __launch_bounds__(kLongBlock) void gather_edge_to_row_long_kernel(
   const uint32_t n_rows = *count;
   for (uint32_t i = blockIdx.x; i < n_rows; i += gridDim.x) {
     const uint32_t r = list[i];
-    block_sum_edge_rows(out + static_cast<size_t>(r) * Fv, msg, perm, off[r], off[r + 1], Fv, tile, accumulate, part);
+    block_sum_edge_rows<V, kLongBlock>(out + static_cast<size_t>(r) * Fv, msg, perm, off[r], off[r + 1], Fv, tile,
+                                       accumulate, part);
   }
 }
 
@@ -581,7 +614,7 @@ __global__ __launch_bounds__(kLongBlock) void giant_sum_pieces_kernel(V *__restr
   const uint32_t n_pieces = hdr[1];
   for (uint32_t p = blockIdx.x; p < n_pieces; p += gridDim.x) {
     const uint4 pc = pieces[p];
-    block_sum_edge_rows(partial + static_cast<size_t>(p) * Fv, msg, perm, pc.z, pc.w, Fv, tile, 0, part);
+    block_sum_edge_rows<V, kLongBlock>(partial + static_cast<size_t>(p) * Fv, msg, perm, pc.z, pc.w, Fv, tile, 0, part);
   }
 }
 
@@ -1737,17 +1770,36 @@ uint32_t coop_limit() {
   return value;
 }
 
+// Blocks of a row launch set aside for the long rows when they are summed in the same launch: as many
+// threads as the long-row kernels of their own bring (512 blocks of 1,024).
+constexpr uint32_t kMergedLongBlocks = 2048;
+// NTS_EDGE_SUM_MERGE in the environment: 0 = long rows always in launches of their own; n > 0 = that many
+// blocks of the row launch for them.
+uint32_t merged_long_blocks() {
+  static const uint32_t value = [] {
+    const char *env = getenv("NTS_EDGE_SUM_MERGE");
+    if (!env) return kMergedLongBlocks;
+    const long v = atol(env);
+    return v <= 0 ? 0u : static_cast<uint32_t>(v);
+  }();
+  return value;
+}
+
+// The row launch whose first blocks also sum the long rows: one-group rows of a vertex set large enough.
+bool rows_launch_takes_long_rows(uint32_t rows, uint32_t Fv) { return Fv <= 64 && rows >= 4096; }
+
 template <typename V>
 void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_t *perm, uint32_t rows, uint32_t Fv,
-                        int accumulate, uint32_t limit, hipStream_t stream) {
-  if (Fv <= 64 && rows >= 4096) {
+                        int accumulate, uint32_t limit, const LongRowWork<V> &lw, hipStream_t stream) {
+  if (rows_launch_takes_long_rows(rows, Fv)) {
     // One group covers a row: wavefronts hand their 64 rows out dynamically (strided launch).
 #define NTS_BALANCED(GG, SS)                                                                                    \
   do {                                                                                                          \
     const uint32_t set = (kWave / ((GG) * (SS))) * 8 < kWave ? (kWave / ((GG) * (SS))) * 8 : kWave;            \
     const uint32_t blocks = ceil_div(rows, 4 * set); /* at most `set` rows per wavefront at a time */          \
-    hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG, SS>), dim3(blocks < 16384u ? blocks : 16384u), \
-                       dim3(256), 0, stream, out, msg, off, perm, rows, Fv, accumulate, limit, coop_limit());   \
+    hipLaunchKernelGGL((gather_edge_to_row_balanced_kernel<V, GG, SS>),                                         \
+                       dim3((blocks < 16384u ? blocks : 16384u) + lw.blocks), dim3(256), 0, stream, out, msg, off, \
+                       perm, rows, Fv, accumulate, limit, coop_limit(), lw);                                    \
   } while (0)
     switch (lanes_for(Fv)) {  // rows narrower than eight lanes are shared by eight lanes all the same
       case 1: NTS_BALANCED(1, 8); break;
@@ -1784,42 +1836,56 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
   LongRows lr;
   if (int rc = collect_long_rows(lr, off, rows, 1u, kLongRowEdges, kGiantRowEdges, stream)) return rc;
   const uint32_t limit = lr.list ? kLongRowEdges : kNoLimit;
-  if (F % 4 == 0 && aligned_to(out, 16) && aligned_to(msg, 16))
-    launch_gather_rows(reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, rows, F / 4,
-                       accumulate, limit, stream);
-  else
-    launch_gather_rows(out, msg, off, perm, rows, F, accumulate, limit, stream);
-  NTS_LAUNCH_CHECK(who);
+  // 16-byte vectors for the row kernels and the block kernels alike
+  const bool v4 = F % 4 == 0 && aligned_to(out, 16) && aligned_to(msg, 16);
+  const uint32_t Fv = v4 ? F / 4 : F;
+  // Long rows: in the first blocks of the row launch where that launch has them (256-thread blocks),
+  // else in launches of their own after it (1,024-thread blocks).  Giant rows: pieces by separate
+  // blocks into stream-ordered scratch, then the ordered combine.
+  const bool merged = lr.list && rows_launch_takes_long_rows(rows, Fv) && merged_long_blocks() > 0;
+  const uint32_t block_threads = merged ? 256u : static_cast<uint32_t>(kLongBlock);
+  uint32_t tile = 1;
+  while (tile < Fv && tile < block_threads) tile <<= 1;
+  ScratchBlock partial_block;
+  float *partial = nullptr;
   if (lr.list) {
-    // The block kernels take 16-byte vectors under the same condition as the row kernels above.
-    const bool v4 = F % 4 == 0 && aligned_to(out, 16) && aligned_to(msg, 16);
-    const uint32_t Fv = v4 ? F / 4 : F;
-    uint32_t tile = 1;
-    while (tile < Fv && tile < static_cast<uint32_t>(kLongBlock)) tile <<= 1;
-    if (v4)
-      hipLaunchKernelGGL(gather_edge_to_row_long_kernel<float4>, dim3(kLongGrid), dim3(kLongBlock), 0, stream,
-                         reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, lr.list,
-                         lr.count, Fv, tile, accumulate);
-    else
-      hipLaunchKernelGGL(gather_edge_to_row_long_kernel<float>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, msg,
-                         off, perm, lr.list, lr.count, Fv, tile, accumulate);
-    NTS_LAUNCH_CHECK(who);
-    // Giant rows: pieces by separate blocks into stream-ordered scratch, then the ordered combine.
-    ScratchBlock partial_block;
     NTS_HIP_TRY(partial_block.alloc(static_cast<size_t>(kPieceCap) * F * sizeof(float), stream));
-    float *partial = static_cast<float *>(partial_block.ptr);
-    if (v4)
-      hipLaunchKernelGGL(giant_sum_pieces_kernel<float4>, dim3(kLongGrid), dim3(kLongBlock), 0, stream,
-                         reinterpret_cast<float4 *>(partial), reinterpret_cast<const float4 *>(msg), perm, lr.hdr,
-                         lr.pieces, Fv, tile);
-    else
-      hipLaunchKernelGGL(giant_sum_pieces_kernel<float>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, partial, msg,
-                         perm, lr.hdr, lr.pieces, Fv, tile);
+    partial = static_cast<float *>(partial_block.ptr);
+  }
+  if (v4) {
+    LongRowWork<float4> lw{lr.list, lr.count, lr.hdr, lr.pieces, reinterpret_cast<float4 *>(partial), tile,
+                           merged ? merged_long_blocks() : 0u};
+    launch_gather_rows(reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, rows, Fv,
+                       accumulate, limit, lw, stream);
+  } else {
+    LongRowWork<float> lw{lr.list, lr.count, lr.hdr, lr.pieces, partial, tile, merged ? merged_long_blocks() : 0u};
+    launch_gather_rows(out, msg, off, perm, rows, Fv, accumulate, limit, lw, stream);
+  }
+  hipError_t launch_err = hipGetLastError();
+  if (lr.list && launch_err == hipSuccess) {
+    if (!merged) {
+      if (v4) {
+        hipLaunchKernelGGL(gather_edge_to_row_long_kernel<float4>, dim3(kLongGrid), dim3(kLongBlock), 0, stream,
+                           reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(msg), off, perm, lr.list,
+                           lr.count, Fv, tile, accumulate);
+        hipLaunchKernelGGL(giant_sum_pieces_kernel<float4>, dim3(kLongGrid), dim3(kLongBlock), 0, stream,
+                           reinterpret_cast<float4 *>(partial), reinterpret_cast<const float4 *>(msg), perm, lr.hdr,
+                           lr.pieces, Fv, tile);
+      } else {
+        hipLaunchKernelGGL(gather_edge_to_row_long_kernel<float>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, msg,
+                           off, perm, lr.list, lr.count, Fv, tile, accumulate);
+        hipLaunchKernelGGL(giant_sum_pieces_kernel<float>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, partial, msg,
+                           perm, lr.hdr, lr.pieces, Fv, tile);
+      }
+    }
     hipLaunchKernelGGL(giant_sum_combine_kernel, dim3(kGiantCap / 4), dim3(256), 0, stream, out, partial, lr.hdr,
                        lr.giant_rows, lr.first, F, accumulate);
-    const hipError_t launch_err = hipGetLastError();
-    NTS_HIP_TRY(partial_block.release());
-    if (launch_err != hipSuccess) return fail_hip(launch_err, who);
+    launch_err = hipGetLastError();
+  }
+  if (lr.list) NTS_HIP_TRY(partial_block.release());
+  if (launch_err != hipSuccess) {
+    (void)release_long_rows(lr);
+    return fail_hip(launch_err, who);
   }
   return release_long_rows(lr);
 }
