@@ -107,7 +107,9 @@ __global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, con
 // ---- edge -> vertex sums ----------------------------------------------------------------------
 //
 // Rows with at most `long_limit` edges: a group of G lanes per row (64/G rows per wavefront) adds
-// the row's edge rows in order.  Longer rows (power-law hubs) are listed first and summed by whole
+// the row's edge rows in order; where the edge rows of consecutive vertices follow each other in
+// memory (no permutation) and are at most 16 lanes wide, a wavefront streams the edges of 64 rows
+// through LDS instead (same sums).  Longer rows (power-law hubs) are listed first and summed by whole
 // blocks -- the first blocks of the same launch where the row launch is the balanced kernel, the
 // block kernels below otherwise -- which spread a row's edges over the slices of the block and add
 // the slices' partial sums in a fixed order.
@@ -256,6 +258,134 @@ __device__ __forceinline__ void block_sum_edge_rows(V *__restrict__ dst, const V
   }
 }
 
+// The first blocks of a row launch take the listed long rows, one 256-thread block per row, and the
+// pieces of the giant ones (their partial sums are combined by a launch of its own afterwards); the
+// rows of the launch proper fill the chip meanwhile.
+template <typename V>
+__device__ __forceinline__ void sum_long_rows_in_this_block(V *__restrict__ out, const V *__restrict__ msg,
+                                                            const uint32_t *__restrict__ off,
+                                                            const uint32_t *__restrict__ perm, uint32_t Fv,
+                                                            int accumulate, const LongRowWork<V> &lw) {
+  __shared__ V long_part[256];
+  const uint32_t n_rows = *lw.count;
+  for (uint32_t i = blockIdx.x; i < n_rows; i += lw.blocks) {
+    const uint32_t r = lw.list[i];
+    block_sum_edge_rows<V, 256>(out + static_cast<size_t>(r) * Fv, msg, perm, off[r], off[r + 1], Fv, lw.tile,
+                                accumulate, long_part);
+  }
+  const uint32_t n_pieces = lw.hdr[1];
+  for (uint32_t p = blockIdx.x; p < n_pieces; p += lw.blocks) {
+    const uint4 pc = lw.pieces[p];
+    block_sum_edge_rows<V, 256>(lw.partial + static_cast<size_t>(p) * Fv, msg, perm, pc.z, pc.w, Fv, lw.tile, 0,
+                                long_part);
+  }
+}
+
+// Edge rows that lie one after the other in memory (no permutation: the sums over a destination's
+// edges) and are at most 16 lanes wide: a wavefront takes 64 consecutive rows, whose edges are one
+// contiguous range, and streams that range through a tile of LDS private to it -- all 64 lanes load
+// consecutive 4- or 16-byte vectors, the next round is requested before this one is added up -- while
+// the lanes that each own one float of an output row walk the tile edge by edge and write a row out
+// where it ends: the running fp32 sum in edge order, as in the kernel below, without a loop per lane
+// group and its hand-out of rows.  Rows above `long_limit` edges are skipped (the first blocks of the
+// launch sum them); empty rows are written as zeros (or left, when accumulating).
+template <typename V, int G>
+__global__ __launch_bounds__(256) void gather_edge_to_row_stream_kernel(V *__restrict__ out, const V *__restrict__ msg,
+                                                                        const uint32_t *__restrict__ off,
+                                                                        uint32_t rows, uint32_t Fv, int accumulate,
+                                                                        uint32_t long_limit, LongRowWork<V> lw) {
+  if (blockIdx.x < lw.blocks) {
+    sum_long_rows_in_this_block(out, msg, off, static_cast<const uint32_t *>(nullptr), Fv, accumulate, lw);
+    return;
+  }
+  constexpr int NF = sizeof(V) / 4;
+  constexpr int U = 8;                            // loads per lane and round
+  constexpr uint32_t kSlots = kWave / G;          // edge rows per load of the wavefront
+  constexpr uint32_t kRound = kSlots * U;         // edge rows per round
+  constexpr uint32_t kPitch = G * NF;             // floats of an edge row in the tile
+  __shared__ float tiles[4][kWave * U * NF];
+  float *tile = tiles[threadIdx.x / kWave];
+  const uint32_t lane = lane_id();
+  const uint32_t col = lane & (G - 1), slot = lane / G;
+  const bool col_live = col < Fv;
+  const uint32_t comps = Fv * NF;  // floats of an output row: lane c < comps owns float c
+  const bool owner = lane < comps;
+  const uint64_t wave = (static_cast<uint64_t>(blockIdx.x - lw.blocks) * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t n_waves = static_cast<uint64_t>(gridDim.x - lw.blocks) * blockDim.x / kWave;
+  for (uint64_t base = wave * kWave; base < rows; base += n_waves * kWave) {
+    const uint32_t n_set = rows - base < kWave ? static_cast<uint32_t>(rows - base) : kWave;
+    uint32_t my_e1 = 0;
+    if (lane < n_set) my_e1 = off[base + lane + 1];
+    uint32_t pos = off[base];                       // next edge to add (wave-uniform)
+    const uint32_t range_end = wave_read(my_e1, n_set - 1);
+    uint32_t j = 0;                                 // current row of the set
+    float acc = 0.f;
+    V cur[U];
+    auto load_round = [&](uint32_t k) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        cur[u] = V{};
+        const uint32_t idx = k + u * kSlots + slot;
+        if (idx < range_end && col_live) cur[u] = msg[static_cast<size_t>(idx) * Fv + col];
+      }
+    };
+    // Rows that end at `pos` are complete: written out (a skipped long row is not), next row.
+    auto finish_rows = [&](bool skip_first) {
+      bool skip = skip_first;
+      while (j < n_set && wave_read(my_e1, j) == pos) {
+        if (owner && !skip) {
+          float *p = reinterpret_cast<float *>(out) + (base + j) * comps + lane;
+          float v = acc;
+          if (accumulate) v += *p;
+          *p = v;
+        }
+        skip = false;
+        acc = 0.f;
+        ++j;
+      }
+    };
+    finish_rows(false);  // empty rows at the head of the set
+    uint32_t loaded = 0xFFFFFFFFu;  // first edge of the round held in `cur`
+    while (j < n_set) {
+      const uint32_t row_end = wave_read(my_e1, j);
+      if (row_end - pos > long_limit) {  // pos is this row's first edge: nothing of it has been added
+        pos = row_end;
+        finish_rows(true);
+        continue;
+      }
+      const uint32_t ts = pos;  // this round covers [ts, ts + kRound)
+      if (loaded != ts) load_round(ts);
+      __builtin_amdgcn_wave_barrier();  // the previous round's reads of the tile are done
+#pragma unroll
+      for (int u = 0; u < U; ++u) reinterpret_cast<V *>(tile)[u * kWave + lane] = cur[u];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      loaded = ts + kRound;
+      if (loaded < range_end) load_round(loaded);  // in flight while this round is added up
+      const uint32_t tile_end = range_end - ts < kRound ? range_end : ts + kRound;
+      while (pos < tile_end && j < n_set) {
+        const uint32_t e1 = wave_read(my_e1, j);
+        if (e1 - pos > long_limit) break;  // a long row starts here (a shorter one never has that much left)
+        const uint32_t end = e1 < tile_end ? e1 : tile_end;
+        if (owner) {
+          const float *t = tile + (pos - ts) * kPitch + lane;
+          uint32_t i = pos;
+          for (; i + 4 <= end; i += 4, t += 4 * kPitch) {
+            acc += t[0];
+            acc += t[kPitch];
+            acc += t[2 * kPitch];
+            acc += t[3 * kPitch];
+          }
+          for (; i < end; ++i, t += kPitch) acc += t[0];
+        }
+        pos = end;
+        if (pos == e1) finish_rows(false);
+      }
+    }
+  }
+}
+
 // The same sums for rows that fit one group (Fv <= G), with the rows of a wavefront handed out
 // dynamically: a wavefront takes 64 consecutive rows, reads their offsets with one coalesced load,
 // and its 64/G groups then pull rows from that set one after the other -- a group that finishes a
@@ -285,22 +415,7 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_balanced_kernel(V *__r
                                                                           uint32_t long_limit, uint32_t coop_limit,
                                                                           LongRowWork<V> lw) {
   if (blockIdx.x < lw.blocks) {
-    // The first blocks of the launch take the listed long rows, one block per row, and the pieces of
-    // the giant ones (their partial sums are combined by a launch of its own afterwards); the rows
-    // below fill the chip meanwhile.
-    __shared__ V long_part[256];
-    const uint32_t n_rows = *lw.count;
-    for (uint32_t i = blockIdx.x; i < n_rows; i += lw.blocks) {
-      const uint32_t r = lw.list[i];
-      block_sum_edge_rows<V, 256>(out + static_cast<size_t>(r) * Fv, msg, perm, off[r], off[r + 1], Fv, lw.tile,
-                                  accumulate, long_part);
-    }
-    const uint32_t n_pieces = lw.hdr[1];
-    for (uint32_t p = blockIdx.x; p < n_pieces; p += lw.blocks) {
-      const uint4 pc = lw.pieces[p];
-      block_sum_edge_rows<V, 256>(lw.partial + static_cast<size_t>(p) * Fv, msg, perm, pc.z, pc.w, Fv, lw.tile, 0,
-                                  long_part);
-    }
+    sum_long_rows_in_this_block(out, msg, off, perm, Fv, accumulate, lw);
     return;
   }
   constexpr bool kCoop = G <= 8;
@@ -1788,9 +1903,35 @@ uint32_t merged_long_blocks() {
 // The row launch whose first blocks also sum the long rows: one-group rows of a vertex set large enough.
 bool rows_launch_takes_long_rows(uint32_t rows, uint32_t Fv) { return Fv <= 64 && rows >= 4096; }
 
+// NTS_EDGE_SUM_STREAM=0 in the environment: contiguous edge rows take the lane-group kernel like permuted ones.
+bool stream_contiguous_rows() {
+  static const bool value = [] {
+    const char *env = getenv("NTS_EDGE_SUM_STREAM");
+    return !(env && atol(env) == 0);
+  }();
+  return value;
+}
+
 template <typename V>
 void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_t *perm, uint32_t rows, uint32_t Fv,
                         int accumulate, uint32_t limit, const LongRowWork<V> &lw, hipStream_t stream) {
+  if (rows_launch_takes_long_rows(rows, Fv) && !perm && lanes_for(Fv) <= 16 && stream_contiguous_rows()) {
+    // a wavefront streams the contiguous edges of 64 rows at a time
+    const uint32_t blocks = ceil_div(rows, 4 * kWave);
+    const dim3 grid((blocks < 16384u ? blocks : 16384u) + lw.blocks);
+#define NTS_STREAM(GG)                                                                                          \
+  hipLaunchKernelGGL((gather_edge_to_row_stream_kernel<V, GG>), grid, dim3(256), 0, stream, out, msg, off, rows, Fv, \
+                     accumulate, limit, lw)
+    switch (lanes_for(Fv)) {
+      case 1: NTS_STREAM(1); break;
+      case 2: NTS_STREAM(2); break;
+      case 4: NTS_STREAM(4); break;
+      case 8: NTS_STREAM(8); break;
+      default: NTS_STREAM(16); break;
+    }
+#undef NTS_STREAM
+    return;
+  }
   if (rows_launch_takes_long_rows(rows, Fv)) {
     // One group covers a row: wavefronts hand their 64 rows out dynamically (strided launch).
 #define NTS_BALANCED(GG, SS)                                                                                    \

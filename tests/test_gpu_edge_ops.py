@@ -538,3 +538,6 @@ def test_long_rows_of_narrow_messages_are_the_edge_order_sum(device, F):
             a = a + msg[k]
         ident[r] = a
     assert np.array_equal(out.cpu().numpy()[chains], ident[chains])
+    acc = dev(init, device)
+    call("nts_gather_edge_to_dst", ptr(acc), ptr(dmsg), ptr(dro), Vs, F, 1, s)
+    assert np.array_equal(acc.cpu().numpy()[chains], (ident + init)[chains])  # empty rows keep their contents
