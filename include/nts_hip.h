@@ -531,7 +531,8 @@ int nts_sample_hop_neighbors(uint32_t *ri_global, const uint32_t *co, const uint
  *   nts_batch_builder_join  makes `stream` wait (on the device; the call returns at once) until every
  *                array of the builder's current batch is complete.  Needed with enable == 3 only;
  *                otherwise the arrays are complete when nts_batch_builder_layers returns and the call
- *                does nothing.
+ *                does nothing.  `stream` must not be recording a graph (the event it waits for is
+ *                recorded outside any recording).
  * Calls on one builder must not overlap: consecutive nts_batch_builder_sample calls go to the same
  * stream, or the earlier batch is waited for first (nts_batch_builder_layers does). */
 typedef struct nts_batch_builder nts_batch_builder_t;
