@@ -281,6 +281,25 @@ __device__ __forceinline__ void sum_long_rows_in_this_block(V *__restrict__ out,
   }
 }
 
+// Smallest row r in [0, rows] whose weight before it, (off[r] - off0) + r, is at least x (x at most the
+// weight before `rows`, the total), searched by the whole wavefront like owner_of_wave.
+__device__ __forceinline__ uint32_t first_row_of_weight(const uint32_t *__restrict__ off, uint32_t rows, uint32_t off0,
+                                                        uint64_t x) {
+  if (x == 0) return 0;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint64_t pos = x - 1;
+  uint32_t lo = 0, hi = rows + 1;  // the largest row whose weight is at most pos lies in [lo, hi)
+  while (hi - lo > 1) {
+    const uint32_t step = (hi - lo + kWave - 1) / kWave;
+    const uint64_t idx = static_cast<uint64_t>(lo) + static_cast<uint64_t>(lane + 1) * step;
+    const bool behind = idx < hi && static_cast<uint64_t>(off[idx] - off0) + idx <= pos;
+    const uint32_t k = __popcll(__ballot(behind));
+    lo += k * step;
+    hi = lo + step < hi ? lo + step : hi;
+  }
+  return lo + 1 < rows ? lo + 1 : rows;  // at most `rows` for ascending offsets; never beyond them for any input
+}
+
 // Edge rows that lie one after the other in memory (no permutation: the sums over a destination's
 // edges) and are at most 16 lanes wide: a wavefront takes 64 consecutive rows, whose edges are one
 // contiguous range, and streams that range through a tile of LDS private to it -- all 64 lanes load
@@ -312,8 +331,18 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_stream_kernel(V *__res
   const bool owner = lane < comps;
   const uint64_t wave = (static_cast<uint64_t>(blockIdx.x - lw.blocks) * blockDim.x + threadIdx.x) / kWave;
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x - lw.blocks) * blockDim.x / kWave;
-  for (uint64_t base = wave * kWave; base < rows; base += n_waves * kWave) {
-    const uint32_t n_set = rows - base < kWave ? static_cast<uint32_t>(rows - base) : kWave;
+  // The wavefronts share the rows by weight, a row counting one plus its edges: wavefront w takes the
+  // rows r with w C <= (off[r] - off[0]) + r < (w + 1) C.
+  const uint32_t off0 = off[0];
+  const uint64_t total = static_cast<uint64_t>(off[rows] - off0) + rows;
+  const uint64_t share = (total + n_waves - 1) / n_waves;
+  const uint64_t x0 = wave * share < total ? wave * share : total;
+  const uint64_t x1 = x0 + share < total ? x0 + share : total;
+  if (x0 == x1) return;
+  const uint32_t r_begin = first_row_of_weight(off, rows, off0, x0);
+  const uint32_t r_end = first_row_of_weight(off, rows, off0, x1);
+  for (uint64_t base = r_begin; base < r_end; base += kWave) {
+    const uint32_t n_set = r_end - base < kWave ? static_cast<uint32_t>(r_end - base) : kWave;
     uint32_t my_e1 = 0;
     if (lane < n_set) my_e1 = off[base + lane + 1];
     uint32_t pos = off[base];                       // next edge to add (wave-uniform)
