@@ -108,8 +108,8 @@ __global__ __launch_bounds__(256) void edge_copy_kernel(V *__restrict__ msg, con
 //
 // Rows with at most `long_limit` edges: a group of G lanes per row (64/G rows per wavefront) adds
 // the row's edge rows in order; where the edge rows of consecutive vertices follow each other in
-// memory (no permutation) and are at most 16 lanes wide, a wavefront streams the edges of 64 rows
-// through LDS instead (same sums).  Longer rows (power-law hubs) are listed first and summed by whole
+// memory (no permutation), a wavefront streams the edges of a run of rows through LDS instead (same
+// sums).  Longer rows (power-law hubs) are listed first and summed by whole
 // blocks -- the first blocks of the same launch where the row launch is the balanced kernel, the
 // block kernels below otherwise -- which spread a row's edges over the slices of the block and add
 // the slices' partial sums in a fixed order.
@@ -301,10 +301,11 @@ __device__ __forceinline__ uint32_t first_row_of_weight(const uint32_t *__restri
 }
 
 // Edge rows that lie one after the other in memory (no permutation: the sums over a destination's
-// edges) and are at most 16 lanes wide: a wavefront takes 64 consecutive rows, whose edges are one
+// edges) and are at most one wavefront wide: a wavefront takes 64 consecutive rows, whose edges are one
 // contiguous range, and streams that range through a tile of LDS private to it -- all 64 lanes load
 // consecutive 4- or 16-byte vectors, the next round is requested before this one is added up -- while
-// the lanes that each own one float of an output row walk the tile edge by edge and write a row out
+// the lanes that each own one float of an output row (up to four from 32 lanes of 16 bytes on) walk the
+// tile edge by edge and write a row out
 // where it ends: the running fp32 sum in edge order, as in the kernel below, without a loop per lane
 // group and its hand-out of rows.  Rows above `long_limit` edges are skipped (the first blocks of the
 // launch sum them); empty rows are written as zeros (or left, when accumulating).
@@ -327,8 +328,8 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_stream_kernel(V *__res
   const uint32_t lane = lane_id();
   const uint32_t col = lane & (G - 1), slot = lane / G;
   const bool col_live = col < Fv;
-  const uint32_t comps = Fv * NF;  // floats of an output row: lane c < comps owns float c
-  const bool owner = lane < comps;
+  const uint32_t comps = Fv * NF;  // floats of an output row: lane c owns the floats c + 64 k below comps
+  constexpr int OWN = (G * NF + kWave - 1) / kWave;  // floats a lane owns at most (1 up to 16 lanes of 16 bytes)
   const uint64_t wave = (static_cast<uint64_t>(blockIdx.x - lw.blocks) * blockDim.x + threadIdx.x) / kWave;
   const uint64_t n_waves = static_cast<uint64_t>(gridDim.x - lw.blocks) * blockDim.x / kWave;
   // The wavefronts share the rows by weight, a row counting one plus its edges: wavefront w takes the
@@ -348,7 +349,9 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_stream_kernel(V *__res
     uint32_t pos = off[base];                       // next edge to add (wave-uniform)
     const uint32_t range_end = wave_read(my_e1, n_set - 1);
     uint32_t j = 0;                                 // current row of the set
-    float acc = 0.f;
+    float acc[OWN];
+#pragma unroll
+    for (int o = 0; o < OWN; ++o) acc[o] = 0.f;
     V cur[U];
     auto load_round = [&](uint32_t k) {
 #pragma unroll
@@ -362,14 +365,21 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_stream_kernel(V *__res
     auto finish_rows = [&](bool skip_first) {
       bool skip = skip_first;
       while (j < n_set && wave_read(my_e1, j) == pos) {
-        if (owner && !skip) {
-          float *p = reinterpret_cast<float *>(out) + (base + j) * comps + lane;
-          float v = acc;
-          if (accumulate) v += *p;
-          *p = v;
+        if (!skip) {
+#pragma unroll
+          for (int o = 0; o < OWN; ++o) {
+            const uint32_t c = lane + o * kWave;
+            if (c < comps) {
+              float *p = reinterpret_cast<float *>(out) + (base + j) * comps + c;
+              float v = acc[o];
+              if (accumulate) v += *p;
+              *p = v;
+            }
+          }
         }
         skip = false;
-        acc = 0.f;
+#pragma unroll
+        for (int o = 0; o < OWN; ++o) acc[o] = 0.f;
         ++j;
       }
     };
@@ -397,16 +407,21 @@ __global__ __launch_bounds__(256) void gather_edge_to_row_stream_kernel(V *__res
         const uint32_t e1 = wave_read(my_e1, j);
         if (e1 - pos > long_limit) break;  // a long row starts here (a shorter one never has that much left)
         const uint32_t end = e1 < tile_end ? e1 : tile_end;
-        if (owner) {
-          const float *t = tile + (pos - ts) * kPitch + lane;
-          uint32_t i = pos;
-          for (; i + 4 <= end; i += 4, t += 4 * kPitch) {
-            acc += t[0];
-            acc += t[kPitch];
-            acc += t[2 * kPitch];
-            acc += t[3 * kPitch];
+#pragma unroll
+        for (int o = 0; o < OWN; ++o) {
+          if (lane + o * kWave < comps) {
+            const float *t = tile + (pos - ts) * kPitch + lane + o * kWave;
+            float a = acc[o];
+            uint32_t i = pos;
+            for (; i + 4 <= end; i += 4, t += 4 * kPitch) {
+              a += t[0];
+              a += t[kPitch];
+              a += t[2 * kPitch];
+              a += t[3 * kPitch];
+            }
+            for (; i < end; ++i, t += kPitch) a += t[0];
+            acc[o] = a;
           }
-          for (; i < end; ++i, t += kPitch) acc += t[0];
         }
         pos = end;
         if (pos == e1) finish_rows(false);
@@ -1944,7 +1959,7 @@ bool stream_contiguous_rows() {
 template <typename V>
 void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_t *perm, uint32_t rows, uint32_t Fv,
                         int accumulate, uint32_t limit, const LongRowWork<V> &lw, hipStream_t stream) {
-  if (rows_launch_takes_long_rows(rows, Fv) && !perm && lanes_for(Fv) <= 16 && stream_contiguous_rows()) {
+  if (rows_launch_takes_long_rows(rows, Fv) && !perm && stream_contiguous_rows()) {
     // a wavefront streams the contiguous edges of 64 rows at a time
     const uint32_t blocks = ceil_div(rows, 4 * kWave);
     const dim3 grid((blocks < 16384u ? blocks : 16384u) + lw.blocks);
@@ -1956,7 +1971,9 @@ void launch_gather_rows(V *out, const V *msg, const uint32_t *off, const uint32_
       case 2: NTS_STREAM(2); break;
       case 4: NTS_STREAM(4); break;
       case 8: NTS_STREAM(8); break;
-      default: NTS_STREAM(16); break;
+      case 16: NTS_STREAM(16); break;
+      case 32: NTS_STREAM(32); break;
+      default: NTS_STREAM(64); break;
     }
 #undef NTS_STREAM
     return;

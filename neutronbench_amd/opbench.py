@@ -110,6 +110,13 @@ def main():
     report("nts_gather_edge_to_dst", lambda: call("nts_gather_edge_to_dst", ptr(o_dst), ptr(msg), ptr(co32), Vd, Fm, 0, s),
            E2 * 4 * Fm + Vd * 4 * Fm, part)
     del msg, feat, o_dst
+    Fw = 128  # edge rows as wide as a hidden layer: what the unfused GAT aggregation sums
+    msg = torch.randn(E2, Fw, device=dev)
+    o_dst = torch.empty(Vd, Fw, device=dev)
+    report("nts_gather_edge_to_dst (wide rows)", lambda: call("nts_gather_edge_to_dst", ptr(o_dst), ptr(msg), ptr(co32), Vd,
+                                                              Fw, 0, s),
+           E2 * 4 * Fw + Vd * 4 * Fw, f"edges of the first {Vd} destinations, E={E2}, F'={Fw}")
+    del msg, o_dst
 
     n = int(1_000_000 * args.scale)
     Ff = 100
