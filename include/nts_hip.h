@@ -5,10 +5,12 @@
  * Every entry point is `extern "C"`, takes plain pointers and sizes, receives the HIP stream
  * explicitly, returns an int status (0 = NTS_OK) and never prints or exits.  State that outlives a
  * call is either in a handle the caller owns (a schedule, a batch builder: calls on one handle are
- * serialised by the library, see each) or one of three process-wide items that are safe to share: a
- * per-device pool that keeps freed scratch (thread-safe, stream-ordered), the per-thread last-error
- * text, and the fixed scratch array of nts_spmm_gather_static_scratch (whose calls a caller must
- * serialise).  Calls on different streams and host threads are otherwise independent, which is what
+ * serialised by the library, see each) or one of four items that are safe to share: a per-device
+ * pool that keeps freed scratch (thread-safe, stream-ordered), the per-thread last-error text, a
+ * stream per host thread and device on which the softmax / attention entry points run the block
+ * kernels of their hub rows beside their other launches (forked from and joined to the caller's
+ * stream inside the call; never while that stream records a graph), and the fixed scratch array of
+ * nts_spmm_gather_static_scratch (whose calls a caller must serialise).  Calls on different streams and host threads are otherwise independent, which is what
  * the reference's pipelined mini-batch loop needs (one Cuda_Stream per host thread,
  * toolkits/GCN_GPU_NEIGHBOR.hpp:1350-1363).
  *

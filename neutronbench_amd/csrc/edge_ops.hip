@@ -2077,6 +2077,81 @@ int gather_edge_impl(float *out, const float *msg, const uint32_t *off, const ui
   return release_long_rows(lr);
 }
 
+// A second stream per host thread and device, for launches that a call runs beside those on the
+// caller's stream (the block kernels of the few hub rows, which leave most of the chip idle, beside the
+// kernels of all other rows).  Created at first use and kept until the process ends; a thread that
+// ends leaves its stream and events behind (destroying them from a thread-exit hook could run after the
+// runtime has shut down).  NTS_SOFTMAX_SIDE_STREAM=0 in the environment: everything on the caller's stream.
+struct SideLane {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+};
+SideLane *side_lane() {
+  static const bool enabled = [] {
+    const char *env = getenv("NTS_SOFTMAX_SIDE_STREAM");
+    return !(env && atol(env) == 0);
+  }();
+  if (!enabled) return nullptr;
+  constexpr int kDevices = 16;
+  thread_local SideLane lanes[kDevices];
+  thread_local bool tried[kDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kDevices) return nullptr;
+  SideLane &l = lanes[dev];
+  if (!tried[dev]) {
+    tried[dev] = true;
+    hipStream_t st = nullptr;
+    hipEvent_t a = nullptr, b = nullptr;
+    if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) == hipSuccess &&
+        hipEventCreateWithFlags(&a, hipEventDisableTiming) == hipSuccess &&
+        hipEventCreateWithFlags(&b, hipEventDisableTiming) == hipSuccess) {
+      l.stream = st;
+      l.fork = a;
+      l.join = b;
+    } else {
+      if (a) (void)hipEventDestroy(a);
+      if (st) (void)hipStreamDestroy(st);
+      (void)hipGetLastError();
+    }
+  }
+  return l.stream ? &l : nullptr;
+}
+
+// The side lane between a fork (it waits for everything enqueued on `main` so far) and the join (`main`
+// waits for it), which also happens on every way out of the scope.
+class SideWork {
+ public:
+  SideWork(hipStream_t main, bool wanted) : main_(main), lane_(wanted ? side_lane() : nullptr) {
+    // a stream that is recording a graph keeps all of the call's launches: the side stream is shared by
+    // the thread's calls and must not become part of a recording
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (lane_ && (hipStreamIsCapturing(main_, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone)) {
+      (void)hipGetLastError();
+      lane_ = nullptr;
+    }
+    if (lane_ && (hipEventRecord(lane_->fork, main_) != hipSuccess ||
+                  hipStreamWaitEvent(lane_->stream, lane_->fork, 0) != hipSuccess)) {
+      (void)hipGetLastError();
+      lane_ = nullptr;  // nothing has been enqueued on the side stream: the caller's stream takes the work
+    }
+  }
+  SideWork(const SideWork &) = delete;
+  SideWork &operator=(const SideWork &) = delete;
+  hipStream_t stream() const { return lane_ ? lane_->stream : main_; }
+  hipError_t join() {
+    if (!lane_) return hipSuccess;
+    SideLane *l = lane_;
+    lane_ = nullptr;
+    const hipError_t e = hipEventRecord(l->join, l->stream);
+    return e != hipSuccess ? e : hipStreamWaitEvent(main_, l->join, 0);
+  }
+  ~SideWork() { (void)join(); }
+
+ private:
+  hipStream_t main_;
+  SideLane *lane_;
+};
+
 // Edge softmax / fused attention, forward (gy == nullptr) or backward; x / el / er / ri / ger are
 // null where the variant does not use them.
 int softmax_impl(bool backward, bool fused, float *out, float *ger, const float *x_or_gy, const float *y,
@@ -2091,6 +2166,14 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   if (pow2 && !no_hubs)
     if (int rc = collect_long_rows(lr, co, Vd, H, kLongRowValues, kGiantValues, stream)) return rc;
   const uint32_t max_values = lr.list ? kLongRowValues : kNoLimit;
+  // The block kernels of the hub rows and the kernels of the giant ones' pieces run on the side lane,
+  // beside the launches for all other rows below (they write other rows); their scratch is taken
+  // before the fork, so that whatever the pool ordered for it on `stream` lies before it too.
+  const size_t stats_floats = static_cast<size_t>(kPieceCap) * 2 * H, row_floats = static_cast<size_t>(kGiantCap) * 2 * H;
+  ScratchBlock stats_block;
+  if (lr.list) NTS_HIP_TRY(stats_block.alloc((stats_floats + row_floats) * sizeof(float), stream));
+  SideWork side(stream, lr.list != nullptr);
+  const hipStream_t hub_stream = side.stream();
   // 16-byte lanes for the segments that do not fit the register paths: whole heads per lane and
   // every array 16-byte aligned (a segment starts at e0 * H floats).
   const uint32_t vec4 = pow2 && H % 4 == 0 && aligned_to(out, 16) && aligned_to(x_or_gy, 16) && aligned_to(y, 16) &&
@@ -2103,6 +2186,60 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
   const dim3 short_grid(short_blocks < 16384u ? short_blocks : 16384u);
   const uint32_t wave_blocks = ceil_div(Vd, 4);  // at most one destination per wavefront
   const dim3 grid(wave_blocks < 8192u ? wave_blocks : 8192u);
+  if (lr.list) {
+    // The hub rows first: their few large blocks take their places on the chip before the launches for
+    // all other rows fill it.
+    if (!backward) {
+      if (fused)
+        hipLaunchKernelGGL(edge_softmax_fwd_long_kernel<true>, dim3(kLongGrid), dim3(kLongBlock), 0, hub_stream, out,
+                           x_or_gy, el, er, co, ri, lr.list, lr.count, H, slope);
+      else
+        hipLaunchKernelGGL(edge_softmax_fwd_long_kernel<false>, dim3(kLongGrid), dim3(kLongBlock), 0, hub_stream, out,
+                           x_or_gy, el, er, co, ri, lr.list, lr.count, H, slope);
+    } else {
+      if (fused)
+        hipLaunchKernelGGL(edge_softmax_bwd_long_kernel<true>, dim3(kLongGrid), dim3(kLongBlock), 0, hub_stream, out, ger,
+                           x_or_gy, y, el, er, co, ri, lr.list, lr.count, H, slope);
+      else
+        hipLaunchKernelGGL(edge_softmax_bwd_long_kernel<false>, dim3(kLongGrid), dim3(kLongBlock), 0, hub_stream, out, ger,
+                           x_or_gy, y, el, er, co, ri, lr.list, lr.count, H, slope);
+    }
+    NTS_LAUNCH_CHECK(who);
+    // Giant segments: per-piece statistics, ordered combine, apply (see the kernels above).
+    float *stats = static_cast<float *>(stats_block.ptr);
+    float *rowstat = stats + stats_floats;
+    const dim3 pgrid(kLongGrid), pblock(kLongBlock), cgrid(kGiantCap / 4), cblock(64);
+    if (!backward) {
+      if (fused)
+        hipLaunchKernelGGL(giant_softmax_stats_kernel<true>, pgrid, pblock, 0, hub_stream, stats, out, x_or_gy, el, er, ri,
+                           lr.hdr, lr.pieces, H, slope);
+      else
+        hipLaunchKernelGGL(giant_softmax_stats_kernel<false>, pgrid, pblock, 0, hub_stream, stats, out, x_or_gy, el, er, ri,
+                           lr.hdr, lr.pieces, H, slope);
+      hipLaunchKernelGGL(giant_softmax_combine_kernel<0>, cgrid, cblock, 0, hub_stream, rowstat,
+                         static_cast<float *>(nullptr), stats, lr.hdr, lr.giant_rows, lr.first, H);
+      if (fused)
+        hipLaunchKernelGGL(giant_softmax_apply_kernel<true>, pgrid, pblock, 0, hub_stream, out, x_or_gy, rowstat, lr.hdr,
+                           lr.pieces, H);
+      else
+        hipLaunchKernelGGL(giant_softmax_apply_kernel<false>, pgrid, pblock, 0, hub_stream, out, x_or_gy, rowstat, lr.hdr,
+                           lr.pieces, H);
+    } else {
+      hipLaunchKernelGGL(giant_softmax_dot_kernel, pgrid, pblock, 0, hub_stream, stats, x_or_gy, y, lr.hdr, lr.pieces, H);
+      hipLaunchKernelGGL(giant_softmax_combine_kernel<1>, cgrid, cblock, 0, hub_stream, rowstat,
+                         static_cast<float *>(nullptr), stats, lr.hdr, lr.giant_rows, lr.first, H);
+      if (fused) {
+        hipLaunchKernelGGL(giant_softmax_bwd_apply_kernel<true>, pgrid, pblock, 0, hub_stream, out, stats, x_or_gy, y, el, er,
+                           ri, rowstat, lr.hdr, lr.pieces, H, slope);
+        hipLaunchKernelGGL(giant_softmax_combine_kernel<1>, cgrid, cblock, 0, hub_stream, rowstat, ger, stats, lr.hdr,
+                           lr.giant_rows, lr.first, H);
+      } else {
+        hipLaunchKernelGGL(giant_softmax_bwd_apply_kernel<false>, pgrid, pblock, 0, hub_stream, out, stats, x_or_gy, y, el, er,
+                           ri, rowstat, lr.hdr, lr.pieces, H, slope);
+      }
+    }
+    NTS_LAUNCH_CHECK(who);
+  }
   if (use_short && fused && max_degree != 0 && static_cast<uint64_t>(max_degree) * H <= kShortValues) {
     // Every segment fits the short class by the caller's word: one launch (which still computes a
     // longer segment, slowly, should there be one).
@@ -2146,15 +2283,6 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
     }
 #undef NTS_FWD
     NTS_LAUNCH_CHECK(who);
-    if (lr.list) {
-      if (fused)
-        hipLaunchKernelGGL(edge_softmax_fwd_long_kernel<true>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out,
-                           x_or_gy, el, er, co, ri, lr.list, lr.count, H, slope);
-      else
-        hipLaunchKernelGGL(edge_softmax_fwd_long_kernel<false>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out,
-                           x_or_gy, el, er, co, ri, lr.list, lr.count, H, slope);
-      NTS_LAUNCH_CHECK(who);
-    }
   } else {
 #define NTS_BWD(FU, P2, PART, LO, HI)                                                                            \
   hipLaunchKernelGGL((edge_softmax_bwd_kernel<FU, P2, PART>), grid, block, 0, stream, out, ger, x_or_gy, y, el, er, co, \
@@ -2172,56 +2300,11 @@ int softmax_impl(bool backward, bool fused, float *out, float *ger, const float 
     }
 #undef NTS_BWD
     NTS_LAUNCH_CHECK(who);
-    if (lr.list) {
-      if (fused)
-        hipLaunchKernelGGL(edge_softmax_bwd_long_kernel<true>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, ger,
-                           x_or_gy, y, el, er, co, ri, lr.list, lr.count, H, slope);
-      else
-        hipLaunchKernelGGL(edge_softmax_bwd_long_kernel<false>, dim3(kLongGrid), dim3(kLongBlock), 0, stream, out, ger,
-                           x_or_gy, y, el, er, co, ri, lr.list, lr.count, H, slope);
-      NTS_LAUNCH_CHECK(who);
-    }
   }
   if (lr.list) {
-    // Giant segments: per-piece statistics, ordered combine, apply (see the kernels above).
-    const size_t stats_floats = static_cast<size_t>(kPieceCap) * 2 * H, row_floats = static_cast<size_t>(kGiantCap) * 2 * H;
-    ScratchBlock stats_block;
-    NTS_HIP_TRY(stats_block.alloc((stats_floats + row_floats) * sizeof(float), stream));
-    float *stats = static_cast<float *>(stats_block.ptr);
-    float *rowstat = stats + stats_floats;
-    const dim3 pgrid(kLongGrid), pblock(kLongBlock), cgrid(kGiantCap / 4), cblock(64);
-    if (!backward) {
-      if (fused)
-        hipLaunchKernelGGL(giant_softmax_stats_kernel<true>, pgrid, pblock, 0, stream, stats, out, x_or_gy, el, er, ri,
-                           lr.hdr, lr.pieces, H, slope);
-      else
-        hipLaunchKernelGGL(giant_softmax_stats_kernel<false>, pgrid, pblock, 0, stream, stats, out, x_or_gy, el, er, ri,
-                           lr.hdr, lr.pieces, H, slope);
-      hipLaunchKernelGGL(giant_softmax_combine_kernel<0>, cgrid, cblock, 0, stream, rowstat,
-                         static_cast<float *>(nullptr), stats, lr.hdr, lr.giant_rows, lr.first, H);
-      if (fused)
-        hipLaunchKernelGGL(giant_softmax_apply_kernel<true>, pgrid, pblock, 0, stream, out, x_or_gy, rowstat, lr.hdr,
-                           lr.pieces, H);
-      else
-        hipLaunchKernelGGL(giant_softmax_apply_kernel<false>, pgrid, pblock, 0, stream, out, x_or_gy, rowstat, lr.hdr,
-                           lr.pieces, H);
-    } else {
-      hipLaunchKernelGGL(giant_softmax_dot_kernel, pgrid, pblock, 0, stream, stats, x_or_gy, y, lr.hdr, lr.pieces, H);
-      hipLaunchKernelGGL(giant_softmax_combine_kernel<1>, cgrid, cblock, 0, stream, rowstat,
-                         static_cast<float *>(nullptr), stats, lr.hdr, lr.giant_rows, lr.first, H);
-      if (fused) {
-        hipLaunchKernelGGL(giant_softmax_bwd_apply_kernel<true>, pgrid, pblock, 0, stream, out, stats, x_or_gy, y, el, er,
-                           ri, rowstat, lr.hdr, lr.pieces, H, slope);
-        hipLaunchKernelGGL(giant_softmax_combine_kernel<1>, cgrid, cblock, 0, stream, rowstat, ger, stats, lr.hdr,
-                           lr.giant_rows, lr.first, H);
-      } else {
-        hipLaunchKernelGGL(giant_softmax_bwd_apply_kernel<false>, pgrid, pblock, 0, stream, out, stats, x_or_gy, y, el, er,
-                           ri, rowstat, lr.hdr, lr.pieces, H, slope);
-      }
-    }
-    const hipError_t launch_err = hipGetLastError();
+    const hipError_t join_err = side.join();  // `stream` waits for the hub rows before their scratch goes back
     NTS_HIP_TRY(stats_block.release());
-    if (launch_err != hipSuccess) return fail_hip(launch_err, who);
+    if (join_err != hipSuccess) return fail_hip(join_err, who);
   }
   return release_long_rows(lr);
 }
