@@ -620,6 +620,10 @@ def run_epochs(torch, names, with_cpu, cpu_batches):
                 "ms_per_batch": round(1e3 * serial["epoch_s"] / max(serial["batches"], 1), 4),
                 "pipelined_epoch_s": piped["epoch_s"], "pipeline_depth": piped["pipeline"],
                 "driver": "lib/nts_epoch (C++ over the C ABI), one stream, a wait after every stage; 2 untimed batches first",
+                # how the whole-batch builder replays its launches (nts_batch_builder_use_graph): 2 = the hops'
+                # transpositions on a side branch of its graph, 3 = as a second graph beside the feature gather
+                # (sample time is then the sampling alone); the pipelined run: 1 = one chain
+                "hop_graph_mode": serial.get("hop_graph_mode"), "pipelined_hop_graph_mode": piped.get("hop_graph_mode"),
                 "check": check, "cpu_baseline": cpu,
             }
     finally:
@@ -648,7 +652,8 @@ def run_epoch_workload(args):
                                "a step = one batch: sampling, layer construction, feature/label gather, aggregation "
                                "fwd+bwd of every layer",
                    **{k: rec[k] for k in ("vertices", "edges", "stage_s", "sampled_edges", "gathered_rows",
-                                          "cache_hit_rate", "pipelined_epoch_s", "pipeline_depth", "driver")}},
+                                          "cache_hit_rate", "pipelined_epoch_s", "pipeline_depth", "driver",
+                                          "hop_graph_mode", "pipelined_hop_graph_mode")}},
         "roofline": None,
         "check": rec["check"],
         "cpu_baseline": rec["cpu_baseline"],
