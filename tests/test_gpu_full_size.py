@@ -396,3 +396,47 @@ def test_config5_full_graph_softmax_and_attention_segments(device, products_grap
     _check_segments("attention bwd (destinations)", ger[rows].cpu().numpy(), oracle.aggregate_dst(gs_ref, sub_off),
                     _seg_reduce(np.add, gs_exact, sub_off), np.repeat(short_rows[:, None], H, 1),
                     _seg_reduce(np.add, scale_gs.astype(np.float64), sub_off))
+
+
+@pytest.mark.parametrize("F", [4, 32])
+def test_config5_full_graph_edge_sums_to_destinations(device, products_graph, F):
+    """nts_gather_edge_to_dst over all 126.2 M edges (F = 4: a value per head; F = 32): wavefronts stream
+    the contiguous edges of their rows, the first blocks of the launch take the rows above 1,024 edges
+    and the pieces of the giant ones.  2,000 seeded destinations and the eight longest against the
+    float64 sum (1e-4 of the sum of magnitudes); rows of at most 1,024 edges equal the running fp32
+    sum in edge order bit for bit; untouched rows of an accumulating call keep their contents."""
+    g = products_graph
+    V, E = g["V"], g["E"]
+    gco = g["gco"]
+    s = stream()
+    off64 = u32_to_i64(gco)
+    deg = off64[1:] - off64[:-1]
+    hubs = torch.topk(deg, 8).indices
+    cand = synth.permutation(V, 19, device)
+    rows = torch.cat([cand[:2000], hubs])
+    sub_off, eid = sub_segments(off64, rows)
+    lens = np.diff(sub_off.astype(np.int64))
+    print(f"F={F}: {rows.numel()} rows, {eid.numel()} edges, longest {int(deg.max())}, empty {int((lens == 0).sum())}",
+          flush=True)
+    msg = synth.normal_features(E, F, seed=230 + F, device=device)
+    out = torch.full((V, F), float("nan"), device=device)
+    call("nts_gather_edge_to_dst", ptr(out), ptr(msg), ptr(gco), V, F, 0, s)
+    got = out[rows].cpu().numpy()
+    m = msg[eid].cpu().numpy()
+    exact = np.zeros((rows.numel(), F))
+    scale = np.zeros((rows.numel(), F))
+    chain = np.zeros((rows.numel(), F), np.float32)
+    for k in range(rows.numel()):
+        seg = m[sub_off[k]:sub_off[k + 1]]
+        exact[k] = seg.astype(np.float64).sum(0)
+        scale[k] = np.abs(seg).astype(np.float64).sum(0)
+        if 0 < lens[k] <= 1024:
+            chain[k] = np.cumsum(seg, axis=0, dtype=np.float32)[-1]
+    assert np.all(np.abs(got - exact) <= 1e-4 * np.maximum(scale, 1e-6)), "beyond 1e-4 of the sum of magnitudes"
+    ordered = lens <= 1024
+    assert np.array_equal(got[ordered].view(np.uint32), chain[ordered].view(np.uint32))
+    assert bool((out == out).all()), "a row was not written"
+    # accumulate: out += sums; a second pass doubles nothing but adds once more
+    call("nts_gather_edge_to_dst", ptr(out), ptr(msg), ptr(gco), V, F, 1, s)
+    twice = out[rows].cpu().numpy()
+    assert np.array_equal(twice[ordered], (chain + chain)[ordered])
