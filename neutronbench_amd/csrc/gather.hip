@@ -116,12 +116,27 @@ struct RowsArgs {
 };
 
 // Blocks of a gather whose table lies in host memory.  Such a launch is bound by the PCIe link
-// (about 57 GB/s here), which 128 blocks of four wavefronts, one row in flight per lane group, keep
-// full: measured alone, a 337 k-row gather takes the same time with 128 blocks as with 16,384, and
-// a 1 GB gather 22.2 ms instead of 24.9.  What the small grid buys is the rest of the chip: a
-// gather of the next batch on a stream of its own then runs beside the aggregation of this one
-// instead of parking wavefronts that wait for the link on every compute unit.
-constexpr uint32_t kHostTableBlocks = 128;
+// (about 57 GB/s here).  Where every row crosses the link, 32 blocks of four wavefronts, one row in
+// flight per lane group, keep it full: the same time as with 128 blocks or 16,384.  In the cached
+// gather the blocks that copy the missed rows also look up, one after the other, the rows that they
+// then skip, and need 128 blocks for the same (32: three times the time; a variant in which a
+// wavefront looks 64 rows up at once and 32 blocks suffice gathered 4-6 % faster and changed no
+// epoch: what runs beside it slowed down by as much).  What the small grid buys is the rest of the
+// chip and of the memory path: kernels that run beside a gather slow down several times over while
+// their requests queue behind outstanding reads of host memory, and the fewer of those a gather keeps
+// in flight beyond what the link needs, the less they do (a sampled batch's sort, CSR and weight
+// kernels beside a plain 128-block gather: 5 to 18 times their usual time; beside 32 blocks: unchanged).
+constexpr uint32_t kHostTableBlocks = 32;   // every row over the link
+constexpr uint32_t kHostMissBlocks = 128;   // the missed rows of a cached gather
+// NTS_GATHER_HOST_BLOCKS in the environment overrides both counts (for measurements).
+uint32_t host_table_blocks(bool cached) {
+  static const uint32_t forced = [] {
+    const char *env = getenv("NTS_GATHER_HOST_BLOCKS");
+    const long n = env ? atol(env) : 0;
+    return n > 0 ? static_cast<uint32_t>(n) : 0u;
+  }();
+  return forced ? forced : (cached ? kHostMissBlocks : kHostTableBlocks);
+}
 constexpr uint32_t kCachedBlocks = 16384;  // table in device memory: fill the chip several times over
 constexpr uint32_t kHitBlocks = 1024;      // table in host memory: blocks that copy the rows the HBM cache holds
 
@@ -149,13 +164,13 @@ void launch_rows(const RowsArgs &a, uint32_t Fv) {
   uint32_t blocks = ceil_div(a.n, per_block);
   const bool host_table = table_in_host_memory(a.table);
   // Both kernels stride over the rows, so any grid covers them.
-  const uint32_t cap = host_table ? kHostTableBlocks : (a.cache ? kCachedBlocks : blocks);
+  const uint32_t cap = host_table ? host_table_blocks(a.cache != nullptr) : (a.cache ? kCachedBlocks : blocks);
   const uint32_t wanted = blocks;
   if (blocks > cap) blocks = cap;
   if (a.cache) {
-    // table in host memory: kHostTableBlocks blocks for the rows that miss, and beside them blocks for
+    // table in host memory: kHostMissBlocks blocks for the rows that miss, and beside them blocks for
     // the rows the cache holds (enough to move them at HBM speed, still a fraction of the chip)
-    const uint32_t miss_blocks = (host_table && wanted > kHostTableBlocks) ? kHostTableBlocks : 0u;
+    const uint32_t miss_blocks = (host_table && wanted > host_table_blocks(true)) ? host_table_blocks(true) : 0u;
     const uint32_t hit_blocks = miss_blocks ? std::min<uint32_t>(wanted, kHitBlocks) : 0u;
     hipLaunchKernelGGL((gather_rows_cached_kernel<V, G>), dim3(blocks + hit_blocks), dim3(256), 0, a.stream,
                        reinterpret_cast<V *>(a.out), reinterpret_cast<const V *>(a.table),

@@ -63,15 +63,12 @@ class Timer:
 def graph_mode(graph, pipeline, cache=0.0):
     """The value for nts_batch_builder_use_graph.  True picks by measurement.  With several batches in
     flight: 1 (one recorded chain of launches; the chains of the other builders already fill the
-    chip, extra branches and streams only cost).  With one batch in flight the transpositions and
-    weights leave the chain: with an HBM feature cache they run as a second graph beside the gather
-    (3); a gather that reads every row over PCIe slows kernels running beside it several times over
-    (their memory requests queue behind the link's), so there they stay inside the batch's one graph,
-    on a side branch beside the next hop's sampling (2)."""
+    chip, extra branches and streams only cost).  With one batch in flight: 3, the transpositions and
+    weights as a second graph beside the feature gather (with and without a feature cache: the gather
+    keeps no more reads of host memory in flight than the link needs, so the kernels beside it run at
+    their usual speed)."""
     if graph is True:
-        if pipeline > 1:
-            return 1
-        return 3 if cache > 0 else 2
+        return 1 if pipeline > 1 else 3
     return int(graph)
 
 

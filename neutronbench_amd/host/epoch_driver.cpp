@@ -105,6 +105,7 @@ struct Args {
   uint32_t V = 0, F = 0, hidden = 128, batch = 1024, pipeline = 1, warmup = 2, max_batches = 0, heads = 0;
   double cache = 0.0;
   int graph = 1, verify = 0, stage_sync = 0;
+  int hw_queues = -1;  // -1: 8 for --pipeline 4, else the runtime's own count
 };
 
 Args parse(int argc, char **argv) {
@@ -124,6 +125,7 @@ Args parse(int argc, char **argv) {
     else if (k == "--graph") a.graph = std::stoi(v);
     else if (k == "--verify") a.verify = std::stoi(v);
     else if (k == "--stage-sync") a.stage_sync = std::stoi(v);
+    else if (k == "--hw-queues") a.hw_queues = std::stoi(v);
     else if (k == "--dump-dir") a.dump_dir = v;
     else if (k == "--dump-batch") a.dump_batch = static_cast<uint32_t>(std::stoul(v));
     else if (k == "--fanout") {
@@ -144,7 +146,7 @@ Args parse(int argc, char **argv) {
     fprintf(stderr,
             "usage: nts_epoch --dir D --V n --F n --fanout a,b[,c] [--batch n] [--hidden n] [--heads n] [--pipeline 1..8]\n"
             "                 [--cache fraction] [--graph 0|1|2|3] [--warmup n] [--max-batches n] [--verify 0|1] [--stage-sync 0|1]\n"
-            "                 [--dump-dir D [--dump-batch b]]\n");
+            "                 [--hw-queues n] [--dump-dir D [--dump-batch b]]\n");
     exit(2);
   }
   return a;
@@ -165,6 +167,18 @@ struct Slot {  // one batch in flight
 
 int main(int argc, char **argv) {
   const Args a = parse(argc, argv);
+  // Hardware queues of the process (the HIP runtime reads GPU_MAX_HW_QUEUES when it starts; its own count
+  // is 4).  With four batches in flight the loop below feeds four streams -- training, gather and two
+  // sampling chains -- beside the streams the library records its graphs on, and with four queues two of
+  // them share one: a gather then waits behind a whole sampling chain.  Measured with 6 to 16 queues
+  // against 4: four in flight 0.0226 -> 0.0174 s (Arxiv-shaped), 0.0255 -> 0.0212 s (Products-shaped),
+  // 0.0151 -> 0.0157 s (GAT); five and six in flight get slower with them (GAT 0.019 -> 0.026-0.035 s), two
+  // and three and the serial loop do not change.  So: 8 for --pipeline 4 unless --hw-queues says otherwise
+  // (0 = leave the environment alone).
+  {
+    const int queues = a.hw_queues >= 0 ? a.hw_queues : (a.pipeline == 4 ? 8 : 0);
+    if (queues > 0) setenv("GPU_MAX_HW_QUEUES", std::to_string(queues).c_str(), 1);
+  }
   const uint32_t hops = static_cast<uint32_t>(a.fanout.size());
   const uint32_t V = a.V, F = a.F;
   std::vector<uint32_t> co = read_file<uint32_t>(a.dir + "/co.bin", static_cast<size_t>(V) + 1);

@@ -5,10 +5,10 @@ from neutronbench_amd import epoch
 def test_graph_mode_picked_by_batches_in_flight_and_feature_cache():
     """nts_batch_builder_use_graph value of the epoch loops: an explicit value is passed through; True
     picks the one recorded chain with several batches in flight, and with one batch in flight the
-    second graph beside the gather when most rows come from the HBM cache, else the side branch."""
+    second graph beside the gather."""
     assert epoch.graph_mode(True, 1, 0.2) == 3
-    assert epoch.graph_mode(True, 1, 0.0) == 2
-    assert epoch.graph_mode(True, 1) == 2
+    assert epoch.graph_mode(True, 1, 0.0) == 3
+    assert epoch.graph_mode(True, 1) == 3
     for p in (2, 3, 4, 6):
         assert epoch.graph_mode(True, p, 0.2) == 1
         assert epoch.graph_mode(True, p, 0.0) == 1
