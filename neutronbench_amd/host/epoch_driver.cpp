@@ -20,6 +20,10 @@
 // chain of hops on a stream of its own, the next batch's features and labels are gathered on a gather
 // stream, the current one is aggregated; events order a batch's gather before its aggregation and
 // an arena's re-use after the aggregation that read it.  One host thread enqueues all of it.
+// --graph g: how the builders replay their launches (nts_batch_builder_use_graph; with 3 the
+// transposed structure is built beside the feature gather and joined before the first aggregation).
+// --hw-queues n: hardware queues asked of the HIP runtime before it starts (default: 8 with
+// --pipeline 4, see main()).
 //
 // The program reads raw arrays written by neutronbench_amd/epoch.py (--native): co.bin, ri.bin (uint32
 // CSC of the whole graph), feat.bin (float32 [V, F]), labels.bin (int64 [V]), train.bin (uint32 ids),
