@@ -541,3 +541,41 @@ def test_long_rows_of_narrow_messages_are_the_edge_order_sum(device, F):
     acc = dev(init, device)
     call("nts_gather_edge_to_dst", ptr(acc), ptr(dmsg), ptr(dro), Vs, F, 1, s)
     assert np.array_equal(acc.cpu().numpy()[chains], (ident + init)[chains])  # empty rows keep their contents
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_edge_sums_to_destinations_random_shapes(device, seed):
+    """nts_gather_edge_to_dst on seeded random shapes -- 4,096 to 30,000 rows, empty stretches at both
+    ends, rows up to and just beyond 1,024 edges, now and then a row beyond 16,384, widths from 1 to 256
+    floats, with and without accumulation: rows of at most 1,024 edges equal the running fp32 sum in
+    edge order bit for bit (whichever kernel takes them: streamed, lane groups, whole wavefronts), longer
+    ones within rounding."""
+    rng = np.random.default_rng(9000 + seed)
+    rows = int(rng.integers(4096, 30000))
+    deg = rng.integers(0, [4, 12, 40, 3][seed % 4], rows)
+    n_mid = int(rng.integers(1, 30))
+    deg[rng.integers(0, rows, n_mid)] = rng.integers(60, 1025, n_mid)
+    deg[rng.integers(0, rows, 3)] = [1024, 1025, int(rng.integers(1026, 6000))]
+    if seed % 3 == 0:
+        deg[rng.integers(0, rows)] = int(rng.integers(16385, 40000))
+    deg[:int(rng.integers(1, 200))] = 0
+    deg[-int(rng.integers(1, 200)):] = 0
+    F = [1, 4, 5, 12, 32, 33, 100, 256][seed]
+    off = np.concatenate([[0], np.cumsum(deg)]).astype(np.uint32)
+    E = int(off[-1])
+    msg = rng.standard_normal((E, F)).astype(np.float32)
+    init = rng.standard_normal((rows, F)).astype(np.float32)
+    accumulate = seed & 1
+    print(f"rows {rows} E {E} F {F} accumulate {accumulate} longest {int(deg.max())}", flush=True)
+    out = dev(init, device) if accumulate else torch.full((rows, F), float("nan"), device=device)
+    d_msg, d_off = dev(msg, device), dev(off, device)  # named: a temporary would be freed, and reused, before the launch
+    call("nts_gather_edge_to_dst", ptr(out), ptr(d_msg), ptr(d_off), rows, F, accumulate, stream())
+    got = out.cpu().numpy()
+    want = np.zeros((rows, F), np.float32)
+    for r in np.flatnonzero(deg):
+        want[r] = np.cumsum(msg[off[r]:off[r + 1]], axis=0, dtype=np.float32)[-1]
+    if accumulate:
+        want = want + init
+    ordered = deg <= 1024
+    assert np.array_equal(got[ordered].view(np.uint32), want[ordered].view(np.uint32))
+    np.testing.assert_allclose(got[~ordered], want[~ordered], rtol=2e-4, atol=2e-3)
