@@ -362,7 +362,7 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
                                                          uint32_t row_edge_limit,
                                                          const uint32_t *__restrict__ edge_ids) {
   using V = typename Vec<VEC>::type;
-  constexpr int U = 4;
+  constexpr int U = G >= 8 ? 8 : 4;  // edges per step: their rows are requested together
   const uint32_t gl = threadIdx.x & (G - 1);
   const uint32_t item = (blockIdx.x * blockDim.x + threadIdx.x) / G;
   if (item >= n_items) return;  // whole groups leave together; shuffles stay inside a group
@@ -448,6 +448,30 @@ __global__ __launch_bounds__(256) void spmm_group_kernel(const float *__restrict
       for (int u = 0; u < U; ++u) {
         vfma(acc, v[u], wv[u]);
       }
+    }
+    if (!RUNS && j < n) {
+      // The last, partial step: its rows are requested together like a full step's (a sampled layer's
+      // rows are a step or two long; one edge after the other, each waited for, doubled their time),
+      // and added in the same order.
+      const uint32_t left = n - j;
+      V v[U];
+      float wv[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t si = __shfl(my_i, (j + u) & (G - 1), G);
+        const uint32_t ss = __shfl(my_s, (j + u) & (G - 1), G);
+        v[u] = vzero<VEC>();
+        wv[u] = 0.f;
+        if (static_cast<uint32_t>(u) < left) {
+          v[u] = *reinterpret_cast<const V *>(in + static_cast<size_t>(si) * F + lcol);
+          wv[u] = HEADS ? w[static_cast<size_t>(ss) * heads.H + head] : __uint_as_float(ss);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (static_cast<uint32_t>(u) < left) vfma(acc, v[u], wv[u]);
+      }
+      j = n;
     }
     for (; j < n; ++j) {
       const uint32_t si = __shfl(my_i, j, G);
