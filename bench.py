@@ -624,6 +624,8 @@ def run_epochs(torch, names, with_cpu, cpu_batches):
                 # transpositions on a side branch of its graph, 3 = as a second graph beside the feature gather
                 # (sample time is then the sampling alone); the pipelined run: 1 = one chain
                 "hop_graph_mode": serial.get("hop_graph_mode"), "pipelined_hop_graph_mode": piped.get("hop_graph_mode"),
+                # the program asks the HIP runtime for eight hardware queues when four batches are in flight
+                "pipelined_hw_queues": 8 if piped["pipeline"] == 4 else None,
                 "check": check, "cpu_baseline": cpu,
             }
     finally:
